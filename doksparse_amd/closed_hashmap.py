@@ -1,0 +1,581 @@
+"""Batched GPU hashmap with the Python surface of the reference's ``CudaClosedHashmap``
+(reference: sparse_dok/components/cuda_closed_hashmap.py:20-477), backed by libdokhip.
+
+What differs underneath (and why callers do not see it):
+
+* Storage is one array of 128-byte buckets (see ``csrc/dok_packed8.h`` / ``csrc/dok_tagged.h``)
+  instead of the reference's three arrays ``_uuid/_keys/_values``.  ``n_buckets`` keeps the
+  reference meaning - the number of key slots asked for - and the physical table has at least
+  that many slots.
+* Key identity is the key row's bytes, not a 63-bit hash of it, so two keys are never confused.
+* ``n_elements`` is maintained by the kernels themselves (fresh inserts are counted where the
+  slot is claimed), which replaces the reference's "get, unique, count" pre-pass in ``set``.
+  The rehash rule is the reference's: grow to ``int((n + n_new) * rehash_factor)`` when
+  ``n + n_new > int(rehash_threshold * n_buckets)``.
+* The hash-constant keyword arguments are accepted and kept for ``get_hash`` / ``get_uuid`` /
+  ``test_uniformity``; slot placement uses the library's own hash.
+* ``coord_dims`` (not in the reference) makes the map coordinate-keyed: key rows are int64
+  coordinates inside ``coord_dims`` and are stored as one linearised 8-byte key.  This is how
+  ``SparseDOKTensor`` uses the map.
+"""
+import ctypes
+import math
+
+import numpy as np
+import torch
+from torch import Tensor
+
+from . import _lib
+from ._lib import DokTable, DOK_BUCKET_BYTES, DOK_HEADER_WORDS, DOK_MAX_DIMS
+
+
+def _stream_ptr(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _next_prime(n):
+    """Smallest prime > n (deterministic Miller-Rabin, exact below 3.3e24)."""
+    def is_prime(m):
+        if m < 2:
+            return False
+        small = (2, 3, 5, 7, 11, 13, 17, 19, 23, 29, 31, 37)
+        for p in small:
+            if m % p == 0:
+                return m == p
+        d, r = m - 1, 0
+        while d % 2 == 0:
+            d //= 2
+            r += 1
+        for a in small:
+            x = pow(a, d, m)
+            if x in (1, m - 1):
+                continue
+            for _ in range(r - 1):
+                x = x * x % m
+                if x == m - 1:
+                    break
+            else:
+                return False
+        return True
+    m = int(n) + 1
+    while not is_prime(m):
+        m += 1
+    return m
+
+
+class CudaClosedHashmap:
+    def __init__(
+        self,
+        n_buckets=1024,
+        device="cuda:0",
+        prime1=None,
+        prime2=None,
+        alpha1=None,
+        alpha2=None,
+        beta1=None,
+        beta2=None,
+        key_size=None,
+        key_perm=None,
+        rehash_factor=2.0,
+        rehash_threshold=0.75,
+        coord_dims=None,
+        seed=None,
+    ):
+        self._empty_marker = -1
+        self._removed_marker = -3
+        self._n_buckets = int(n_buckets)
+        self.device = torch.device(device)
+        self._key_size = key_size
+        self._prime1, self._prime2 = prime1, prime2
+        self._alpha1, self._alpha2 = alpha1, alpha2
+        self._beta1, self._beta2 = beta1, beta2
+        self._rehash_factor = rehash_factor
+        self._rehash_threshold = rehash_threshold
+        self._key_perm = None
+        if key_perm is not None:
+            if not isinstance(key_perm, Tensor):
+                key_perm = torch.tensor(key_perm, dtype=torch.long, device=self.device)
+            self._key_perm = key_perm.to(device=self.device, dtype=torch.long)
+        self._coord_dims = None if coord_dims is None else tuple(int(d) for d in coord_dims)
+        self._seed = int(seed) if seed is not None else int(np.random.randint(1, 2**62, dtype=np.int64))
+
+        # physical state; the table itself is allocated at the first set(), when the key and
+        # value widths are known (the reference allocates _keys/_values there too)
+        self._header = torch.zeros(DOK_HEADER_WORDS, device=self.device, dtype=torch.long)
+        self._table = None
+        self._desc = None
+        self._n_phys = 0
+        self._slots_per_bucket = 0
+        self._layout = 0
+        self._key_shape = None
+        self._key_dtype = None
+        self._value_shape = None
+        self._value_dtype = None
+        self._key_bytes = 0
+        self._value_bytes = 0
+        # host-side upper bound of n_elements; lets set() skip the device read-back
+        self._n_upper = 0
+
+    # ------------------------------------------------------------------ physical table
+    @property
+    def _allocated(self):
+        return self._table is not None
+
+    def _make_desc(self, table, header, n_phys):
+        d = DokTable()
+        d.buckets = table.data_ptr()
+        d.header = header.data_ptr()
+        d.n_phys_buckets = n_phys
+        d.seed = self._seed
+        d.key_bytes = 8 if self._coord_dims is not None else self._key_bytes
+        d.value_bytes = self._value_bytes
+        if self._coord_dims is not None:
+            d.lin_ndim = len(self._coord_dims)
+            for i, s in enumerate(self._coord_dims):
+                d.lin_dims[i] = s
+        else:
+            d.lin_ndim = 0
+        return d
+
+    def _alloc_table(self, n_buckets):
+        lib = _lib.load()
+        kb = 8 if self._coord_dims is not None else self._key_bytes
+        slots = ctypes.c_int32(0)
+        layout = lib.dok_layout_of(kb, self._value_bytes, ctypes.byref(slots))
+        _lib.check(min(layout, 0), "CudaClosedHashmap")
+        n_phys = int(lib.dok_phys_buckets_for(max(int(n_buckets), 1), kb, self._value_bytes))
+        assert 1 <= n_phys < 2**32, "table too large"
+        table = torch.empty(n_phys * DOK_BUCKET_BYTES, device=self.device, dtype=torch.uint8)
+        assert table.data_ptr() % DOK_BUCKET_BYTES == 0
+        header = torch.empty(DOK_HEADER_WORDS, device=self.device, dtype=torch.long)
+        desc = self._make_desc(table, header, n_phys)
+        _lib.check(lib.dok_table_clear(ctypes.byref(desc), _stream_ptr(self.device)), "clear")
+        return table, header, desc, n_phys, int(slots.value), int(layout)
+
+    def _init_storage(self, keys, values):
+        self._key_shape = tuple(keys.shape[1:])
+        self._key_dtype = keys.dtype
+        self._value_shape = tuple(values.shape[1:])
+        self._value_dtype = values.dtype
+        self._key_bytes = int(np.prod(self._key_shape, dtype=np.int64)) * keys.element_size()
+        self._value_bytes = int(np.prod(self._value_shape, dtype=np.int64)) * values.element_size()
+        if self._coord_dims is not None:
+            assert keys.dtype == torch.long and self._key_shape == (len(self._coord_dims),), \
+                "a coordinate-keyed map takes int64 key rows of one coordinate per dimension"
+        (self._table, self._header, self._desc, self._n_phys,
+         self._slots_per_bucket, self._layout) = self._alloc_table(self._n_buckets)
+        self._n_upper = 0
+
+    def _read_header(self):
+        h = self._header.cpu()
+        n_full = int(h[_lib.DOK_H_NFULL])
+        if n_full:
+            raise RuntimeError(f"hashmap is full: {n_full} rows could not be stored")
+        return h
+
+    # ------------------------------------------------------------------ reference-compatible state
+    @property
+    def _n_elements(self):
+        """0-dim int64 device tensor, as in the reference (a view of the table header)."""
+        return self._header[_lib.DOK_H_NELEM]
+
+    @property
+    def n_elements(self):
+        n = int(self._read_header()[_lib.DOK_H_NELEM])
+        self._n_upper = n
+        return n
+
+    @property
+    def n_buckets(self):
+        return self._n_buckets
+
+    @property
+    def load_factor(self):
+        return self.n_elements / self.n_buckets
+
+    @property
+    def key_shape(self):
+        assert self._allocated
+        return torch.Size(self._key_shape)
+
+    @property
+    def value_shape(self):
+        assert self._allocated
+        return torch.Size(self._value_shape)
+
+    @property
+    def key_type(self):
+        return self._key_dtype
+
+    @property
+    def value_type(self):
+        return self._value_dtype
+
+    def __len__(self):
+        return self.n_elements
+
+    # raw-table attributes of the reference.  The physical layout is different, so these are
+    # materialised on demand from the live entries; None means "nothing stored yet", which is
+    # the only thing the reference's own callers test them for.
+    @property
+    def _keys(self):
+        return None if not self._allocated else self.keys().reshape(-1, *self._key_shape)
+
+    @property
+    def _values(self):
+        return None if not self._allocated else self.values()
+
+    @property
+    def _uuid(self):
+        if not self._allocated:
+            return torch.full((self._n_buckets,), self._empty_marker, device=self.device, dtype=torch.long)
+        return self.get_uuid(self.keys().reshape(-1, *self._key_shape))
+
+    def uuid(self):
+        return self._uuid
+
+    @property
+    def nonempty_mask(self):
+        n = 0 if not self._allocated else self.n_elements
+        return torch.ones(n, device=self.device, dtype=torch.bool)
+
+    # ------------------------------------------------------------------ hash constants (compat)
+    def _flat_key_size(self):
+        assert self._allocated or self._key_size is not None
+        if self._allocated:
+            return int(np.prod(self._key_shape, dtype=np.int64))
+        return int(self._key_size)
+
+    def _draw(self, bounds):
+        return torch.tensor([int(np.random.randint(int(b))) - 1 for b in bounds], device=self.device)
+
+    @property
+    def prime1(self):
+        if self._prime1 is None:
+            ks = self._flat_key_size()
+            draws = [np.random.randint(self.n_buckets, self.n_buckets * 2) for _ in range(ks)]
+            self._prime1 = torch.tensor([_next_prime(int(i)) for i in draws], device=self.device)
+        return self._prime1
+
+    @property
+    def prime2(self):
+        if self._prime2 is None:
+            ks = self._flat_key_size()
+            draws = [np.random.randint(0, 2**60, dtype="int64") for _ in range(ks)]
+            self._prime2 = torch.tensor([_next_prime(int(i)) for i in draws], device=self.device)
+        return self._prime2
+
+    @property
+    def alpha1(self):
+        if self._alpha1 is None:
+            self._alpha1 = self._draw(self.prime1.cpu())
+        return self._alpha1
+
+    @property
+    def alpha2(self):
+        if self._alpha2 is None:
+            self._alpha2 = self._draw(self.prime1.cpu())
+        return self._alpha2
+
+    @property
+    def beta1(self):
+        if self._beta1 is None:
+            self._beta1 = self._draw(self.prime1.cpu())
+        return self._beta1
+
+    @property
+    def beta2(self):
+        if self._beta2 is None:
+            self._beta2 = self._draw(self.prime1.cpu())
+        return self._beta2
+
+    @property
+    def key_perm(self):
+        if self._key_perm is None:
+            assert self._allocated
+            self._key_perm = torch.arange(int(np.prod(self._key_shape, dtype=np.int64)), device=self.device)
+        else:
+            assert self._key_perm.shape[0] == int(np.prod(self._key_shape, dtype=np.int64))
+        return self._key_perm
+
+    @staticmethod
+    def _hash_words(keys):
+        n = keys.shape[0]
+        keys = keys.reshape(n, -1).clone()
+        if keys.dtype == torch.float:
+            keys = keys.view(dtype=torch.int32).long()
+            keys[keys == -2**31] = 0
+        elif keys.dtype == torch.half:
+            keys = keys.view(dtype=torch.int16).long()
+            keys[keys == -2**15] = 0
+        elif keys.dtype == torch.double:
+            keys = keys.view(dtype=torch.int64)
+            keys[keys == -2**63] = 0
+        else:
+            keys = keys.to(torch.long)
+        return keys
+
+    def get_hash(self, keys):
+        """The reference's bucket hash of each key row (cuda_closed_hashmap.py:278-300)."""
+        w = self._hash_words(keys)
+        t = (self.alpha1[None] * w + self.beta1[None]) % self.prime1[None]
+        if self._key_perm is not None:
+            t = t[:, self._key_perm]
+        return t.prod(dim=-1).abs() % self.n_buckets
+
+    def get_uuid(self, keys):
+        """The reference's 63-bit identity hash of each key row (cuda_closed_hashmap.py:302-319)."""
+        w = self._hash_words(keys)
+        return ((self.alpha2[None] * w + self.beta2[None]) % self.prime2[None]).prod(dim=-1).abs()
+
+    def test_uniformity(self, keys):
+        codes = self.get_hash(keys)
+        logits = (torch.bincount(codes, minlength=self.n_buckets) + 1).log()
+        logp = torch.log_softmax(logits, dim=-1)
+        return (-(logp * logp.exp()).sum(dim=-1)).exp() / self.n_buckets
+
+    # ------------------------------------------------------------------ batch preparation
+    def _prep_rows(self, t, what):
+        t = t.contiguous()
+        if t.numel() and t.data_ptr() % 8 != 0:
+            t = t.clone()
+        return t
+
+    def _check_keys(self, keys):
+        assert keys.dtype == self._key_dtype
+        assert keys.device == self.device
+        assert tuple(keys.shape[1:]) == self._key_shape
+
+    # ------------------------------------------------------------------ set / get / remove
+    def _launch_set(self, keys, values):
+        lib = _lib.load()
+        _lib.check(lib.dok_map_set(ctypes.byref(self._desc), keys.data_ptr(), values.data_ptr(),
+                                   keys.shape[0], None, _stream_ptr(self.device)), "set")
+
+    def _physical_slots(self):
+        return self._n_phys * self._slots_per_bucket
+
+    def set(self, new_keys, new_values):
+        """Upsert a batch (reference: cuda_closed_hashmap.py:321-384).  Returns None."""
+        assert new_keys.shape[0] == new_values.shape[0]
+        if not self._allocated:
+            assert new_keys.device == new_values.device == self.device
+            self._init_storage(new_keys, new_values)
+        else:
+            self._check_keys(new_keys)
+            assert new_values.dtype == self._value_dtype
+            assert new_values.device == self.device
+            assert tuple(new_values.shape[1:]) == self._value_shape
+        n = new_keys.shape[0]
+        if n == 0:
+            return
+        keys = self._prep_rows(new_keys, "keys")
+        values = self._prep_rows(new_values, "values")
+
+        limit = int(self._rehash_threshold * self._n_buckets)
+        if self._n_upper + n <= limit:
+            # cannot cross the threshold whatever the batch holds: no read-back, no sync
+            self._launch_set(keys, values)
+            self._n_upper += n
+            return
+        n_old = self.n_elements
+        if n_old + n <= limit:
+            self._launch_set(keys, values)
+            self._n_upper = n_old + n
+            return
+        if n_old + n <= int(0.9 * self._physical_slots()):
+            # the batch fits physically: insert, then apply the reference's growth rule to the
+            # count the kernel produced (same final size and contents as growing first)
+            self._launch_set(keys, values)
+            n_now = self.n_elements
+            if n_now > limit:
+                self.rehash(int(n_now * self._rehash_factor))
+            return
+        # the batch may not fit: count its distinct new keys first, as the reference does
+        _, is_found = self.get(keys)
+        n_new = int(keys[~is_found].unique(dim=0).shape[0])
+        if n_old + n_new > limit:
+            self.rehash(int((n_old + n_new) * self._rehash_factor))
+        self._launch_set(keys, values)
+        self._n_upper = n_old + n_new
+
+    def get(self, keys, fallback_value=None):
+        """(values, is_found) for a batch of keys (reference: cuda_closed_hashmap.py:386-421)."""
+        if not self._allocated:
+            raise RuntimeError("store something first")
+        if keys.shape[0] == 0:
+            return (torch.empty(0, *self._value_shape, device=self.device, dtype=self._value_dtype),
+                    torch.empty(0, device=self.device, dtype=torch.bool))
+        self._check_keys(keys)
+        fb = None
+        if fallback_value is not None:
+            if not isinstance(fallback_value, Tensor):
+                fallback_value = torch.tensor(fallback_value, device=self.device, dtype=self._value_dtype)
+            assert fallback_value.dtype == self._value_dtype
+            row = torch.empty(self._value_shape, dtype=self._value_dtype)
+            row.copy_(torch.broadcast_to(fallback_value.cpu(), self._value_shape))
+            fb = row.reshape(-1).view(torch.uint8).numpy().tobytes()
+        keys = self._prep_rows(keys, "keys")
+        n = keys.shape[0]
+        values = torch.empty(n, *self._value_shape, device=self.device, dtype=self._value_dtype)
+        is_found = torch.empty(n, device=self.device, dtype=torch.bool)
+        lib = _lib.load()
+        _lib.check(lib.dok_map_get(ctypes.byref(self._desc), keys.data_ptr(), n, values.data_ptr(),
+                                   fb, is_found.data_ptr(), _stream_ptr(self.device)), "get")
+        return values, is_found
+
+    def remove(self, keys):
+        """Remove a batch of keys; returns the mask over ``keys.unique(dim=0)``
+        (reference: cuda_closed_hashmap.py:423-454)."""
+        if not self._allocated:
+            raise RuntimeError("store something first")
+        if keys.shape[0] == 0:
+            return torch.zeros(0, device=keys.device, dtype=torch.bool)
+        self._check_keys(keys)
+        unique_keys = self._prep_rows(keys.unique(dim=0), "keys")
+        return self._remove_rows(unique_keys)
+
+    def _remove_rows(self, keys):
+        """Remove without the sort: mask aligned with ``keys`` (equal rows: one reports True)."""
+        n = keys.shape[0]
+        is_removed = torch.empty(n, device=self.device, dtype=torch.bool)
+        lib = _lib.load()
+        _lib.check(lib.dok_map_remove(ctypes.byref(self._desc), keys.data_ptr(), n,
+                                      is_removed.data_ptr(), _stream_ptr(self.device)), "remove")
+        return is_removed
+
+    def count_existing(self, keys):
+        """How many rows of ``keys`` are present (device int64 scalar)."""
+        if not self._allocated:
+            raise RuntimeError("store something first")
+        self._check_keys(keys)
+        keys = self._prep_rows(keys, "keys")
+        count = torch.zeros((), device=self.device, dtype=torch.long)
+        lib = _lib.load()
+        _lib.check(lib.dok_map_count_existing(ctypes.byref(self._desc), keys.data_ptr(), keys.shape[0],
+                                              count.data_ptr(), _stream_ptr(self.device)), "count")
+        return count
+
+    # ------------------------------------------------------------------ read-out
+    def _compact(self, want_keys, want_values):
+        lib = _lib.load()
+        scratch_bytes = int(lib.dok_compact_scratch_bytes(ctypes.byref(self._desc)))
+        scratch = torch.empty(scratch_bytes // 8, device=self.device, dtype=torch.long)
+        count = torch.zeros(1, device=self.device, dtype=torch.long)
+        stream = _stream_ptr(self.device)
+        # pass 1: count only, to size the outputs
+        _lib.check(lib.dok_map_compact(ctypes.byref(self._desc), None, None, 0, count.data_ptr(),
+                                       scratch.data_ptr(), stream), "compact")
+        n = int(count.item())
+        keys = values = None
+        if want_keys:
+            keys = torch.empty(n, *self._key_shape, device=self.device, dtype=self._key_dtype)
+        if want_values:
+            values = torch.empty(n, *self._value_shape, device=self.device, dtype=self._value_dtype)
+        if n:
+            _lib.check(lib.dok_map_compact(
+                ctypes.byref(self._desc),
+                keys.data_ptr() if keys is not None else None,
+                values.data_ptr() if values is not None else None,
+                n, count.data_ptr(), scratch.data_ptr(), stream), "compact")
+        return keys, values
+
+    def keys(self):
+        """Live key rows, [n, prod(key_shape)], in slot order (reference: :161-166)."""
+        if not self._allocated:
+            return None
+        keys, _ = self._compact(True, False)
+        return keys.reshape(keys.shape[0], -1)
+
+    def values(self):
+        """Live value rows in the same order as ``keys()`` (reference: :168-172)."""
+        if not self._allocated:
+            return None
+        _, values = self._compact(False, True)
+        return values
+
+    def items(self):
+        """(keys, values) from one pass."""
+        if not self._allocated:
+            return None, None
+        keys, values = self._compact(True, True)
+        return keys.reshape(keys.shape[0], -1), values
+
+    def set_values(self, selectors, new_values):
+        """Overwrite values of live entries picked by position in ``values()`` order (:174-177)."""
+        keys, values = self.items()
+        values[selectors] = new_values
+        self._launch_set(self._prep_rows(keys.reshape(-1, *self._key_shape), "keys"), values.contiguous())
+
+    # ------------------------------------------------------------------ rehash / clone
+    def rehash(self, n_buckets):
+        """Move every entry into a fresh table of ``n_buckets`` slots (reference: :456-468)."""
+        n_buckets = int(n_buckets)
+        if not self._allocated:
+            self._n_buckets = n_buckets
+            return
+        lib = _lib.load()
+        old = (self._table, self._header, self._desc)
+        self._seed = int(np.random.randint(1, 2**62, dtype=np.int64))
+        table, header, desc, n_phys, slots, layout = self._alloc_table(n_buckets)
+        if layout == _lib.DOK_LAYOUT_PACKED8:
+            _lib.check(lib.dok_map_rehash(ctypes.byref(old[2]), ctypes.byref(desc), _stream_ptr(self.device)), "rehash")
+            self._table, self._header, self._desc, self._n_phys = table, header, desc, n_phys
+            self._n_buckets = n_buckets
+        else:
+            keys, values = self.items()
+            self._table, self._header, self._desc, self._n_phys = table, header, desc, n_phys
+            self._n_buckets = n_buckets
+            if keys.shape[0]:
+                self._launch_set(self._prep_rows(keys.reshape(-1, *self._key_shape), "keys"), values.contiguous())
+        # the old table tensors stay referenced by `old` until the copies above are enqueued;
+        # torch's allocator orders their reuse on the same stream
+        del old
+
+    def clone(self, deepclone=False):
+        """Shallow clone shares the table; deep clone copies it (reference: :193-231)."""
+        new = CudaClosedHashmap(
+            n_buckets=self._n_buckets, device=self.device,
+            prime1=self._prime1, prime2=self._prime2, alpha1=self._alpha1, alpha2=self._alpha2,
+            beta1=self._beta1, beta2=self._beta2, key_perm=self._key_perm,
+            rehash_factor=self._rehash_factor, rehash_threshold=self._rehash_threshold,
+            coord_dims=self._coord_dims, seed=self._seed,
+        )
+        for name in ("_key_shape", "_key_dtype", "_value_shape", "_value_dtype", "_key_bytes",
+                     "_value_bytes", "_n_phys", "_slots_per_bucket", "_layout", "_n_upper"):
+            setattr(new, name, getattr(self, name))
+        if self._allocated:
+            if deepclone:
+                new._table = self._table.clone()
+                new._header = self._header.clone()
+            else:
+                new._table = self._table
+                new._header = self._header
+            new._desc = new._make_desc(new._table, new._header, new._n_phys)
+        return new
+
+    # ------------------------------------------------------------------ probe statistics
+    def probe_stats(self, keys):
+        """Mean number of buckets a lookup of each of ``keys`` visits."""
+        self._check_keys(keys)
+        keys = self._prep_rows(keys, "keys")
+        n = keys.shape[0]
+        values = torch.empty(n, *self._value_shape, device=self.device, dtype=self._value_dtype)
+        is_found = torch.empty(n, device=self.device, dtype=torch.bool)
+        before = self._header.cpu()
+        lib = _lib.load()
+        _lib.check(lib.dok_map_get_stats(ctypes.byref(self._desc), keys.data_ptr(), n, values.data_ptr(),
+                                         None, is_found.data_ptr(), _stream_ptr(self.device)), "get_stats")
+        after = self._header.cpu()
+        probes = int(after[_lib.DOK_H_NPROBE] - before[_lib.DOK_H_NPROBE])
+        ops = int(after[_lib.DOK_H_NOPS] - before[_lib.DOK_H_NOPS])
+        return probes / max(ops, 1)
+
+    def __getitem__(self, keys):
+        return self.get(keys)
+
+    def __setitem__(self, keys, values):
+        return self.set(keys, values)
+
+    def __delitem__(self, keys):
+        return self.remove(keys)

@@ -1,0 +1,211 @@
+// Device-side building blocks shared by every kernel of libdokhip: integer types, the key
+// hash, wave64 helpers and the kernel-argument form of a table.
+//
+// Execution model used throughout: one workgroup = 256 threads = 4 wave64s.  Each lane
+// "owns" one batch row (its key, its result).  A 128-byte bucket is probed by a *group* of 16
+// adjacent lanes, each lane loading one 8-byte word, so a wave inspects four buckets per
+// load instruction and a bucket costs exactly one 128-byte line.  The group works through
+// the rows its 16 lanes own one at a time; the row being served is broadcast with a lane
+// shuffle, matches are found with a wave ballot, and the owning lane takes the result.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/dokhip.h"
+
+typedef unsigned long long u64;
+typedef long long i64;
+typedef unsigned int u32;
+typedef unsigned short u16;
+typedef unsigned char u8;
+
+#define DOK_TPB 256          // threads per workgroup
+#define DOK_NONE32 0xffffffffu
+
+// Kernel-argument copy of dok_table_t plus what the host precomputes from it.
+struct DevTable {
+  u64 *buckets;
+  i64 *header;
+  u64 nb;                    // physical buckets
+  u64 seed;
+  int key_bytes;
+  int value_bytes;
+  int lin_ndim;
+  int pad_;
+  i64 lin_dims[DOK_MAX_DIMS];
+  i64 lin_strides[DOK_MAX_DIMS];   // row-major strides of lin_dims
+};
+
+// Kernel-argument form of dok_index_t (+ optional source-value view).
+struct DevIndex {
+  int ndim;
+  int sel_ndim;
+  i64 n_elems;
+  i64 shape[DOK_MAX_DIMS];
+  i64 estride[DOK_MAX_DIMS];       // C-contiguous strides of `shape`
+  const i64 *sel[DOK_MAX_DIMS];
+  i64 sstride[DOK_MAX_DIMS][DOK_MAX_DIMS];
+  const void *src;
+  i64 vstride[DOK_MAX_DIMS];
+};
+
+__device__ __forceinline__ u64 dok_fmix64(u64 x) {
+  x ^= x >> 33; x *= 0xff51afd7ed558ccdULL;
+  x ^= x >> 33; x *= 0xc4ceb9fe1a85ec53ULL;
+  x ^= x >> 33;
+  return x;
+}
+
+// Multiply-high range reduction: maps a 64-bit hash uniformly onto [0, nb) without division.
+__device__ __forceinline__ u32 dok_reduce(u64 h, u64 nb) { return (u32)__umul64hi(h, nb); }
+
+__device__ __forceinline__ u64 dok_ballot(bool p) { return __ballot(p); }
+
+__device__ __forceinline__ u64 dok_shfl64(u64 v, int src) { return __shfl(v, src, 64); }
+__device__ __forceinline__ u32 dok_shfl32(u32 v, int src) { return __shfl(v, src, 64); }
+
+// Loads that must observe what other workgroups (possibly on another XCD, behind another L2)
+// wrote earlier in the same kernel.
+__device__ __forceinline__ u64 dok_load_coherent(const u64 *p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void dok_store_coherent(u64 *p, u64 v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// One add per wave instead of one per lane.
+__device__ __forceinline__ void dok_wave_add(i64 *counter, bool flag, i64 sign = 1) {
+  u64 m = dok_ballot(flag);
+  if (m != 0 && (threadIdx.x & 63) == 0) atomicAdd((u64 *)counter, (u64)(sign * (i64)__popcll(m)));
+}
+__device__ __forceinline__ void dok_wave_add_n(i64 *counter, int v) {
+  // sum of a small per-lane non-negative int over the wave
+  #pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  if (v != 0 && (threadIdx.x & 63) == 0) atomicAdd((u64 *)counter, (u64)(i64)v);
+}
+
+// Zero `words` 8-byte words (a multiple of 4) and the table header.
+__global__ __launch_bounds__(DOK_TPB) void dok_fill_kernel(u64 *p, i64 words, i64 *header) {
+  const i64 i = ((i64)blockIdx.x * DOK_TPB + threadIdx.x) * 4;
+  if (i + 3 < words) {
+    ulonglong2 z; z.x = 0; z.y = 0;
+    ((ulonglong2 *)(p + i))[0] = z;
+    ((ulonglong2 *)(p + i))[1] = z;
+  }
+  if (blockIdx.x == 0 && threadIdx.x < DOK_HEADER_WORDS) header[threadIdx.x] = 0;
+}
+
+// Row-major linearisation of an int64 coordinate row; false if any coordinate is outside
+// [0, dim).  Negative coordinates are not wrapped (the reference does not wrap them either).
+__device__ __forceinline__ bool dok_linearise(const DevTable &t, const i64 *row, u64 &key) {
+  bool ok = true;
+  u64 k = 0;
+  for (int d = 0; d < t.lin_ndim; d++) {
+    i64 c = row[d];
+    ok = ok && ((u64)c < (u64)t.lin_dims[d]);
+    k += (u64)c * (u64)t.lin_strides[d];
+  }
+  key = k;
+  return ok;
+}
+
+// Key of batch row i as an 8-byte integer (packed layout): narrower keys are zero-extended.
+__device__ __forceinline__ bool dok_load_key8(const DevTable &t, const void *keys, i64 i, u64 &key) {
+  if (t.lin_ndim > 0) return dok_linearise(t, (const i64 *)keys + i * t.lin_ndim, key);
+  switch (t.key_bytes) {
+    case 8: key = ((const u64 *)keys)[i]; break;
+    case 4: key = ((const u32 *)keys)[i]; break;
+    case 2: key = ((const u16 *)keys)[i]; break;
+    default: key = ((const u8 *)keys)[i]; break;
+  }
+  return true;
+}
+
+__device__ __forceinline__ void dok_store_key8(const DevTable &t, void *keys_out, i64 i, u64 key) {
+  if (t.lin_ndim > 0) {
+    i64 *row = (i64 *)keys_out + i * t.lin_ndim;
+    u64 rem = key;
+    for (int d = 0; d < t.lin_ndim; d++) {
+      u64 s = (u64)t.lin_strides[d];
+      u64 c = rem / s;
+      rem -= c * s;
+      row[d] = (i64)c;
+    }
+    return;
+  }
+  switch (t.key_bytes) {
+    case 8: ((u64 *)keys_out)[i] = key; break;
+    case 4: ((u32 *)keys_out)[i] = (u32)key; break;
+    case 2: ((u16 *)keys_out)[i] = (u16)key; break;
+    default: ((u8 *)keys_out)[i] = (u8)key; break;
+  }
+}
+
+template <int V> struct ValT;
+template <> struct ValT<1> { typedef u8 type; };
+template <> struct ValT<2> { typedef u16 type; };
+template <> struct ValT<4> { typedef u32 type; };
+template <> struct ValT<8> { typedef u64 type; };
+
+template <int V> __device__ __forceinline__ u64 dok_load_val(const void *values, i64 i) {
+  return (u64)((const typename ValT<V>::type *)values)[i];
+}
+template <int V> __device__ __forceinline__ void dok_store_val(void *values, i64 i, u64 v) {
+  ((typename ValT<V>::type *)values)[i] = (typename ValT<V>::type)v;
+}
+
+// Coordinate of element e of the broadcast index space along every tensor dimension,
+// linearised.  Unravel e over `shape`, then read each selector through its strides
+// (stride 0 = broadcast axis).  `voff` receives the element offset into the source view.
+// Loops run to the compile-time maximum with uniform guards so that idx[] stays in registers;
+// the host zeroes the strides of unused axes.
+__device__ __forceinline__ bool dok_gather_key(const DevTable &t, const DevIndex &ix, i64 e,
+                                               u64 &key, i64 &voff) {
+  i64 idx[DOK_MAX_DIMS];
+  if (ix.n_elems <= 0x7fffffffLL) {
+    u32 rem = (u32)e;
+    #pragma unroll
+    for (int j = 0; j < DOK_MAX_DIMS; j++) {
+      idx[j] = 0;
+      if (j < ix.sel_ndim) {
+        u32 s = (u32)ix.estride[j];
+        u32 q = rem / s;
+        rem -= q * s;
+        idx[j] = q;
+      }
+    }
+  } else {
+    u64 rem = (u64)e;
+    #pragma unroll
+    for (int j = 0; j < DOK_MAX_DIMS; j++) {
+      idx[j] = 0;
+      if (j < ix.sel_ndim) {
+        u64 s = (u64)ix.estride[j];
+        u64 q = rem / s;
+        rem -= q * s;
+        idx[j] = (i64)q;
+      }
+    }
+  }
+  bool ok = true;
+  u64 k = 0;
+  #pragma unroll
+  for (int d = 0; d < DOK_MAX_DIMS; d++) {
+    if (d < ix.ndim) {
+      i64 off = 0;
+      #pragma unroll
+      for (int j = 0; j < DOK_MAX_DIMS; j++)
+        if (j < ix.sel_ndim) off += idx[j] * ix.sstride[d][j];
+      i64 c = ix.sel[d][off];
+      ok = ok && ((u64)c < (u64)t.lin_dims[d]);
+      k += (u64)c * (u64)t.lin_strides[d];
+    }
+  }
+  i64 vo = 0;
+  #pragma unroll
+  for (int j = 0; j < DOK_MAX_DIMS; j++)
+    if (j < ix.sel_ndim) vo += idx[j] * ix.vstride[j];
+  voff = vo;
+  key = k;
+  return ok;
+}

@@ -1,0 +1,359 @@
+// libdokhip: host side of the C ABI declared in include/dokhip.h.  Validates arguments,
+// turns the caller's descriptors into kernel-argument structs, picks the kernel instantiation
+// from the table's widths and enqueues it on the caller's stream.  Nothing here allocates
+// device memory or synchronises.
+#include <hip/hip_runtime.h>
+#include <string.h>
+#include "dok_device.h"
+#include "dok_packed8.h"
+#include "dok_tagged.h"
+
+namespace {
+
+thread_local char g_last_error[256] = "";
+
+int note_launch() {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    strncpy(g_last_error, hipGetErrorString(e), sizeof(g_last_error) - 1);
+    g_last_error[sizeof(g_last_error) - 1] = 0;
+    return DOK_ELAUNCH;
+  }
+  return DOK_OK;
+}
+
+bool is_pow2_le8(int v) { return v == 1 || v == 2 || v == 4 || v == 8; }
+
+int layout_of(int kb, int vb, int *slots) {
+  if (kb <= 0 || vb <= 0) return DOK_EUNSUPPORTED;
+  if (is_pow2_le8(kb) && is_pow2_le8(vb)) {
+    if (slots) *slots = 128 / (8 + vb);
+    return DOK_LAYOUT_PACKED8;
+  }
+  const int w = 1 + (kb + 7) / 8 + (vb + 7) / 8;
+  if (w > 16) return DOK_EUNSUPPORTED;
+  if (slots) *slots = 16 / w;
+  return DOK_LAYOUT_TAGGED;
+}
+
+// Validate a table descriptor and build its kernel-argument form.
+int make_dev_table(const dok_table_t *t, DevTable &d, int &layout) {
+  if (!t || !t->buckets || !t->header) return DOK_EINVAL;
+  if (t->n_phys_buckets < 1 || t->n_phys_buckets > 0xffffffffLL) return DOK_EINVAL;
+  if (((uintptr_t)t->buckets & 127) != 0 || ((uintptr_t)t->header & 7) != 0) return DOK_EINVAL;
+  if (t->lin_ndim < 0 || t->lin_ndim > DOK_MAX_DIMS) return DOK_EINVAL;
+  if (t->lin_ndim > 0 && t->key_bytes != 8) return DOK_EINVAL;
+  layout = layout_of(t->key_bytes, t->value_bytes, nullptr);
+  if (layout < 0) return layout;
+  if (t->lin_ndim > 0 && layout != DOK_LAYOUT_PACKED8) return DOK_EUNSUPPORTED;
+  memset(&d, 0, sizeof(d));
+  d.buckets = (u64 *)t->buckets;
+  d.header = (i64 *)t->header;
+  d.nb = (u64)t->n_phys_buckets;
+  d.seed = t->seed;
+  d.key_bytes = t->key_bytes;
+  d.value_bytes = t->value_bytes;
+  d.lin_ndim = t->lin_ndim;
+  if (t->lin_ndim > 0) {
+    // volume must fit in 63 bits so that a linear key never meets the reserved patterns
+    unsigned __int128 vol = 1;
+    for (int k = t->lin_ndim - 1; k >= 0; k--) {
+      if (t->lin_dims[k] < 0) return DOK_EINVAL;
+      d.lin_dims[k] = t->lin_dims[k];
+      d.lin_strides[k] = (i64)vol;
+      vol *= (unsigned __int128)(t->lin_dims[k] > 0 ? t->lin_dims[k] : 1);
+      if (vol >> 63) return DOK_EUNSUPPORTED;
+    }
+  }
+  return DOK_OK;
+}
+
+// Validate an index descriptor against the table; build its kernel-argument form.
+int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *src, DevIndex &d) {
+  if (!ix || t.lin_ndim == 0) return DOK_EINVAL;
+  if (ix->ndim != t.lin_ndim) return DOK_EINVAL;
+  if (ix->sel_ndim < 0 || ix->sel_ndim > DOK_MAX_DIMS) return DOK_EINVAL;
+  memset(&d, 0, sizeof(d));
+  d.ndim = ix->ndim;
+  d.sel_ndim = ix->sel_ndim;
+  unsigned __int128 n = 1;
+  for (int j = ix->sel_ndim - 1; j >= 0; j--) {
+    if (ix->shape[j] < 0) return DOK_EINVAL;
+    d.shape[j] = ix->shape[j];
+    d.estride[j] = n ? (i64)n : 1;          // never 0: it is a divisor in the unravel
+    n *= (unsigned __int128)ix->shape[j];
+    if (n >> 62) return DOK_EINVAL;
+  }
+  d.n_elems = (i64)n;
+  for (int k = 0; k < ix->ndim; k++) {
+    if (!ix->sel[k].data && d.n_elems > 0) return DOK_EINVAL;
+    d.sel[k] = (const i64 *)ix->sel[k].data;
+    for (int j = 0; j < ix->sel_ndim; j++) {
+      if (ix->sel[k].strides[j] < 0) return DOK_EINVAL;
+      d.sstride[k][j] = ix->sel[k].strides[j];
+    }
+  }
+  if (src) {
+    if (!src->data && d.n_elems > 0) return DOK_EINVAL;
+    d.src = src->data;
+    for (int j = 0; j < ix->sel_ndim; j++) {
+      if (src->strides[j] < 0) return DOK_EINVAL;
+      d.vstride[j] = src->strides[j];
+    }
+  }
+  return DOK_OK;
+}
+
+inline unsigned grid_for(i64 n) { return (unsigned)((n + DOK_TPB - 1) / DOK_TPB); }
+inline i64 chunks_of(const DevTable &d) { return ((i64)d.nb + DOK_CHUNK - 1) / DOK_CHUNK; }
+inline unsigned chunk_grid(i64 n_chunks) { return (unsigned)((n_chunks + 3) / 4); }
+
+u64 fallback_word(const void *fallback, int vb) {
+  u64 f = 0;
+  if (fallback) memcpy(&f, fallback, vb);
+  return f;
+}
+
+// Rows per launch are bounded so that the 32-bit grid dimension cannot overflow.
+const i64 kMaxRows = (i64)0x7fffffff * DOK_TPB;
+
+#define P8_DISPATCH(vb, CALL)        \
+  switch (vb) {                      \
+    case 1: { constexpr int V = 1; CALL; } break; \
+    case 2: { constexpr int V = 2; CALL; } break; \
+    case 4: { constexpr int V = 4; CALL; } break; \
+    default: { constexpr int V = 8; CALL; } break; \
+  }
+
+}  // namespace
+
+extern "C" {
+
+int dok_layout_of(int32_t key_bytes, int32_t value_bytes, int32_t *slots_per_bucket) {
+  return layout_of(key_bytes, value_bytes, slots_per_bucket);
+}
+
+int64_t dok_phys_buckets_for(int64_t capacity, int32_t key_bytes, int32_t value_bytes) {
+  int slots = 0;
+  const int lay = layout_of(key_bytes, value_bytes, &slots);
+  if (lay < 0) return lay;
+  if (capacity < 1) capacity = 1;
+  return (capacity + slots - 1) / slots;
+}
+
+const char *dok_last_hip_error(void) { return g_last_error; }
+
+int dok_table_clear(const dok_table_t *t, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  // a fill kernel rather than a memset node, so that the call can be captured into a graph
+  const i64 words = (i64)d.nb * 16;
+  dok_fill_kernel<<<(unsigned)((words / 4 + DOK_TPB - 1) / DOK_TPB), DOK_TPB, 0, s>>>(d.buckets, words, d.header);
+  return note_launch();
+}
+
+int dok_map_get(const dok_table_t *t, const void *keys, int64_t n, void *values_out,
+                const void *fallback, uint8_t *found, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (n < 0 || n > kMaxRows) return DOK_EINVAL;
+  if (n == 0) return DOK_OK;
+  if (!keys || !values_out || !found) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (layout == DOK_LAYOUT_PACKED8) {
+    const u64 fb = fallback_word(fallback, d.value_bytes);
+    P8_DISPATCH(d.value_bytes, (p8_get_kernel<V, false><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
+  } else {
+    rc = tg_launch_get(d, keys, n, values_out, fallback, found, false, s);
+    if (rc) return rc;
+  }
+  return note_launch();
+}
+
+int dok_map_get_stats(const dok_table_t *t, const void *keys, int64_t n, void *values_out,
+                      const void *fallback, uint8_t *found, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (n < 0 || n > kMaxRows) return DOK_EINVAL;
+  if (n == 0) return DOK_OK;
+  if (!keys || !values_out || !found) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (layout == DOK_LAYOUT_PACKED8) {
+    const u64 fb = fallback_word(fallback, d.value_bytes);
+    P8_DISPATCH(d.value_bytes, (p8_get_kernel<V, true><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
+  } else {
+    rc = tg_launch_get(d, keys, n, values_out, fallback, found, true, s);
+    if (rc) return rc;
+  }
+  return note_launch();
+}
+
+int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int64_t n,
+                uint8_t *stored, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (n < 0 || n > kMaxRows) return DOK_EINVAL;
+  if (n == 0) return DOK_OK;
+  if (!keys || !values) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (layout == DOK_LAYOUT_PACKED8) {
+    P8_DISPATCH(d.value_bytes, (p8_set_kernel<V><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, values, n, stored)));
+  } else {
+    rc = tg_launch_set(d, keys, values, n, stored, s);
+    if (rc) return rc;
+  }
+  return note_launch();
+}
+
+int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t *removed, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (n < 0 || n > kMaxRows) return DOK_EINVAL;
+  if (n == 0) return DOK_OK;
+  if (!keys) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (layout == DOK_LAYOUT_PACKED8) {
+    P8_DISPATCH(d.value_bytes, (p8_remove_kernel<V><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
+  } else {
+    rc = tg_launch_remove(d, keys, n, removed, s);
+    if (rc) return rc;
+  }
+  return note_launch();
+}
+
+int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n, int64_t *count, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (n < 0 || n > kMaxRows) return DOK_EINVAL;
+  if (n == 0) return DOK_OK;
+  if (!keys || !count) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (layout == DOK_LAYOUT_PACKED8) {
+    P8_DISPATCH(d.value_bytes, (p8_count_kernel<V><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, (i64 *)count)));
+  } else {
+    rc = tg_launch_count(d, keys, n, (i64 *)count, s);
+    if (rc) return rc;
+  }
+  return note_launch();
+}
+
+int64_t dok_compact_scratch_bytes(const dok_table_t *t) {
+  if (!t || t->n_phys_buckets < 1) return DOK_EINVAL;
+  const i64 n_chunks = (t->n_phys_buckets + DOK_CHUNK - 1) / DOK_CHUNK;
+  return (n_chunks + 1) * 8;
+}
+
+int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out, int64_t capacity_rows,
+                    int64_t *count_out, void *scratch, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (!count_out || !scratch || capacity_rows < 0) return DOK_EINVAL;
+  if (((uintptr_t)scratch & 7) != 0) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  const i64 n_chunks = chunks_of(d);
+  i64 *offs = (i64 *)scratch;
+  if (layout == DOK_LAYOUT_PACKED8) {
+    P8_DISPATCH(d.value_bytes, (p8_chunk_count_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks)));
+    dok_scan_kernel<<<1, 1024, 0, s>>>(offs, n_chunks, d.lin_ndim == 0 ? d.header : nullptr, (i64 *)count_out);
+    if (keys_out || values_out) {
+      P8_DISPATCH(d.value_bytes, (p8_chunk_write_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks, keys_out, values_out, capacity_rows)));
+    }
+  } else {
+    rc = tg_launch_compact(d, offs, n_chunks, keys_out, values_out, capacity_rows, (i64 *)count_out, s);
+    if (rc) return rc;
+  }
+  return note_launch();
+}
+
+int dok_map_rehash(const dok_table_t *src, const dok_table_t *dst, void *stream) {
+  DevTable a, b; int la, lb;
+  int rc = make_dev_table(src, a, la);
+  if (rc) return rc;
+  rc = make_dev_table(dst, b, lb);
+  if (rc) return rc;
+  if (a.key_bytes != b.key_bytes || a.value_bytes != b.value_bytes || a.lin_ndim != b.lin_ndim) return DOK_EINVAL;
+  if (a.buckets == b.buckets) return DOK_EINVAL;
+  for (int k = 0; k < a.lin_ndim; k++) if (a.lin_dims[k] != b.lin_dims[k]) return DOK_EINVAL;
+  if (la != DOK_LAYOUT_PACKED8) return DOK_EUNSUPPORTED;   // tagged tables rehash through compact + set
+  hipStream_t s = (hipStream_t)stream;
+  const i64 n_chunks = chunks_of(a);
+  P8_DISPATCH(a.value_bytes, (p8_rehash_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(a, b, n_chunks)));
+  return note_launch();
+}
+
+int dok_getitem_dense(const dok_table_t *t, const dok_index_t *ix, void *out, void *stream) {
+  DevTable d; int layout; DevIndex di;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  rc = make_dev_index(d, ix, nullptr, di);
+  if (rc) return rc;
+  if (di.n_elems == 0) return DOK_OK;
+  if (!out || di.n_elems > kMaxRows) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  P8_DISPATCH(d.value_bytes, (p8_getitem_kernel<V><<<grid_for(di.n_elems), DOK_TPB, 0, s>>>(d, di, out)));
+  return note_launch();
+}
+
+int dok_setitem_dense(const dok_table_t *t, const dok_index_t *ix, const dok_view_t *src, void *stream) {
+  DevTable d; int layout; DevIndex di;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (!src) return DOK_EINVAL;
+  rc = make_dev_index(d, ix, src, di);
+  if (rc) return rc;
+  if (di.n_elems == 0) return DOK_OK;
+  if (di.n_elems > kMaxRows) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  P8_DISPATCH(d.value_bytes, (p8_setitem_kernel<V><<<grid_for(di.n_elems), DOK_TPB, 0, s>>>(d, di)));
+  return note_launch();
+}
+
+int dok_count_items(const dok_table_t *t, const dok_index_t *ix, int64_t *count, void *stream) {
+  DevTable d; int layout; DevIndex di;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  rc = make_dev_index(d, ix, nullptr, di);
+  if (rc) return rc;
+  if (di.n_elems == 0) return DOK_OK;
+  if (!count || di.n_elems > kMaxRows) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  P8_DISPATCH(d.value_bytes, (p8_countitems_kernel<V><<<grid_for(di.n_elems), DOK_TPB, 0, s>>>(d, di, (i64 *)count)));
+  return note_launch();
+}
+
+int dok_zero_items(const dok_table_t *t, const dok_index_t *ix, void *stream) {
+  DevTable d; int layout; DevIndex di;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  rc = make_dev_index(d, ix, nullptr, di);
+  if (rc) return rc;
+  if (di.n_elems == 0) return DOK_OK;
+  if (di.n_elems > kMaxRows) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  P8_DISPATCH(d.value_bytes, (p8_zeroitems_kernel<V><<<grid_for(di.n_elems), DOK_TPB, 0, s>>>(d, di)));
+  return note_launch();
+}
+
+int dok_to_dense(const dok_table_t *t, void *dense, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (d.lin_ndim == 0 || !dense) return DOK_EINVAL;
+  i64 volume = 1;
+  for (int k = 0; k < d.lin_ndim; k++) volume *= d.lin_dims[k];
+  if (volume == 0) return DOK_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const i64 n_chunks = chunks_of(d);
+  P8_DISPATCH(d.value_bytes, (p8_to_dense_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, dense, n_chunks, volume)));
+  return note_launch();
+}
+
+}  // extern "C"

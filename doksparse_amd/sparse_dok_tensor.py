@@ -1,0 +1,513 @@
+"""Dictionary-of-keys sparse tensor with the Python surface of the reference's
+``SparseDOKTensor`` (reference: sparse_dok/components/sparse_dok_tensor.py:17-561).
+
+The tensor is a size plus a coordinate-keyed ``CudaClosedHashmap`` whose key rows are int64
+coordinates and whose values have shape ``(1,)``.  The hot methods run as single fused HIP
+kernels of libdokhip:
+
+* ``__getitem__``  : selector gather -> linearise -> table lookup -> dense write
+                     (the reference stacks and transposes the selectors first, :302-315)
+* ``__setitem__``  : selector gather -> linearise -> upsert (dense source, :317-327 and
+                     sparse_dok_tensor_impl.py:412-474)
+* ``to_dense``     : one scan of the table scattering into a zero tensor (:195-209)
+* ``indices/values``: one compaction pass (:156-169)
+
+Selector handling follows the reference's ``_handle_selectors`` (:220-300), including its axis
+placement rule (the broadcast axes of all tensor selectors sit at the position of the first
+tensor selector; every slice keeps an axis of its own, in order) and its squeeze of axes named
+by scalar selectors.  Where the reference raises by accident (a bare ``int`` selector, numpy
+selectors, a scalar selector behind a slice) the intended result is returned instead; a slice
+step other than 1, which the reference silently ignores, raises ``ValueError``.
+"""
+import ctypes
+
+import numpy as np
+import torch
+from torch import Tensor
+
+from . import _lib
+from ._lib import DokIndex, DokView, DOK_MAX_DIMS
+from .closed_hashmap import CudaClosedHashmap, _stream_ptr
+from .util import str2dtype, next_power_of_2, shape_to_stride
+
+_INT_DTYPES = {torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8}
+
+
+class SparseDOKTensor(object):
+    def __init__(self, size, indices=None, values=None, device=None, dtype=None, storage=None):
+        assert isinstance(size, (list, tuple))
+        self._size = torch.Size(size)
+
+        if storage is None:
+            self.device = torch.device("cuda:0") if device is None else torch.device(device)
+        else:
+            assert isinstance(storage, CudaClosedHashmap)
+            self.device = storage.device
+
+        if storage is not None and storage._allocated:
+            assert len(storage.key_shape) == 1 and storage.key_shape[0] == self.ndim
+            self._dtype = storage.value_type
+        elif dtype is None:
+            self._dtype = torch.float32 if values is None else values.dtype
+        else:
+            self._dtype = str2dtype(dtype)
+
+        if storage is not None:
+            self._hashmap = self._adopt_storage(storage)
+        else:
+            n_buckets = 32 if indices is None else next_power_of_2(values.shape[0])
+            self._hashmap = CudaClosedHashmap(n_buckets=n_buckets, device=self.device,
+                                              coord_dims=tuple(self._size))
+        if indices is not None:
+            assert values is not None
+            assert len(indices.shape) == 2
+            assert len(values.shape) == 1
+            assert indices.shape[1] == values.shape[0]
+            assert indices.shape[0] == self.ndim
+            self._hashmap.set(
+                indices.T.to(self.device),
+                values.to(device=self.device, dtype=self.dtype)[:, None],
+            )
+
+    def _adopt_storage(self, storage):
+        """Use `storage` directly if it is keyed by coordinates of this size; otherwise move its
+        entries into a coordinate-keyed map (the fused kernels need the linearised key)."""
+        if storage._coord_dims == tuple(self._size):
+            return storage
+        new = CudaClosedHashmap(n_buckets=storage.n_buckets, device=storage.device,
+                                coord_dims=tuple(self._size),
+                                rehash_factor=storage._rehash_factor,
+                                rehash_threshold=storage._rehash_threshold)
+        if storage._allocated:
+            keys, values = storage.items()
+            if keys.shape[0]:
+                new.set(keys.reshape(-1, self.ndim).long(), values)
+        return new
+
+    # ------------------------------------------------------------------ constructors
+    @classmethod
+    def from_sparse_coo(cls, tensor):
+        assert isinstance(tensor, Tensor)
+        assert tensor.layout == torch.sparse_coo
+        tensor = tensor.coalesce()
+        return cls(size=tuple(tensor.shape), indices=tensor._indices(), values=tensor._values(),
+                   device=tensor.device)
+
+    @classmethod
+    def from_dense(cls, tensor):
+        assert isinstance(tensor, Tensor)
+        assert tensor.layout == torch.strided
+        return cls.from_sparse_coo(tensor.to_sparse())
+
+    @classmethod
+    def from_storage(cls, storage, size=None):
+        assert isinstance(storage, CudaClosedHashmap)
+        assert storage.value_shape == (1,)
+        assert len(storage.key_shape) == 1
+        ndims = storage.key_shape[0]
+        if size is None:
+            if storage._coord_dims is not None:
+                size = storage._coord_dims
+            else:
+                size = tuple((storage.keys().max(dim=0).values + 1).cpu().tolist())
+        else:
+            assert len(size) == ndims
+            assert all(i >= 0 for i in size)
+        return cls(size=tuple(size), storage=storage)
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        kwargs = {} if kwargs is None else kwargs
+        args = [a.to_sparse_coo() if isinstance(a, cls) else a for a in args]
+        kwargs = {k: (a.to_sparse_coo() if isinstance(a, cls) else a) for k, a in kwargs.items()}
+        return func(*args, **kwargs)
+
+    # ------------------------------------------------------------------ simple properties
+    @property
+    def is_sparse(self):
+        return True
+
+    def _is_coalesced(self):
+        return False
+
+    def is_coalesced(self):
+        return False
+
+    def size(self):
+        return self._size
+
+    @property
+    def shape(self):
+        return self._size
+
+    @property
+    def ndim(self):
+        return len(self._size)
+
+    @property
+    def dtype(self):
+        return self._dtype
+
+    def _stride(self, dim=None):
+        stride = shape_to_stride(self.shape)
+        return stride if dim is None else stride[dim]
+
+    def storage(self):
+        return self._hashmap
+
+    def _nnz(self):
+        return self._hashmap.n_elements
+
+    @property
+    def sparsity(self):
+        return 1 - self._nnz() / float(np.prod(self.shape))
+
+    def clone(self, deepclone=True):
+        new = SparseDOKTensor(size=tuple(self._size), device=self.device, dtype=self.dtype)
+        new._hashmap = self._hashmap.clone(deepclone=deepclone)
+        return new
+
+    # ------------------------------------------------------------------ read-out
+    def indices(self):
+        keys = self._hashmap.keys()
+        if keys is None:
+            return torch.empty(self.ndim, 0, device=self.device, dtype=torch.long)
+        return keys.T
+
+    def values(self):
+        values = self._hashmap.values()
+        if values is None:
+            return torch.empty(0, device=self.device, dtype=self.dtype)
+        return values.flatten()
+
+    def _indices(self):
+        return self._hashmap._keys
+
+    def _values(self):
+        return self._hashmap._values
+
+    def set_values(self, selectors, new_values):
+        self._hashmap.set_values(selectors=selectors, new_values=new_values[:, None])
+
+    def to_sparse_coo(self):
+        keys, values = self._hashmap.items()
+        if keys is None:
+            keys = torch.empty(0, self.ndim, device=self.device, dtype=torch.long)
+            values = torch.empty(0, 1, device=self.device, dtype=self.dtype)
+        return torch.sparse_coo_tensor(indices=keys.T, values=values.flatten(), size=tuple(self.shape),
+                                       device=self.device)
+
+    @property
+    def _as_sparse_coo_tensor(self):
+        return self.to_sparse_coo()
+
+    def to_sparse_csr(self):
+        return self.to_sparse_coo().to_sparse_csr()
+
+    def to_dense(self):
+        dense = torch.zeros(tuple(self.shape), device=self.device, dtype=self.dtype)
+        hm = self._hashmap
+        if hm._allocated and dense.numel():
+            lib = _lib.load()
+            _lib.check(lib.dok_to_dense(ctypes.byref(hm._desc), dense.data_ptr(), _stream_ptr(self.device)),
+                       "to_dense")
+        return dense
+
+    def resize(self, *new_size):
+        new_size = tuple(new_size) + (self.ndim - len(new_size)) * (-1,)
+        assert len(new_size) == self.ndim
+        new_size = torch.Size([self.shape[i] if new_size[i] == -1 else new_size[i] for i in range(self.ndim)])
+        if new_size != self._size:
+            self._rekey(new_size, lambda idx: idx)
+        return self
+
+    def _rekey(self, new_size, fn):
+        """Rebuild the storage for `new_size`, mapping the [ndim, nnz] indices through fn."""
+        old = self._hashmap
+        new = CudaClosedHashmap(n_buckets=old.n_buckets, device=self.device, coord_dims=tuple(new_size),
+                                rehash_factor=old._rehash_factor, rehash_threshold=old._rehash_threshold)
+        if old._allocated:
+            keys, values = old.items()
+            if keys.shape[0]:
+                new.set(fn(keys.T).T.contiguous(), values)
+                new._header[_lib.DOK_H_NOOB] = 0      # entries outside the new size are dropped
+        self._hashmap = new
+        self._size = torch.Size(new_size)
+
+    # ------------------------------------------------------------------ selectors
+    def _normalise_slice(self, sl, dim):
+        if sl.step not in (None, 1):
+            raise ValueError("only slices with step 1 are supported")
+        size = self.shape[dim]
+        start = 0 if sl.start is None else int(sl.start)
+        stop = size if sl.stop is None else int(sl.stop)
+        if start < 0:
+            start = max(start + size, 0)
+        if stop < 0:
+            stop = stop + size
+        stop = max(min(stop, size), start)
+        return start, stop
+
+    def _handle_selectors(self, selectors, return_slice_as_tensor=True):
+        """Turn an indexing expression into one int64 selector per tensor dimension, all
+        broadcast (as views) to the shape of the result, plus the positions of the scalar
+        selectors.  Reference: sparse_dok_tensor.py:220-300."""
+        if not isinstance(selectors, tuple):
+            selectors = (selectors,)
+
+        flat = []
+        for sel in selectors:
+            if isinstance(sel, np.ndarray):
+                sel = torch.from_numpy(sel)
+            if isinstance(sel, Tensor) and sel.dtype == torch.bool:
+                flat.extend(sel.to(self.device).nonzero(as_tuple=True))
+            elif isinstance(sel, Tensor) and sel.dtype in _INT_DTYPES:
+                flat.append(sel.to(self.device).long())
+            elif isinstance(sel, (bool, np.bool_)):
+                raise ValueError("boolean scalars are not valid selectors")
+            elif isinstance(sel, (int, np.integer)):
+                flat.append(torch.tensor(int(sel), device=self.device, dtype=torch.long))
+            elif isinstance(sel, slice):
+                flat.append(sel)
+            elif isinstance(sel, (tuple, list)):
+                flat.append(torch.tensor(sel, device=self.device, dtype=torch.long))
+            else:
+                raise ValueError(f"unsupported selector {type(sel)}")
+        if len(flat) > self.ndim:
+            raise IndexError(f"too many indices for tensor of dimension {self.ndim}")
+        flat += [slice(None)] * (self.ndim - len(flat))
+
+        scalar_positions = [i for i, s in enumerate(flat) if isinstance(s, Tensor) and s.ndim == 0]
+        tensors = [s for s in flat if isinstance(s, Tensor)]
+        n_slices = len(flat) - len(tensors)
+        bshape = tuple(torch.broadcast_shapes(*[t.shape for t in tensors])) if tensors else tuple()
+        out_ndim = len(bshape) + n_slices
+        first_tensor = next((i for i, s in enumerate(flat) if isinstance(s, Tensor)), None)
+
+        out = []
+        axis = 0          # next free output axis for a slice
+        met_tensor = False
+        for i, sel in enumerate(flat):
+            if isinstance(sel, Tensor):
+                # broadcast axes of every tensor selector sit together at the first tensor's position
+                view_shape = [1] * out_ndim
+                view_shape[first_tensor:first_tensor + len(bshape)] = bshape
+                out.append(torch.broadcast_to(sel, bshape).reshape(view_shape))
+                if not met_tensor:
+                    axis += len(bshape)
+                    met_tensor = True
+            else:
+                start, stop = self._normalise_slice(sel, i)
+                if return_slice_as_tensor:
+                    view_shape = [1] * out_ndim
+                    view_shape[axis] = stop - start
+                    out.append(torch.arange(start, stop, device=self.device).reshape(view_shape))
+                    axis += 1
+                else:
+                    out.append(slice(start, stop))
+        if return_slice_as_tensor:
+            out = list(torch.broadcast_tensors(*out))
+        return out, scalar_positions
+
+    def _index_desc(self, selectors):
+        out_shape = tuple(selectors[0].shape)
+        if len(out_shape) > DOK_MAX_DIMS or self.ndim > DOK_MAX_DIMS:
+            raise NotImplementedError(f"indexing expressions with more than {DOK_MAX_DIMS} axes")
+        ix = DokIndex()
+        ix.ndim = self.ndim
+        ix.sel_ndim = len(out_shape)
+        for j, s in enumerate(out_shape):
+            ix.shape[j] = s
+        for d, sel in enumerate(selectors):
+            assert sel.dtype == torch.long and sel.device == self.device
+            ix.sel[d].data = sel.data_ptr()
+            for j, st in enumerate(sel.stride()):
+                ix.sel[d].strides[j] = st
+        return ix, out_shape
+
+    # ------------------------------------------------------------------ indexing
+    def __getitem__(self, selectors):
+        selectors, scalar_positions = self._handle_selectors(selectors)
+        ix, out_shape = self._index_desc(selectors)
+        hm = self._hashmap
+        if not hm._allocated:
+            values = torch.zeros(out_shape, device=self.device, dtype=self.dtype)
+        else:
+            values = torch.empty(out_shape, device=self.device, dtype=self.dtype)
+            if values.numel():
+                lib = _lib.load()
+                _lib.check(lib.dok_getitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), values.data_ptr(),
+                                                 _stream_ptr(self.device)), "__getitem__")
+        # the reference squeezes the output axis numbered like each scalar selector's position
+        for i in reversed(scalar_positions):
+            if i < values.ndim:
+                values = values.squeeze(i)
+        return values
+
+    def __setitem__(self, selectors, values):
+        selectors, _ = self._handle_selectors(selectors)
+        out_shape = tuple(selectors[0].shape)
+        if isinstance(values, SparseDOKTensor) or (isinstance(values, Tensor) and values.is_sparse):
+            raise NotImplementedError("sparse-valued __setitem__")
+        if not isinstance(values, Tensor):
+            values = torch.tensor(values, device=self.device, dtype=self.dtype)
+        values = torch.broadcast_to(values.to(device=self.device, dtype=self.dtype), out_shape)
+        self._set_items_dense(values, selectors)
+
+    def _set_items_dense(self, src, selectors):
+        """Reference: SparseDOKTensorImplCuda.set_items_dense (sparse_dok_tensor_impl.py:412-474)."""
+        n_sel = int(np.prod(src.shape, dtype=np.int64))
+        if n_sel == 0:
+            return
+        hm = self._hashmap
+        if not hm._allocated:
+            # fixes the key/value widths; the entry itself is written again by the kernel below
+            first_key = torch.stack([s.reshape(-1)[0] for s in selectors], dim=0)[None]
+            hm.set(first_key, src.reshape(-1)[:1, None].contiguous())
+        ix, _ = self._index_desc(selectors)
+        view = DokView()
+        view.data = src.data_ptr()
+        for j, st in enumerate(src.stride()):
+            view.strides[j] = st
+        # growth rule of the reference: decided on the number of selector elements
+        n_now = hm.n_elements
+        if n_now + n_sel > hm.n_buckets * hm._rehash_threshold:
+            hm.rehash(int(np.ceil((n_now + n_sel) * hm._rehash_factor)))
+        lib = _lib.load()
+        _lib.check(lib.dok_setitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), ctypes.byref(view),
+                                         _stream_ptr(self.device)), "__setitem__")
+        hm._n_upper = n_now + n_sel
+        n_oob = int(hm._header[_lib.DOK_H_NOOB].item())
+        if n_oob:
+            hm._header[_lib.DOK_H_NOOB] = 0
+            raise IndexError(f"{n_oob} coordinates fall outside the tensor of size {tuple(self.shape)}")
+
+    def count_items(self, selectors):
+        """Number of addressed elements that are stored (reference: count_items,
+        sparse_dok_tensor_impl.py:56-108)."""
+        selectors, _ = self._handle_selectors(selectors)
+        count = torch.zeros(1, device=self.device, dtype=torch.long)
+        hm = self._hashmap
+        if hm._allocated and selectors[0].numel():
+            ix, _ = self._index_desc(selectors)
+            lib = _lib.load()
+            _lib.check(lib.dok_count_items(ctypes.byref(hm._desc), ctypes.byref(ix), count.data_ptr(),
+                                           _stream_ptr(self.device)), "count_items")
+        return count
+
+    def zero_items(self, selectors):
+        """Remove every addressed element (reference: zero_items, sparse_dok_tensor_impl.py:110-146)."""
+        selectors, _ = self._handle_selectors(selectors)
+        hm = self._hashmap
+        if hm._allocated and selectors[0].numel():
+            ix, _ = self._index_desc(selectors)
+            lib = _lib.load()
+            _lib.check(lib.dok_zero_items(ctypes.byref(hm._desc), ctypes.byref(ix), _stream_ptr(self.device)),
+                       "zero_items")
+
+    # ------------------------------------------------------------------ torch.sparse pass-throughs
+    def sum(self, dim=None, keepdim=False):
+        coo = self.to_sparse_coo()
+        if dim is None:
+            return torch.sparse.sum(coo)
+        out = torch.sparse.sum(coo, dim=dim)
+        return out
+
+    def index_select(self, dim, index):
+        return self.to_sparse_coo().index_select(dim=dim, index=index)
+
+    def select(self, dim, index):
+        return self.to_sparse_coo().select(dim=dim, index=index)
+
+    # ------------------------------------------------------------------ re-layout (rebuilds the storage)
+    def permute_(self, *ordering):
+        ordering = [int(o) for o in ordering]
+        assert sorted(ordering) == list(range(self.ndim))
+        new_size = torch.Size(self._size[i] for i in ordering)
+        self._rekey(new_size, lambda idx: idx[ordering])
+        return self
+
+    def permute(self, *ordering):
+        return self.clone(deepclone=False)._detach_storage().permute_(*ordering)
+
+    def _detach_storage(self):
+        self._hashmap = self._hashmap.clone(deepclone=False)
+        return self
+
+    def transpose_(self, dim0, dim1):
+        assert dim0 != dim1
+        order = list(range(self.ndim))
+        dim0, dim1 = dim0 % self.ndim, dim1 % self.ndim
+        order[dim0], order[dim1] = dim1, dim0
+        return self.permute_(*order)
+
+    def transpose(self, dim0, dim1):
+        assert dim0 != dim1
+        order = list(range(self.ndim))
+        dim0, dim1 = dim0 % self.ndim, dim1 % self.ndim
+        order[dim0], order[dim1] = dim1, dim0
+        return self.permute(*order)
+
+    def t(self):
+        assert self.ndim == 2, "tensor isn't 2 dimensional, try x.transpose(dim1, dim2)"
+        return self.transpose(0, 1)
+
+    @property
+    def T(self):
+        return self.t()
+
+    def flatten(self):
+        stride = torch.tensor(self._stride(), device=self.device, dtype=torch.long)[:, None]
+        flat = (self.indices() * stride).sum(dim=0, keepdim=True)
+        return SparseDOKTensor(size=[int(np.prod(self.shape))], indices=flat, values=self.values(),
+                               device=self.device)
+
+    def reshape(self, *new_shape):
+        assert np.prod(new_shape) == np.prod(self.shape)
+        flat = self.flatten()
+        if len(new_shape) == 1:
+            return flat
+        idx = flat.indices()
+        strides = torch.tensor(shape_to_stride(new_shape), device=self.device, dtype=torch.long)[:, None]
+        sizes = torch.tensor(new_shape, device=self.device, dtype=torch.long)[:, None]
+        new_idx = torch.div(idx.expand(len(new_shape), -1), strides, rounding_mode="floor") % sizes
+        return SparseDOKTensor(size=tuple(new_shape), indices=new_idx, values=flat.values(), device=self.device)
+
+    # ------------------------------------------------------------------ unary ops on the stored values
+    def _map_values(self, fn):
+        keys, values = self._hashmap.items()
+        new = SparseDOKTensor(size=tuple(self._size), device=self.device, dtype=self.dtype)
+        new._hashmap = CudaClosedHashmap(n_buckets=self._hashmap.n_buckets, device=self.device,
+                                         coord_dims=tuple(self._size),
+                                         rehash_factor=self._hashmap._rehash_factor,
+                                         rehash_threshold=self._hashmap._rehash_threshold)
+        if keys is not None and keys.shape[0]:
+            new._hashmap.set(keys, fn(values))
+        return new
+
+    def abs(self):
+        return self._map_values(torch.abs)
+
+    def _float_only(self):
+        assert self.dtype in {torch.half, torch.float, torch.double}
+
+    def sqrt(self):
+        self._float_only()
+        return self._map_values(torch.sqrt)
+
+    def ceil(self):
+        self._float_only()
+        return self._map_values(torch.ceil)
+
+    def floor(self):
+        self._float_only()
+        return self._map_values(torch.floor)
+
+    def round(self, decimals=0):
+        self._float_only()
+        return self._map_values(lambda v: torch.round(v, decimals=decimals or 0))
+
+    def __repr__(self):
+        return (f"SparseDOKTensor(indices={self.indices()},\n"
+                f"                values={self.values()},\n"
+                f"                size={self.size()}, nnz={self._nnz()}, sparsity={round(self.sparsity, 6)})")

@@ -1,0 +1,181 @@
+/*
+ * dokhip.h - C ABI of libdokhip.so: a batched open-addressing hash table and the
+ * dictionary-of-keys (DOK) sparse-tensor indexing kernels that run on it, written
+ * for AMD gfx950 (MI355X).
+ *
+ * Conventions
+ *   - Every pointer documented as "device" is a HIP device pointer owned by the
+ *     caller.  The library never allocates or frees device memory; scratch space
+ *     is passed in.  Batch buffers are row-major and contiguous.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Calls
+ *     enqueue work and return; they do not synchronise.  Operations on one table
+ *     must be ordered on one stream (or by events); distinct tables are independent.
+ *   - Return value: DOK_OK or a negative DOK_E* code.  No call throws or aborts.
+ *   - Flags (`found`, `stored`, `removed`) are one byte per row, 0 or 1.
+ *
+ * Each entry point names the interface of the reference implementation
+ * (DeMoriarty/DOKSparse, paths relative to its checkout) that it stands in for.
+ */
+#ifndef DOKHIP_H
+#define DOKHIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DOK_OK            0
+#define DOK_EINVAL       -1   /* bad argument (null pointer, negative count, misaligned buffer)   */
+#define DOK_EUNSUPPORTED -2   /* key/value width the table layouts cannot hold                   */
+#define DOK_ELAUNCH      -3   /* the HIP runtime refused a launch; see dok_last_hip_error()      */
+
+#define DOK_BUCKET_BYTES  128
+#define DOK_MAX_DIMS      8
+
+/* Table header: DOK_HEADER_WORDS int64 words in device memory, zeroed by dok_table_clear.     */
+#define DOK_HEADER_WORDS  16
+#define DOK_H_NELEM       0   /* live entries (set adds fresh inserts, remove subtracts)          */
+#define DOK_H_NFULL       1   /* rows a set could not place because every bucket was full         */
+#define DOK_H_NPROBE      2   /* buckets visited, accumulated by the *_stats entry points         */
+#define DOK_H_NOOB        3   /* rows whose coordinates fell outside lin_dims (skipped)           */
+#define DOK_H_NOPS        4   /* rows processed by the *_stats entry points                       */
+/* words 8..11: side slots for the two 8-byte key patterns the packed layout reserves            */
+
+/* Physical layouts (chosen from the key/value widths by dok_layout_of). */
+#define DOK_LAYOUT_PACKED8 1  /* key <= 8 bytes (1,2,4,8), value 1,2,4 or 8 bytes: the key word
+                                 itself is the CAS-claimed slot word; S = 128/(8+V) slots/bucket  */
+#define DOK_LAYOUT_TAGGED  2  /* any widths with 8*(1+ceil(K/8)+ceil(V/8)) <= 128: an 8-byte
+                                 tag/lock word per slot, then the key words, then the value words */
+
+typedef struct dok_table {
+  void    *buckets;            /* device, 128-byte aligned, n_phys_buckets * 128 bytes            */
+  int64_t *header;             /* device, DOK_HEADER_WORDS int64                                  */
+  int64_t  n_phys_buckets;     /* 1 .. 2^32-1                                                     */
+  uint64_t seed;               /* hash seed; placement depends on it, results do not              */
+  int32_t  key_bytes;          /* bytes per key row as stored (8 when lin_ndim > 0)               */
+  int32_t  value_bytes;        /* bytes per value row                                             */
+  int32_t  lin_ndim;           /* 0: key rows are raw bytes.  n>0: key rows handed to the batch
+                                  entry points are n int64 coordinates that are linearised
+                                  row-major over lin_dims into one 8-byte key                     */
+  int32_t  reserved_;
+  int64_t  lin_dims[DOK_MAX_DIMS];
+} dok_table_t;
+
+/* A strided int64 (selector) or value (source) view over the broadcast index space.
+ * Strides are in elements; 0 means the axis is broadcast. */
+typedef struct dok_view {
+  const void *data;                    /* device */
+  int64_t     strides[DOK_MAX_DIMS];
+} dok_view_t;
+
+/* The broadcast index space of one advanced-indexing expression plus one selector per
+ * tensor dimension: what SparseDOKTensor._handle_selectors (sparse_dok_tensor.py:220-300)
+ * produces and get_tensor_accessor_argument_array (util.py:295-310) packs for the kernels. */
+typedef struct dok_index {
+  int32_t    ndim;                     /* tensor dimensions = number of selectors (<= 8)         */
+  int32_t    sel_ndim;                 /* dimensions of the broadcast index space (<= 8)         */
+  int64_t    shape[DOK_MAX_DIMS];      /* broadcast shape                                        */
+  dok_view_t sel[DOK_MAX_DIMS];        /* int64 selector views, one per tensor dimension         */
+} dok_index_t;
+
+/* ---- layout helpers (host only, no GPU needed) ------------------------------------------ */
+
+/* Layout id for the widths, or DOK_EUNSUPPORTED.  *slots_per_bucket may be NULL. */
+int dok_layout_of(int32_t key_bytes, int32_t value_bytes, int32_t *slots_per_bucket);
+
+/* Physical bucket count that gives at least `capacity` slots. */
+int64_t dok_phys_buckets_for(int64_t capacity, int32_t key_bytes, int32_t value_bytes);
+
+/* Text of the last HIP error a launch hit on this thread ("" if none). */
+const char *dok_last_hip_error(void);
+
+/* ---- table lifetime --------------------------------------------------------------------- */
+
+/* Mark every slot empty and zero the header.
+ * Reference: CudaClosedHashmap.__init__ filling _uuid with -1 (cuda_closed_hashmap.py:40). */
+int dok_table_clear(const dok_table_t *t, void *stream);
+
+/* ---- batched map operations -------------------------------------------------------------- */
+
+/* values_out[r] = value of keys[r] if present else the fallback row; found[r] = present.
+ * `fallback` is a HOST pointer to value_bytes bytes (NULL = zeros).
+ * Reference: closed_hashmap_get (closed_hashmap_impl.cu:7-85) together with the fallback
+ * pre-fill of ClosedHashmapImplCuda.get (closed_hashmap_impl.py:50-145). */
+int dok_map_get(const dok_table_t *t, const void *keys, int64_t n,
+                void *values_out, const void *fallback, uint8_t *found, void *stream);
+
+/* Same, and adds the buckets visited / rows processed to header[DOK_H_NPROBE/NOPS]. */
+int dok_map_get_stats(const dok_table_t *t, const void *keys, int64_t n,
+                      void *values_out, const void *fallback, uint8_t *found, void *stream);
+
+/* Upsert.  A key present is overwritten in place; a key absent takes the first tombstone on
+ * its probe chain, else the first empty slot.  Equal keys inside one batch end up in ONE slot
+ * holding one of their values.  header[DOK_H_NELEM] grows by the number of fresh inserts.
+ * stored (may be NULL): 1 = placed, 0 = table full or coordinate out of range.
+ * Reference: closed_hashmap_set (closed_hashmap_impl.cu:88-156, ClosedHashmap::set
+ * closed_hashmap_impl_class.cu:368-427); the in-kernel count replaces the host-side
+ * "get, unique, count" pre-pass of CudaClosedHashmap.set (cuda_closed_hashmap.py:350-384). */
+int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int64_t n,
+                uint8_t *stored, void *stream);
+
+/* Tombstone each present key; header[DOK_H_NELEM] shrinks by the number removed.  Equal keys
+ * in one batch: exactly one row reports 1.
+ * Reference: closed_hashmap_remove (closed_hashmap_impl.cu:159-220, ClosedHashmap::remove
+ * closed_hashmap_impl_class.cu:459-484). */
+int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n,
+                   uint8_t *removed, void *stream);
+
+/* count[0] += number of rows whose key is present.  count is a device int64.
+ * Reference: ClosedHashmap::exists (closed_hashmap_impl_class.cu:253-278). */
+int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n,
+                           int64_t *count, void *stream);
+
+/* ---- read-out ----------------------------------------------------------------------------- */
+
+/* Bytes of device scratch dok_map_compact needs for this table. */
+int64_t dok_compact_scratch_bytes(const dok_table_t *t);
+
+/* Write the live entries in slot order: keys_out[i] (key_bytes each; lin_ndim int64
+ * coordinates each when lin_ndim > 0) and values_out[i].  Either output may be NULL.  Two
+ * calls on an unchanged table give the same order.  `capacity_rows` bounds the rows written;
+ * count_out[0] (device int64) receives the number of live entries.
+ * Reference: nonempty_mask / keys() / values() (cuda_closed_hashmap.py:157-172). */
+int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out,
+                    int64_t capacity_rows, int64_t *count_out, void *scratch, void *stream);
+
+/* Re-insert every live entry of src into dst (same key/value widths; dst cleared by the
+ * caller; dst may have another size, seed or lin_dims of equal volume).
+ * Reference: CudaClosedHashmap.rehash (cuda_closed_hashmap.py:456-468). */
+int dok_map_rehash(const dok_table_t *src, const dok_table_t *dst, void *stream);
+
+/* ---- DOK indexing (tables with lin_ndim > 0) ------------------------------------------------ */
+
+/* out[e] = value stored at the coordinate the selectors give for element e of the broadcast
+ * index space, or zero; out is C-contiguous with value_bytes per element.
+ * Reference: SparseDOKTensor.__getitem__ (sparse_dok_tensor.py:302-315): stack + transpose +
+ * closed_hashmap_get with fallback 0, fused into one pass. */
+int dok_getitem_dense(const dok_table_t *t, const dok_index_t *ix, void *out, void *stream);
+
+/* Upsert src[e] at the coordinate of every element e (zeros are stored too).
+ * Reference: sparse_dok_set_items_dense (sparse_dok_tensor_impl.cu:271-313). */
+int dok_setitem_dense(const dok_table_t *t, const dok_index_t *ix, const dok_view_t *src,
+                      void *stream);
+
+/* count[0] += number of elements whose coordinate is stored.
+ * Reference: sparse_dok_count_items (sparse_dok_tensor_impl.cu:4-56). */
+int dok_count_items(const dok_table_t *t, const dok_index_t *ix, int64_t *count, void *stream);
+
+/* Tombstone the coordinate of every element; header[DOK_H_NELEM] shrinks accordingly.
+ * Reference: sparse_dok_zero_items (sparse_dok_tensor_impl.cu:59-108). */
+int dok_zero_items(const dok_table_t *t, const dok_index_t *ix, void *stream);
+
+/* dense[linear coordinate] = value for every live entry; `dense` holds prod(lin_dims) elements
+ * of value_bytes and must be zero-filled by the caller.
+ * Reference: SparseDOKTensor.to_dense (sparse_dok_tensor.py:195-209). */
+int dok_to_dense(const dok_table_t *t, void *dense, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DOKHIP_H */
