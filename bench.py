@@ -1,0 +1,281 @@
+#!/usr/bin/env python3
+"""Headline benchmark: batched hashmap get / set at 64M int64 keys -> float32 values on one
+MI355X, load factors 0.5 and 0.9 (synthetic data).
+
+One "step" is one `get` of a 64M-query batch (50% hits drawn Zipf(1.1) over the stored keys,
+50% uniform misses) against the load-factor-0.5 table.  The JSON line also carries set
+throughput, the load-factor-0.9 figures, mean probe lengths, the HBM roofline of the get kernel
+and a CPU baseline (the reference algorithm restated in C, timed on this machine's cores over a
+bounded sample of the same workload).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--keys N] [--no-cpu]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+# algorithmic bytes per op for 8-byte keys and 4-byte values: one 128-byte bucket line per op,
+# plus the batch row and the outputs
+B_GET = 8 + 128 + 4 + 1           # key in, bucket line, value out, flag out
+B_SET = 8 + 4 + 128 + 128         # key+value in, bucket line read, dirtied line written back
+
+
+def make_unique_keys(n, gen, device):
+    k = torch.randint(0, 2**62, (int(n * 1.002) + 1024,), generator=gen, device=device, dtype=torch.long)
+    k = torch.unique(k)
+    assert k.shape[0] >= n
+    perm = torch.randperm(k.shape[0], generator=gen, device=device)[:n]
+    return k[perm].contiguous()
+
+
+def make_queries(keys, n_q, gen, device, zipf_s=1.1):
+    """50% hits with rank ~ r^-s over the stored keys (rank -> key through the keys' own random
+    order), 50% uniform misses, shuffled."""
+    n = keys.shape[0]
+    n_hit = n_q // 2
+    w = torch.arange(1, n + 1, device=device, dtype=torch.float64).pow_(-zipf_s)
+    cdf = torch.cumsum(w, 0)
+    del w
+    u = torch.rand(n_hit, generator=gen, device=device, dtype=torch.float64) * cdf[-1]
+    rank = torch.searchsorted(cdf, u).clamp_(max=n - 1)
+    del cdf, u
+    hits = keys[rank]
+    del rank
+    misses = torch.randint(0, 2**62, (n_q - n_hit,), generator=gen, device=device, dtype=torch.long)
+    q = torch.cat([hits, misses])
+    del hits, misses
+    q = q[torch.randperm(n_q, generator=gen, device=device)].contiguous()
+    return q, n_hit
+
+
+def time_kernel(fn, reps, prep=None):
+    """Average / min milliseconds of fn() over reps, measured with events on the current stream
+    (the stream the library launches on).  prep() runs untimed before each rep."""
+    times = []
+    for _ in range(reps):
+        if prep is not None:
+            prep()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1))
+    return float(np.mean(times)), float(np.min(times))
+
+
+def build_map(keys, values, capacity, device):
+    from doksparse_amd import CudaClosedHashmap
+    hm = CudaClosedHashmap(n_buckets=capacity, device=device, rehash_threshold=1.0, seed=12345)
+    hm.set(keys[:, None], values[:, None])
+    return hm
+
+
+def raw_calls(hm):
+    """Closures that launch the get / set / clear kernels through the C ABI on preallocated
+    buffers, so that a timed region holds nothing but the kernel."""
+    from doksparse_amd import _lib
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    lib = _lib.load()
+    desc = ctypes.byref(hm._desc)
+    dev = hm.device
+
+    def get(q, out_v, out_f):
+        _lib.check(lib.dok_map_get(desc, q.data_ptr(), q.shape[0], out_v.data_ptr(), None,
+                                   out_f.data_ptr(), _stream_ptr(dev)), "get")
+
+    def set_(k, v):
+        _lib.check(lib.dok_map_set(desc, k.data_ptr(), v.data_ptr(), k.shape[0], None, _stream_ptr(dev)), "set")
+
+    def clear():
+        _lib.check(lib.dok_table_clear(desc, _stream_ptr(dev)), "clear")
+
+    return get, set_, clear
+
+
+def cpu_baseline(n_keys, seed):
+    """The reference algorithm (oracle/closed_hashmap_ref.c) on the host cores, on a bounded
+    sample of the workload: n_keys unique keys at load factor 0.5, n_keys queries (50% Zipf hits,
+    50% misses)."""
+    from oracle.ref_hashmap import RefClosedHashmap, _rows
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    rng = np.random.default_rng(seed)
+    keys = np.unique(rng.integers(0, 2**62, size=int(n_keys * 1.01) + 64, dtype=np.int64))
+    rng.shuffle(keys)
+    keys = keys[:n_keys]
+    vals = rng.standard_normal(n_keys).astype(np.float32)
+    n_hit = n_keys // 2
+    w = np.arange(1, n_keys + 1, dtype=np.float64) ** -1.1
+    cdf = np.cumsum(w)
+    rank = np.minimum(np.searchsorted(cdf, rng.random(n_hit) * cdf[-1]), n_keys - 1)
+    q = np.concatenate([keys[rank], rng.integers(0, 2**62, size=n_keys - n_hit, dtype=np.int64)])
+    rng.shuffle(q)
+
+    ref = RefClosedHashmap(n_buckets=2 * n_keys, rehash_threshold=1.0, rng=np.random.default_rng(seed + 1),
+                           n_threads=cores)
+    ref._allocate(keys[:, None], vals[:, None])
+    ref._keys.fill(0)          # touch the pages before timing
+    ref._values.fill(0)
+    kr, vr, qr = _rows(keys[:, None]), _rows(vals[:, None]), _rows(q[:, None])
+    t0 = time.perf_counter()
+    ref._kernel_set(kr, vr)
+    t_set = time.perf_counter() - t0
+    best_get = 1e30
+    for _ in range(3):
+        t0 = time.perf_counter()
+        _, found = ref._kernel_get(qr)
+        best_get = min(best_get, time.perf_counter() - t0)
+    assert abs(int(found.sum()) - n_hit) <= 2, "oracle get disagrees with the workload"
+    return {
+        "value": round(n_keys / best_get / 1e6, 2),
+        "unit": "Mops/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{n_keys} unique int64 keys -> f32 at load factor 0.5, get of {n_keys} queries "
+                  f"(50% Zipf(1.1) hits, 50% misses), best of 3; set of the same keys "
+                  f"{round(n_keys / t_set / 1e6, 2)} Mops/s",
+        "set_mops": round(n_keys / t_set / 1e6, 2),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--keys", type=int, default=1 << 26, help="stored keys and queries per batch")
+    ap.add_argument("--cpu-keys", type=int, default=1 << 24)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--quick", action="store_true", help="skip the set and load-factor-0.9 legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the hashmap path has no multi-GPU leg in this build "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    n = args.keys
+    gen = torch.Generator(device=device)
+    gen.manual_seed(1003)
+    keys = make_unique_keys(n, gen, device)
+    values = torch.randn(n, generator=gen, device=device, dtype=torch.float32)
+    queries, n_hit = make_queries(keys, n, gen, device)
+
+    cap05 = 2 * n
+    cap09 = int(np.ceil(n / 0.9))
+    results = {}
+
+    # ---------------- load factor 0.5: the timed steps -------------------------------------
+    hm = build_map(keys, values, cap05, device)
+    assert hm.n_elements == n
+    out_v = torch.empty(n, 1, device=device, dtype=torch.float32)
+    out_f = torch.empty(n, device=device, dtype=torch.bool)
+    raw_get, raw_set, raw_clear = raw_calls(hm)
+
+    # correctness gate before any timing: hits return their value, misses are misses
+    v, f = hm.get(queries[:, None])
+    assert int(f.sum().item()) == n_hit, "unexpected hit count"
+    chk = torch.randperm(n, generator=gen, device=device)[: 1 << 20]
+    vv, ff = hm.get(keys[chk][:, None])
+    assert bool(ff.all()) and torch.equal(vv[:, 0], values[chk])
+    del v, f, vv, ff
+
+    for _ in range(args.warmup):
+        hm.get(queries[:, None])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        hm.get(queries[:, None])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    get_mops = n / (ms_per_step * 1e-3) / 1e6
+
+    # kernel-only duration for the roofline
+    k_avg, k_min = time_kernel(lambda: raw_get(queries, out_v, out_f), max(args.steps, 5))
+    results["get_kernel_ms_lf05"] = round(k_avg, 4)
+    results["get_mops_lf05"] = round(n / k_avg / 1e3, 1)
+    results["probe_len_lf05"] = round(hm.probe_stats(queries[:, None]), 4)
+
+    if not args.quick:
+        s_avg, s_min = time_kernel(lambda: raw_set(keys, values), 5, prep=raw_clear)
+        results["set_kernel_ms_lf05"] = round(s_avg, 4)
+        results["set_mops_lf05"] = round(n / s_avg / 1e3, 1)
+        results["set_algo_gbs_lf05"] = round(n * B_SET / s_avg / 1e6, 1)
+        assert hm.n_elements == n
+        # overwrite pass (every key present)
+        o_avg, _ = time_kernel(lambda: raw_set(keys, values), 5)
+        results["overwrite_mops_lf05"] = round(n / o_avg / 1e3, 1)
+        del hm
+        torch.cuda.empty_cache()
+
+        # ---------------- load factor 0.9 ---------------------------------------------------
+        hm9 = build_map(keys, values, cap09, device)
+        assert hm9.n_elements == n
+        raw_get9, raw_set9, raw_clear9 = raw_calls(hm9)
+        v, f = hm9.get(queries[:, None])
+        assert int(f.sum().item()) == n_hit
+        del v, f
+        g9, _ = time_kernel(lambda: raw_get9(queries, out_v, out_f), 10)
+        s9, _ = time_kernel(lambda: raw_set9(keys, values), 3, prep=raw_clear9)
+        results["get_kernel_ms_lf09"] = round(g9, 4)
+        results["get_mops_lf09"] = round(n / g9 / 1e3, 1)
+        results["set_mops_lf09"] = round(n / s9 / 1e3, 1)
+        results["probe_len_lf09"] = round(hm9.probe_stats(queries[:, None]), 4)
+        results["load_factor_09_physical"] = round(n / (hm9._n_phys * hm9._slots_per_bucket), 4)
+        del hm9
+
+    achieved = n * B_GET / (k_avg * 1e-3) / 1e9
+    line = {
+        "metric": "hashmap get/set Mops/s at 64M keys LF 0.5/0.9; achieved HBM GB/s % of peak",
+        "value": round(get_mops, 1),
+        "unit": "Mops/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int64",
+        "data": "synthetic",
+        "config": {
+            "workload": f"get of {n} queries (50% Zipf(1.1) hits, 50% uniform misses) against {n} "
+                        f"unique int64 keys -> float32 values, capacity {cap05} (load factor 0.5)",
+            "keys": n, "capacity": cap05, "key_bytes": 8, "value_bytes": 4,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "kernel": "p8_get_kernel<4,false>",
+            "bytes_per_op": B_GET,
+            "kernel_ms": round(k_avg, 4),
+        },
+        "extra": results,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(args.cpu_keys, 1003)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -485,7 +485,7 @@ class CudaClosedHashmap:
         if not self._allocated:
             return None
         keys, _ = self._compact(True, False)
-        return keys.reshape(keys.shape[0], -1)
+        return keys.reshape(keys.shape[0], self._flat_key_size())
 
     def values(self):
         """Live value rows in the same order as ``keys()`` (reference: :168-172)."""
@@ -499,7 +499,7 @@ class CudaClosedHashmap:
         if not self._allocated:
             return None, None
         keys, values = self._compact(True, True)
-        return keys.reshape(keys.shape[0], -1), values
+        return keys.reshape(keys.shape[0], self._flat_key_size()), values
 
     def set_values(self, selectors, new_values):
         """Overwrite values of live entries picked by position in ``values()`` order (:174-177)."""

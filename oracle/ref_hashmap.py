@@ -200,7 +200,7 @@ class RefClosedHashmap:
         if self._keys is None:
             return None
         k = self._keys[self.nonempty_mask]
-        return k.view(self._key_dtype).reshape(k.shape[0], -1)
+        return k.view(self._key_dtype).reshape(k.shape[0], self._key_size)
 
     def values(self):                                                      # :168-172
         if self._values is None:

@@ -10,9 +10,10 @@ pytestmark = pytest.mark.gpu
 
 def _sorted_items(keys, values):
     """Order-independent view of a key->value map: rows sorted by key bytes."""
-    k = np.ascontiguousarray(keys).reshape(keys.shape[0], -1)
-    v = np.ascontiguousarray(values).reshape(values.shape[0], -1)
-    kb = k.view(np.uint8).reshape(k.shape[0], -1)
+    n = keys.shape[0]
+    k = np.ascontiguousarray(keys).reshape(n, int(np.prod(keys.shape[1:])))
+    v = np.ascontiguousarray(values).reshape(n, int(np.prod(values.shape[1:])))
+    kb = k.view(np.uint8).reshape(n, k.shape[1] * k.itemsize)
     order = np.lexsort(kb.T[::-1])
     return k[order], v[order]
 
@@ -23,8 +24,8 @@ def _assert_same_map(hm, ref):
     assert hm.n_elements == ref.n_elements == keys.shape[0] == rk.shape[0]
     a = _sorted_items(keys.cpu().numpy(), values.cpu().numpy())
     b = _sorted_items(rk, rv)
-    assert a[0].tobytes() == b[0].tobytes()
-    assert a[1].tobytes() == b[1].tobytes()
+    assert np.array_equal(a[0].view(np.uint8), b[0].view(np.uint8)), "key sets differ"
+    assert np.array_equal(a[1].view(np.uint8), b[1].view(np.uint8)), "values differ"
 
 
 def _unique_i64(rng, n, hi=2**62):
@@ -75,3 +76,236 @@ def test_cfg1_int64_scalar_keys(cuda):
     assert np.array_equal(f.cpu().numpy(), rf)
     assert np.array_equal(v.cpu().numpy(), rv)
     _assert_same_map(hm, ref)
+
+
+def _to(dev, *arrays):
+    return [torch.from_numpy(np.ascontiguousarray(a)).to(dev) for a in arrays]
+
+
+def _check_get(hm, ref, q, dev, fallback=None):
+    v, f = hm.get(torch.from_numpy(q).to(dev), fallback_value=fallback)
+    rv, rf = ref.get(q, fallback_value=fallback)
+    assert np.array_equal(f.cpu().numpy(), rf)
+    assert np.array_equal(np.ascontiguousarray(v.cpu().numpy()).view(np.uint8), np.ascontiguousarray(rv).view(np.uint8))
+
+
+def test_cfg2_float_triple_keys_wide_values(cuda):
+    """README-shaped map at 1/8 scale: float32[3] keys hashed over raw bytes, int64[5] values
+    (tagged layout): set, get hits+misses, remove 25 %, get again."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(1002)
+    n = 131072
+    keys = rng.random((n, 3), dtype=np.float32)
+    keys = np.unique(keys, axis=0)
+    rng.shuffle(keys)
+    n = keys.shape[0]
+    vals = rng.integers(0, 2**63 - 1, size=(n, 5), dtype=np.int64)
+    misses = rng.random((n, 3), dtype=np.float32) + 1.0            # disjoint from [0, 1)
+
+    hm = CudaClosedHashmap(n_buckets=2**18, device=cuda)
+    ref = RefClosedHashmap(n_buckets=2**18, rng=np.random.default_rng(8))
+    k, v = _to(cuda, keys, vals)
+    hm.set(k, v)
+    ref.set(keys, vals)
+    assert hm.n_elements == ref.n_elements == n and hm.n_buckets == ref.n_buckets
+    q = np.concatenate([keys, misses])[rng.permutation(2 * n)]
+    _check_get(hm, ref, q, cuda)
+    _check_get(hm, ref, q, cuda, fallback=-1)
+    gone = keys[rng.permutation(n)[: n // 4]]
+    m = hm.remove(torch.from_numpy(gone).to(cuda))
+    rm = ref.remove(gone)
+    assert np.array_equal(m.cpu().numpy(), rm) and hm.n_elements == ref.n_elements
+    _check_get(hm, ref, q, cuda)
+    _assert_same_map(hm, ref)
+    # overwrite half of the survivors and re-insert the removed quarter
+    again = np.unique(np.concatenate([keys[: n // 2], gone]), axis=0)    # no repeats inside the batch
+    vals2 = rng.integers(0, 2**63 - 1, size=(again.shape[0], 5), dtype=np.int64)
+    a, b = _to(cuda, again, vals2)
+    hm.set(a, b)
+    ref.set(again, vals2)
+    assert hm.n_elements == ref.n_elements
+    _assert_same_map(hm, ref)
+
+
+@pytest.mark.parametrize("key_shape,key_dtype,value_shape,value_dtype", [
+    ((1,), np.int64, (1,), np.float32),
+    ((1,), np.int64, (1,), np.float64),
+    ((1,), np.int64, (1,), np.float16),
+    ((1,), np.int64, (1,), np.int8),
+    ((1,), np.int32, (1,), np.int32),
+    ((2,), np.int32, (1,), np.int64),
+    ((1,), np.int16, (2,), np.int16),
+    ((2,), np.int64, (1,), np.float32),
+    ((4,), np.int64, (1,), np.float16),
+    ((3,), np.int16, (3,), np.int8),
+    ((5,), np.int8, (7,), np.int8),
+    ((1,), np.float64, (3,), np.float32),
+])
+def test_random_op_sequences_all_layouts(cuda, key_shape, key_dtype, value_shape, value_dtype):
+    """Random interleaved set / get / remove batches with many repeated keys, growing from 16
+    slots through several rehashes; state compared with the oracle after every step."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(77)
+    hm = CudaClosedHashmap(n_buckets=16, device=cuda)
+    ref = RefClosedHashmap(n_buckets=16, rng=np.random.default_rng(3))
+    universe = rng.integers(0, 40, size=(400, *key_shape)).astype(key_dtype)
+    for step in range(30):
+        op = rng.integers(0, 3)
+        idx = rng.permutation(universe.shape[0])[: rng.integers(0, 90)]
+        ks = int(np.prod(key_shape))
+        keys = np.unique(universe[idx].reshape(idx.shape[0], ks), axis=0).reshape(-1, *key_shape)
+        if op <= 1:
+            vals = rng.integers(-100, 100, size=(keys.shape[0], *value_shape)).astype(value_dtype)
+            k, v = _to(cuda, keys, vals)
+            hm.set(k, v)
+            ref.set(keys, vals)
+        elif hm._allocated:
+            m = hm.remove(torch.from_numpy(keys).to(cuda))
+            rm = ref.remove(keys)
+            assert np.array_equal(m.cpu().numpy(), rm)
+        if hm._allocated:
+            assert hm.n_elements == ref.n_elements
+            assert hm.n_buckets == ref.n_buckets
+            _check_get(hm, ref, universe, cuda, fallback=-7)
+            _assert_same_map(hm, ref)
+
+
+def test_equal_keys_inside_one_batch(cuda):
+    """Every key 64 times in one set batch: one slot per key, holding one of its values."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(5)
+    for key_shape, vshape, vdtype in [((1,), (1,), np.int64), ((3,), (5,), np.int64)]:
+        base = np.unique(rng.integers(0, 2**40, size=(3000, *key_shape), dtype=np.int64), axis=0)[:2048]
+        keys = np.repeat(base, 64, axis=0)
+        perm = rng.permutation(keys.shape[0])
+        keys = keys[perm]
+        # value rows carry (key id, copy id) so that a torn row would be visible
+        ids = np.repeat(np.arange(base.shape[0]), 64)[perm]
+        copy = rng.integers(0, 2**30, size=keys.shape[0])
+        vals = np.stack([ids * 2**32 + copy] * int(np.prod(vshape)), axis=1).reshape(-1, *vshape).astype(vdtype)
+        hm = CudaClosedHashmap(n_buckets=8192, device=cuda)
+        k, v = _to(cuda, keys, vals)
+        hm.set(k, v)
+        assert hm.n_elements == base.shape[0]
+        gk, gv = hm.items()
+        assert gk.shape[0] == base.shape[0]
+        out, found = hm.get(torch.from_numpy(base).to(cuda))
+        assert bool(found.all())
+        out = out.cpu().numpy().reshape(base.shape[0], -1)
+        assert (out == out[:, :1]).all(), "a value row mixes two writers"
+        written = {}
+        for i_, c_ in zip(ids, copy):
+            written.setdefault(int(i_), set()).add(int(c_))
+        for i_ in range(base.shape[0]):
+            assert out[i_, 0] >> 32 == i_ and int(out[i_, 0] & (2**32 - 1)) in written[i_]
+        # a second identical batch changes nothing but values
+        hm.set(k, v)
+        assert hm.n_elements == base.shape[0]
+        # removing with repeats removes each key once
+        m = hm._remove_rows(k)
+        assert int(m.sum().item()) == base.shape[0] and hm.n_elements == 0
+
+
+def test_reserved_patterns_and_extreme_keys(cuda):
+    """The packed layout keeps two key patterns in side slots; they and the extreme integers
+    must behave like any other key."""
+    from doksparse_amd import CudaClosedHashmap
+    X = np.uint64(0x9E3779B97F4A7C15)
+    special = np.array([X, X ^ np.uint64(1), 0, 1, np.uint64(2**64 - 1), np.uint64(2**63), np.uint64(2**63 - 1),
+                        np.uint64(2**64 - 3)], dtype=np.uint64).view(np.int64)[:, None]
+    vals = np.arange(1, special.shape[0] + 1, dtype=np.float32)[:, None]
+    hm = CudaClosedHashmap(n_buckets=64, device=cuda)
+    ref = RefClosedHashmap(n_buckets=64)
+    k, v = _to(cuda, special, vals)
+    hm.set(k, v)
+    ref.set(special, vals)
+    assert hm.n_elements == ref.n_elements == special.shape[0]
+    _check_get(hm, ref, special, cuda)
+    _assert_same_map(hm, ref)
+    hm.set(k, v * 2)                                    # overwrite: still 8 entries
+    ref.set(special, vals * 2)
+    assert hm.n_elements == special.shape[0]
+    _check_get(hm, ref, special, cuda)
+    m = hm.remove(k[:3])
+    rm = ref.remove(special[:3])
+    assert np.array_equal(m.cpu().numpy(), rm) and hm.n_elements == ref.n_elements
+    _check_get(hm, ref, special, cuda, fallback=9)
+    _assert_same_map(hm, ref)
+    hm.rehash(256)                                      # side slots survive a rehash
+    assert hm.n_elements == ref.n_elements
+    _check_get(hm, ref, special, cuda)
+
+
+def test_tiny_and_full_tables(cuda):
+    from doksparse_amd import CudaClosedHashmap
+    for vdtype in (np.float32, np.float64):
+        for cap in (1, 2, 3, 8):
+            hm = CudaClosedHashmap(n_buckets=cap, device=cuda, rehash_threshold=1.0)
+            ref = RefClosedHashmap(n_buckets=cap, rehash_threshold=1.0)
+            keys = (np.arange(cap, dtype=np.int64) * 1000003 + 17)[:, None]
+            vals = np.arange(cap, dtype=vdtype)[:, None] + 0.5
+            k, v = _to(cuda, keys, vals)
+            hm.set(k, v)
+            ref.set(keys, vals)
+            assert hm.n_elements == ref.n_elements == cap and hm.n_buckets == cap
+            q = np.concatenate([keys, keys + 1])
+            _check_get(hm, ref, q, cuda)
+            # tombstone everything, then reuse the slots
+            assert bool(hm.remove(k).all()) and hm.n_elements == 0
+            v2, f2 = hm.get(torch.from_numpy(q).to(cuda))
+            assert not bool(f2.any())
+            hm.set(k + 5, v)
+            assert hm.n_elements == cap
+            v3, f3 = hm.get(k + 5)
+            assert bool(f3.all()) and torch.equal(v3, v)
+    # a table that is physically full reports it
+    hm = CudaClosedHashmap(n_buckets=8, device=cuda, rehash_threshold=100.0)
+    n_slots = 10   # one packed bucket of 8-byte keys / 4-byte values
+    keys = torch.arange(n_slots + 6, device=cuda)[:, None]
+    hm.set(keys, torch.ones(n_slots + 6, 1, device=cuda))
+    with pytest.raises(RuntimeError, match="full"):
+        hm.n_elements
+
+
+def test_api_edges(cuda):
+    from doksparse_amd import CudaClosedHashmap
+    hm = CudaClosedHashmap(n_buckets=32, device=cuda)
+    hm.set(torch.zeros(0, 1, dtype=torch.long, device=cuda), torch.zeros(0, 1, device=cuda))
+    assert hm.n_elements == 0 and hm.key_shape == (1,) and hm.value_type == torch.float32
+    v, f = hm.get(torch.zeros(0, 1, dtype=torch.long, device=cuda))
+    assert v.shape == (0, 1) and f.shape == (0,) and f.dtype == torch.bool
+    assert hm.remove(torch.zeros(0, 1, dtype=torch.long, device=cuda)).shape == (0,)
+    with pytest.raises(AssertionError):
+        hm.set(torch.zeros(2, 1, dtype=torch.int32, device=cuda), torch.zeros(2, 1, device=cuda))
+    with pytest.raises(AssertionError):
+        hm.get(torch.zeros(2, 2, dtype=torch.long, device=cuda))
+    hm[torch.tensor([[4], [6]], device=cuda)] = torch.tensor([[1.0], [2.0]], device=cuda)
+    v, f = hm[torch.tensor([[6], [5]], device=cuda)]
+    assert v.flatten().tolist() == [2.0, 0.0] and f.tolist() == [True, False]
+    mask = hm.remove(torch.tensor([[6], [9], [6], [4]], device=cuda))     # over sorted unique rows 4, 6, 9
+    assert mask.tolist() == [True, True, False] and len(hm) == 0
+    # clone: shallow shares the table, deep does not
+    hm.set(torch.tensor([[1]], device=cuda), torch.tensor([[3.0]], device=cuda))
+    sh, dp = hm.clone(), hm.clone(deepclone=True)
+    hm.set(torch.tensor([[2]], device=cuda), torch.tensor([[4.0]], device=cuda))
+    assert sh.n_elements == 2 and dp.n_elements == 1
+    assert hm.load_factor == 2 / 32
+    # non-contiguous inputs are accepted
+    kk = torch.arange(20, device=cuda).reshape(10, 2)[:, :1]
+    hm.set(kk, torch.ones(10, 1, device=cuda))
+    assert bool(hm.get(kk)[1].all())
+    assert hm.count_existing(torch.arange(0, 25, device=cuda)[:, None]).item() == sum(
+        1 for x in range(25) if x in {1, 2} | set(range(0, 20, 2)))
+
+
+def test_probe_stats_are_in_the_expected_band(cuda):
+    """Mean buckets visited per lookup at load factor 0.5 with 10-slot buckets is barely above 1."""
+    from doksparse_amd import CudaClosedHashmap
+    g = torch.Generator(device=cuda).manual_seed(3)
+    n = 1 << 20
+    keys = torch.unique(torch.randint(0, 2**62, (n + 4096,), generator=g, device=cuda))[:n, None]
+    hm = CudaClosedHashmap(n_buckets=2 * n, device=cuda, rehash_threshold=1.0)
+    hm.set(keys, torch.randn(n, 1, device=cuda))
+    hits = hm.probe_stats(keys)
+    misses = hm.probe_stats(torch.randint(0, 2**62, (n, 1), generator=g, device=cuda))
+    assert 1.0 <= hits < 1.05 and 1.0 <= misses < 1.1
