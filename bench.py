@@ -158,6 +158,10 @@ def main():
     ap.add_argument("--cpu-keys", type=int, default=1 << 24)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--quick", action="store_true", help="skip the set and load-factor-0.9 legs")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run one read-only pass over the whole table (the live-entry count of "
+                         "the read-out path); with the table clear that every run does, this gives "
+                         "a profiler a read kernel and a write kernel of known size")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the hashmap path has no multi-GPU leg in this build "
@@ -187,13 +191,25 @@ def main():
     out_f = torch.empty(n, device=device, dtype=torch.bool)
     raw_get, raw_set, raw_clear = raw_calls(hm)
 
-    # correctness gate before any timing: hits return their value, misses are misses
+    # correctness gate before any timing: hits return their value, misses are misses.  The value
+    # check goes through the *_stats entry point, a separate kernel instantiation, so that a
+    # profiler's per-kernel average of the plain get kernel covers identical launches only.
     v, f = hm.get(queries[:, None])
     assert int(f.sum().item()) == n_hit, "unexpected hit count"
-    chk = torch.randperm(n, generator=gen, device=device)[: 1 << 20]
-    vv, ff = hm.get(keys[chk][:, None])
-    assert bool(ff.all()) and torch.equal(vv[:, 0], values[chk])
-    del v, f, vv, ff
+    chk = keys[torch.randperm(n, generator=gen, device=device)[: 1 << 20]].contiguous()
+    vv = torch.empty(chk.shape[0], 1, device=device, dtype=torch.float32)
+    ff = torch.empty(chk.shape[0], device=device, dtype=torch.bool)
+    from doksparse_amd import _lib as _dl
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    _dl.check(_dl.load().dok_map_get_stats(ctypes.byref(hm._desc), chk.data_ptr(), chk.shape[0], vv.data_ptr(),
+                                           None, ff.data_ptr(), _stream_ptr(device)), "get_stats")
+    vref, _ = hm.get(queries[:, None])          # same launch as the timed one; determinism check
+    assert bool(ff.all()) and torch.equal(v, vref)
+    idx = torch.searchsorted(torch.sort(keys).values, chk)      # independent of the table: sorted lookup
+    assert torch.equal(torch.sort(keys).values[idx], chk)
+    order = torch.argsort(keys)
+    assert torch.equal(vv[:, 0], values[order[idx]]), "get returned a wrong value"
+    del v, f, vv, ff, vref, idx, order
 
     for _ in range(args.warmup):
         hm.get(queries[:, None])
@@ -211,6 +227,9 @@ def main():
     results["get_kernel_ms_lf05"] = round(k_avg, 4)
     results["get_mops_lf05"] = round(n / k_avg / 1e3, 1)
     results["probe_len_lf05"] = round(hm.probe_stats(queries[:, None]), 4)
+    results["table_bytes_lf05"] = hm._n_phys * 128
+    if args.calibrate:
+        hm._compact(False, False)
 
     if not args.quick:
         s_avg, s_min = time_kernel(lambda: raw_set(keys, values), 5, prep=raw_clear)
