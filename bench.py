@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0
 # algorithmic bytes per op for 8-byte keys and 4-byte values: one 128-byte bucket line per op,
 # plus the batch row and the outputs
 B_GET = 8 + 128 + 4 + 1           # key in, bucket line, value out, flag out
-B_SET = 8 + 4 + 128 + 128         # key+value in, bucket line read, dirtied line written back
+B_SET = 8 + 4 + 128 + 128 + 1     # key+value in, bucket line read, dirtied line written back, flag
 
 
 def make_unique_keys(n, gen, device):
