@@ -21,6 +21,16 @@ typedef unsigned char u8;
 #define DOK_TPB 256          // threads per workgroup
 #define DOK_NONE32 0xffffffffu
 
+// Batch kernels walk the rows in tiles of DOK_TPB; a workgroup takes tiles blockIdx.x,
+// blockIdx.x + gridDim.x, ...  The host launches one workgroup per tile for kernels without
+// counters and a fixed, machine-filling grid for kernels that count (fresh inserts, removals,
+// hits): a wave then adds to the table header once, after its last tile, instead of once per
+// tile - a million same-address atomics would otherwise serialise the whole kernel.
+#define DOK_TILE_LOOP(n_rows)                                          \
+  const i64 n_tiles_ = ((i64)(n_rows) + DOK_TPB - 1) / DOK_TPB;        \
+  for (i64 tile_ = blockIdx.x; tile_ < n_tiles_; tile_ += gridDim.x)
+#define DOK_TILE_ROW() (tile_ * DOK_TPB + (i64)threadIdx.x)
+
 // Kernel-argument copy of dok_table_t plus what the host precomputes from it.
 struct DevTable {
   u64 *buckets;
@@ -78,7 +88,7 @@ __device__ __forceinline__ void dok_wave_add(i64 *counter, bool flag, i64 sign =
   if (m != 0 && (threadIdx.x & 63) == 0) atomicAdd((u64 *)counter, (u64)(sign * (i64)__popcll(m)));
 }
 __device__ __forceinline__ void dok_wave_add_n(i64 *counter, int v) {
-  // sum of a small per-lane non-negative int over the wave
+  // sum of a small per-lane int (either sign) over the wave, one atomic per wave
   #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   if (v != 0 && (threadIdx.x & 63) == 0) atomicAdd((u64 *)counter, (u64)(i64)v);

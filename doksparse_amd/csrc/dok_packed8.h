@@ -1,28 +1,33 @@
 // Packed layout: keys of at most 8 bytes, values of 1, 2, 4 or 8 bytes.
 //
-// A 128-byte bucket holds S = 128 / (8 + V) slots:
+// A 128-byte bucket holds S = 120 / (8 + V) slots and one metadata word:
 //     words 0 .. S-1           the S stored key words (8 bytes each)
 //     bytes 8*S .. 8*S + V*S   the S values, value s at byte 8*S + V*s
-// (V=4: 10 slots, V=8: 8, V=2: 12, V=1: 14).  The stored key word is  key XOR DOK_P8_XOR,
+//     word 15                  metadata: low 32 bits = the largest displacement (in buckets)
+//                              at which a key whose home is this bucket was ever placed
+// (V=4: 10 slots, V=8: 7, V=2: 12, V=1: 13).  The stored key word is  key XOR DOK_P8_XOR,
 // and the two words 0 and 1 mean EMPTY and TOMBSTONE, so a cleared table is all zero bytes and
 // the slot word itself is the target of the claiming 64-bit compare-and-swap: an insert is one
 // CAS plus one value store into the same line.  The two keys whose stored word would be 0 or 1
 // live in two side slots of the table header instead (state word + value word each).
 //
-// Probing is linear over buckets.  A chain ends at the first bucket that still has an EMPTY
-// slot; a bucket never regains an EMPTY slot (remove leaves a TOMBSTONE), so a key that was
-// placed past a full bucket stays reachable.
+// Probing is linear over buckets.  A lookup of a key with home bucket h visits h, h+1, ... and
+// stops at a match, at a bucket that still has an EMPTY slot (a bucket never regains one:
+// remove leaves a TOMBSTONE), or once it has gone further than h's recorded largest
+// displacement.  The last rule is what keeps misses short in a nearly full table: most home
+// buckets never overflowed, so a miss is decided by the home bucket alone.
 #pragma once
 #include "dok_device.h"
 
 #define DOK_P8_XOR   0x9E3779B97F4A7C15ULL
 #define DOK_P8_EMPTY 0ULL
 #define DOK_P8_TOMB  1ULL
+#define DOK_P8_META  15       // word index of the bucket metadata
 #define DOK_H_SIDE_STATE 8    // header words 8,9: side slot occupied (0/1)
 #define DOK_H_SIDE_VALUE 10   // header words 10,11: side slot values
 
 template <int V> struct P8 {
-  static constexpr int S = 128 / (8 + V);
+  static constexpr int S = 120 / (8 + V);
   __device__ static __forceinline__ u64 extract(u64 vword, int s) {
     if (V == 8) return vword;
     return (vword >> (((s * V) & 7) * 8)) & ((1ULL << (8 * (V & 7))) - 1ULL);
@@ -46,8 +51,7 @@ __device__ __forceinline__ u32 p8_home(u64 sk, const DevTable &t) {
 // Phase 1 serves the home bucket of each of the group's 16 rows.  It is written as "issue U
 // loads, then resolve U rounds" with no branch in between, so that a wave keeps U*4 bucket
 // lines in flight; everything a round decides is folded into the owner lane with selects.
-// Phase 2 walks the few rows whose home bucket was full and held no match, one row per group
-// per turn.
+// Phase 2 walks the few rows whose home bucket overflowed, one row per group per turn.
 #define DOK_P8_U 8
 template <int V>
 __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 nb, u64 sk, u32 b,
@@ -59,6 +63,7 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
   const int l = lane & 15;
   const bool inb = l < S;
   const u32 home = b;
+  u32 maxd = 0;                 // largest displacement recorded in the row's home bucket
   slot_b = home;
 
   const u64 pend0 = dok_ballot(pend);
@@ -83,6 +88,7 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
         const u64 be = dok_ballot(has && inb && w[u] == DOK_P8_EMPTY);
         const u32 gm = (u32)(bm >> gbase) & 0xffffu;
         const u32 ge = (u32)(be >> gbase) & 0xffffu;
+        const u32 md = dok_shfl32((u32)w[u], gbase + DOK_P8_META);
         const int s = gm ? __builtin_ctz(gm) : 0;
         const u64 vword = dok_shfl64(w[u], gbase + P8<V>::value_word(s));
         const bool mine = has && l == r;
@@ -90,14 +96,15 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
         found = found || hit;
         val = hit ? P8<V>::extract(vword, s) : val;
         slot_s = hit ? s : slot_s;
-        pend = pend && !(mine && (gm | ge) != 0);
+        maxd = mine ? md : maxd;
+        pend = pend && !(mine && ((gm | ge) != 0 || md == 0));
       }
     }
   }
   nprobe += (pend0 >> lane) & 1ULL;
 
   // Phase 2
-  u64 iters = 1;
+  u32 d = 1;
   if (pend) b = (home + 1 == nb) ? 0u : home + 1;
   if (pend && nb == 1) pend = false;
   u64 pm = dok_ballot(pend);
@@ -123,7 +130,8 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
         pend = false;
       } else {
         b = (b + 1 == nb) ? 0u : b + 1;
-        if (++iters >= nb) pend = false;      // walked the whole ring: absent
+        d++;
+        if (d > maxd || d >= nb) pend = false;   // beyond every key homed at `home`: absent
       }
     }
     pm = dok_ballot(pend);
@@ -137,11 +145,23 @@ __device__ __forceinline__ bool p8_side_get(const DevTable &t, u64 sk, u64 &val)
 }
 
 // ---- cooperative upsert -------------------------------------------------------------------
-// In: per-lane stored key, value, `pend`.  Out: st (1 placed / 0 table full), fresh (took a new
-// slot).  All table reads are device-coherent: other workgroups insert into the same buckets
-// during the kernel.  The claim is one CAS on the slot's key word; whoever loses re-examines:
-// if the winner wrote the same key (equal keys inside one batch) the loser is done and the
-// winner's value stands, otherwise it restarts from its home bucket.
+// In: per-lane stored key, value, home bucket, `pend`.  Out: st (1 placed / 0 table full),
+// fresh (took a new slot).
+//
+// The claim is one CAS on the slot's key word; whoever loses re-examines: if the winner wrote
+// the same key (equal keys inside one batch) the loser is done and the winner's value stands,
+// otherwise it walks again.  A key absent from the table takes the first tombstone on its chain,
+// else the first empty slot of the chain-end bucket.  Because slots only ever move
+// EMPTY/TOMBSTONE -> key inside a set kernel, two rows with the same key can never both win a
+// claim: the later one either sees the earlier one's key or competes for the same slot.  The
+// same monotonicity makes a stale (cached) view of a bucket harmless - it can only show a slot
+// as free that is in fact taken, and the CAS then fails - so phase 1 uses plain loads; the
+// retry loop reads device-coherently.
+//
+// Phase 1 inspects the home bucket of all 64 rows (batched loads as in the lookup), then the
+// whole wave issues its CAS / value stores together.  Phase 2 is the general walk for rows whose
+// home bucket was full or whose claim was lost.  A key placed d > 0 buckets past its home
+// raises the home bucket's recorded largest displacement to d.
 template <int V>
 __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val, u32 home,
                                           bool pend, int &st, int &fresh) {
@@ -150,10 +170,65 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
   const int gbase = lane & 48;
   const int l = lane & 15;
   const bool inb = l < S;
-  u32 b = home;
-  u32 tomb_b = DOK_NONE32;
+
+  int act = 0;                  // 0 walk on, 1 overwrite slot, 2 claim slot
+  int slot = 0;
+  bool tomb_here = false;       // the chosen slot of the home bucket is a tombstone
+  u32 md_home = 0;
+
+  const u64 pend0 = dok_ballot(pend);
+  if (pend0 != 0) {
+    const u32 gp = (u32)(pend0 >> gbase) & 0xffffu;
+    #pragma unroll
+    for (int r0 = 0; r0 < 16; r0 += DOK_P8_U) {
+      u64 w[DOK_P8_U];
+      #pragma unroll
+      for (int u = 0; u < DOK_P8_U; u++) {
+        const int r = r0 + u;
+        const u32 qb = dok_shfl32(home, gbase + r);
+        const bool has = (gp >> r) & 1u;
+        w[u] = buckets[(u64)(has ? qb : 0u) * 16 + l];
+      }
+      #pragma unroll
+      for (int u = 0; u < DOK_P8_U; u++) {
+        const int r = r0 + u;
+        const bool has = (gp >> r) & 1u;
+        const u64 q = dok_shfl64(sk, gbase + r);
+        const u32 gm = (u32)(dok_ballot(has && inb && w[u] == q) >> gbase) & 0xffffu;
+        const u32 ge = (u32)(dok_ballot(has && inb && w[u] == DOK_P8_EMPTY) >> gbase) & 0xffffu;
+        const u32 gt = (u32)(dok_ballot(has && inb && w[u] == DOK_P8_TOMB) >> gbase) & 0xffffu;
+        const u32 md = dok_shfl32((u32)w[u], gbase + DOK_P8_META);
+        const bool mine = has && l == r;
+        const int a = gm ? 1 : (ge ? 2 : 0);
+        const u32 pick = gm ? gm : (gt ? gt : ge);
+        act = mine ? a : act;
+        slot = mine ? (pick ? __builtin_ctz(pick) : 0) : slot;
+        tomb_here = mine ? (gm == 0 && gt != 0) : tomb_here;
+        md_home = mine ? md : md_home;
+      }
+    }
+  }
+
+  u64 *hb = buckets + (u64)home * 16;
+  u32 b = home, d = 0;
+  u32 tomb_b = DOK_NONE32, tomb_d = 0;
   int tomb_s = 0;
   u64 iters = 0;
+  if (pend && act == 1) {
+    P8<V>::store(hb, slot, val);
+    st = 1; pend = false;
+  } else if (pend && act == 2) {
+    const u64 expect = tomb_here ? DOK_P8_TOMB : DOK_P8_EMPTY;
+    const u64 old = atomicCAS(hb + slot, expect, sk);
+    if (old == expect) { P8<V>::store(hb, slot, val); st = 1; fresh = 1; pend = false; }
+    else if (old == sk) { st = 1; pend = false; }
+    // else: lost to another key; phase 2 starts over at the home bucket
+  } else if (pend) {
+    // home bucket full without a match: walk on, remembering its first tombstone
+    if (tomb_here) { tomb_b = home; tomb_s = slot; tomb_d = 0; }
+    b = (home + 1 == nb) ? 0u : home + 1;
+    d = 1; iters = 1;
+  }
 
   u64 pm = dok_ballot(pend);
   while (pm != 0) {
@@ -164,42 +239,40 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
     const u64 q = dok_shfl64(sk, j);
     const u32 qb = dok_shfl32(b, j);
     const u64 w = dok_load_coherent(buckets + (u64)(has ? qb : 0u) * 16 + l);
-    const u64 bm = dok_ballot(has && inb && w == q);
-    const u64 be = dok_ballot(has && inb && w == DOK_P8_EMPTY);
-    const u64 bt = dok_ballot(has && inb && w == DOK_P8_TOMB);
-    const u32 gm = (u32)(bm >> gbase) & 0xffffu;
-    const u32 ge = (u32)(be >> gbase) & 0xffffu;
-    const u32 gt = (u32)(bt >> gbase) & 0xffffu;
+    const u32 gm = (u32)(dok_ballot(has && inb && w == q) >> gbase) & 0xffffu;
+    const u32 ge = (u32)(dok_ballot(has && inb && w == DOK_P8_EMPTY) >> gbase) & 0xffffu;
+    const u32 gt = (u32)(dok_ballot(has && inb && w == DOK_P8_TOMB) >> gbase) & 0xffffu;
     if (has && l == r) {
       if (gm) {
         // key present: overwrite its value in place
         P8<V>::store(buckets + (u64)b * 16, __builtin_ctz(gm), val);
         st = 1; pend = false;
       } else {
-        if (tomb_b == DOK_NONE32 && gt) { tomb_b = b; tomb_s = __builtin_ctz(gt); }
+        if (tomb_b == DOK_NONE32 && gt) { tomb_b = b; tomb_s = __builtin_ctz(gt); tomb_d = d; }
         const bool ring_done = (ge == 0) && (++iters >= nb);
         if (ge || ring_done) {
-          // chain end: the key is absent.  Take the first tombstone seen on the way, else the
-          // first empty slot of this bucket.
+          // chain end: the key is absent
           if (tomb_b == DOK_NONE32 && ge == 0) {
             st = 0; pend = false;                       // no free slot anywhere
           } else {
-            u32 tb; int ts; u64 expect;
-            if (tomb_b != DOK_NONE32) { tb = tomb_b; ts = tomb_s; expect = DOK_P8_TOMB; }
-            else { tb = b; ts = __builtin_ctz(ge); expect = DOK_P8_EMPTY; }
+            u32 tb, td; int ts; u64 expect;
+            if (tomb_b != DOK_NONE32) { tb = tomb_b; ts = tomb_s; td = tomb_d; expect = DOK_P8_TOMB; }
+            else { tb = b; ts = __builtin_ctz(ge); td = d; expect = DOK_P8_EMPTY; }
             u64 *tp = buckets + (u64)tb * 16;
             const u64 old = atomicCAS(tp + ts, expect, sk);
             if (old == expect) {
               P8<V>::store(tp, ts, val);
+              if (td > md_home) atomicMax((u32 *)(hb + DOK_P8_META), td);
               st = 1; fresh = 1; pend = false;
             } else if (old == sk) {
               st = 1; pend = false;                     // an equal key of this batch won the slot
             } else {
-              b = home; tomb_b = DOK_NONE32; iters = 0; // somebody else's key: look again
+              b = home; d = 0; tomb_b = DOK_NONE32; iters = 0;   // somebody else's key: look again
             }
           }
         } else {
           b = (b + 1 == nb) ? 0u : b + 1;
+          d++;
         }
       }
     }
@@ -215,29 +288,33 @@ __device__ __forceinline__ int p8_side_set(const DevTable &t, u64 sk, u64 val) {
 }
 
 // ---- kernels ------------------------------------------------------------------------------
-
 template <int V, bool STATS>
 __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                          void *__restrict__ values, u8 *__restrict__ found_out,
                                                          u64 fallback) {
-  const i64 i = (i64)blockIdx.x * DOK_TPB + threadIdx.x;
-  const bool active = i < n;
-  u64 key = 0;
-  const bool ok = active && dok_load_key8(t, keys, i, key);
-  const u64 sk = key ^ DOK_P8_XOR;
-  bool found = false;
-  u64 val = fallback;
-  bool pend = ok;
-  if (ok && sk < 2) { found = p8_side_get(t, sk, val); pend = false; }
-  u32 sb = 0; int ss = 0, nprobe = 0;
-  p8_lookup<V>(t.buckets, t.nb, sk, pend ? p8_home(sk, t) : 0u, pend, found, val, sb, ss, nprobe);
-  if (active) {
-    dok_store_val<V>(values, i, val);
-    found_out[i] = found ? 1 : 0;
+  int n_probe = 0, n_ops = 0;
+  DOK_TILE_LOOP(n) {
+    const i64 i = DOK_TILE_ROW();
+    const bool active = i < n;
+    u64 key = 0;
+    const bool ok = active && dok_load_key8(t, keys, i, key);
+    const u64 sk = key ^ DOK_P8_XOR;
+    bool found = false;
+    u64 val = fallback;
+    bool pend = ok;
+    if (ok && sk < 2) { found = p8_side_get(t, sk, val); pend = false; }
+    u32 sb = 0; int ss = 0, nprobe = 0;
+    p8_lookup<V>(t.buckets, t.nb, sk, pend ? p8_home(sk, t) : 0u, pend, found, val, sb, ss, nprobe);
+    if (active) {
+      dok_store_val<V>(values, i, val);
+      found_out[i] = found ? 1 : 0;
+    }
+    n_probe += nprobe;
+    n_ops += active;
   }
   if (STATS) {
-    dok_wave_add_n(&t.header[DOK_H_NPROBE], nprobe);
-    dok_wave_add(&t.header[DOK_H_NOPS], active);
+    dok_wave_add_n(&t.header[DOK_H_NPROBE], n_probe);
+    dok_wave_add_n(&t.header[DOK_H_NOPS], n_ops);
   }
 }
 
@@ -245,60 +322,74 @@ template <int V>
 __global__ __launch_bounds__(DOK_TPB) void p8_set_kernel(DevTable t, const void *__restrict__ keys,
                                                          const void *__restrict__ values, i64 n,
                                                          u8 *__restrict__ stored) {
-  const i64 i = (i64)blockIdx.x * DOK_TPB + threadIdx.x;
-  const bool active = i < n;
-  u64 key = 0;
-  const bool ok = active && dok_load_key8(t, keys, i, key);
-  const u64 sk = key ^ DOK_P8_XOR;
-  const u64 val = ok ? dok_load_val<V>(values, i) : 0;
-  int st = 0, fresh = 0;
-  bool pend = ok;
-  if (ok && sk < 2) { fresh = p8_side_set(t, sk, val); st = 1; pend = false; }
-  p8_insert<V>(t.buckets, t.nb, sk, val, pend ? p8_home(sk, t) : 0u, pend, st, fresh);
-  if (active && stored) stored[i] = (u8)st;
-  dok_wave_add(&t.header[DOK_H_NELEM], fresh != 0);
-  dok_wave_add(&t.header[DOK_H_NFULL], ok && st == 0);
-  dok_wave_add(&t.header[DOK_H_NOOB], active && !ok);
+  int n_fresh = 0, n_full = 0, n_oob = 0;
+  DOK_TILE_LOOP(n) {
+    const i64 i = DOK_TILE_ROW();
+    const bool active = i < n;
+    u64 key = 0;
+    const bool ok = active && dok_load_key8(t, keys, i, key);
+    const u64 sk = key ^ DOK_P8_XOR;
+    const u64 val = ok ? dok_load_val<V>(values, i) : 0;
+    int st = 0, fresh = 0;
+    bool pend = ok;
+    if (ok && sk < 2) { fresh = p8_side_set(t, sk, val); st = 1; pend = false; }
+    p8_insert<V>(t.buckets, t.nb, sk, val, pend ? p8_home(sk, t) : 0u, pend, st, fresh);
+    if (active && stored) stored[i] = (u8)st;
+    n_fresh += fresh;
+    n_full += (ok && st == 0);
+    n_oob += (active && !ok);
+  }
+  dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
+  dok_wave_add_n(&t.header[DOK_H_NFULL], n_full);
+  dok_wave_add_n(&t.header[DOK_H_NOOB], n_oob);
 }
 
 // Tombstone the matching slot with a CAS so that equal keys in one batch remove it once.
 template <int V>
 __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                             u8 *__restrict__ removed_out) {
-  const i64 i = (i64)blockIdx.x * DOK_TPB + threadIdx.x;
-  const bool active = i < n;
-  u64 key = 0;
-  const bool ok = active && dok_load_key8(t, keys, i, key);
-  const u64 sk = key ^ DOK_P8_XOR;
-  bool found = false, removed = false;
-  u64 val = 0;
-  bool pend = ok;
-  if (ok && sk < 2) {
-    removed = atomicExch((u64 *)&t.header[DOK_H_SIDE_STATE + sk], 0ULL) != 0;
-    pend = false;
+  int n_removed = 0;
+  DOK_TILE_LOOP(n) {
+    const i64 i = DOK_TILE_ROW();
+    const bool active = i < n;
+    u64 key = 0;
+    const bool ok = active && dok_load_key8(t, keys, i, key);
+    const u64 sk = key ^ DOK_P8_XOR;
+    bool found = false, removed = false;
+    u64 val = 0;
+    bool pend = ok;
+    if (ok && sk < 2) {
+      removed = atomicExch((u64 *)&t.header[DOK_H_SIDE_STATE + sk], 0ULL) != 0;
+      pend = false;
+    }
+    u32 sb = 0; int ss = 0, nprobe = 0;
+    p8_lookup<V>(t.buckets, t.nb, sk, pend ? p8_home(sk, t) : 0u, pend, found, val, sb, ss, nprobe);
+    if (found) removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
+    if (active && removed_out) removed_out[i] = removed ? 1 : 0;
+    n_removed += removed;
   }
-  u32 sb = 0; int ss = 0, nprobe = 0;
-  p8_lookup<V>(t.buckets, t.nb, sk, pend ? p8_home(sk, t) : 0u, pend, found, val, sb, ss, nprobe);
-  if (found) removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
-  if (active && removed_out) removed_out[i] = removed ? 1 : 0;
-  dok_wave_add(&t.header[DOK_H_NELEM], removed, -1);
+  dok_wave_add_n(&t.header[DOK_H_NELEM], -n_removed);
 }
 
 template <int V>
 __global__ __launch_bounds__(DOK_TPB) void p8_count_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                            i64 *count) {
-  const i64 i = (i64)blockIdx.x * DOK_TPB + threadIdx.x;
-  const bool active = i < n;
-  u64 key = 0;
-  const bool ok = active && dok_load_key8(t, keys, i, key);
-  const u64 sk = key ^ DOK_P8_XOR;
-  bool found = false;
-  u64 val = 0;
-  bool pend = ok;
-  if (ok && sk < 2) { found = p8_side_get(t, sk, val); pend = false; }
-  u32 sb = 0; int ss = 0, nprobe = 0;
-  p8_lookup<V>(t.buckets, t.nb, sk, pend ? p8_home(sk, t) : 0u, pend, found, val, sb, ss, nprobe);
-  dok_wave_add(count, found);
+  int n_found = 0;
+  DOK_TILE_LOOP(n) {
+    const i64 i = DOK_TILE_ROW();
+    const bool active = i < n;
+    u64 key = 0;
+    const bool ok = active && dok_load_key8(t, keys, i, key);
+    const u64 sk = key ^ DOK_P8_XOR;
+    bool found = false;
+    u64 val = 0;
+    bool pend = ok;
+    if (ok && sk < 2) { found = p8_side_get(t, sk, val); pend = false; }
+    u32 sb = 0; int ss = 0, nprobe = 0;
+    p8_lookup<V>(t.buckets, t.nb, sk, pend ? p8_home(sk, t) : 0u, pend, found, val, sb, ss, nprobe);
+    n_found += found;
+  }
+  dok_wave_add_n(count, n_found);
 }
 
 // ---- table scans: read-out, rehash, densify ------------------------------------------------
@@ -452,58 +543,74 @@ __global__ __launch_bounds__(DOK_TPB) void p8_to_dense_kernel(DevTable t, void *
 
 template <int V>
 __global__ __launch_bounds__(DOK_TPB) void p8_getitem_kernel(DevTable t, DevIndex ix, void *__restrict__ out) {
-  const i64 e = (i64)blockIdx.x * DOK_TPB + threadIdx.x;
-  const bool active = e < ix.n_elems;
-  u64 key = 0; i64 voff = 0;
-  const bool ok = active && dok_gather_key(t, ix, e, key, voff);
-  const u64 sk = key ^ DOK_P8_XOR;
-  bool found = false;
-  u64 val = 0;
-  u32 sb = 0; int ss = 0, nprobe = 0;
-  p8_lookup<V>(t.buckets, t.nb, sk, ok ? p8_home(sk, t) : 0u, ok, found, val, sb, ss, nprobe);
-  if (active) dok_store_val<V>(out, e, val);
+  DOK_TILE_LOOP(ix.n_elems) {
+    const i64 e = DOK_TILE_ROW();
+    const bool active = e < ix.n_elems;
+    u64 key = 0; i64 voff = 0;
+    const bool ok = active && dok_gather_key(t, ix, e, key, voff);
+    const u64 sk = key ^ DOK_P8_XOR;
+    bool found = false;
+    u64 val = 0;
+    u32 sb = 0; int ss = 0, nprobe = 0;
+    p8_lookup<V>(t.buckets, t.nb, sk, ok ? p8_home(sk, t) : 0u, ok, found, val, sb, ss, nprobe);
+    if (active) dok_store_val<V>(out, e, val);
+  }
 }
 
 template <int V>
 __global__ __launch_bounds__(DOK_TPB) void p8_setitem_kernel(DevTable t, DevIndex ix) {
-  const i64 e = (i64)blockIdx.x * DOK_TPB + threadIdx.x;
-  const bool active = e < ix.n_elems;
-  u64 key = 0; i64 voff = 0;
-  const bool ok = active && dok_gather_key(t, ix, e, key, voff);
-  const u64 sk = key ^ DOK_P8_XOR;
-  const u64 val = ok ? dok_load_val<V>(ix.src, voff) : 0;
-  int st = 0, fresh = 0;
-  p8_insert<V>(t.buckets, t.nb, sk, val, ok ? p8_home(sk, t) : 0u, ok, st, fresh);
-  dok_wave_add(&t.header[DOK_H_NELEM], fresh != 0);
-  dok_wave_add(&t.header[DOK_H_NFULL], ok && st == 0);
-  dok_wave_add(&t.header[DOK_H_NOOB], active && !ok);
+  int n_fresh = 0, n_full = 0, n_oob = 0;
+  DOK_TILE_LOOP(ix.n_elems) {
+    const i64 e = DOK_TILE_ROW();
+    const bool active = e < ix.n_elems;
+    u64 key = 0; i64 voff = 0;
+    const bool ok = active && dok_gather_key(t, ix, e, key, voff);
+    const u64 sk = key ^ DOK_P8_XOR;
+    const u64 val = ok ? dok_load_val<V>(ix.src, voff) : 0;
+    int st = 0, fresh = 0;
+    p8_insert<V>(t.buckets, t.nb, sk, val, ok ? p8_home(sk, t) : 0u, ok, st, fresh);
+    n_fresh += fresh;
+    n_full += (ok && st == 0);
+    n_oob += (active && !ok);
+  }
+  dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
+  dok_wave_add_n(&t.header[DOK_H_NFULL], n_full);
+  dok_wave_add_n(&t.header[DOK_H_NOOB], n_oob);
 }
 
 template <int V>
 __global__ __launch_bounds__(DOK_TPB) void p8_countitems_kernel(DevTable t, DevIndex ix, i64 *count) {
-  const i64 e = (i64)blockIdx.x * DOK_TPB + threadIdx.x;
-  const bool active = e < ix.n_elems;
-  u64 key = 0; i64 voff = 0;
-  const bool ok = active && dok_gather_key(t, ix, e, key, voff);
-  const u64 sk = key ^ DOK_P8_XOR;
-  bool found = false;
-  u64 val = 0;
-  u32 sb = 0; int ss = 0, nprobe = 0;
-  p8_lookup<V>(t.buckets, t.nb, sk, ok ? p8_home(sk, t) : 0u, ok, found, val, sb, ss, nprobe);
-  dok_wave_add(count, found);
+  int n_found = 0;
+  DOK_TILE_LOOP(ix.n_elems) {
+    const i64 e = DOK_TILE_ROW();
+    const bool active = e < ix.n_elems;
+    u64 key = 0; i64 voff = 0;
+    const bool ok = active && dok_gather_key(t, ix, e, key, voff);
+    const u64 sk = key ^ DOK_P8_XOR;
+    bool found = false;
+    u64 val = 0;
+    u32 sb = 0; int ss = 0, nprobe = 0;
+    p8_lookup<V>(t.buckets, t.nb, sk, ok ? p8_home(sk, t) : 0u, ok, found, val, sb, ss, nprobe);
+    n_found += found;
+  }
+  dok_wave_add_n(count, n_found);
 }
 
 template <int V>
 __global__ __launch_bounds__(DOK_TPB) void p8_zeroitems_kernel(DevTable t, DevIndex ix) {
-  const i64 e = (i64)blockIdx.x * DOK_TPB + threadIdx.x;
-  const bool active = e < ix.n_elems;
-  u64 key = 0; i64 voff = 0;
-  const bool ok = active && dok_gather_key(t, ix, e, key, voff);
-  const u64 sk = key ^ DOK_P8_XOR;
-  bool found = false, removed = false;
-  u64 val = 0;
-  u32 sb = 0; int ss = 0, nprobe = 0;
-  p8_lookup<V>(t.buckets, t.nb, sk, ok ? p8_home(sk, t) : 0u, ok, found, val, sb, ss, nprobe);
-  if (found) removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
-  dok_wave_add(&t.header[DOK_H_NELEM], removed, -1);
+  int n_removed = 0;
+  DOK_TILE_LOOP(ix.n_elems) {
+    const i64 e = DOK_TILE_ROW();
+    const bool active = e < ix.n_elems;
+    u64 key = 0; i64 voff = 0;
+    const bool ok = active && dok_gather_key(t, ix, e, key, voff);
+    const u64 sk = key ^ DOK_P8_XOR;
+    bool found = false, removed = false;
+    u64 val = 0;
+    u32 sb = 0; int ss = 0, nprobe = 0;
+    p8_lookup<V>(t.buckets, t.nb, sk, ok ? p8_home(sk, t) : 0u, ok, found, val, sb, ss, nprobe);
+    if (found) removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
+    n_removed += removed;
+  }
+  dok_wave_add_n(&t.header[DOK_H_NELEM], -n_removed);
 }

@@ -124,7 +124,9 @@ __device__ __forceinline__ TgView tg_inspect(const TgGeom &g, const TgLane &L, b
   return v;
 }
 
-// mode 0: get (write value or fallback + flag), 1: count, 2: remove
+// mode 0: get (write value or fallback + flag), 1: count, 2: remove.
+// Rows are taken in tiles of DOK_TPB (see DOK_TILE_LOOP); a wave only ever reads the LDS rows its
+// own lanes staged, so the tiles need no workgroup barrier between them.
 template <int MODE, bool STATS>
 __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g, const u8 *__restrict__ keys, i64 n,
                                                             u8 *__restrict__ values, u8 *__restrict__ flags,
@@ -132,74 +134,77 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
   extern __shared__ u64 lds[];
   u64 *lds_keys = lds;                          // [DOK_TPB][KW]
   u64 *lds_fb = lds + DOK_TPB * g.KW;           // [VW]
-  const i64 i = (i64)blockIdx.x * DOK_TPB + threadIdx.x;
-  const bool active = i < n;
-  u32 b; u64 tag_full;
-  tg_stage(t, g, keys, i, active, lds_keys, b, tag_full);
   if (MODE == 0 && threadIdx.x < g.VW) lds_fb[threadIdx.x] = g.fallback[threadIdx.x];
   __syncthreads();
-
   const TgLane L(g);
   const int wave_row0 = threadIdx.x & ~63;      // first LDS row of this wave
-  const i64 wave_i0 = i - L.lane;               // batch row of lane 0
-  bool pend = active, found = false, removed = false;
-  u64 iters = 0;
-  int nprobe = 0;
+  int n_found = 0, n_removed = 0, n_probe = 0, n_ops = 0;
 
-  u64 pm = dok_ballot(pend);
-  while (pm != 0) {
-    const u32 sub = (u32)(pm >> L.gbase) & 0xffffu;
-    const bool has = sub != 0;
-    const int r = has ? __builtin_ctz(sub) : 0;
-    const int j = L.gbase + r;
-    const u32 qb = dok_shfl32(b, j);
-    const u64 qfull = dok_shfl64(tag_full, j);
-    const u64 w = t.buckets[(u64)(has ? qb : 0u) * 16 + L.l];
-    const TgView v = tg_inspect(g, L, has, w, qfull, lds_keys + (wave_row0 + j) * g.KW);
-    const bool resolved = v.hit != 0 || v.empty != 0;
-    if (MODE == 0 && has && resolved) {
-      // the value lanes of the matching slot (or, on a miss, of slot 0 with the fallback) write
-      // the output row directly
-      const int hit_slot = v.hit ? (__builtin_ctz(v.hit) / g.W) : 0;
-      if (L.is_val && L.slot == hit_slot) {
-        const int k = L.p - 1 - g.KW;
-        const u64 word = v.hit ? w : lds_fb[k];
-        tg_store_word(values + (size_t)(wave_i0 + j) * g.V, k, g.V, g.unit_v, word);
-      }
-    }
-    if (has && L.l == r) {
-      nprobe++;
-      if (v.hit) {
-        found = true; pend = false;
-        if (MODE == 2) {
-          u64 *tagp = t.buckets + (u64)b * 16 + __builtin_ctz(v.hit);
-          removed = atomicCAS(tagp, qfull, DOK_TG_TOMB) == qfull;
+  DOK_TILE_LOOP(n) {
+    const i64 i = DOK_TILE_ROW();
+    const bool active = i < n;
+    u32 b; u64 tag_full;
+    tg_stage(t, g, keys, i, active, lds_keys, b, tag_full);
+    const i64 wave_i0 = i - L.lane;             // batch row of lane 0
+    bool pend = active, found = false, removed = false;
+    u64 iters = 0;
+
+    u64 pm = dok_ballot(pend);
+    while (pm != 0) {
+      const u32 sub = (u32)(pm >> L.gbase) & 0xffffu;
+      const bool has = sub != 0;
+      const int r = has ? __builtin_ctz(sub) : 0;
+      const int j = L.gbase + r;
+      const u32 qb = dok_shfl32(b, j);
+      const u64 qfull = dok_shfl64(tag_full, j);
+      const u64 w = t.buckets[(u64)(has ? qb : 0u) * 16 + L.l];
+      const TgView v = tg_inspect(g, L, has, w, qfull, lds_keys + (wave_row0 + j) * g.KW);
+      const bool resolved = v.hit != 0 || v.empty != 0;
+      if (MODE == 0 && has && resolved) {
+        // the value lanes of the matching slot (or, on a miss, of slot 0 with the fallback)
+        // write the output row directly
+        const int hit_slot = v.hit ? (__builtin_ctz(v.hit) / g.W) : 0;
+        if (L.is_val && L.slot == hit_slot) {
+          const int k = L.p - 1 - g.KW;
+          const u64 word = v.hit ? w : lds_fb[k];
+          tg_store_word(values + (size_t)(wave_i0 + j) * g.V, k, g.V, g.unit_v, word);
         }
-      } else if (v.empty) {
-        pend = false;
-      } else {
-        b = (b + 1 == t.nb) ? 0u : b + 1;
-        if (++iters >= t.nb) {
+      }
+      if (has && L.l == r) {
+        n_probe++;
+        if (v.hit) {
+          found = true; pend = false;
+          if (MODE == 2) {
+            u64 *tagp = t.buckets + (u64)b * 16 + __builtin_ctz(v.hit);
+            removed = atomicCAS(tagp, qfull, DOK_TG_TOMB) == qfull;
+          }
+        } else if (v.empty) {
           pend = false;
-          if (MODE == 0) {
-            // full ring without an empty slot: absent; the owner writes the fallback itself
-            for (int k = 0; k < g.VW; k++)
-              tg_store_word(values + (size_t)i * g.V, k, g.V, g.unit_v, lds_fb[k]);
+        } else {
+          b = (b + 1 == t.nb) ? 0u : b + 1;
+          if (++iters >= t.nb) {
+            pend = false;
+            if (MODE == 0) {
+              // full ring without an empty slot: absent; the owner writes the fallback itself
+              for (int k = 0; k < g.VW; k++)
+                tg_store_word(values + (size_t)i * g.V, k, g.V, g.unit_v, lds_fb[k]);
+            }
           }
         }
       }
+      pm = dok_ballot(pend);
     }
-    pm = dok_ballot(pend);
+    if (MODE == 0 && active) flags[i] = found ? 1 : 0;
+    if (MODE == 2 && active && flags) flags[i] = removed ? 1 : 0;
+    n_found += found;
+    n_removed += removed;
+    n_ops += active;
   }
-  if (MODE == 0 && active) flags[i] = found ? 1 : 0;
-  if (MODE == 1) dok_wave_add(count, found);
-  if (MODE == 2) {
-    if (active && flags) flags[i] = removed ? 1 : 0;
-    dok_wave_add(&t.header[DOK_H_NELEM], removed, -1);
-  }
+  if (MODE == 1) dok_wave_add_n(count, n_found);
+  if (MODE == 2) dok_wave_add_n(&t.header[DOK_H_NELEM], -n_removed);
   if (STATS) {
-    dok_wave_add_n(&t.header[DOK_H_NPROBE], nprobe);
-    dok_wave_add(&t.header[DOK_H_NOPS], active);
+    dok_wave_add_n(&t.header[DOK_H_NPROBE], n_probe);
+    dok_wave_add_n(&t.header[DOK_H_NOPS], n_ops);
   }
 }
 
@@ -221,81 +226,85 @@ __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, c
                                                          u8 *__restrict__ stored) {
   extern __shared__ u64 lds[];
   u64 *lds_keys = lds;
-  const i64 i = (i64)blockIdx.x * DOK_TPB + threadIdx.x;
-  const bool active = i < n;
-  u32 home; u64 tag_full;
-  tg_stage(t, g, keys, i, active, lds_keys, home, tag_full);
-  __syncthreads();
-
   const TgLane L(g);
   const int wave_row0 = threadIdx.x & ~63;
-  u32 b = home, tomb_b = DOK_NONE32;
-  int tomb_w = 0;
-  bool pend = active, confirm = false;
-  int st = 0, fresh = 0;
-  u64 iters = 0;
-  const u8 *vrow = values + (size_t)i * g.V;
   const u64 *krow = lds_keys + threadIdx.x * g.KW;
+  int n_fresh = 0, n_full = 0;
 
-  u64 pm = dok_ballot(pend);
-  while (pm != 0) {
-    if (dok_ballot(confirm) != 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    const u32 sub = (u32)(pm >> L.gbase) & 0xffffu;
-    const bool has = sub != 0;
-    const int r = has ? __builtin_ctz(sub) : 0;
-    const int j = L.gbase + r;
-    const u32 qb = dok_shfl32(b, j);
-    const u64 qfull = dok_shfl64(tag_full, j);
-    const u64 w = dok_load_coherent(t.buckets + (u64)(has ? qb : 0u) * 16 + L.l);
-    const TgView v = tg_inspect(g, L, has, w, qfull, lds_keys + (wave_row0 + j) * g.KW);
-    if (has && L.l == r) {
-      u64 *bucket = t.buckets + (u64)b * 16;
-      const u64 qbusy = qfull & ~1ULL;
-      if (v.hit) {
-        u64 *slot = bucket + __builtin_ctz(v.hit);
-        if (atomicCAS(slot, qfull, qbusy) == qfull) {
-          for (int k = 0; k < g.VW; k++)
-            dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-          dok_store_coherent(slot, qfull);
-        }
-        st = 1; pend = false;
-      } else if (v.busy) {
-        // wait for the holder to publish
-      } else if ((v.tagonly & ~v.hit) != 0 && !confirm) {
-        confirm = true;
-      } else {
-        confirm = false;
-        if (tomb_b == DOK_NONE32 && v.tomb) { tomb_b = b; tomb_w = __builtin_ctz(v.tomb); }
-        const bool ring_done = (v.empty == 0) && (++iters >= t.nb);
-        if (v.empty || ring_done) {
-          if (tomb_b == DOK_NONE32 && v.empty == 0) {
-            st = 0; pend = false;                         // no free slot anywhere
-          } else {
-            u64 *slot; u64 expect;
-            if (tomb_b != DOK_NONE32) { slot = t.buckets + (u64)tomb_b * 16 + tomb_w; expect = DOK_TG_TOMB; }
-            else { slot = bucket + __builtin_ctz(v.empty); expect = DOK_TG_EMPTY; }
-            if (atomicCAS(slot, expect, qbusy) == expect) {
-              for (int k = 0; k < g.KW; k++) dok_store_coherent(slot + 1 + k, krow[k]);
-              for (int k = 0; k < g.VW; k++)
-                dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
-              __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-              dok_store_coherent(slot, qfull);
-              st = 1; fresh = 1; pend = false;
-            } else {
-              b = home; tomb_b = DOK_NONE32; iters = 0;   // lost the claim: walk again
-            }
+  DOK_TILE_LOOP(n) {
+    const i64 i = DOK_TILE_ROW();
+    const bool active = i < n;
+    u32 home; u64 tag_full;
+    tg_stage(t, g, keys, i, active, lds_keys, home, tag_full);
+    u32 b = home, tomb_b = DOK_NONE32;
+    int tomb_w = 0;
+    bool pend = active, confirm = false;
+    int st = 0, fresh = 0;
+    u64 iters = 0;
+    const u8 *vrow = values + (size_t)i * g.V;
+
+    u64 pm = dok_ballot(pend);
+    while (pm != 0) {
+      if (dok_ballot(confirm) != 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      const u32 sub = (u32)(pm >> L.gbase) & 0xffffu;
+      const bool has = sub != 0;
+      const int r = has ? __builtin_ctz(sub) : 0;
+      const int j = L.gbase + r;
+      const u32 qb = dok_shfl32(b, j);
+      const u64 qfull = dok_shfl64(tag_full, j);
+      const u64 w = dok_load_coherent(t.buckets + (u64)(has ? qb : 0u) * 16 + L.l);
+      const TgView v = tg_inspect(g, L, has, w, qfull, lds_keys + (wave_row0 + j) * g.KW);
+      if (has && L.l == r) {
+        u64 *bucket = t.buckets + (u64)b * 16;
+        const u64 qbusy = qfull & ~1ULL;
+        if (v.hit) {
+          u64 *slot = bucket + __builtin_ctz(v.hit);
+          if (atomicCAS(slot, qfull, qbusy) == qfull) {
+            for (int k = 0; k < g.VW; k++)
+              dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            dok_store_coherent(slot, qfull);
           }
+          st = 1; pend = false;
+        } else if (v.busy) {
+          // wait for the holder to publish
+        } else if ((v.tagonly & ~v.hit) != 0 && !confirm) {
+          confirm = true;
         } else {
-          b = (b + 1 == t.nb) ? 0u : b + 1;
+          confirm = false;
+          if (tomb_b == DOK_NONE32 && v.tomb) { tomb_b = b; tomb_w = __builtin_ctz(v.tomb); }
+          const bool ring_done = (v.empty == 0) && (++iters >= t.nb);
+          if (v.empty || ring_done) {
+            if (tomb_b == DOK_NONE32 && v.empty == 0) {
+              st = 0; pend = false;                         // no free slot anywhere
+            } else {
+              u64 *slot; u64 expect;
+              if (tomb_b != DOK_NONE32) { slot = t.buckets + (u64)tomb_b * 16 + tomb_w; expect = DOK_TG_TOMB; }
+              else { slot = bucket + __builtin_ctz(v.empty); expect = DOK_TG_EMPTY; }
+              if (atomicCAS(slot, expect, qbusy) == expect) {
+                for (int k = 0; k < g.KW; k++) dok_store_coherent(slot + 1 + k, krow[k]);
+                for (int k = 0; k < g.VW; k++)
+                  dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+                dok_store_coherent(slot, qfull);
+                st = 1; fresh = 1; pend = false;
+              } else {
+                b = home; tomb_b = DOK_NONE32; iters = 0;   // lost the claim: walk again
+              }
+            }
+          } else {
+            b = (b + 1 == t.nb) ? 0u : b + 1;
+          }
         }
       }
+      pm = dok_ballot(pend);
     }
-    pm = dok_ballot(pend);
+    if (active && stored) stored[i] = (u8)st;
+    n_fresh += fresh;
+    n_full += (active && st == 0);
   }
-  if (active && stored) stored[i] = (u8)st;
-  dok_wave_add(&t.header[DOK_H_NELEM], fresh != 0);
-  dok_wave_add(&t.header[DOK_H_NFULL], active && st == 0);
+  dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
+  dok_wave_add_n(&t.header[DOK_H_NFULL], n_full);
 }
 
 // ---- read-out ---------------------------------------------------------------------------------
@@ -372,8 +381,9 @@ static int tg_launch_get(const DevTable &d, const void *keys, i64 n, void *value
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k) || !tg_aligned(values, g.unit_v)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
+  const unsigned cgrid = grid < 2048u ? grid : 2048u;
   if (stats)
-    tg_lookup_kernel<0, true><<<grid, DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr);
+    tg_lookup_kernel<0, true><<<cgrid, DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr);
   else
     tg_lookup_kernel<0, false><<<grid, DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr);
   return DOK_OK;
@@ -385,7 +395,7 @@ static int tg_launch_count(const DevTable &d, const void *keys, i64 n, i64 *coun
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_lookup_kernel<1, false><<<grid, DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, nullptr, nullptr, count);
+  tg_lookup_kernel<1, false><<<(grid < 2048u ? grid : 2048u), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, nullptr, nullptr, count);
   return DOK_OK;
 }
 
@@ -395,7 +405,7 @@ static int tg_launch_remove(const DevTable &d, const void *keys, i64 n, u8 *remo
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_lookup_kernel<2, false><<<grid, DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, nullptr, removed, nullptr);
+  tg_lookup_kernel<2, false><<<(grid < 2048u ? grid : 2048u), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, nullptr, removed, nullptr);
   return DOK_OK;
 }
 
@@ -405,7 +415,7 @@ static int tg_launch_set(const DevTable &d, const void *keys, const void *values
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k) || !tg_aligned(values, g.unit_v)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_set_kernel<<<grid, DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, (const u8 *)values, n, stored);
+  tg_set_kernel<<<(grid < 2048u ? grid : 2048u), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, (const u8 *)values, n, stored);
   return DOK_OK;
 }
 

@@ -27,7 +27,7 @@ bool is_pow2_le8(int v) { return v == 1 || v == 2 || v == 4 || v == 8; }
 int layout_of(int kb, int vb, int *slots) {
   if (kb <= 0 || vb <= 0) return DOK_EUNSUPPORTED;
   if (is_pow2_le8(kb) && is_pow2_le8(vb)) {
-    if (slots) *slots = 128 / (8 + vb);
+    if (slots) *slots = 120 / (8 + vb);    // word 15 of a packed bucket is metadata
     return DOK_LAYOUT_PACKED8;
   }
   const int w = 1 + (kb + 7) / 8 + (vb + 7) / 8;
@@ -104,7 +104,14 @@ int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *s
   return DOK_OK;
 }
 
+// One workgroup per tile of DOK_TPB rows (kernels without counters) ...
 inline unsigned grid_for(i64 n) { return (unsigned)((n + DOK_TPB - 1) / DOK_TPB); }
+// ... or a fixed grid that fills the machine (8 workgroups on each of 256 CUs) and loops over the
+// tiles, for kernels that end with per-wave atomics on the table header.
+inline unsigned grid_counting(i64 n) {
+  const i64 tiles = (n + DOK_TPB - 1) / DOK_TPB;
+  return (unsigned)(tiles < 2048 ? tiles : 2048);
+}
 inline i64 chunks_of(const DevTable &d) { return ((i64)d.nb + DOK_CHUNK - 1) / DOK_CHUNK; }
 inline unsigned chunk_grid(i64 n_chunks) { return (unsigned)((n_chunks + 3) / 4); }
 
@@ -184,7 +191,7 @@ int dok_map_get_stats(const dok_table_t *t, const void *keys, int64_t n, void *v
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
     const u64 fb = fallback_word(fallback, d.value_bytes);
-    P8_DISPATCH(d.value_bytes, (p8_get_kernel<V, true><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
+    P8_DISPATCH(d.value_bytes, (p8_get_kernel<V, true><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
   } else {
     rc = tg_launch_get(d, keys, n, values_out, fallback, found, true, s);
     if (rc) return rc;
@@ -202,7 +209,7 @@ int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int6
   if (!keys || !values) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
-    P8_DISPATCH(d.value_bytes, (p8_set_kernel<V><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, values, n, stored)));
+    P8_DISPATCH(d.value_bytes, (p8_set_kernel<V><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, values, n, stored)));
   } else {
     rc = tg_launch_set(d, keys, values, n, stored, s);
     if (rc) return rc;
@@ -219,7 +226,7 @@ int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t *r
   if (!keys) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
-    P8_DISPATCH(d.value_bytes, (p8_remove_kernel<V><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
+    P8_DISPATCH(d.value_bytes, (p8_remove_kernel<V><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
   } else {
     rc = tg_launch_remove(d, keys, n, removed, s);
     if (rc) return rc;
@@ -236,7 +243,7 @@ int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n, in
   if (!keys || !count) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
-    P8_DISPATCH(d.value_bytes, (p8_count_kernel<V><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, (i64 *)count)));
+    P8_DISPATCH(d.value_bytes, (p8_count_kernel<V><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, (i64 *)count)));
   } else {
     rc = tg_launch_count(d, keys, n, (i64 *)count, s);
     if (rc) return rc;
@@ -312,7 +319,7 @@ int dok_setitem_dense(const dok_table_t *t, const dok_index_t *ix, const dok_vie
   if (di.n_elems == 0) return DOK_OK;
   if (di.n_elems > kMaxRows) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
-  P8_DISPATCH(d.value_bytes, (p8_setitem_kernel<V><<<grid_for(di.n_elems), DOK_TPB, 0, s>>>(d, di)));
+  P8_DISPATCH(d.value_bytes, (p8_setitem_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di)));
   return note_launch();
 }
 
@@ -325,7 +332,7 @@ int dok_count_items(const dok_table_t *t, const dok_index_t *ix, int64_t *count,
   if (di.n_elems == 0) return DOK_OK;
   if (!count || di.n_elems > kMaxRows) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
-  P8_DISPATCH(d.value_bytes, (p8_countitems_kernel<V><<<grid_for(di.n_elems), DOK_TPB, 0, s>>>(d, di, (i64 *)count)));
+  P8_DISPATCH(d.value_bytes, (p8_countitems_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di, (i64 *)count)));
   return note_launch();
 }
 
@@ -338,7 +345,7 @@ int dok_zero_items(const dok_table_t *t, const dok_index_t *ix, void *stream) {
   if (di.n_elems == 0) return DOK_OK;
   if (di.n_elems > kMaxRows) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
-  P8_DISPATCH(d.value_bytes, (p8_zeroitems_kernel<V><<<grid_for(di.n_elems), DOK_TPB, 0, s>>>(d, di)));
+  P8_DISPATCH(d.value_bytes, (p8_zeroitems_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di)));
   return note_launch();
 }
 

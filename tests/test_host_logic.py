@@ -56,7 +56,7 @@ def test_struct_sizes_match_the_header():
 def test_layout_selection():
     lib = _lib.load()
     s = ctypes.c_int32()
-    expect = {(8, 4): (1, 10), (8, 8): (1, 8), (8, 2): (1, 12), (8, 1): (1, 14), (4, 4): (1, 10),
+    expect = {(8, 4): (1, 10), (8, 8): (1, 7), (8, 2): (1, 12), (8, 1): (1, 13), (4, 4): (1, 10),
               (12, 40): (2, 2), (16, 4): (2, 4), (32, 2): (2, 2), (3, 3): (2, 5)}
     for (kb, vb), (layout, slots) in expect.items():
         assert lib.dok_layout_of(kb, vb, ctypes.byref(s)) == layout and s.value == slots
