@@ -8,7 +8,8 @@ import os
 from ctypes import c_int32, c_int64, c_uint64, c_void_p, c_char_p, POINTER
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libdokhip.so")
+# DOKHIP_LIB points at another build of the same ABI (e.g. a tuning variant)
+LIB_PATH = os.environ.get("DOKHIP_LIB") or os.path.join(_HERE, "libdokhip.so")
 
 DOK_OK = 0
 DOK_EINVAL = -1

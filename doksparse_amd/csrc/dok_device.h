@@ -120,8 +120,11 @@ __device__ __forceinline__ bool dok_linearise(const DevTable &t, const i64 *row,
 }
 
 // Key of batch row i as an 8-byte integer (packed layout): narrower keys are zero-extended.
+// LIN selects the coordinate-keyed form at compile time, so that kernels of plain tables never
+// touch (or hold in scalar registers) the sixteen dimension / stride words of the descriptor.
+template <bool LIN>
 __device__ __forceinline__ bool dok_load_key8(const DevTable &t, const void *keys, i64 i, u64 &key) {
-  if (t.lin_ndim > 0) return dok_linearise(t, (const i64 *)keys + i * t.lin_ndim, key);
+  if (LIN) return dok_linearise(t, (const i64 *)keys + i * t.lin_ndim, key);
   switch (t.key_bytes) {
     case 8: key = ((const u64 *)keys)[i]; break;
     case 4: key = ((const u32 *)keys)[i]; break;
@@ -131,8 +134,9 @@ __device__ __forceinline__ bool dok_load_key8(const DevTable &t, const void *key
   return true;
 }
 
+template <bool LIN>
 __device__ __forceinline__ void dok_store_key8(const DevTable &t, void *keys_out, i64 i, u64 key) {
-  if (t.lin_ndim > 0) {
+  if (LIN) {
     i64 *row = (i64 *)keys_out + i * t.lin_ndim;
     u64 rem = key;
     for (int d = 0; d < t.lin_ndim; d++) {

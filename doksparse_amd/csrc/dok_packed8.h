@@ -43,98 +43,188 @@ __device__ __forceinline__ u32 p8_home(u64 sk, const DevTable &t) {
   return dok_reduce(dok_fmix64(sk ^ t.seed), t.nb);
 }
 
+// Keeps the compiler from hoisting the 16 per-round "is this my row" masks out of the tile loop
+// (32 scalar registers that then spill) and from interleaving the rounds (which keeps every
+// round's ballot masks alive at once).
+#define DOK_OPAQUE(v) asm volatile("" : "+v"(v))
+#define DOK_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// ---- shared pieces of the cooperative probe ---------------------------------------------------
+
+// Lane geometry of the 16-lane probe groups of a wave64.
+struct P8Lane {
+  int lane, gbase, l;
+  bool upper;        // lane >= 32: the group's ballot bits sit in the high word
+  int sh;            // bit offset of the group inside that word (0 or 16)
+  __device__ __forceinline__ P8Lane() {
+    lane = threadIdx.x & 63;
+    gbase = lane & 48;
+    l = lane & 15;
+    upper = lane >= 32;
+    sh = lane & 16;
+  }
+  // the 16 ballot bits that belong to this lane's group
+  __device__ __forceinline__ u32 group(u64 m) const {
+    const u32 x = upper ? (u32)(m >> 32) : (u32)m;
+    return (x >> sh) & 0xffffu;
+  }
+};
+
+// One probe of one bucket by one group: which slots hold `q`, which are EMPTY / TOMBSTONE.
+// Masks are restricted to the S key lanes on the scalar side.
+template <int V> struct P8Probe {
+  static constexpr u64 KEY_LANES = ((1ULL << P8<V>::S) - 1ULL) * 0x0001000100010001ULL;
+  u32 gm, ge, gt;
+  __device__ __forceinline__ void match(const P8Lane &L, u64 w, u64 q) {
+    gm = L.group(__builtin_amdgcn_ballot_w64(w == q) & KEY_LANES);
+    ge = L.group(__builtin_amdgcn_ballot_w64(w == DOK_P8_EMPTY) & KEY_LANES);
+  }
+  __device__ __forceinline__ void tombs(const P8Lane &L, u64 w) {
+    gt = L.group(__builtin_amdgcn_ballot_w64(w == DOK_P8_TOMB) & KEY_LANES);
+  }
+  // index of the matching slot, 16 if none
+  __device__ __forceinline__ int slot() const { return __builtin_ctz(gm | 0x10000u); }
+  // value of slot s, fetched from the lane of the group that holds it: the holding lanes
+  // pre-shift their word so that one 32-bit shuffle suffices for values up to 4 bytes
+  __device__ __forceinline__ u64 value(const P8Lane &L, u64 w, int s) const {
+    const int vlane = L.gbase + ((P8<V>::S + ((s * V) >> 3)) & 15);
+    if (V == 8) return dok_shfl64(w, vlane);
+    u32 pre;
+    if (V == 4) pre = (s & 1) ? (u32)(w >> 32) : (u32)w;
+    else pre = (u32)(w >> (((s * V) & 7) * 8));
+    const u32 got = dok_shfl32(pre, vlane);
+    return V == 4 ? (u64)got : (u64)(got & ((1u << (8 * (V & 3))) - 1u));
+  }
+};
+
 // ---- cooperative lookup -------------------------------------------------------------------
-// In: per-lane stored key `sk`, home bucket `b`, `pend` (row needs a table probe).
-// Out: found / value for the lane's own row; slot_b / slot_s locate the matching slot;
-// nprobe counts the buckets visited for the lane's row.
+// In: per-lane stored key `sk`, home bucket `b` (0 for rows that need no probe), `pend` (row
+// needs a table probe).  Out: found / value for the lane's own row; slot_b / slot_s locate the
+// matching slot; nprobe counts the buckets visited for the lane's row.
 //
 // Phase 1 serves the home bucket of each of the group's 16 rows.  It is written as "issue U
 // loads, then resolve U rounds" with no branch in between, so that a wave keeps U*4 bucket
-// lines in flight; everything a round decides is folded into the owner lane with selects.
-// Phase 2 walks the few rows whose home bucket overflowed, one row per group per turn.
+// lines in flight; everything a round decides is folded into the owner lane with selects
+// (rows that need no probe are carried through it and their outcome discarded).
+// Phase 2 walks the rows whose home bucket overflowed: per turn every group serves up to four
+// of its open rows (loads first, then the four outcomes folded into their owners, which then
+// act together).
+#ifndef DOK_P8_U
 #define DOK_P8_U 8
+#endif
+#define DOK_P8_W 4   // rows per group per phase-2 turn
+#ifndef DOK_P8_VALUE_RELOAD
+#define DOK_P8_VALUE_RELOAD 1
+#endif
 template <int V>
 __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 nb, u64 sk, u32 b,
                                           bool pend, bool &found, u64 &val, u32 &slot_b,
                                           int &slot_s, int &nprobe) {
-  constexpr int S = P8<V>::S;
-  const int lane = threadIdx.x & 63;
-  const int gbase = lane & 48;
-  const int l = lane & 15;
-  const bool inb = l < S;
+  const P8Lane L;
+  const int gbase = L.gbase;
+  int l = L.l;
+  DOK_OPAQUE(l);
   const u32 home = b;
   u32 maxd = 0;                 // largest displacement recorded in the row's home bucket
+  bool open = false;            // row still unresolved after its home bucket
   slot_b = home;
 
-  const u64 pend0 = dok_ballot(pend);
-  if (pend0 != 0) {
-    const u32 gp = (u32)(pend0 >> gbase) & 0xffffu;      // pending rows of this group
+  if (dok_ballot(pend) != 0) {
+    // per-owner outcome of the row's own round, kept as plain words (lane-mask booleans would
+    // occupy a scalar register pair per round)
+    u32 my_gm = 0, my_ge = 0;
+    u64 my_v = 0;
     #pragma unroll
     for (int r0 = 0; r0 < 16; r0 += DOK_P8_U) {
       u64 w[DOK_P8_U];
       #pragma unroll
       for (int u = 0; u < DOK_P8_U; u++) {
-        const int r = r0 + u;
-        const u32 qb = dok_shfl32(home, gbase + r);
-        const bool has = (gp >> r) & 1u;
-        w[u] = buckets[(u64)(has ? qb : 0u) * 16 + l];
+        const u32 qb = dok_shfl32(home, gbase + r0 + u);
+        w[u] = buckets[(u64)qb * 16 + l];
       }
       #pragma unroll
       for (int u = 0; u < DOK_P8_U; u++) {
         const int r = r0 + u;
-        const bool has = (gp >> r) & 1u;
         const u64 q = dok_shfl64(sk, gbase + r);
-        const u64 bm = dok_ballot(has && inb && w[u] == q);
-        const u64 be = dok_ballot(has && inb && w[u] == DOK_P8_EMPTY);
-        const u32 gm = (u32)(bm >> gbase) & 0xffffu;
-        const u32 ge = (u32)(be >> gbase) & 0xffffu;
+        P8Probe<V> pr;
+        pr.match(L, w[u], q);
         const u32 md = dok_shfl32((u32)w[u], gbase + DOK_P8_META);
-        const int s = gm ? __builtin_ctz(gm) : 0;
-        const u64 vword = dok_shfl64(w[u], gbase + P8<V>::value_word(s));
-        const bool mine = has && l == r;
-        const bool hit = mine && gm != 0;
-        found = found || hit;
-        val = hit ? P8<V>::extract(vword, s) : val;
-        slot_s = hit ? s : slot_s;
+#if !DOK_P8_VALUE_RELOAD
+        const u64 v = pr.value(L, w[u], pr.slot());
+#endif
+        const bool mine = l == r;
+        my_gm = mine ? pr.gm : my_gm;
+        my_ge = mine ? pr.ge : my_ge;
         maxd = mine ? md : maxd;
-        pend = pend && !(mine && ((gm | ge) != 0 || md == 0));
+#if !DOK_P8_VALUE_RELOAD
+        my_v = mine ? v : my_v;
+#endif
+        DOK_SCHED_FENCE();
       }
     }
+    const bool hit1 = pend && my_gm != 0;
+    const int s1 = __builtin_ctz(my_gm | 0x10000u);
+#if DOK_P8_VALUE_RELOAD
+    // the bucket line was fetched a moment ago: read the value of the matching slot from it
+    if (hit1) {
+      typedef typename ValT<V>::type T;
+      my_v = *(const T *)((const char *)(buckets + (u64)home * 16) + 8 * P8<V>::S + V * s1);
+    }
+#endif
+    if (pend) { found = hit1; slot_s = s1; if (hit1) val = my_v; }
+    open = pend && (my_gm | my_ge) == 0 && maxd != 0;
+    nprobe += pend;
   }
-  nprobe += (pend0 >> lane) & 1ULL;
 
   // Phase 2
   u32 d = 1;
-  if (pend) b = (home + 1 == nb) ? 0u : home + 1;
-  if (pend && nb == 1) pend = false;
-  u64 pm = dok_ballot(pend);
+  if (open) b = (home + 1 == nb) ? 0u : home + 1;
+  if (nb == 1) open = false;
+  u64 pm = dok_ballot(open);
   while (pm != 0) {
-    const u32 sub = (u32)(pm >> gbase) & 0xffffu;
-    const bool has = sub != 0;
-    const int r = has ? __builtin_ctz(sub) : 0;
-    const int j = gbase + r;
-    const u64 q = dok_shfl64(sk, j);
-    const u32 qb = dok_shfl32(b, j);
-    const u64 w = buckets[(u64)(has ? qb : 0u) * 16 + l];
-    const u64 bm = dok_ballot(has && inb && w == q);
-    const u64 be = dok_ballot(has && inb && w == DOK_P8_EMPTY);
-    const u32 gm = (u32)(bm >> gbase) & 0xffffu;
-    const u32 ge = (u32)(be >> gbase) & 0xffffu;
-    const int s = gm ? __builtin_ctz(gm) : 0;
-    const u64 vword = dok_shfl64(w, gbase + P8<V>::value_word(s));
-    if (has && l == r) {
+    u32 rest = L.group(pm);
+    int rr[DOK_P8_W];
+    bool hs[DOK_P8_W];
+    u64 w[DOK_P8_W];
+    #pragma unroll
+    for (int k = 0; k < DOK_P8_W; k++) {
+      hs[k] = rest != 0;
+      rr[k] = hs[k] ? __builtin_ctz(rest) : 0;
+      rest &= rest - 1;
+      const u32 qb = dok_shfl32(b, gbase + rr[k]);
+      w[k] = buckets[(u64)(hs[k] ? qb : 0u) * 16 + l];
+    }
+    bool act = false;
+    u32 my_gm = 0, my_ge = 0;
+    u64 my_v = 0;
+    int my_s = 0;
+    #pragma unroll
+    for (int k = 0; k < DOK_P8_W; k++) {
+      const u64 q = dok_shfl64(sk, gbase + rr[k]);
+      P8Probe<V> pr;
+      pr.match(L, w[k], q);
+      const int s = pr.slot();
+      const u64 v = pr.value(L, w[k], s);
+      const bool mine = hs[k] && l == rr[k];
+      act = act || mine;
+      my_gm = mine ? pr.gm : my_gm;
+      my_ge = mine ? pr.ge : my_ge;
+      my_v = mine ? v : my_v;
+      my_s = mine ? s : my_s;
+    }
+    if (act) {
       nprobe++;
-      if (gm) {
-        found = true; val = P8<V>::extract(vword, s); slot_b = b; slot_s = s; pend = false;
-      } else if (ge) {
-        pend = false;
+      if (my_gm) {
+        found = true; val = my_v; slot_b = b; slot_s = my_s; open = false;
+      } else if (my_ge) {
+        open = false;
       } else {
         b = (b + 1 == nb) ? 0u : b + 1;
         d++;
-        if (d > maxd || d >= nb) pend = false;   // beyond every key homed at `home`: absent
+        if (d > maxd || d >= nb) open = false;   // beyond every key homed at `home`: absent
       }
     }
-    pm = dok_ballot(pend);
+    pm = dok_ballot(open);
   }
 }
 
@@ -145,8 +235,8 @@ __device__ __forceinline__ bool p8_side_get(const DevTable &t, u64 sk, u64 &val)
 }
 
 // ---- cooperative upsert -------------------------------------------------------------------
-// In: per-lane stored key, value, home bucket, `pend`.  Out: st (1 placed / 0 table full),
-// fresh (took a new slot).
+// In: per-lane stored key, value, home bucket (0 for rows that need no probe), `pend`.
+// Out: st (1 placed / 0 table full), fresh (took a new slot).
 //
 // The claim is one CAS on the slot's key word; whoever loses re-examines: if the winner wrote
 // the same key (equal keys inside one batch) the loser is done and the winner's value stands,
@@ -160,51 +250,47 @@ __device__ __forceinline__ bool p8_side_get(const DevTable &t, u64 sk, u64 &val)
 //
 // Phase 1 inspects the home bucket of all 64 rows (batched loads as in the lookup), then the
 // whole wave issues its CAS / value stores together.  Phase 2 is the general walk for rows whose
-// home bucket was full or whose claim was lost.  A key placed d > 0 buckets past its home
-// raises the home bucket's recorded largest displacement to d.
+// home bucket was full or whose claim was lost, four rows per group per turn, the owners acting
+// together.  A key placed d > 0 buckets past its home raises the home bucket's recorded largest
+// displacement to d.
 template <int V>
 __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val, u32 home,
                                           bool pend, int &st, int &fresh) {
-  constexpr int S = P8<V>::S;
-  const int lane = threadIdx.x & 63;
-  const int gbase = lane & 48;
-  const int l = lane & 15;
-  const bool inb = l < S;
+  const P8Lane L;
+  const int gbase = L.gbase;
+  int l = L.l;
+  DOK_OPAQUE(l);
 
-  int act = 0;                  // 0 walk on, 1 overwrite slot, 2 claim slot
+  int act1 = 0;                 // 0 walk on, 1 overwrite slot, 2 claim slot
   int slot = 0;
   bool tomb_here = false;       // the chosen slot of the home bucket is a tombstone
   u32 md_home = 0;
 
-  const u64 pend0 = dok_ballot(pend);
-  if (pend0 != 0) {
-    const u32 gp = (u32)(pend0 >> gbase) & 0xffffu;
+  if (dok_ballot(pend) != 0) {
     #pragma unroll
     for (int r0 = 0; r0 < 16; r0 += DOK_P8_U) {
       u64 w[DOK_P8_U];
       #pragma unroll
       for (int u = 0; u < DOK_P8_U; u++) {
-        const int r = r0 + u;
-        const u32 qb = dok_shfl32(home, gbase + r);
-        const bool has = (gp >> r) & 1u;
-        w[u] = buckets[(u64)(has ? qb : 0u) * 16 + l];
+        const u32 qb = dok_shfl32(home, gbase + r0 + u);
+        w[u] = buckets[(u64)qb * 16 + l];
       }
       #pragma unroll
       for (int u = 0; u < DOK_P8_U; u++) {
         const int r = r0 + u;
-        const bool has = (gp >> r) & 1u;
         const u64 q = dok_shfl64(sk, gbase + r);
-        const u32 gm = (u32)(dok_ballot(has && inb && w[u] == q) >> gbase) & 0xffffu;
-        const u32 ge = (u32)(dok_ballot(has && inb && w[u] == DOK_P8_EMPTY) >> gbase) & 0xffffu;
-        const u32 gt = (u32)(dok_ballot(has && inb && w[u] == DOK_P8_TOMB) >> gbase) & 0xffffu;
+        P8Probe<V> pr;
+        pr.match(L, w[u], q);
+        pr.tombs(L, w[u]);
         const u32 md = dok_shfl32((u32)w[u], gbase + DOK_P8_META);
-        const bool mine = has && l == r;
-        const int a = gm ? 1 : (ge ? 2 : 0);
-        const u32 pick = gm ? gm : (gt ? gt : ge);
-        act = mine ? a : act;
-        slot = mine ? (pick ? __builtin_ctz(pick) : 0) : slot;
-        tomb_here = mine ? (gm == 0 && gt != 0) : tomb_here;
+        const bool mine = l == r;
+        const int a = pr.gm ? 1 : (pr.ge ? 2 : 0);
+        const u32 pick = pr.gm ? pr.gm : (pr.gt ? pr.gt : pr.ge);
+        act1 = mine ? a : act1;
+        slot = mine ? __builtin_ctz(pick | 0x10000u) : slot;
+        tomb_here = mine ? (pr.gm == 0 && pr.gt != 0) : tomb_here;
         md_home = mine ? md : md_home;
+        DOK_SCHED_FENCE();
       }
     }
   }
@@ -214,10 +300,10 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
   u32 tomb_b = DOK_NONE32, tomb_d = 0;
   int tomb_s = 0;
   u64 iters = 0;
-  if (pend && act == 1) {
+  if (pend && act1 == 1) {
     P8<V>::store(hb, slot, val);
     st = 1; pend = false;
-  } else if (pend && act == 2) {
+  } else if (pend && act1 == 2) {
     const u64 expect = tomb_here ? DOK_P8_TOMB : DOK_P8_EMPTY;
     const u64 old = atomicCAS(hb + slot, expect, sk);
     if (old == expect) { P8<V>::store(hb, slot, val); st = 1; fresh = 1; pend = false; }
@@ -232,17 +318,33 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
 
   u64 pm = dok_ballot(pend);
   while (pm != 0) {
-    const u32 sub = (u32)(pm >> gbase) & 0xffffu;
-    const bool has = sub != 0;
-    const int r = has ? __builtin_ctz(sub) : 0;
-    const int j = gbase + r;
-    const u64 q = dok_shfl64(sk, j);
-    const u32 qb = dok_shfl32(b, j);
-    const u64 w = dok_load_coherent(buckets + (u64)(has ? qb : 0u) * 16 + l);
-    const u32 gm = (u32)(dok_ballot(has && inb && w == q) >> gbase) & 0xffffu;
-    const u32 ge = (u32)(dok_ballot(has && inb && w == DOK_P8_EMPTY) >> gbase) & 0xffffu;
-    const u32 gt = (u32)(dok_ballot(has && inb && w == DOK_P8_TOMB) >> gbase) & 0xffffu;
-    if (has && l == r) {
+    u32 rest = L.group(pm);
+    int rr[DOK_P8_W];
+    bool hs[DOK_P8_W];
+    u64 w[DOK_P8_W];
+    #pragma unroll
+    for (int k = 0; k < DOK_P8_W; k++) {
+      hs[k] = rest != 0;
+      rr[k] = hs[k] ? __builtin_ctz(rest) : 0;
+      rest &= rest - 1;
+      const u32 qb = dok_shfl32(b, gbase + rr[k]);
+      w[k] = dok_load_coherent(buckets + (u64)(hs[k] ? qb : 0u) * 16 + l);
+    }
+    bool act = false;
+    u32 gm = 0, ge = 0, gt = 0;
+    #pragma unroll
+    for (int k = 0; k < DOK_P8_W; k++) {
+      const u64 q = dok_shfl64(sk, gbase + rr[k]);
+      P8Probe<V> pr;
+      pr.match(L, w[k], q);
+      pr.tombs(L, w[k]);
+      const bool mine = hs[k] && l == rr[k];
+      act = act || mine;
+      gm = mine ? pr.gm : gm;
+      ge = mine ? pr.ge : ge;
+      gt = mine ? pr.gt : gt;
+    }
+    if (act) {
       if (gm) {
         // key present: overwrite its value in place
         P8<V>::store(buckets + (u64)b * 16, __builtin_ctz(gm), val);
@@ -288,7 +390,7 @@ __device__ __forceinline__ int p8_side_set(const DevTable &t, u64 sk, u64 val) {
 }
 
 // ---- kernels ------------------------------------------------------------------------------
-template <int V, bool STATS>
+template <int V, bool STATS, bool LIN>
 __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                          void *__restrict__ values, u8 *__restrict__ found_out,
                                                          u64 fallback) {
@@ -297,7 +399,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
     const i64 i = DOK_TILE_ROW();
     const bool active = i < n;
     u64 key = 0;
-    const bool ok = active && dok_load_key8(t, keys, i, key);
+    const bool ok = active && dok_load_key8<LIN>(t, keys, i, key);
     const u64 sk = key ^ DOK_P8_XOR;
     bool found = false;
     u64 val = fallback;
@@ -318,7 +420,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
   }
 }
 
-template <int V>
+template <int V, bool LIN>
 __global__ __launch_bounds__(DOK_TPB) void p8_set_kernel(DevTable t, const void *__restrict__ keys,
                                                          const void *__restrict__ values, i64 n,
                                                          u8 *__restrict__ stored) {
@@ -327,7 +429,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_set_kernel(DevTable t, const void 
     const i64 i = DOK_TILE_ROW();
     const bool active = i < n;
     u64 key = 0;
-    const bool ok = active && dok_load_key8(t, keys, i, key);
+    const bool ok = active && dok_load_key8<LIN>(t, keys, i, key);
     const u64 sk = key ^ DOK_P8_XOR;
     const u64 val = ok ? dok_load_val<V>(values, i) : 0;
     int st = 0, fresh = 0;
@@ -345,7 +447,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_set_kernel(DevTable t, const void 
 }
 
 // Tombstone the matching slot with a CAS so that equal keys in one batch remove it once.
-template <int V>
+template <int V, bool LIN>
 __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                             u8 *__restrict__ removed_out) {
   int n_removed = 0;
@@ -353,7 +455,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const vo
     const i64 i = DOK_TILE_ROW();
     const bool active = i < n;
     u64 key = 0;
-    const bool ok = active && dok_load_key8(t, keys, i, key);
+    const bool ok = active && dok_load_key8<LIN>(t, keys, i, key);
     const u64 sk = key ^ DOK_P8_XOR;
     bool found = false, removed = false;
     u64 val = 0;
@@ -371,7 +473,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const vo
   dok_wave_add_n(&t.header[DOK_H_NELEM], -n_removed);
 }
 
-template <int V>
+template <int V, bool LIN>
 __global__ __launch_bounds__(DOK_TPB) void p8_count_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                            i64 *count) {
   int n_found = 0;
@@ -379,7 +481,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_count_kernel(DevTable t, const voi
     const i64 i = DOK_TILE_ROW();
     const bool active = i < n;
     u64 key = 0;
-    const bool ok = active && dok_load_key8(t, keys, i, key);
+    const bool ok = active && dok_load_key8<LIN>(t, keys, i, key);
     const u64 sk = key ^ DOK_P8_XOR;
     bool found = false;
     u64 val = 0;
@@ -456,7 +558,7 @@ __global__ __launch_bounds__(1024) void dok_scan_kernel(i64 *counts, i64 n, cons
   }
 }
 
-template <int V>
+template <int V, bool LIN>
 __global__ __launch_bounds__(DOK_TPB) void p8_chunk_write_kernel(DevTable t, const i64 *chunk_offsets, i64 n_chunks,
                                                                  void *keys_out, void *values_out, i64 cap) {
   const i64 wid = (i64)blockIdx.x * (DOK_TPB / 64) + (threadIdx.x >> 6);
@@ -472,18 +574,18 @@ __global__ __launch_bounds__(DOK_TPB) void p8_chunk_write_kernel(DevTable t, con
     const u64 vword = dok_shfl64(w, gbase + vw);
     const i64 row = base + __popcll(m & ((1ULL << lane) - 1ULL));
     if (live && row < cap) {
-      if (keys_out) dok_store_key8(t, keys_out, row, w ^ DOK_P8_XOR);
+      if (keys_out) dok_store_key8<LIN>(t, keys_out, row, w ^ DOK_P8_XOR);
       if (values_out) dok_store_val<V>(values_out, row, P8<V>::extract(vword, l));
     }
     base += __popcll(m);
   }
   // the two side slots come last
-  if (wid == 0 && lane == 0 && t.lin_ndim == 0) {
+  if (!LIN && wid == 0 && lane == 0) {
     i64 row = chunk_offsets[n_chunks];
     for (u64 k = 0; k < 2; k++) {
       if (t.header[DOK_H_SIDE_STATE + k] != 0) {
         if (row < cap) {
-          if (keys_out) dok_store_key8(t, keys_out, row, k ^ DOK_P8_XOR);
+          if (keys_out) dok_store_key8<LIN>(t, keys_out, row, k ^ DOK_P8_XOR);
           if (values_out) dok_store_val<V>(values_out, row, (u64)t.header[DOK_H_SIDE_VALUE + k]);
         }
         row++;

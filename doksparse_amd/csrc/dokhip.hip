@@ -105,7 +105,14 @@ int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *s
 }
 
 // One workgroup per tile of DOK_TPB rows (kernels without counters) ...
-inline unsigned grid_for(i64 n) { return (unsigned)((n + DOK_TPB - 1) / DOK_TPB); }
+#ifndef DOK_GET_GRID_CAP
+#define DOK_GET_GRID_CAP 0
+#endif
+inline unsigned grid_for(i64 n) {
+  const i64 tiles = (n + DOK_TPB - 1) / DOK_TPB;
+  if (DOK_GET_GRID_CAP > 0 && tiles > DOK_GET_GRID_CAP) return DOK_GET_GRID_CAP;
+  return (unsigned)tiles;
+}
 // ... or a fixed grid that fills the machine (8 workgroups on each of 256 CUs) and loops over the
 // tiles, for kernels that end with per-wave atomics on the table header.
 inline unsigned grid_counting(i64 n) {
@@ -131,6 +138,10 @@ const i64 kMaxRows = (i64)0x7fffffff * DOK_TPB;
     case 4: { constexpr int V = 4; CALL; } break; \
     default: { constexpr int V = 8; CALL; } break; \
   }
+// the same, also binding LIN (coordinate-keyed table) for the kernels that read key rows
+#define P8_DISPATCH_LIN(vb, lin, CALL)                                   \
+  if (lin) { constexpr bool LIN = true; P8_DISPATCH(vb, CALL) }          \
+  else { constexpr bool LIN = false; P8_DISPATCH(vb, CALL) }
 
 }  // namespace
 
@@ -172,7 +183,7 @@ int dok_map_get(const dok_table_t *t, const void *keys, int64_t n, void *values_
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
     const u64 fb = fallback_word(fallback, d.value_bytes);
-    P8_DISPATCH(d.value_bytes, (p8_get_kernel<V, false><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, false, LIN><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
   } else {
     rc = tg_launch_get(d, keys, n, values_out, fallback, found, false, s);
     if (rc) return rc;
@@ -191,7 +202,7 @@ int dok_map_get_stats(const dok_table_t *t, const void *keys, int64_t n, void *v
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
     const u64 fb = fallback_word(fallback, d.value_bytes);
-    P8_DISPATCH(d.value_bytes, (p8_get_kernel<V, true><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, true, LIN><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
   } else {
     rc = tg_launch_get(d, keys, n, values_out, fallback, found, true, s);
     if (rc) return rc;
@@ -209,7 +220,7 @@ int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int6
   if (!keys || !values) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
-    P8_DISPATCH(d.value_bytes, (p8_set_kernel<V><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, values, n, stored)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_set_kernel<V, LIN><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, values, n, stored)));
   } else {
     rc = tg_launch_set(d, keys, values, n, stored, s);
     if (rc) return rc;
@@ -226,7 +237,7 @@ int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t *r
   if (!keys) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
-    P8_DISPATCH(d.value_bytes, (p8_remove_kernel<V><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_remove_kernel<V, LIN><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
   } else {
     rc = tg_launch_remove(d, keys, n, removed, s);
     if (rc) return rc;
@@ -243,7 +254,7 @@ int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n, in
   if (!keys || !count) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
-    P8_DISPATCH(d.value_bytes, (p8_count_kernel<V><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, (i64 *)count)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_count_kernel<V, LIN><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, (i64 *)count)));
   } else {
     rc = tg_launch_count(d, keys, n, (i64 *)count, s);
     if (rc) return rc;
@@ -271,7 +282,7 @@ int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out, int6
     P8_DISPATCH(d.value_bytes, (p8_chunk_count_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks)));
     dok_scan_kernel<<<1, 1024, 0, s>>>(offs, n_chunks, d.lin_ndim == 0 ? d.header : nullptr, (i64 *)count_out);
     if (keys_out || values_out) {
-      P8_DISPATCH(d.value_bytes, (p8_chunk_write_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks, keys_out, values_out, capacity_rows)));
+      P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_chunk_write_kernel<V, LIN><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks, keys_out, values_out, capacity_rows)));
     }
   } else {
     rc = tg_launch_compact(d, offs, n_chunks, keys_out, values_out, capacity_rows, (i64 *)count_out, s);
