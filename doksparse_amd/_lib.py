@@ -77,6 +77,9 @@ SIGNATURES = {
     "dok_setitem_dense": (c_int32, [POINTER(DokTable), POINTER(DokIndex), POINTER(DokView), c_void_p]),
     "dok_count_items": (c_int32, [POINTER(DokTable), POINTER(DokIndex), c_void_p, c_void_p]),
     "dok_zero_items": (c_int32, [POINTER(DokTable), POINTER(DokIndex), c_void_p]),
+    "dok_getitem_sparse": (c_int32, [POINTER(DokTable), POINTER(DokIndex), POINTER(DokTable), c_void_p]),
+    "dok_setitem_sparse": (c_int32, [POINTER(DokTable), POINTER(DokIndex), c_void_p, c_void_p, c_int64,
+                                     c_uint64, c_void_p]),
     "dok_to_dense": (c_int32, [POINTER(DokTable), c_void_p, c_void_p]),
 }
 

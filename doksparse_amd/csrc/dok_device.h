@@ -168,11 +168,37 @@ template <int V> __device__ __forceinline__ void dok_store_val(void *values, i64
   ((typename ValT<V>::type *)values)[i] = (typename ValT<V>::type)v;
 }
 
-// Coordinate of element e of the broadcast index space along every tensor dimension,
-// linearised.  Unravel e over `shape`, then read each selector through its strides
-// (stride 0 = broadcast axis).  `voff` receives the element offset into the source view.
-// Loops run to the compile-time maximum with uniform guards so that idx[] stays in registers;
-// the host zeroes the strides of unused axes.
+// Coordinate selected by index vector idx[] of the broadcast index space along every tensor
+// dimension, linearised: read each selector through its strides (stride 0 = broadcast axis).
+// `voff` receives the element offset into the source view.  Loops run to the compile-time
+// maximum with uniform guards so that idx[] stays in registers; the host zeroes the strides of
+// unused axes.
+__device__ __forceinline__ bool dok_gather_at(const DevTable &t, const DevIndex &ix,
+                                              const i64 (&idx)[DOK_MAX_DIMS], u64 &key, i64 &voff) {
+  bool ok = true;
+  u64 k = 0;
+  #pragma unroll
+  for (int d = 0; d < DOK_MAX_DIMS; d++) {
+    if (d < ix.ndim) {
+      i64 off = 0;
+      #pragma unroll
+      for (int j = 0; j < DOK_MAX_DIMS; j++)
+        if (j < ix.sel_ndim) off += idx[j] * ix.sstride[d][j];
+      i64 c = ix.sel[d][off];
+      ok = ok && ((u64)c < (u64)t.lin_dims[d]);
+      k += (u64)c * (u64)t.lin_strides[d];
+    }
+  }
+  i64 vo = 0;
+  #pragma unroll
+  for (int j = 0; j < DOK_MAX_DIMS; j++)
+    if (j < ix.sel_ndim) vo += idx[j] * ix.vstride[j];
+  voff = vo;
+  key = k;
+  return ok;
+}
+
+// The same for element e (row-major offset) of the index space: unravel e over `shape` first.
 __device__ __forceinline__ bool dok_gather_key(const DevTable &t, const DevIndex &ix, i64 e,
                                                u64 &key, i64 &voff) {
   i64 idx[DOK_MAX_DIMS];
@@ -201,25 +227,5 @@ __device__ __forceinline__ bool dok_gather_key(const DevTable &t, const DevIndex
       }
     }
   }
-  bool ok = true;
-  u64 k = 0;
-  #pragma unroll
-  for (int d = 0; d < DOK_MAX_DIMS; d++) {
-    if (d < ix.ndim) {
-      i64 off = 0;
-      #pragma unroll
-      for (int j = 0; j < DOK_MAX_DIMS; j++)
-        if (j < ix.sel_ndim) off += idx[j] * ix.sstride[d][j];
-      i64 c = ix.sel[d][off];
-      ok = ok && ((u64)c < (u64)t.lin_dims[d]);
-      k += (u64)c * (u64)t.lin_strides[d];
-    }
-  }
-  i64 vo = 0;
-  #pragma unroll
-  for (int j = 0; j < DOK_MAX_DIMS; j++)
-    if (j < ix.sel_ndim) vo += idx[j] * ix.vstride[j];
-  voff = vo;
-  key = k;
-  return ok;
+  return dok_gather_at(t, ix, idx, key, voff);
 }

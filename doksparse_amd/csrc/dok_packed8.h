@@ -716,3 +716,66 @@ __global__ __launch_bounds__(DOK_TPB) void p8_zeroitems_kernel(DevTable t, DevIn
   }
   dok_wave_add_n(&t.header[DOK_H_NELEM], -n_removed);
 }
+
+// Sparse-valued getitem: every element of the index space whose coordinate is stored in `t` is
+// inserted into `out`, a coordinate-keyed table over the index space itself (key = e).
+template <int V>
+__global__ __launch_bounds__(DOK_TPB) void p8_getitem_sparse_kernel(DevTable t, DevIndex ix, DevTable out) {
+  int n_fresh = 0, n_full = 0;
+  DOK_TILE_LOOP(ix.n_elems) {
+    const i64 e = DOK_TILE_ROW();
+    const bool active = e < ix.n_elems;
+    u64 key = 0; i64 voff = 0;
+    const bool ok = active && dok_gather_key(t, ix, e, key, voff);
+    const u64 sk = key ^ DOK_P8_XOR;
+    bool found = false;
+    u64 val = 0;
+    u32 sb = 0; int ss = 0, nprobe = 0;
+    p8_lookup<V>(t.buckets, t.nb, sk, ok ? p8_home(sk, t) : 0u, ok, found, val, sb, ss, nprobe);
+    const u64 ok2 = (u64)e ^ DOK_P8_XOR;
+    int st = 0, fresh = 0;
+    p8_insert<V>(out.buckets, out.nb, ok2, val, found ? p8_home(ok2, out) : 0u, found, st, fresh);
+    n_fresh += fresh;
+    n_full += (found && st == 0);
+  }
+  dok_wave_add_n(&out.header[DOK_H_NELEM], n_fresh);
+  dok_wave_add_n(&out.header[DOK_H_NFULL], n_full);
+}
+
+// Sparse-valued setitem: source entry k has index vector src_indices[j*n_src + k] (j over the
+// axes of the index space) and value src_values[k]; entries whose value is zero under
+// `nonzero_mask` (all ones for integers, sign bit cleared for floating values) are skipped.
+template <int V>
+__global__ __launch_bounds__(DOK_TPB) void p8_setitem_sparse_kernel(DevTable t, DevIndex ix,
+                                                                    const i64 *__restrict__ src_indices,
+                                                                    const void *__restrict__ src_values,
+                                                                    i64 n_src, u64 nonzero_mask) {
+  int n_fresh = 0, n_full = 0, n_oob = 0;
+  DOK_TILE_LOOP(n_src) {
+    const i64 k = DOK_TILE_ROW();
+    const bool active = k < n_src;
+    i64 idx[DOK_MAX_DIMS];
+    bool inside = active;
+    #pragma unroll
+    for (int j = 0; j < DOK_MAX_DIMS; j++) {
+      idx[j] = 0;
+      if (j < ix.sel_ndim && active) {
+        idx[j] = src_indices[(i64)j * n_src + k];
+        inside = inside && ((u64)idx[j] < (u64)ix.shape[j]);
+      }
+    }
+    const u64 val = active ? dok_load_val<V>(src_values, k) : 0;
+    const bool nonzero = (val & nonzero_mask) != 0;
+    u64 key = 0; i64 voff = 0;
+    const bool ok = inside && nonzero && dok_gather_at(t, ix, idx, key, voff);
+    const u64 sk = key ^ DOK_P8_XOR;
+    int st = 0, fresh = 0;
+    p8_insert<V>(t.buckets, t.nb, sk, val, ok ? p8_home(sk, t) : 0u, ok, st, fresh);
+    n_fresh += fresh;
+    n_full += (ok && st == 0);
+    n_oob += (active && nonzero && !ok);
+  }
+  dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
+  dok_wave_add_n(&t.header[DOK_H_NFULL], n_full);
+  dok_wave_add_n(&t.header[DOK_H_NOOB], n_oob);
+}

@@ -360,6 +360,41 @@ int dok_zero_items(const dok_table_t *t, const dok_index_t *ix, void *stream) {
   return note_launch();
 }
 
+int dok_getitem_sparse(const dok_table_t *t, const dok_index_t *ix, const dok_table_t *out, void *stream) {
+  DevTable d, o; int layout, lo; DevIndex di;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  rc = make_dev_table(out, o, lo);
+  if (rc) return rc;
+  rc = make_dev_index(d, ix, nullptr, di);
+  if (rc) return rc;
+  // `out` must be keyed by the index space itself
+  if (o.lin_ndim != di.sel_ndim || o.lin_ndim == 0 || o.value_bytes != d.value_bytes || o.buckets == d.buckets)
+    return DOK_EINVAL;
+  for (int j = 0; j < di.sel_ndim; j++) if (o.lin_dims[j] != di.shape[j]) return DOK_EINVAL;
+  if (di.n_elems == 0) return DOK_OK;
+  if (di.n_elems > kMaxRows) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  P8_DISPATCH(d.value_bytes, (p8_getitem_sparse_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di, o)));
+  return note_launch();
+}
+
+int dok_setitem_sparse(const dok_table_t *t, const dok_index_t *ix, const int64_t *src_indices,
+                       const void *src_values, int64_t n_src, uint64_t nonzero_mask, void *stream) {
+  DevTable d; int layout; DevIndex di;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  rc = make_dev_index(d, ix, nullptr, di);
+  if (rc) return rc;
+  if (n_src < 0 || n_src > kMaxRows) return DOK_EINVAL;
+  if (n_src == 0) return DOK_OK;
+  if (!src_values || (!src_indices && di.sel_ndim > 0)) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  P8_DISPATCH(d.value_bytes, (p8_setitem_sparse_kernel<V><<<grid_counting(n_src), DOK_TPB, 0, s>>>(
+      d, di, (const i64 *)src_indices, src_values, n_src, nonzero_mask)));
+  return note_launch();
+}
+
 int dok_to_dense(const dok_table_t *t, void *dense, void *stream) {
   DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);

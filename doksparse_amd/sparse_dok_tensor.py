@@ -348,7 +348,9 @@ class SparseDOKTensor(object):
         selectors, _ = self._handle_selectors(selectors)
         out_shape = tuple(selectors[0].shape)
         if isinstance(values, SparseDOKTensor) or (isinstance(values, Tensor) and values.is_sparse):
-            raise NotImplementedError("sparse-valued __setitem__")
+            assert tuple(values.shape) == out_shape, \
+                f"expecting the value shape to be {out_shape}, got {tuple(values.shape)} instead"
+            return self._set_items_sparse(values, selectors)
         if not isinstance(values, Tensor):
             values = torch.tensor(values, device=self.device, dtype=self.dtype)
         values = torch.broadcast_to(values.to(device=self.device, dtype=self.dtype), out_shape)
@@ -381,6 +383,73 @@ class SparseDOKTensor(object):
         if n_oob:
             hm._header[_lib.DOK_H_NOOB] = 0
             raise IndexError(f"{n_oob} coordinates fall outside the tensor of size {tuple(self.shape)}")
+
+    def __spgetitem__(self, selectors):
+        """Sparse-valued gather: a SparseDOKTensor over the index space holding the addressed
+        entries (reference: :342-350 and get_items, sparse_dok_tensor_impl.py:148-233)."""
+        selectors, _ = self._handle_selectors(selectors)
+        ix, out_shape = self._index_desc(selectors)
+        if len(out_shape) == 0:
+            raise NotImplementedError("sparse-valued indexing needs at least one result axis")
+        out = SparseDOKTensor(size=out_shape, device=self.device, dtype=self.dtype)
+        hm = self._hashmap
+        if not hm._allocated:
+            return out
+        lib = _lib.load()
+        stream = _stream_ptr(self.device)
+        n = 0
+        if selectors[0].numel():
+            count = torch.zeros(1, device=self.device, dtype=torch.long)
+            _lib.check(lib.dok_count_items(ctypes.byref(hm._desc), ctypes.byref(ix), count.data_ptr(), stream),
+                       "count_items")
+            n = int(count.item())
+        om = CudaClosedHashmap(n_buckets=int(n * 2.0), device=self.device, coord_dims=out_shape)
+        om.set(torch.zeros(0, len(out_shape), device=self.device, dtype=torch.long),
+               torch.zeros(0, 1, device=self.device, dtype=self.dtype))          # fixes widths, allocates
+        if n:
+            _lib.check(lib.dok_getitem_sparse(ctypes.byref(hm._desc), ctypes.byref(ix), ctypes.byref(om._desc),
+                                              stream), "__spgetitem__")
+        om._n_upper = n
+        out._hashmap = om
+        return out
+
+    def _set_items_sparse(self, src, selectors):
+        """Reference: set_items_sparse (sparse_dok_tensor_impl.py:235-340): clear every addressed
+        element, grow, then store the source's nonzero entries through the selectors."""
+        if isinstance(src, SparseDOKTensor):
+            keys, vals = src.storage().items()
+            if keys is None:
+                src_indices = torch.empty(src.ndim, 0, device=self.device, dtype=torch.long)
+                src_values = torch.empty(0, device=self.device, dtype=self.dtype)
+            else:
+                src_indices, src_values = keys.T.contiguous(), vals.flatten()
+        else:
+            if src.layout != torch.sparse_coo:
+                src = src.to_sparse_coo()
+            src = src.coalesce()
+            src_indices, src_values = src.indices().contiguous(), src.values()
+        src_indices = src_indices.to(self.device)
+        src_values = src_values.to(device=self.device, dtype=self.dtype).contiguous()
+        hm = self._hashmap
+        if not hm._allocated:
+            first_key = torch.stack([s.reshape(-1)[0] for s in selectors], dim=0)[None]
+            hm.set(first_key, torch.zeros(1, 1, device=self.device, dtype=self.dtype))
+        ix, _ = self._index_desc(selectors)
+        lib = _lib.load()
+        stream = _stream_ptr(self.device)
+        if selectors[0].numel():
+            _lib.check(lib.dok_zero_items(ctypes.byref(hm._desc), ctypes.byref(ix), stream), "zero_items")
+        n_src = int(src_values.shape[0])
+        n_now = hm.n_elements
+        hm.rehash(int(np.ceil((n_now + n_src) * hm._rehash_factor * 2)))
+        if n_src:
+            bits = 8 * src_values.element_size()
+            mask = (1 << bits) - 1
+            if src_values.dtype.is_floating_point:
+                mask >>= 1                                   # minus zero counts as zero
+            _lib.check(lib.dok_setitem_sparse(ctypes.byref(hm._desc), ctypes.byref(ix), src_indices.data_ptr(),
+                                              src_values.data_ptr(), n_src, mask, stream), "__setitem__")
+        hm._n_upper = n_now + n_src
 
     def count_items(self, selectors):
         """Number of addressed elements that are stored (reference: count_items,

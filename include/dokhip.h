@@ -44,7 +44,8 @@ extern "C" {
 
 /* Physical layouts (chosen from the key/value widths by dok_layout_of). */
 #define DOK_LAYOUT_PACKED8 1  /* key <= 8 bytes (1,2,4,8), value 1,2,4 or 8 bytes: the key word
-                                 itself is the CAS-claimed slot word; S = 128/(8+V) slots/bucket  */
+                                 itself is the CAS-claimed slot word; S = 120/(8+V) slots per bucket
+                                 and one metadata word                                            */
 #define DOK_LAYOUT_TAGGED  2  /* any widths with 8*(1+ceil(K/8)+ceil(V/8)) <= 128: an 8-byte
                                  tag/lock word per slot, then the key words, then the value words */
 
@@ -169,6 +170,22 @@ int dok_count_items(const dok_table_t *t, const dok_index_t *ix, int64_t *count,
 /* Tombstone the coordinate of every element; header[DOK_H_NELEM] shrinks accordingly.
  * Reference: sparse_dok_zero_items (sparse_dok_tensor_impl.cu:59-108). */
 int dok_zero_items(const dok_table_t *t, const dok_index_t *ix, void *stream);
+
+/* Sparse-valued gather: every element e of the index space whose coordinate is stored in t is
+ * inserted into `out` under the key e.  `out` is a cleared coordinate-keyed table whose
+ * lin_dims are the broadcast shape of ix and whose value_bytes equal t's.
+ * Reference: sparse_dok_get_items (sparse_dok_tensor_impl.cu:111-160). */
+int dok_getitem_sparse(const dok_table_t *t, const dok_index_t *ix, const dok_table_t *out,
+                       void *stream);
+
+/* Sparse-valued scatter: source entry k has index vector src_indices[j*n_src + k] (j over the
+ * axes of the index space, device int64) and value src_values[k]; every entry whose value,
+ * ANDed with nonzero_mask, is not zero is upserted at the coordinate its index vector selects
+ * (nonzero_mask: all ones for integer values, sign bit cleared for floating values, so that
+ * minus zero counts as zero).
+ * Reference: sparse_dok_set_items_sparse_v1 (sparse_dok_tensor_impl.cu:163-211). */
+int dok_setitem_sparse(const dok_table_t *t, const dok_index_t *ix, const int64_t *src_indices,
+                       const void *src_values, int64_t n_src, uint64_t nonzero_mask, void *stream);
 
 /* dense[linear coordinate] = value for every live entry; `dense` holds prod(lin_dims) elements
  * of value_bytes and must be zero-filled by the caller.

@@ -18,7 +18,9 @@
  *   sparse_dok/components/cuda/tensor_accessor.cu
  *       get_offset :50-58, get_index_from_offset :82-87
  *   sparse_dok/components/cuda/sparse_dok_tensor_impl.cu
- *       sparse_dok_count_items :4-56, sparse_dok_set_items_dense :271-313
+ *       sparse_dok_count_items :4-56, sparse_dok_zero_items :59-108,
+ *       sparse_dok_get_items :111-160, sparse_dok_set_items_sparse_v1 :163-211,
+ *       sparse_dok_set_items_dense :271-313
  *
  * Table layout is the reference's structure-of-arrays:
  *   uuid[B] int64 (-1 empty, -3 removed), keys[B][key_bytes], values[B][value_bytes].
@@ -327,10 +329,10 @@ ll_t ref_dok_set_items_dense(const ref_table_t *t, const ref_accessor_t *sel, co
 
 /* Lookup half of SparseDOKTensor.__getitem__ (sparse_dok_tensor.py:302-315) without the
  * stack/transpose copies: gather the coordinate of each selector element and read its value
- * (zero when absent) into the C-contiguous dense output. */
+ * (zero when absent) into the C-contiguous dense output; found (may be NULL) gets the hit flags. */
 void ref_dok_get_items_dense(const ref_table_t *t, const ref_accessor_t *sel, int ndim, int sel_ndim,
                              const ll_t *elem_sizes, const ll_t *elem_strides, ll_t n_elems,
-                             uint8_t *out, int n_threads) {
+                             uint8_t *out, uint8_t *found, int n_threads) {
   const int vb = t->value_bytes;
   ref_set_threads(n_threads);
   #pragma omp parallel for schedule(static) if (n_threads != 1)
@@ -341,7 +343,62 @@ void ref_dok_get_items_dense(const ref_table_t *t, const ref_accessor_t *sel, in
     ll_t addr = ref_find(t, (const uint8_t *)coord, NULL);
     if (addr >= 0) memcpy(out + (size_t)e * vb, t->values + (size_t)addr * vb, vb);
     else memset(out + (size_t)e * vb, 0, vb);
+    if (found) found[e] = addr >= 0;
   }
+}
+
+/* sparse_dok_zero_items :59-108: remove the coordinate of every selector element.
+ * Returns the number removed. */
+ll_t ref_dok_zero_items(const ref_table_t *t, const ref_accessor_t *sel, int ndim, int sel_ndim,
+                        const ll_t *elem_sizes, const ll_t *elem_strides, ll_t n_elems) {
+  ll_t cnt = 0;
+  for (ll_t e = 0; e < n_elems; e++) {
+    ll_t idx[REF_MAX_DIMS], coord[REF_MAX_DIMS];
+    ref_unravel(elem_sizes, elem_strides, sel_ndim, e, idx);
+    ref_gather_coord(sel, ndim, sel_ndim, idx, coord);
+    cnt += ref_remove(t, (const uint8_t *)coord);
+  }
+  return cnt;
+}
+
+/* sparse_dok_get_items :111-160: every selector element whose coordinate is stored is inserted
+ * into `out`, keyed by its index vector in the selector space (sel_ndim int64 words). */
+void ref_dok_get_items(const ref_table_t *t, const ref_table_t *out, const ref_accessor_t *sel,
+                       int ndim, int sel_ndim, const ll_t *elem_sizes, const ll_t *elem_strides,
+                       ll_t n_elems) {
+  for (ll_t e = 0; e < n_elems; e++) {
+    ll_t idx[REF_MAX_DIMS], coord[REF_MAX_DIMS];
+    ref_unravel(elem_sizes, elem_strides, sel_ndim, e, idx);
+    ref_gather_coord(sel, ndim, sel_ndim, idx, coord);
+    ll_t addr = ref_find(t, (const uint8_t *)coord, NULL);
+    if (addr >= 0) ref_set(out, (const uint8_t *)idx, t->values + (size_t)addr * t->value_bytes);
+  }
+}
+
+/* sparse_dok_set_items_sparse_v1 :163-211: src_indices is [sel_ndim][n_src] (index vectors in the
+ * selector space), src_values [n_src]; each nonzero source value is stored at the coordinate
+ * its index vector selects.  "Nonzero" is the numeric test of the device code: for floating
+ * values minus zero counts as zero (value_is_float).  Returns the number of fresh slots. */
+ll_t ref_dok_set_items_sparse_v1(const ref_table_t *t, const ref_accessor_t *sel, int ndim, int sel_ndim,
+                                 const ll_t *src_indices, const uint8_t *src_values, ll_t n_src,
+                                 int value_is_float) {
+  const int vb = t->value_bytes;
+  ll_t fresh = 0;
+  for (ll_t k = 0; k < n_src; k++) {
+    ll_t idx[REF_MAX_DIMS], coord[REF_MAX_DIMS];
+    for (int j = 0; j < sel_ndim; j++) idx[j] = src_indices[(size_t)j * n_src + k];
+    const uint8_t *v = src_values + (size_t)k * vb;
+    int nonzero = 0;
+    for (int q = 0; q < vb; q++) {
+      uint8_t byte = v[q];
+      if (value_is_float && q == vb - 1) byte &= 0x7f;      /* little endian: sign bit last */
+      nonzero |= byte != 0;
+    }
+    if (!nonzero) continue;
+    ref_gather_coord(sel, ndim, sel_ndim, idx, coord);
+    fresh += ref_set(t, (const uint8_t *)coord, v) == 1;
+  }
+  return fresh;
 }
 
 int ref_max_threads(void) {

@@ -16,6 +16,12 @@ Restated, with the reference lines each method follows:
   set_items_dense      sparse_dok_tensor_impl.py:412-474: bootstrap insert when unallocated,
                                    count existing, rehash when n + n_sel > B*threshold to
                                    ceil((n + n_sel)*factor), scatter, n += n_sel - n_existing
+  __spgetitem__        :342-350 + get_items (sparse_dok_tensor_impl.py:148-233): count the hits,
+                                   new map of int(2n) buckets keyed by selector-space index, insert
+                                   every hit
+  __setitem__ (sparse) :321-323 + set_items_sparse (sparse_dok_tensor_impl.py:235-340): remove every
+                                   addressed element, rehash to ceil((n + n_src)*factor*2), store the
+                                   source's nonzero entries through the selectors, n += n_src
   indices/values/to_dense :156-209
 
 Deliberate differences: numpy selectors are converted with torch.from_numpy (the reference's
@@ -184,6 +190,9 @@ class RefSparseDOKTensor:
     def __setitem__(self, selectors, values):
         sel, _ = self._handle_selectors(selectors)
         bshape = sel[0].shape
+        if isinstance(values, RefSparseDOKTensor) or (isinstance(values, Tensor) and values.is_sparse):
+            assert tuple(values.shape) == tuple(bshape)
+            return self._set_items_sparse(values, sel)
         if not isinstance(values, Tensor):
             # the reference ignores non-tensor values here; its README documents scalar
             # assignment, which is what is restated
@@ -212,3 +221,52 @@ class RefSparseDOKTensor:
         lib().ref_dok_set_items_dense(hm._table(), acc, ctypes.byref(vacc), ndim, sel_ndim,
                                       _ptr(esizes), _ptr(estrides), n_sel, 1)               # :464-473
         hm._n_elements += n_sel - int(n_existing)                                           # :474
+
+    def _index_space(self, sel):
+        ndim, sel_ndim = len(sel), sel[0].dim()
+        shape = tuple(sel[0].shape)
+        esizes = np.array(list(shape) + [0] * (8 - sel_ndim), dtype=np.int64)
+        estrides = np.array(list(shape_to_stride(shape)) + [0] * (8 - sel_ndim), dtype=np.int64)
+        acc = (RefAccessor * ndim)(*[_accessor(s) for s in sel])
+        return ndim, sel_ndim, esizes, estrides, acc, int(np.prod(shape))
+
+    # ---- sparse-valued getitem (:342-350, get_items sparse_dok_tensor_impl.py:148-233) ------
+    def __spgetitem__(self, selectors):
+        sel, _ = self._handle_selectors(selectors)
+        bshape = tuple(sel[0].shape)
+        out = RefSparseDOKTensor(bshape, dtype=self._dtype, rng=self._rng)
+        hm = self._hashmap
+        if hm._values is None:
+            return out
+        ndim, sel_ndim, esizes, estrides, acc, n_sel = self._index_space(sel)
+        n = lib().ref_dok_count_items(hm._table(), acc, ndim, sel_ndim, _ptr(esizes), _ptr(estrides), n_sel, 1)
+        oh = RefClosedHashmap(n_buckets=int(n * 2.0), rng=self._rng)
+        if n:
+            oh._allocate(np.zeros((1, sel_ndim), dtype=np.int64), np.zeros((1, 1), dtype=hm._value_dtype))
+            lib().ref_dok_get_items(hm._table(), oh._table(), acc, ndim, sel_ndim, _ptr(esizes), _ptr(estrides), n_sel)
+            oh._n_elements += int(n)
+        out._hashmap = oh
+        return out
+
+    # ---- setitem, sparse source (:321-323, set_items_sparse sparse_dok_tensor_impl.py:235-340) ----
+    def _set_items_sparse(self, src, sel):
+        hm = self._hashmap
+        if isinstance(src, RefSparseDOKTensor):
+            src_indices, src_values = src.indices().contiguous(), src.values().contiguous()
+        else:
+            src = src.coalesce() if not src.is_coalesced() else src
+            src_indices, src_values = src.indices().contiguous(), src.values().contiguous()
+        src_values = src_values.to(self._dtype)
+        if hm._keys is None:
+            first_key = torch.stack([s.reshape(-1)[0] for s in sel], dim=0)[None]
+            hm.set(first_key.numpy(), np.zeros((1, 1), dtype=src_values.numpy().dtype))
+        ndim, sel_ndim, esizes, estrides, acc, n_sel = self._index_space(sel)
+        n_removed = lib().ref_dok_zero_items(hm._table(), acc, ndim, sel_ndim, _ptr(esizes), _ptr(estrides), n_sel)
+        hm._n_elements -= int(n_removed)
+        n_src = int(src_values.shape[0])
+        hm.rehash(int(np.ceil((hm.n_elements + n_src) * hm._rehash_factor * 2)))
+        acc = (RefAccessor * ndim)(*[_accessor(s) for s in sel])
+        si, sv = src_indices.numpy(), src_values.numpy()
+        lib().ref_dok_set_items_sparse_v1(hm._table(), acc, ndim, sel_ndim, _ptr(si), _ptr(sv), n_src,
+                                          int(src_values.dtype.is_floating_point))
+        hm._n_elements += n_src

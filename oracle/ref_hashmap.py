@@ -83,7 +83,13 @@ def lib():
         L.ref_dok_set_items_dense.restype = i64
         L.ref_dok_set_items_dense.argtypes = [T, A, A, i32, i32, vp, vp, i64, i32]
         L.ref_dok_get_items_dense.restype = None
-        L.ref_dok_get_items_dense.argtypes = [T, A, i32, i32, vp, vp, i64, vp, i32]
+        L.ref_dok_get_items_dense.argtypes = [T, A, i32, i32, vp, vp, i64, vp, vp, i32]
+        L.ref_dok_zero_items.restype = i64
+        L.ref_dok_zero_items.argtypes = [T, A, i32, i32, vp, vp, i64]
+        L.ref_dok_get_items.restype = None
+        L.ref_dok_get_items.argtypes = [T, T, A, i32, i32, vp, vp, i64]
+        L.ref_dok_set_items_sparse_v1.restype = i64
+        L.ref_dok_set_items_sparse_v1.argtypes = [T, A, i32, i32, vp, vp, i64, i32]
         L.ref_max_threads.restype = i32
         L.ref_max_threads.argtypes = []
         _lib = L

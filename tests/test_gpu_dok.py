@@ -284,3 +284,55 @@ def test_cfg5_shape_scaled_with_tombstone_churn(cuda):
     assert dok._nnz() == ref._nnz() and dok.storage().n_buckets == ref._hashmap.n_buckets
     assert run_gets() > 1000
     assert same_entries(dok, ref)
+
+
+def test_sparse_valued_getitem(cuda):
+    dok, ref = make((9, 11, 6), 250, 9, cuda)
+    sels = [(slice(2, 7), torch.tensor([1, 3, 5, 10]), slice(None)),
+            (torch.tensor([0, 8, 3])[:, None], torch.tensor([2, 2, 9])[None, :], 4),
+            (slice(None), slice(None), slice(None)),
+            (torch.tensor([1, 1, 2]), slice(0, 0), slice(None))]
+    for sel in sels:
+        dsel = tuple(s.to(cuda) if isinstance(s, torch.Tensor) else s for s in sel)
+        got, exp = dok.__spgetitem__(dsel), ref.__spgetitem__(sel)
+        assert tuple(got.shape) == tuple(exp.shape)
+        assert got._nnz() == exp._nnz()
+        assert got.storage().n_buckets == exp._hashmap.n_buckets
+        assert same_entries(got, exp)
+        assert torch.equal(got.to_dense().cpu(), exp.to_dense())
+    # explicit zeros are entries: they survive the sparse gather
+    dok[0, 0, 0] = 0.0
+    ref[0, 0, 0] = 0.0
+    got, exp = dok.__spgetitem__((slice(0, 2),)), ref.__spgetitem__((slice(0, 2),))
+    assert got._nnz() == exp._nnz() and same_entries(got, exp)
+
+
+def test_sparse_valued_setitem(cuda):
+    from doksparse_amd import SparseDOKTensor
+    dok, ref = make((9, 11), 40, 10, cuda)
+    src = torch.zeros(5, 4)
+    src[0, 1], src[3, 2], src[4, 0], src[2, 2] = 7.0, -2.0, 5.0, 1.5
+    cols = torch.tensor([1, 3, 5, 10])
+    dok[2:7, cols.to(cuda)] = src.to_sparse().to(cuda)
+    ref[2:7, cols] = src.to_sparse()
+    assert dok.storage().n_buckets == ref._hashmap.n_buckets
+    assert same_entries(dok, ref)
+    dense = ref.to_dense()
+    assert torch.equal(dok.to_dense().cpu(), dense)
+    assert dok._nnz() == int((dense != 0).sum())
+    # a DOK tensor as the source, into an empty destination
+    sdok = SparseDOKTensor.from_dense(src.to(cuda))
+    rsrc = RefSparseDOKTensor((5, 4), src.nonzero().T, src[tuple(src.nonzero().T)])
+    d2 = SparseDOKTensor((20, 20), device=cuda)
+    r2 = RefSparseDOKTensor((20, 20))
+    rows = torch.tensor([3, 19, 0, 7, 8])
+    d2[rows.to(cuda), 4:8] = sdok
+    r2[rows, 4:8] = rsrc
+    assert torch.equal(d2.to_dense().cpu(), r2.to_dense())
+    assert d2.storage().n_buckets == r2._hashmap.n_buckets
+    # minus zero in a floating source counts as zero
+    s3 = torch.sparse_coo_tensor(torch.tensor([[0, 1], [0, 1]]), torch.tensor([-0.0, 4.0]), (5, 4))
+    d2[rows.to(cuda), 4:8] = s3.to(cuda)
+    r2[rows, 4:8] = s3
+    assert torch.equal(d2.to_dense().cpu(), r2.to_dense())
+    assert same_entries(d2, r2)

@@ -146,3 +146,41 @@ def test_empty_tensor_reads_zero():
     dok = RefSparseDOKTensor((5, 6))
     assert torch.equal(dok[1:3, :], torch.zeros(2, 6))
     assert dok.indices().shape == (2, 0) and dok.values().shape == (0,)
+
+
+def test_sparse_valued_getitem_matches_dense_slice():
+    dok, dense = make((9, 11, 6), 250, 9)
+    for sel in [(slice(2, 7), torch.tensor([1, 3, 5, 10]), slice(None)),
+                (torch.tensor([0, 8, 3])[:, None], torch.tensor([2, 2, 9])[None, :], 4),
+                (slice(None), slice(None), slice(None))]:
+        sp = dok.__spgetitem__(sel)
+        exp = dense[sel]
+        assert tuple(sp.shape) == tuple(exp.shape)
+        assert torch.equal(sp.to_dense(), exp)
+        assert sp._nnz() == int((exp != 0).sum())
+        assert sp._hashmap.n_buckets == int(sp._nnz() * 2.0)
+    # an explicitly stored zero is an entry of the result
+    dok[0, 0, 0] = 0.0
+    n0 = int((dense[0:2] != 0).sum()) + (1 if dense[0, 0, 0] == 0 else 0)
+    assert dok.__spgetitem__((slice(0, 2),))._nnz() == n0
+
+
+def test_sparse_valued_setitem_matches_dense_assignment():
+    dok, dense = make((9, 11), 40, 10)
+    src = torch.zeros(5, 4)
+    src[0, 1], src[3, 2], src[4, 0], src[2, 2] = 7.0, -2.0, 5.0, 1.5
+    cols = torch.tensor([1, 3, 5, 10])
+    n_before = dok._nnz()
+    n_removed = int((dense[2:7][:, cols] != 0).sum())
+    dok[2:7, cols] = src.to_sparse()
+    dense[2:7, cols] = src                      # zeros of the source clear the destination
+    assert torch.equal(dok.to_dense(), dense)
+    assert dok._nnz() == int((dense != 0).sum())
+    assert dok._hashmap.n_buckets == int(np.ceil((n_before - n_removed + 4) * 2.0 * 2))
+    # DOK source; minus zero in a floating source is skipped
+    src2 = RefSparseDOKTensor((5, 4), torch.tensor([[0, 1, 4], [0, 1, 3]]), torch.tensor([-0.0, 4.0, 2.0]))
+    dok[2:7, cols] = src2
+    d2 = torch.zeros(5, 4)
+    d2[1, 1], d2[4, 3] = 4.0, 2.0
+    dense[2:7, cols] = d2
+    assert torch.equal(dok.to_dense(), dense)
