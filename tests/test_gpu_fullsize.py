@@ -1,0 +1,139 @@
+"""GPU checks at the full sizes of the benchmark configurations, through properties that do not
+need the CPU oracle: a sorted-array lookup (torch.sort + searchsorted over linearised
+coordinates) as the independent map, entry counts, and read-out round trips."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+class SortedMap:
+    """key -> value by binary search over sorted unique int64 keys (independent of the table)."""
+    def __init__(self, keys, values):
+        self.keys, order = torch.sort(keys)
+        self.values = values[order]
+
+    def get(self, q):
+        pos = torch.searchsorted(self.keys, q).clamp_(max=self.keys.numel() - 1)
+        hit = self.keys[pos] == q
+        return torch.where(hit, self.values[pos], torch.zeros((), dtype=self.values.dtype, device=q.device)), hit
+
+
+def unique_coords(gen, dev, n, size):
+    """~n distinct coordinates uniform over `size` (duplicates of the draw are dropped)."""
+    strides = torch.tensor(np.cumprod((list(size[1:]) + [1])[::-1])[::-1].copy(), device=dev)
+    coords = torch.stack([torch.randint(0, s, (n,), generator=gen, device=dev) for s in size])
+    lin = (coords * strides[:, None]).sum(0)
+    lin = torch.unique(lin)
+    lin = lin[torch.randperm(lin.numel(), generator=gen, device=dev)]
+    coords = torch.stack([(lin // st) % s for st, s in zip(strides.tolist(), size)])
+    return coords, lin
+
+
+def test_cfg4_full_size(cuda):
+    """2-D 1e6 x 1e6 float32, 50M entries: construct, 4096 x 256 advanced-index gather (uniform and
+    planted), scatter of 10M coordinates (overwrites + inserts), read-out round trip."""
+    from doksparse_amd import SparseDOKTensor
+    gen = torch.Generator(device=cuda).manual_seed(1004)
+    size = (1_000_000, 1_000_000)
+    coords, lin = unique_coords(gen, cuda, 50_000_000, size)
+    vals = torch.randn(lin.numel(), generator=gen, device=cuda)
+    dok = SparseDOKTensor(size, coords, vals, device=cuda)
+    nnz = lin.numel()
+    assert dok._nnz() == nnz
+    assert dok.storage().n_buckets == 2**26              # 50M <= int(0.75 * 2^26): no growth
+    smap = SortedMap(lin, vals)
+
+    rows = torch.randint(0, size[0], (4096,), generator=gen, device=cuda)
+    cols = torch.randint(0, size[1], (256,), generator=gen, device=cuda)
+    prow, pcol = coords[0, :4096], coords[1, 1000:1256]
+    for rr, cc in ((rows, cols), (prow, pcol)):
+        got = dok[rr[:, None], cc[None, :]]
+        exp, hit = smap.get((rr[:, None] * size[1] + cc[None, :]).reshape(-1))
+        assert got.shape == (4096, 256) and torch.equal(got.reshape(-1), exp)
+    assert int(hit.sum()) >= 200                          # the planted gather really hits
+
+    # scatter: 5M stored coordinates + ~5M fresh ones
+    fresh, flin = unique_coords(gen, cuda, 5_000_000, size)
+    keep = ~smap.get(flin)[1]
+    fresh, flin = fresh[:, keep], flin[keep]
+    sc = torch.cat([coords[:, :5_000_000], fresh], dim=1)
+    sv = torch.randn(sc.shape[1], generator=gen, device=cuda)
+    dok[sc[0], sc[1]] = sv
+    assert dok._nnz() == nnz + flin.numel()
+    assert dok.storage().n_buckets == int(np.ceil((nnz + sc.shape[1]) * 2.0))   # grown as the reference would
+    lin2 = torch.cat([lin[5_000_000:], lin[:5_000_000], flin])
+    val2 = torch.cat([vals[5_000_000:], sv])
+    smap2 = SortedMap(lin2, val2)
+    probe = torch.randint(0, lin2.numel(), (4_000_000,), generator=gen, device=cuda)
+    got = dok[lin2[probe] // size[1], lin2[probe] % size[1]]
+    assert torch.equal(got, smap2.get(lin2[probe])[0])
+    del smap, got, probe
+
+    # read-out: the entries, sorted by coordinate, are exactly what went in
+    idx, v = dok.indices(), dok.values()
+    assert idx.shape == (2, lin2.numel())
+    out_lin = idx[0] * size[1] + idx[1]
+    order = torch.argsort(out_lin)
+    assert torch.equal(out_lin[order], smap2.keys) and torch.equal(v[order], smap2.values)
+
+
+def test_cfg5_full_size_churn(cuda):
+    """4-D (4096, 4096, 64, 8) float16, 100M entries at load factor 0.85: mixed indexing
+    dok[i, :512, idx, mask] for 64 values of i, then remove 20 % / insert as many fresh / repeat."""
+    from doksparse_amd import SparseDOKTensor, CudaClosedHashmap
+    gen = torch.Generator(device=cuda).manual_seed(1005)
+    size = (4096, 4096, 64, 8)
+    strides = (4096 * 64 * 8, 64 * 8, 8, 1)
+    coords, lin = unique_coords(gen, cuda, 100_000_000, size)
+    vals = torch.randn(lin.numel(), generator=gen, device=cuda).half()
+    nnz = lin.numel()
+    cap = int(np.ceil(nnz / 0.85))
+    store = CudaClosedHashmap(n_buckets=cap, device=cuda, rehash_threshold=0.9, coord_dims=size)
+    dok = SparseDOKTensor(size, coords, vals, device=cuda, storage=store)
+    del coords
+    assert dok._nnz() == nnz and dok.storage().n_buckets == cap
+
+    i_list = torch.randint(0, 4096, (64,), generator=gen, device=cuda).tolist()
+    sel_idx = torch.randint(0, 64, (128,), generator=gen, device=cuda)
+    mask = torch.tensor([True, False, True, True, False, False, True, False], device=cuda)
+    mcols = mask.nonzero()[:, 0]
+
+    def run_gets(smap):
+        hits = 0
+        for i in i_list:
+            got = dok[i, :512, sel_idx[:, None], mask]
+            q = (i * strides[0] + torch.arange(512, device=cuda)[None, None, :] * strides[1]
+                 + sel_idx[:, None, None] * strides[2] + mcols[None, :, None])
+            exp, hit = smap.get(q.reshape(-1))
+            assert got.shape == (128, 4, 512) and got.dtype == torch.float16
+            assert torch.equal(got.reshape(-1), exp)
+            hits += int(hit.sum())
+        return hits
+
+    smap = SortedMap(lin, vals)
+    assert run_gets(smap) > 100            # density 1.8e-4 over 16.8M lookups
+    # churn: remove 20 %, insert as many fresh coordinates
+    n_gone = nnz // 5
+    gone = lin[:n_gone]
+    gc = torch.stack([(gone // st) % s for st, s in zip(strides, size)], dim=1)
+    removed = dok.storage()._remove_rows(gc.contiguous())
+    assert bool(removed.all()) and dok._nnz() == nnz - n_gone
+    del gc, removed
+    fresh, flin = unique_coords(gen, cuda, n_gone + n_gone // 50, size)
+    keep = ~smap.get(flin)[1]
+    fresh, flin = fresh[:, keep][:, :n_gone], flin[keep][:n_gone]
+    fv = torch.randn(flin.numel(), generator=gen, device=cuda).half()
+    dok.storage().set(fresh.T.contiguous(), fv[:, None])
+    assert dok._nnz() == nnz - n_gone + flin.numel()
+    assert dok.storage().n_buckets == cap
+    del smap
+    smap = SortedMap(torch.cat([lin[n_gone:], flin]), torch.cat([vals[n_gone:], fv]))
+    assert run_gets(smap) > 100
+    # removed keys are gone, fresh keys are there
+    q = torch.cat([gone[:1_000_000], flin[:1_000_000]])
+    qc = torch.stack([(q // st) % s for st, s in zip(strides, size)], dim=1).contiguous()
+    v, f = dok.storage().get(qc)
+    assert not bool(f[:1_000_000].any()) and bool(f[1_000_000:].all())
+    assert torch.equal(v[1_000_000:, 0], fv[:1_000_000])
