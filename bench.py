@@ -149,6 +149,97 @@ def cpu_baseline(n_keys, seed):
     }
 
 
+def timed(fn):
+    """Milliseconds of fn() (everything it enqueues on the current stream), by events."""
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    out = fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1), out
+
+
+def other_configs(device):
+    """Timings of the four non-headline configurations (API level, inputs resident in HBM)."""
+    from doksparse_amd import CudaClosedHashmap, SparseDOKTensor
+    res = {}
+    gen = torch.Generator(device=device)
+
+    def uniq_lin(n, volume):
+        lin = torch.unique(torch.randint(0, volume, (n,), generator=gen, device=device))
+        return lin[torch.randperm(lin.numel(), generator=gen, device=device)]
+
+    # cfg1: 65,536 int64 keys -> int64, capacity 131,072
+    gen.manual_seed(1001)
+    k = make_unique_keys(131072, gen, device)
+    v = torch.randint(-2**62, 2**62, (65536, 1), generator=gen, device=device)
+    hm = CudaClosedHashmap(n_buckets=131072, device=device)
+    hm.set(k[:8, None], v[:8]); hm.remove(k[:8, None])        # warm-up (allocation, first launches)
+    res["cfg1_set_ms"] = round(timed(lambda: hm.set(k[:65536, None], v))[0], 4)
+    res["cfg1_get_ms"] = round(timed(lambda: hm.get(k[:, None]))[0], 4)
+    res["cfg1_remove_ms"] = round(timed(lambda: hm._remove_rows(k[:32768, None].contiguous()))[0], 4)
+
+    # cfg2: 1M float32[3] keys -> int64[5], capacity 2^21 (tagged layout)
+    gen.manual_seed(1002)
+    k2 = torch.rand(1_000_000, 3, generator=gen, device=device)
+    v2 = torch.randint(0, 2**63 - 1, (1_000_000, 5), generator=gen, device=device)
+    q2 = torch.cat([k2, torch.rand(1_000_000, 3, generator=gen, device=device) + 1.0])
+    hm2 = CudaClosedHashmap(n_buckets=2**21, device=device)
+    hm2.set(k2[:8], v2[:8])
+    res["cfg2_set_ms"] = round(timed(lambda: hm2.set(k2, v2))[0], 4)
+    res["cfg2_get_ms"] = round(timed(lambda: hm2.get(q2))[0], 4)
+    res["cfg2_remove_ms"] = round(timed(lambda: hm2._remove_rows(k2[:250_000].contiguous()))[0], 4)
+    del hm, hm2, k2, v2, q2
+
+    # cfg4: 2-D 1e6 x 1e6 float32, 50M entries
+    gen.manual_seed(1004)
+    lin = uniq_lin(50_000_000, 10**12)
+    coords = torch.stack([lin // 10**6, lin % 10**6])
+    vals = torch.randn(lin.numel(), generator=gen, device=device)
+    ms, dok = timed(lambda: SparseDOKTensor((10**6, 10**6), coords, vals, device=device))
+    res["cfg4_construct_50M_ms"] = round(ms, 3)
+    rows = torch.randint(0, 10**6, (4096, 1), generator=gen, device=device)
+    cols = torch.randint(0, 10**6, (1, 256), generator=gen, device=device)
+    dok[rows, cols]
+    res["cfg4_getitem_4096x256_ms"] = round(min(timed(lambda: dok[rows, cols])[0] for _ in range(5)), 4)
+    sc = torch.cat([coords[:, :5_000_000], torch.randint(0, 10**6, (2, 5_000_000), generator=gen, device=device)], dim=1)
+    sv = torch.randn(sc.shape[1], generator=gen, device=device)
+    def scatter():
+        dok[sc[0], sc[1]] = sv
+    res["cfg4_setitem_10M_ms"] = round(timed(scatter)[0], 3)           # includes the growth to 120M slots
+    res["cfg4_setitem_10M_again_ms"] = round(timed(scatter)[0], 3)     # all overwrites, no growth
+    res["cfg4_readout_ms"] = round(timed(lambda: dok.storage().items())[0], 3)
+    del dok, coords, vals, lin, sc, sv
+
+    # cfg5: 4-D (4096, 4096, 64, 8) float16, 100M entries at load factor 0.85
+    gen.manual_seed(1005)
+    size, strides = (4096, 4096, 64, 8), (4096 * 64 * 8, 64 * 8, 8, 1)
+    lin = uniq_lin(100_000_000, 2**39)
+    coords = torch.stack([(lin // st) % s for st, s in zip(strides, size)])
+    vals = torch.randn(lin.numel(), generator=gen, device=device).half()
+    store = CudaClosedHashmap(n_buckets=int(np.ceil(lin.numel() / 0.85)), device=device, rehash_threshold=0.9,
+                              coord_dims=size)
+    ms, dok = timed(lambda: SparseDOKTensor(size, coords, vals, device=device, storage=store))
+    res["cfg5_construct_100M_ms"] = round(ms, 3)
+    i_list = torch.randint(0, 4096, (64,), generator=gen, device=device).tolist()
+    idx = torch.randint(0, 64, (128, 1), generator=gen, device=device)
+    mask = torch.tensor([True, False, True, True, False, False, True, False], device=device)
+    def gets():
+        for i in i_list:
+            dok[i, :512, idx, mask]
+    gets()
+    res["cfg5_64_getitems_ms"] = round(timed(gets)[0], 3)
+    n_gone = lin.numel() // 5
+    gone = coords[:, :n_gone].T.contiguous()
+    res["cfg5_remove_20M_ms"] = round(timed(lambda: dok.storage()._remove_rows(gone))[0], 3)
+    fresh = torch.stack([torch.randint(0, s, (n_gone,), generator=gen, device=device) for s in size], dim=1)
+    fv = torch.randn(n_gone, 1, generator=gen, device=device).half()
+    res["cfg5_reinsert_20M_ms"] = round(timed(lambda: dok.storage().set(fresh, fv))[0], 3)
+    res["cfg5_64_getitems_after_churn_ms"] = round(timed(gets)[0], 3)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -158,6 +249,8 @@ def main():
     ap.add_argument("--cpu-keys", type=int, default=1 << 24)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--quick", action="store_true", help="skip the set and load-factor-0.9 legs")
+    ap.add_argument("--configs", action="store_true",
+                    help="also time the four non-headline configurations (reported under extra)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one read-only pass over the whole table (the live-entry count of "
                          "the read-out path); with the table clear that every run does, this gives "
@@ -259,6 +352,11 @@ def main():
         results["load_factor_09_physical"] = round(n / (hm9._n_phys * hm9._slots_per_bucket), 4)
         del hm9
 
+    if args.configs:
+        del keys, values, queries, out_v, out_f
+        torch.cuda.empty_cache()
+        results.update(other_configs(device))
+
     achieved = n * B_GET / (k_avg * 1e-3) / 1e9
     line = {
         "metric": "hashmap get/set Mops/s at 64M keys LF 0.5/0.9; achieved HBM GB/s % of peak",
@@ -285,7 +383,7 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": None,
-            "kernel": "p8_get_kernel<4,false>",
+            "kernel": "p8_get_kernel<4,false,false>",
             "bytes_per_op": B_GET,
             "kernel_ms": round(k_avg, 4),
         },

@@ -391,8 +391,15 @@ class CudaClosedHashmap:
             if n_now > limit:
                 self.rehash(int(n_now * self._rehash_factor))
             return
-        # the batch may not fit: count its distinct new keys first, as the reference does
+        # the batch may not fit.  Rows that miss bound the distinct new keys from above; if even
+        # that bound stays under the threshold nothing can grow and no sort is needed
         _, is_found = self.get(keys)
+        n_miss = int((~is_found).sum().item())
+        if n_old + n_miss <= limit:
+            self._launch_set(keys, values)
+            self._n_upper = n_old + n_miss
+            return
+        # otherwise count the distinct new keys exactly, as the reference does
         n_new = int(keys[~is_found].unique(dim=0).shape[0])
         if n_old + n_new > limit:
             self.rehash(int((n_old + n_new) * self._rehash_factor))

@@ -22,6 +22,16 @@
 #define DOK_TG_EMPTY 0ULL
 #define DOK_TG_TOMB  1ULL
 #define DOK_TG_MAXW  15
+// Ordering of "write the slot's key and value words" before "publish the FULL tag".  The data
+// words are written with agent-scope atomic stores, which gfx950 performs write-through to the
+// level every XCD shares; what remains to be ensured is that those stores have completed before
+// the tag store is issued, i.e. a wait for the wave's outstanding memory operations.  A
+// workgroup-scope release fence compiles to exactly that wait.  (An agent-scope release fence
+// adds a write-back of the whole L2, which exists for plain stores - there are none here - and
+// costs ten times the kernel's run time when issued once per inserted row.)
+#ifndef DOK_TG_RELEASE
+#define DOK_TG_RELEASE() __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup")
+#endif
 
 struct TgGeom {
   int KW, VW, W, S;
@@ -262,7 +272,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, c
           if (atomicCAS(slot, qfull, qbusy) == qfull) {
             for (int k = 0; k < g.VW; k++)
               dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            DOK_TG_RELEASE();
             dok_store_coherent(slot, qfull);
           }
           st = 1; pend = false;
@@ -285,7 +295,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, c
                 for (int k = 0; k < g.KW; k++) dok_store_coherent(slot + 1 + k, krow[k]);
                 for (int k = 0; k < g.VW; k++)
                   dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+                DOK_TG_RELEASE();
                 dok_store_coherent(slot, qfull);
                 st = 1; fresh = 1; pend = false;
               } else {
