@@ -63,6 +63,26 @@ def _next_prime(n):
     return m
 
 
+class _TableState:
+    """Physical state of one table.  Shallow clones of a map share one instance, so a rehash or
+    an insert through any of them is seen by all."""
+    pass
+
+
+_SHARED = ("_table", "_header", "_desc", "_n_phys", "_slots_per_bucket", "_layout", "_n_buckets",
+           "_key_shape", "_key_dtype", "_value_shape", "_value_dtype", "_key_bytes", "_value_bytes",
+           "_n_upper", "_seed")
+
+
+def _forward(name):
+    def fget(self):
+        return getattr(self._st, name)
+
+    def fset(self, value):
+        setattr(self._st, name, value)
+    return property(fget, fset)
+
+
 class CudaClosedHashmap:
     def __init__(
         self,
@@ -81,6 +101,7 @@ class CudaClosedHashmap:
         coord_dims=None,
         seed=None,
     ):
+        self._st = _TableState()
         self._empty_marker = -1
         self._removed_marker = -3
         self._n_buckets = int(n_buckets)
@@ -117,6 +138,10 @@ class CudaClosedHashmap:
         self._n_upper = 0
 
     # ------------------------------------------------------------------ physical table
+    for _name in _SHARED:
+        locals()[_name] = _forward(_name)
+    del _name
+
     @property
     def _allocated(self):
         return self._table is not None
@@ -548,17 +573,17 @@ class CudaClosedHashmap:
             rehash_factor=self._rehash_factor, rehash_threshold=self._rehash_threshold,
             coord_dims=self._coord_dims, seed=self._seed,
         )
-        for name in ("_key_shape", "_key_dtype", "_value_shape", "_value_dtype", "_key_bytes",
-                     "_value_bytes", "_n_phys", "_slots_per_bucket", "_layout", "_n_upper"):
+        if not deepclone:
+            new._st = self._st
+            return new
+        for name in _SHARED:
             setattr(new, name, getattr(self, name))
         if self._allocated:
-            if deepclone:
-                new._table = self._table.clone()
-                new._header = self._header.clone()
-            else:
-                new._table = self._table
-                new._header = self._header
+            new._table = self._table.clone()
+            new._header = self._header.clone()
             new._desc = new._make_desc(new._table, new._header, new._n_phys)
+        else:
+            new._header = self._header.clone()
         return new
 
     # ------------------------------------------------------------------ probe statistics

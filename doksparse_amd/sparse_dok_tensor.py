@@ -37,6 +37,9 @@ class SparseDOKTensor(object):
     def __init__(self, size, indices=None, values=None, device=None, dtype=None, storage=None):
         assert isinstance(size, (list, tuple))
         self._size = torch.Size(size)
+        # view dimension i addresses dimension _perm[i] of the storage (identity unless the tensor
+        # was made by permute/transpose, which share the storage)
+        self._perm = tuple(range(len(size)))
 
         if storage is None:
             self.device = torch.device("cuda:0") if device is None else torch.device(device)
@@ -83,6 +86,16 @@ class SparseDOKTensor(object):
             if keys.shape[0]:
                 new.set(keys.reshape(-1, self.ndim).long(), values)
         return new
+
+    def _is_permuted(self):
+        return self._perm != tuple(range(self.ndim))
+
+    def _to_storage_order(self, per_view_dim):
+        """Reorder a per-view-dimension list into the storage's dimension order."""
+        out = [None] * self.ndim
+        for i, item in enumerate(per_view_dim):
+            out[self._perm[i]] = item
+        return out
 
     # ------------------------------------------------------------------ constructors
     @classmethod
@@ -165,6 +178,7 @@ class SparseDOKTensor(object):
     def clone(self, deepclone=True):
         new = SparseDOKTensor(size=tuple(self._size), device=self.device, dtype=self.dtype)
         new._hashmap = self._hashmap.clone(deepclone=deepclone)
+        new._perm = self._perm
         return new
 
     # ------------------------------------------------------------------ read-out
@@ -172,7 +186,7 @@ class SparseDOKTensor(object):
         keys = self._hashmap.keys()
         if keys is None:
             return torch.empty(self.ndim, 0, device=self.device, dtype=torch.long)
-        return keys.T
+        return keys.T[list(self._perm)] if self._is_permuted() else keys.T
 
     def values(self):
         values = self._hashmap.values()
@@ -194,7 +208,8 @@ class SparseDOKTensor(object):
         if keys is None:
             keys = torch.empty(0, self.ndim, device=self.device, dtype=torch.long)
             values = torch.empty(0, 1, device=self.device, dtype=self.dtype)
-        return torch.sparse_coo_tensor(indices=keys.T, values=values.flatten(), size=tuple(self.shape),
+        idx = keys.T[list(self._perm)] if self._is_permuted() else keys.T
+        return torch.sparse_coo_tensor(indices=idx, values=values.flatten(), size=tuple(self.shape),
                                        device=self.device)
 
     @property
@@ -205,13 +220,14 @@ class SparseDOKTensor(object):
         return self.to_sparse_coo().to_sparse_csr()
 
     def to_dense(self):
-        dense = torch.zeros(tuple(self.shape), device=self.device, dtype=self.dtype)
         hm = self._hashmap
+        storage_shape = self._to_storage_order(list(self.shape))
+        dense = torch.zeros(tuple(storage_shape), device=self.device, dtype=self.dtype)
         if hm._allocated and dense.numel():
             lib = _lib.load()
             _lib.check(lib.dok_to_dense(ctypes.byref(hm._desc), dense.data_ptr(), _stream_ptr(self.device)),
                        "to_dense")
-        return dense
+        return dense.permute(*self._perm).contiguous() if self._is_permuted() else dense
 
     def resize(self, *new_size):
         new_size = tuple(new_size) + (self.ndim - len(new_size)) * (-1,)
@@ -229,10 +245,12 @@ class SparseDOKTensor(object):
         if old._allocated:
             keys, values = old.items()
             if keys.shape[0]:
-                new.set(fn(keys.T).T.contiguous(), values)
+                idx = keys.T[list(self._perm)] if self._is_permuted() else keys.T
+                new.set(fn(idx).T.contiguous(), values)
                 new._header[_lib.DOK_H_NOOB] = 0      # entries outside the new size are dropped
         self._hashmap = new
         self._size = torch.Size(new_size)
+        self._perm = tuple(range(len(new_size)))
 
     # ------------------------------------------------------------------ selectors
     def _normalise_slice(self, sl, dim):
@@ -318,7 +336,7 @@ class SparseDOKTensor(object):
         ix.sel_ndim = len(out_shape)
         for j, s in enumerate(out_shape):
             ix.shape[j] = s
-        for d, sel in enumerate(selectors):
+        for d, sel in enumerate(self._to_storage_order(selectors)):
             assert sel.dtype == torch.long and sel.device == self.device
             ix.sel[d].data = sel.data_ptr()
             for j, st in enumerate(sel.stride()):
@@ -364,7 +382,7 @@ class SparseDOKTensor(object):
         hm = self._hashmap
         if not hm._allocated:
             # fixes the key/value widths; the entry itself is written again by the kernel below
-            first_key = torch.stack([s.reshape(-1)[0] for s in selectors], dim=0)[None]
+            first_key = torch.stack([s.reshape(-1)[0] for s in self._to_storage_order(selectors)], dim=0)[None]
             hm.set(first_key, src.reshape(-1)[:1, None].contiguous())
         ix, _ = self._index_desc(selectors)
         view = DokView()
@@ -432,7 +450,7 @@ class SparseDOKTensor(object):
         src_values = src_values.to(device=self.device, dtype=self.dtype).contiguous()
         hm = self._hashmap
         if not hm._allocated:
-            first_key = torch.stack([s.reshape(-1)[0] for s in selectors], dim=0)[None]
+            first_key = torch.stack([s.reshape(-1)[0] for s in self._to_storage_order(selectors)], dim=0)[None]
             hm.set(first_key, torch.zeros(1, 1, device=self.device, dtype=self.dtype))
         ix, _ = self._index_desc(selectors)
         lib = _lib.load()
@@ -488,20 +506,19 @@ class SparseDOKTensor(object):
     def select(self, dim, index):
         return self.to_sparse_coo().select(dim=dim, index=index)
 
-    # ------------------------------------------------------------------ re-layout (rebuilds the storage)
+    # ------------------------------------------------------------------ views and re-layout
     def permute_(self, *ordering):
-        ordering = [int(o) for o in ordering]
+        """Reorder the dimensions in place; nothing is moved (reference: :439-443)."""
+        ordering = [int(o) % self.ndim for o in ordering]
         assert sorted(ordering) == list(range(self.ndim))
-        new_size = torch.Size(self._size[i] for i in ordering)
-        self._rekey(new_size, lambda idx: idx[ordering])
+        self._perm = tuple(self._perm[o] for o in ordering)
+        self._size = torch.Size(self._size[o] for o in ordering)
         return self
 
     def permute(self, *ordering):
-        return self.clone(deepclone=False)._detach_storage().permute_(*ordering)
-
-    def _detach_storage(self):
-        self._hashmap = self._hashmap.clone(deepclone=False)
-        return self
+        """A view with reordered dimensions that shares this tensor's storage: writes through
+        either are seen by both (reference: :445-450)."""
+        return self.clone(deepclone=False).permute_(*ordering)
 
     def transpose_(self, dim0, dim1):
         assert dim0 != dim1
@@ -551,6 +568,8 @@ class SparseDOKTensor(object):
                                          rehash_factor=self._hashmap._rehash_factor,
                                          rehash_threshold=self._hashmap._rehash_threshold)
         if keys is not None and keys.shape[0]:
+            if self._is_permuted():
+                keys = keys[:, list(self._perm)].contiguous()
             new._hashmap.set(keys, fn(values))
         return new
 

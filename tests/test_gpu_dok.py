@@ -336,3 +336,50 @@ def test_sparse_valued_setitem(cuda):
     r2[rows, 4:8] = s3
     assert torch.equal(d2.to_dense().cpu(), r2.to_dense())
     assert same_entries(d2, r2)
+
+
+def test_views_share_storage(cuda):
+    """permute / transpose / T give views over the same table: reads follow the permuted
+    dimensions, writes through a view land in the base tensor and vice versa."""
+    dok, ref = make((6, 7, 5), 120, 11, cuda)
+    dense = ref.to_dense()
+    v = dok.permute(2, 0, 1)
+    assert tuple(v.shape) == (5, 6, 7) and v._nnz() == dok._nnz()
+    assert torch.equal(v.to_dense().cpu(), dense.permute(2, 0, 1))
+    i, j = torch.tensor([0, 4, 2]), torch.tensor([5, 1, 3])
+    assert torch.equal(v[i.to(cuda), j.to(cuda)].cpu(), dense.permute(2, 0, 1)[i, j])
+    assert torch.equal(v[1:4, :, 2].cpu(), dense.permute(2, 0, 1)[1:4, :, 2])
+    order = np.lexsort(v.indices().cpu().numpy()[::-1])
+    assert torch.equal(v.indices().cpu()[:, order], dense.permute(2, 0, 1).nonzero().T)
+    # write through the view, read through the base
+    v[4, 5, 6] = 42.0
+    dense[5, 6, 4] = 42.0
+    assert dok[5, 6, 4].item() == 42.0 and torch.equal(dok.to_dense().cpu(), dense)
+    # write through the base (enough to force a rehash), read through the view
+    g = torch.Generator().manual_seed(3)
+    flat = torch.randperm(6 * 7 * 5, generator=g)[:150]
+    a, b, c = flat // 35, (flat // 5) % 7, flat % 5
+    x = torch.randn(150, generator=g)
+    dok[a.to(cuda), b.to(cuda), c.to(cuda)] = x.to(cuda)
+    dense[a, b, c] = x
+    assert torch.equal(v.to_dense().cpu(), dense.permute(2, 0, 1))
+    assert v._nnz() == dok._nnz() == int((dense != 0).sum())
+    # transpose of a view composes; T on 2-D
+    w = v.transpose(0, 2)
+    assert tuple(w.shape) == (7, 6, 5) and torch.equal(w.to_dense().cpu(), dense.permute(1, 0, 2))
+    d2, r2 = make((8, 9), 30, 12, cuda)
+    t = d2.T
+    assert torch.equal(t.to_dense().cpu(), r2.to_dense().T)
+    t[torch.arange(9, device=cuda), torch.arange(9, device=cuda) % 8] = 1.0
+    dd = r2.to_dense()
+    dd[torch.arange(9) % 8, torch.arange(9)] = 1.0
+    assert torch.equal(d2.to_dense().cpu(), dd)
+    # in-place permutation moves nothing
+    table_ptr = d2.storage()._table.data_ptr()
+    d2.permute_(1, 0)
+    assert tuple(d2.shape) == (9, 8) and d2.storage()._table.data_ptr() == table_ptr
+    assert torch.equal(d2.to_dense().cpu(), dd.T)
+    # flatten / reshape / unary ops go through the view order
+    assert torch.equal(v.flatten().to_dense().cpu(), dense.permute(2, 0, 1).reshape(-1))
+    assert torch.equal(v.reshape(30, 7).to_dense().cpu(), dense.permute(2, 0, 1).reshape(30, 7))
+    assert torch.equal(v.abs().to_dense().cpu(), dense.permute(2, 0, 1).abs())
