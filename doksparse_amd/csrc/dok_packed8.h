@@ -3,19 +3,23 @@
 // A 128-byte bucket holds S = 120 / (8 + V) slots and one metadata word:
 //     words 0 .. S-1           the S stored key words (8 bytes each)
 //     bytes 8*S .. 8*S + V*S   the S values, value s at byte 8*S + V*s
-//     word 15                  metadata: low 32 bits = the largest displacement (in buckets)
-//                              at which a key whose home is this bucket was ever placed
+//     word 15                  metadata about the keys whose HOME is this bucket:
+//                              bits 1..31  displacement map: bit d set = some key was placed d
+//                                          buckets past this one
+//                              bit 0       a key was placed 32 or more buckets past this one
+//                              bits 32..63 the largest such far displacement
 // (V=4: 10 slots, V=8: 7, V=2: 12, V=1: 13).  The stored key word is  key XOR DOK_P8_XOR,
 // and the two words 0 and 1 mean EMPTY and TOMBSTONE, so a cleared table is all zero bytes and
 // the slot word itself is the target of the claiming 64-bit compare-and-swap: an insert is one
 // CAS plus one value store into the same line.  The two keys whose stored word would be 0 or 1
 // live in two side slots of the table header instead (state word + value word each).
 //
-// Probing is linear over buckets.  A lookup of a key with home bucket h visits h, h+1, ... and
-// stops at a match, at a bucket that still has an EMPTY slot (a bucket never regains one:
-// remove leaves a TOMBSTONE), or once it has gone further than h's recorded largest
-// displacement.  The last rule is what keeps misses short in a nearly full table: most home
-// buckets never overflowed, so a miss is decided by the home bucket alone.
+// Placement is linear probing over buckets: a new key goes to the first tombstone on its chain,
+// else to the first empty slot, where the chain h, h+1, ... ends at the first bucket that still
+// has an EMPTY slot (a bucket never regains one: remove leaves a TOMBSTONE).  A lookup does not
+// walk that chain: after the home bucket it visits exactly the displacements marked in the home
+// bucket's map, and those loads do not depend on each other.  Most home buckets never
+// overflowed, so most misses are decided by the home bucket alone, also in a nearly full table.
 #pragma once
 #include "dok_device.h"
 
@@ -106,9 +110,9 @@ template <int V> struct P8Probe {
 // loads, then resolve U rounds" with no branch in between, so that a wave keeps U*4 bucket
 // lines in flight; everything a round decides is folded into the owner lane with selects
 // (rows that need no probe are carried through it and their outcome discarded).
-// Phase 2 walks the rows whose home bucket overflowed: per turn every group serves up to four
-// of its open rows (loads first, then the four outcomes folded into their owners, which then
-// act together).
+// Phase 2 serves the rows whose home bucket carries overflow marks: per turn every group takes
+// up to four of its open rows and loads the next two marked buckets of each (eight independent
+// loads per group), folds the outcomes into the owners, which then act together.
 #ifndef DOK_P8_U
 #define DOK_P8_U 8
 #endif
@@ -125,7 +129,7 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
   int l = L.l;
   DOK_OPAQUE(l);
   const u32 home = b;
-  u32 maxd = 0;                 // largest displacement recorded in the row's home bucket
+  u32 meta = 0;                 // low word of the home bucket's metadata
   bool open = false;            // row still unresolved after its home bucket
   slot_b = home;
 
@@ -155,7 +159,7 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
         const bool mine = l == r;
         my_gm = mine ? pr.gm : my_gm;
         my_ge = mine ? pr.ge : my_ge;
-        maxd = mine ? md : maxd;
+        meta = mine ? md : meta;
 #if !DOK_P8_VALUE_RELOAD
         my_v = mine ? v : my_v;
 #endif
@@ -172,59 +176,85 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
     }
 #endif
     if (pend) { found = hit1; slot_s = s1; if (hit1) val = my_v; }
-    open = pend && (my_gm | my_ge) == 0 && maxd != 0;
+    open = pend && my_gm == 0 && meta != 0;
     nprobe += pend;
   }
 
-  // Phase 2
-  u32 d = 1;
-  if (open) b = (home + 1 == nb) ? 0u : home + 1;
-  if (nb == 1) open = false;
+  // Phase 2: rows whose home bucket carries overflow marks.  `cand` holds the displacements still
+  // to be visited; the far walk (displacements >= 32, rare even in a 97 % full table) follows.
+  u32 cand = open ? (meta & ~1u) : 0u;
+  bool far = open && (meta & 1u);
+  u32 far_d = 32, far_max = 0;
+  if (far) far_max = (u32)(buckets[(u64)home * 16 + DOK_P8_META] >> 32);
+  bool hit2 = false;
   u64 pm = dok_ballot(open);
   while (pm != 0) {
+    // every open row offers its next two buckets
+    u32 d0 = 0, d1 = 0;
+    if (open) {
+      if (cand) {
+        d0 = __builtin_ctz(cand);
+        const u32 c2 = cand & (cand - 1);
+        if (c2) d1 = __builtin_ctz(c2);
+        else if (far && far_d <= far_max) d1 = far_d;
+      } else {
+        d0 = far_d;
+        if (far_d + 1 <= far_max) d1 = far_d + 1;
+      }
+    }
+    u64 t0 = (u64)home + d0, t1 = (u64)home + d1;
+    const u32 b0 = (u32)(t0 >= nb ? t0 - nb : t0), b1 = (u32)(t1 >= nb ? t1 - nb : t1);
     u32 rest = L.group(pm);
     int rr[DOK_P8_W];
-    bool hs[DOK_P8_W];
-    u64 w[DOK_P8_W];
+    bool hs[DOK_P8_W], h1[DOK_P8_W];
+    u64 w0[DOK_P8_W], w1[DOK_P8_W];
     #pragma unroll
     for (int k = 0; k < DOK_P8_W; k++) {
       hs[k] = rest != 0;
       rr[k] = hs[k] ? __builtin_ctz(rest) : 0;
       rest &= rest - 1;
-      const u32 qb = dok_shfl32(b, gbase + rr[k]);
-      w[k] = buckets[(u64)(hs[k] ? qb : 0u) * 16 + l];
+      const u32 qb0 = dok_shfl32(b0, gbase + rr[k]);
+      const u32 qb1 = dok_shfl32(b1, gbase + rr[k]);
+      h1[k] = hs[k] && dok_shfl32(d1, gbase + rr[k]) != 0;
+      w0[k] = buckets[(u64)(hs[k] ? qb0 : 0u) * 16 + l];
+      w1[k] = buckets[(u64)(h1[k] ? qb1 : 0u) * 16 + l];
     }
     bool act = false;
-    u32 my_gm = 0, my_ge = 0;
-    u64 my_v = 0;
-    int my_s = 0;
+    u32 gm0 = 0, gm1 = 0;
     #pragma unroll
     for (int k = 0; k < DOK_P8_W; k++) {
       const u64 q = dok_shfl64(sk, gbase + rr[k]);
-      P8Probe<V> pr;
-      pr.match(L, w[k], q);
-      const int s = pr.slot();
-      const u64 v = pr.value(L, w[k], s);
+      P8Probe<V> p0, p1;
+      p0.match(L, w0[k], q);
+      p1.match(L, w1[k], q);
       const bool mine = hs[k] && l == rr[k];
       act = act || mine;
-      my_gm = mine ? pr.gm : my_gm;
-      my_ge = mine ? pr.ge : my_ge;
-      my_v = mine ? v : my_v;
-      my_s = mine ? s : my_s;
+      gm0 = mine ? p0.gm : gm0;
+      gm1 = mine ? (h1[k] ? p1.gm : 0u) : gm1;
     }
     if (act) {
-      nprobe++;
-      if (my_gm) {
-        found = true; val = my_v; slot_b = b; slot_s = my_s; open = false;
-      } else if (my_ge) {
-        open = false;
+      nprobe += 1 + (d1 != 0);
+      if (gm0 | gm1) {
+        hit2 = true; open = false;
+        slot_b = gm0 ? b0 : b1;
+        slot_s = __builtin_ctz(gm0 ? gm0 : gm1);
       } else {
-        b = (b + 1 == nb) ? 0u : b + 1;
-        d++;
-        if (d > maxd || d >= nb) open = false;   // beyond every key homed at `home`: absent
+        // drop the visited displacements
+        if (cand) {
+          cand &= cand - 1;
+          if (d1 != 0) { if (cand) cand &= cand - 1; else far_d++; }
+        } else {
+          far_d += 1 + (d1 != 0);
+        }
+        open = cand != 0 || (far && far_d <= far_max);
       }
     }
     pm = dok_ballot(open);
+  }
+  if (hit2) {
+    typedef typename ValT<V>::type T;
+    found = true;
+    val = *(const T *)((const char *)(buckets + (u64)slot_b * 16) + 8 * P8<V>::S + V * slot_s);
   }
 }
 
@@ -364,7 +394,14 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
             const u64 old = atomicCAS(tp + ts, expect, sk);
             if (old == expect) {
               P8<V>::store(tp, ts, val);
-              if (td > md_home) atomicMax((u32 *)(hb + DOK_P8_META), td);
+              // mark the displacement in the home bucket's metadata (skipped when the view
+              // of it taken in phase 1 already shows the mark)
+              if (td >= 32) {
+                atomicMax((u32 *)(hb + DOK_P8_META) + 1, td);
+                if (!(md_home & 1u)) atomicOr((u32 *)(hb + DOK_P8_META), 1u);
+              } else if (td > 0 && !((md_home >> td) & 1u)) {
+                atomicOr((u32 *)(hb + DOK_P8_META), 1u << td);
+              }
               st = 1; fresh = 1; pend = false;
             } else if (old == sk) {
               st = 1; pend = false;                     // an equal key of this batch won the slot

@@ -500,6 +500,24 @@ class SparseDOKTensor(object):
         out = torch.sparse.sum(coo, dim=dim)
         return out
 
+    def norm(self, dim=None, p=2, keepdim=False):
+        coo = self.to_sparse_coo().coalesce()
+        v = coo.values()
+        powered = v.bool().to(v.dtype) if p == 0 else v.abs() if p == 1 else v.square() if p == 2 else v.abs().pow(p)
+        t = torch.sparse_coo_tensor(coo.indices(), powered, size=tuple(self.shape), device=self.device)
+        y = torch.sparse.sum(t) if dim is None else torch.sparse.sum(t, dim=dim)
+        y = y.to_dense() if y.is_sparse else y
+        if keepdim and dim is not None:
+            for d in sorted([dim] if isinstance(dim, int) else list(dim)):
+                y = y.unsqueeze(d)
+        return y.sqrt() if p == 2 else y.pow(1.0 / p) if p not in (0, 1) else y
+
+    def softmax(self, dim=-1):
+        return torch.sparse.softmax(self.to_sparse_coo().coalesce(), dim=dim % self.ndim)
+
+    def log_softmax(self, dim=-1):
+        return torch.sparse.log_softmax(self.to_sparse_coo().coalesce(), dim=dim % self.ndim)
+
     def index_select(self, dim, index):
         return self.to_sparse_coo().index_select(dim=dim, index=index)
 
