@@ -309,3 +309,44 @@ def test_probe_stats_are_in_the_expected_band(cuda):
     hits = hm.probe_stats(keys)
     misses = hm.probe_stats(torch.randint(0, 2**62, (n, 1), generator=g, device=cuda))
     assert 1.0 <= hits < 1.05 and 1.0 <= misses < 1.1
+
+
+def test_get_and_set_inside_a_hip_graph(cuda):
+    """The entry points allocate nothing and only enqueue kernels, so they can be captured: a
+    captured clear + set + get is replayed several times, with eager work and synchronisation
+    between the replays, and every replay must equal the eager result."""
+    import ctypes
+    from doksparse_amd import CudaClosedHashmap, _lib
+    lib = _lib.load()
+    g = torch.Generator(device=cuda).manual_seed(11)
+    n = 100_000
+    keys = torch.unique(torch.randint(0, 2**62, (n + 1000,), generator=g, device=cuda))[:n].contiguous()
+    vals = torch.randn(n, generator=g, device=cuda)
+    q = torch.cat([keys[: n // 2], torch.randint(0, 2**62, (n // 2,), generator=g, device=cuda)]).contiguous()
+    hm = CudaClosedHashmap(n_buckets=2 * n, device=cuda, rehash_threshold=1.0)
+    hm.set(keys[:, None], vals[:, None])
+    eager_v, eager_f = hm.get(q[:, None])
+    out_v = torch.zeros(n, 1, device=cuda)
+    out_f = torch.zeros(n, device=cuda, dtype=torch.bool)
+    desc = ctypes.byref(hm._desc)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            assert lib.dok_table_clear(desc, st) == 0
+            assert lib.dok_map_set(desc, keys.data_ptr(), vals.data_ptr(), n, None, st) == 0
+            assert lib.dok_map_get(desc, q.data_ptr(), n, out_v.data_ptr(), None, out_f.data_ptr(), st) == 0
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(4):
+        out_v.zero_()
+        out_f.zero_()
+        if rep == 2:
+            vals.mul_(2.0)                      # the graph reads the buffers, not a snapshot
+            eager_v = eager_v * 2.0
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_f, eager_f) and torch.equal(out_v, eager_v)
+        assert hm.n_elements == n               # the captured clear + set rebuilt the table
+        (torch.randn(1000, device=cuda) @ torch.randn(1000, device=cuda)).item()   # unrelated eager work
