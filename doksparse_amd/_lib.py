@@ -46,6 +46,7 @@ class DokTable(ctypes.Structure):
 class DokView(ctypes.Structure):
     _fields_ = [
         ("data", c_void_p),
+        ("base", c_int64),
         ("strides", c_int64 * DOK_MAX_DIMS),
     ]
 

@@ -52,7 +52,8 @@ struct DevIndex {
   i64 n_elems;
   i64 shape[DOK_MAX_DIMS];
   i64 estride[DOK_MAX_DIMS];       // C-contiguous strides of `shape`
-  const i64 *sel[DOK_MAX_DIMS];
+  const i64 *sel[DOK_MAX_DIMS];              // NULL: the coordinate is sbase + offset itself
+  i64 sbase[DOK_MAX_DIMS];
   i64 sstride[DOK_MAX_DIMS][DOK_MAX_DIMS];
   const void *src;
   i64 vstride[DOK_MAX_DIMS];
@@ -184,7 +185,8 @@ __device__ __forceinline__ bool dok_gather_at(const DevTable &t, const DevIndex 
       #pragma unroll
       for (int j = 0; j < DOK_MAX_DIMS; j++)
         if (j < ix.sel_ndim) off += idx[j] * ix.sstride[d][j];
-      i64 c = ix.sel[d][off];
+      const i64 *sp = ix.sel[d];
+      const i64 c = ix.sbase[d] + (sp ? sp[off] : off);
       ok = ok && ((u64)c < (u64)t.lin_dims[d]);
       k += (u64)c * (u64)t.lin_strides[d];
     }

@@ -86,8 +86,8 @@ int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *s
   }
   d.n_elems = (i64)n;
   for (int k = 0; k < ix->ndim; k++) {
-    if (!ix->sel[k].data && d.n_elems > 0) return DOK_EINVAL;
     d.sel[k] = (const i64 *)ix->sel[k].data;
+    d.sbase[k] = ix->sel[k].base;
     for (int j = 0; j < ix->sel_ndim; j++) {
       if (ix->sel[k].strides[j] < 0) return DOK_EINVAL;
       d.sstride[k][j] = ix->sel[k].strides[j];

@@ -266,13 +266,11 @@ class SparseDOKTensor(object):
         stop = max(min(stop, size), start)
         return start, stop
 
-    def _handle_selectors(self, selectors, return_slice_as_tensor=True):
-        """Turn an indexing expression into one int64 selector per tensor dimension, all
-        broadcast (as views) to the shape of the result, plus the positions of the scalar
-        selectors.  Reference: sparse_dok_tensor.py:220-300."""
+    def _normalise(self, selectors):
+        """One entry per tensor dimension: an int64 device tensor, a Python int, or a
+        (start, stop) pair for a slice."""
         if not isinstance(selectors, tuple):
             selectors = (selectors,)
-
         flat = []
         for sel in selectors:
             if isinstance(sel, np.ndarray):
@@ -284,7 +282,7 @@ class SparseDOKTensor(object):
             elif isinstance(sel, (bool, np.bool_)):
                 raise ValueError("boolean scalars are not valid selectors")
             elif isinstance(sel, (int, np.integer)):
-                flat.append(torch.tensor(int(sel), device=self.device, dtype=torch.long))
+                flat.append(int(sel))
             elif isinstance(sel, slice):
                 flat.append(sel)
             elif isinstance(sel, (tuple, list)):
@@ -294,40 +292,80 @@ class SparseDOKTensor(object):
         if len(flat) > self.ndim:
             raise IndexError(f"too many indices for tensor of dimension {self.ndim}")
         flat += [slice(None)] * (self.ndim - len(flat))
+        return [self._normalise_slice(s, i) if isinstance(s, slice) else s for i, s in enumerate(flat)]
 
-        scalar_positions = [i for i, s in enumerate(flat) if isinstance(s, Tensor) and s.ndim == 0]
-        tensors = [s for s in flat if isinstance(s, Tensor)]
-        n_slices = len(flat) - len(tensors)
-        bshape = tuple(torch.broadcast_shapes(*[t.shape for t in tensors])) if tensors else tuple()
-        out_ndim = len(bshape) + n_slices
-        first_tensor = next((i for i, s in enumerate(flat) if isinstance(s, Tensor)), None)
-
+    @staticmethod
+    def _broadcast_shape(shapes):
         out = []
-        axis = 0          # next free output axis for a slice
-        met_tensor = False
+        for shape in shapes:
+            shape = tuple(shape)
+            if len(shape) > len(out):
+                out = [1] * (len(shape) - len(out)) + out
+            off = len(out) - len(shape)
+            for k, n in enumerate(shape):
+                if out[off + k] == 1:
+                    out[off + k] = n
+                elif n != 1 and n != out[off + k]:
+                    raise RuntimeError(f"selector shapes {shapes} do not broadcast")
+        return tuple(out)
+
+    def _layout(self, flat):
+        """Where every selector lands in the result (reference rule, :255-296): the broadcast
+        axes of all tensor selectors (integers count as 0-dim tensors) sit together at the
+        position of the first of them; every slice keeps an axis of its own, in order.
+        Returns (bshape, first axis of the broadcast block, {dim: axis} for slices, out_shape,
+        scalar positions)."""
+        is_t = [not isinstance(s, tuple) for s in flat]
+        scalar_positions = [i for i, s in enumerate(flat)
+                            if isinstance(s, int) or (isinstance(s, Tensor) and s.ndim == 0)]
+        bshape = self._broadcast_shape([() if isinstance(s, int) else s.shape
+                                        for s, t in zip(flat, is_t) if t]) if any(is_t) else tuple()
+        first = is_t.index(True) if any(is_t) else None
+        out_shape, slice_axis = [], {}
         for i, sel in enumerate(flat):
-            if isinstance(sel, Tensor):
-                # broadcast axes of every tensor selector sit together at the first tensor's position
-                view_shape = [1] * out_ndim
-                view_shape[first_tensor:first_tensor + len(bshape)] = bshape
-                out.append(torch.broadcast_to(sel, bshape).reshape(view_shape))
-                if not met_tensor:
-                    axis += len(bshape)
-                    met_tensor = True
+            if is_t[i]:
+                if i == first:
+                    out_shape.extend(bshape)
             else:
-                start, stop = self._normalise_slice(sel, i)
+                slice_axis[i] = len(out_shape)
+                out_shape.append(sel[1] - sel[0])
+        return bshape, first, slice_axis, tuple(out_shape), scalar_positions
+
+    def _handle_selectors(self, selectors, return_slice_as_tensor=True):
+        """Turn an indexing expression into one int64 selector per tensor dimension, all
+        broadcast (as views) to the shape of the result, plus the positions of the scalar
+        selectors.  Reference: sparse_dok_tensor.py:220-300."""
+        flat = self._normalise(selectors)
+        bshape, first, slice_axis, out_shape, scalar_positions = self._layout(flat)
+        out_ndim = len(out_shape)
+        out = []
+        for i, sel in enumerate(flat):
+            if isinstance(sel, tuple):
                 if return_slice_as_tensor:
                     view_shape = [1] * out_ndim
-                    view_shape[axis] = stop - start
-                    out.append(torch.arange(start, stop, device=self.device).reshape(view_shape))
-                    axis += 1
+                    view_shape[slice_axis[i]] = sel[1] - sel[0]
+                    out.append(torch.arange(sel[0], sel[1], device=self.device).reshape(view_shape))
                 else:
-                    out.append(slice(start, stop))
+                    out.append(slice(sel[0], sel[1]))
+            else:
+                if isinstance(sel, int):
+                    sel = torch.tensor(sel, device=self.device, dtype=torch.long)
+                view_shape = [1] * out_ndim
+                view_shape[first:first + len(bshape)] = bshape
+                out.append(torch.broadcast_to(sel, bshape).reshape(view_shape))
         if return_slice_as_tensor:
             out = list(torch.broadcast_tensors(*out))
         return out, scalar_positions
 
+    def _fill_index(self, ix, storage_dim, data_ptr, base, strides):
+        view = ix.sel[storage_dim]
+        view.data = data_ptr
+        view.base = base
+        for j, st in enumerate(strides):
+            view.strides[j] = st
+
     def _index_desc(self, selectors):
+        """dok_index_t of materialised selectors (the result of _handle_selectors)."""
         out_shape = tuple(selectors[0].shape)
         if len(out_shape) > DOK_MAX_DIMS or self.ndim > DOK_MAX_DIMS:
             raise NotImplementedError(f"indexing expressions with more than {DOK_MAX_DIMS} axes")
@@ -336,17 +374,46 @@ class SparseDOKTensor(object):
         ix.sel_ndim = len(out_shape)
         for j, s in enumerate(out_shape):
             ix.shape[j] = s
-        for d, sel in enumerate(self._to_storage_order(selectors)):
+        keep = []
+        for d, sel in enumerate(selectors):
             assert sel.dtype == torch.long and sel.device == self.device
-            ix.sel[d].data = sel.data_ptr()
-            for j, st in enumerate(sel.stride()):
-                ix.sel[d].strides[j] = st
+            self._fill_index(ix, self._perm[d], sel.data_ptr(), 0, sel.stride())
+            keep.append(sel)
         return ix, out_shape
+
+    def _plan(self, selectors):
+        """dok_index_t straight from the expression: integers and slices become affine
+        selectors that need no device tensor (no arange kernel, no host-to-device copy of a
+        scalar); only real index tensors are passed by pointer.  Returns (descriptor, result
+        shape, scalar positions, tensors to keep alive until the launch)."""
+        flat = self._normalise(selectors)
+        bshape, first, slice_axis, out_shape, scalar_positions = self._layout(flat)
+        if len(out_shape) > DOK_MAX_DIMS or self.ndim > DOK_MAX_DIMS:
+            raise NotImplementedError(f"indexing expressions with more than {DOK_MAX_DIMS} axes")
+        ix = DokIndex()
+        ix.ndim = self.ndim
+        ix.sel_ndim = len(out_shape)
+        for j, s in enumerate(out_shape):
+            ix.shape[j] = s
+        keep = []
+        zeros = [0] * len(out_shape)
+        for d, sel in enumerate(flat):
+            strides = list(zeros)
+            if isinstance(sel, tuple):
+                strides[slice_axis[d]] = 1
+                self._fill_index(ix, self._perm[d], None, sel[0], strides)
+            elif isinstance(sel, int):
+                self._fill_index(ix, self._perm[d], None, sel, strides)
+            else:
+                view = torch.broadcast_to(sel, bshape)
+                strides[first:first + len(bshape)] = view.stride()
+                self._fill_index(ix, self._perm[d], view.data_ptr(), 0, strides)
+                keep.append(view)
+        return ix, out_shape, scalar_positions, keep
 
     # ------------------------------------------------------------------ indexing
     def __getitem__(self, selectors):
-        selectors, scalar_positions = self._handle_selectors(selectors)
-        ix, out_shape = self._index_desc(selectors)
+        ix, out_shape, scalar_positions, keep = self._plan(selectors)
         hm = self._hashmap
         if not hm._allocated:
             values = torch.zeros(out_shape, device=self.device, dtype=self.dtype)

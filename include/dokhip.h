@@ -64,9 +64,14 @@ typedef struct dok_table {
 } dok_table_t;
 
 /* A strided int64 (selector) or value (source) view over the broadcast index space.
- * Strides are in elements; 0 means the axis is broadcast. */
+ * Strides are in elements; 0 means the axis is broadcast.  For index vector idx[] the element
+ * offset is off = sum_j idx[j]*strides[j].  A selector yields the coordinate
+ * base + data[off], or, when data is NULL, base + off: an integer selector is {NULL, value, all
+ * strides 0}, a slice start:stop on result axis a is {NULL, start, strides[a] = 1} - neither
+ * needs a device tensor.  For a source-value view data must be set and base is ignored. */
 typedef struct dok_view {
-  const void *data;                    /* device */
+  const void *data;                    /* device, or NULL (selectors only)                       */
+  int64_t     base;
   int64_t     strides[DOK_MAX_DIMS];
 } dok_view_t;
 

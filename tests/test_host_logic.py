@@ -49,8 +49,8 @@ def test_library_exports_every_declared_symbol():
 def test_struct_sizes_match_the_header():
     # dok_table_t: 2 pointers + 2 x 8 + 4 x 4 + 8 x 8 bytes; dok_view_t: pointer + 8 x 8
     assert ctypes.sizeof(_lib.DokTable) == 8 + 8 + 8 + 8 + 16 + 64
-    assert ctypes.sizeof(_lib.DokView) == 8 + 64
-    assert ctypes.sizeof(_lib.DokIndex) == 8 + 64 + 8 * (8 + 64)
+    assert ctypes.sizeof(_lib.DokView) == 8 + 8 + 64
+    assert ctypes.sizeof(_lib.DokIndex) == 8 + 64 + 8 * (8 + 8 + 64)
 
 
 def test_layout_selection():
@@ -183,3 +183,60 @@ def test_empty_dok_tensor_on_cpu_reads_zero():
     assert torch.equal(dok.to_dense(), torch.zeros(5, 6))
     assert dok.indices().shape == (2, 0) and dok.values().shape == (0,)
     assert dok[:, 2, ].shape == (5,)
+
+
+def _coords_from_plan(ix, out_shape, ndim):
+    """Evaluate a dok_index_t the way the kernels do: coordinate = base + (data[off] | off)."""
+    grids = np.indices(out_shape).reshape(len(out_shape), -1) if len(out_shape) else np.zeros((0, 1), dtype=np.int64)
+    n = grids.shape[1] if len(out_shape) else 1
+    out = []
+    for d in range(ndim):
+        v = ix.sel[d]
+        off = np.zeros(n, dtype=np.int64)
+        for j in range(len(out_shape)):
+            off += grids[j] * v.strides[j]
+        if v.data:
+            buf = (ctypes.c_int64 * (int(off.max()) + 1 if n else 1)).from_address(v.data)
+            vals = np.frombuffer(buf, dtype=np.int64)[off]
+        else:
+            vals = off
+        out.append(vals + v.base)
+    return out
+
+
+@pytest.mark.parametrize("case", range(len(SELECTOR_CASES)))
+def test_affine_plan_equals_materialised_selectors(case):
+    g = torch.Generator().manual_seed(case)
+    r = torch.randint(0, 13, (6,), generator=g)
+    c = torch.randint(0, 17, (6,), generator=g)
+    m = torch.rand(17, generator=g) < 0.5
+    sel = SELECTOR_CASES[case](r, c, m)
+    dok = SparseDOKTensor(size=(13, 17), device="cpu")
+    mats, sc1 = dok._handle_selectors(sel)
+    ix, out_shape, sc2, keep = dok._plan(sel)
+    assert sc1 == sc2 and tuple(mats[0].shape) == out_shape
+    if int(np.prod(out_shape)) == 0:
+        return
+    for got, exp in zip(_coords_from_plan(ix, out_shape, 2), mats):
+        assert np.array_equal(got, exp.reshape(-1).numpy())
+
+
+def test_affine_plan_4d_and_views():
+    dok = SparseDOKTensor(size=(6, 7, 5, 4), device="cpu")
+    i, k = torch.tensor([0, 5, 2]), torch.tensor([3, 0, 1])
+    mask = torch.tensor([True, False, True, True])
+    for sel in [(slice(None), i, slice(None), k), (i, slice(None), k), (4, slice(0, 3), i[:2], k[:2]),
+                (2, slice(1, 5), i[:, None], mask), (3,), (3, 2, 1, 0), (slice(2, 2),)]:
+        mats, sc1 = dok._handle_selectors(sel)
+        ix, out_shape, sc2, keep = dok._plan(sel)
+        assert sc1 == sc2 and tuple(mats[0].shape) == out_shape
+        if int(np.prod(out_shape)) == 0:
+            continue
+        for got, exp in zip(_coords_from_plan(ix, out_shape, 4), mats):
+            assert np.array_equal(got, exp.reshape(-1).numpy())
+    # a permuted view fills the descriptor in the storage's dimension order
+    v = dok.permute(2, 0, 3, 1)
+    ix, out_shape, _, keep = v._plan((1, slice(None), 2, slice(0, 3)))
+    assert out_shape == (6, 3)
+    assert ix.sel[2].base == 1 and ix.sel[3].base == 2          # view dims 0, 2 -> storage dims 2, 3
+    assert list(ix.sel[0].strides)[:2] == [1, 0] and list(ix.sel[1].strides)[:2] == [0, 1]
