@@ -430,41 +430,47 @@ class SparseDOKTensor(object):
         return values
 
     def __setitem__(self, selectors, values):
-        selectors, _ = self._handle_selectors(selectors)
-        out_shape = tuple(selectors[0].shape)
         if isinstance(values, SparseDOKTensor) or (isinstance(values, Tensor) and values.is_sparse):
+            mats, _ = self._handle_selectors(selectors)
+            out_shape = tuple(mats[0].shape)
             assert tuple(values.shape) == out_shape, \
                 f"expecting the value shape to be {out_shape}, got {tuple(values.shape)} instead"
-            return self._set_items_sparse(values, selectors)
+            return self._set_items_sparse(values, mats)
+        ix, out_shape, _, keep = self._plan(selectors)
         if not isinstance(values, Tensor):
             values = torch.tensor(values, device=self.device, dtype=self.dtype)
         values = torch.broadcast_to(values.to(device=self.device, dtype=self.dtype), out_shape)
-        self._set_items_dense(values, selectors)
+        self._set_items_dense(values, ix, selectors)
 
-    def _set_items_dense(self, src, selectors):
-        """Reference: SparseDOKTensorImplCuda.set_items_dense (sparse_dok_tensor_impl.py:412-474)."""
+    def _set_items_dense(self, src, ix, expr):
+        """Reference: SparseDOKTensorImplCuda.set_items_dense (sparse_dok_tensor_impl.py:412-474).
+        One device read-back per call (after the kernel: entry count and error counters); the
+        reference's count kernel + `.item()` before the scatter is replaced by the in-kernel count."""
         n_sel = int(np.prod(src.shape, dtype=np.int64))
         if n_sel == 0:
             return
         hm = self._hashmap
         if not hm._allocated:
             # fixes the key/value widths; the entry itself is written again by the kernel below
-            first_key = torch.stack([s.reshape(-1)[0] for s in self._to_storage_order(selectors)], dim=0)[None]
+            mats, _ = self._handle_selectors(expr)
+            first_key = torch.stack([s.reshape(-1)[0] for s in self._to_storage_order(mats)], dim=0)[None]
             hm.set(first_key, src.reshape(-1)[:1, None].contiguous())
-        ix, _ = self._index_desc(selectors)
         view = DokView()
         view.data = src.data_ptr()
         for j, st in enumerate(src.stride()):
             view.strides[j] = st
         # growth rule of the reference: decided on the number of selector elements
-        n_now = hm.n_elements
-        if n_now + n_sel > hm.n_buckets * hm._rehash_threshold:
-            hm.rehash(int(np.ceil((n_now + n_sel) * hm._rehash_factor)))
+        limit = hm.n_buckets * hm._rehash_threshold
+        if hm._n_upper + n_sel > limit:
+            n_now = hm.n_elements
+            if n_now + n_sel > limit:
+                hm.rehash(int(np.ceil((n_now + n_sel) * hm._rehash_factor)))
         lib = _lib.load()
         _lib.check(lib.dok_setitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), ctypes.byref(view),
                                          _stream_ptr(self.device)), "__setitem__")
-        hm._n_upper = n_now + n_sel
-        n_oob = int(hm._header[_lib.DOK_H_NOOB].item())
+        header = hm._read_header()
+        hm._n_upper = int(header[_lib.DOK_H_NELEM])
+        n_oob = int(header[_lib.DOK_H_NOOB])
         if n_oob:
             hm._header[_lib.DOK_H_NOOB] = 0
             raise IndexError(f"{n_oob} coordinates fall outside the tensor of size {tuple(self.shape)}")
