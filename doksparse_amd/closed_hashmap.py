@@ -425,11 +425,37 @@ class CudaClosedHashmap:
             self._n_upper = n_old + n_miss
             return
         # otherwise count the distinct new keys exactly, as the reference does
-        n_new = int(keys[~is_found].unique(dim=0).shape[0])
+        n_new = self._count_distinct(keys[~is_found])
         if n_old + n_new > limit:
             self.rehash(int((n_old + n_new) * self._rehash_factor))
         self._launch_set(keys, values)
         self._n_upper = n_old + n_new
+
+    def _count_distinct(self, keys):
+        """Number of distinct rows of `keys` (the reference's `unique(dim=0).shape[0]`,
+        cuda_closed_hashmap.py:363).  For the packed layout the rows are inserted into a scratch
+        table of one-byte values and its entry count is read back - two kernels instead of a
+        sort of the whole batch."""
+        n = keys.shape[0]
+        if n == 0:
+            return 0
+        if self._layout != _lib.DOK_LAYOUT_PACKED8:
+            return int(keys.unique(dim=0).shape[0])
+        lib = _lib.load()
+        kb = 8 if self._coord_dims is not None else self._key_bytes
+        n_phys = int(lib.dok_phys_buckets_for(2 * n, kb, 1))
+        table = torch.empty(n_phys * DOK_BUCKET_BYTES, device=self.device, dtype=torch.uint8)
+        header = torch.empty(DOK_HEADER_WORDS, device=self.device, dtype=torch.long)
+        desc = self._make_desc(table, header, n_phys)
+        desc.value_bytes = 1
+        stream = _stream_ptr(self.device)
+        ones = torch.zeros(n, device=self.device, dtype=torch.uint8)
+        keys = self._prep_rows(keys, "keys")
+        _lib.check(lib.dok_table_clear(ctypes.byref(desc), stream), "clear")
+        _lib.check(lib.dok_map_set(ctypes.byref(desc), keys.data_ptr(), ones.data_ptr(), n, None, stream), "set")
+        h = header.cpu()
+        # out-of-range coordinate rows are skipped by the real insert as well
+        return int(h[_lib.DOK_H_NELEM])
 
     def get(self, keys, fallback_value=None):
         """(values, is_found) for a batch of keys (reference: cuda_closed_hashmap.py:386-421)."""

@@ -350,3 +350,30 @@ def test_get_and_set_inside_a_hip_graph(cuda):
         assert torch.equal(out_f, eager_f) and torch.equal(out_v, eager_v)
         assert hm.n_elements == n               # the captured clear + set rebuilt the table
         (torch.randn(1000, device=cuda) @ torch.randn(1000, device=cuda)).item()   # unrelated eager work
+
+
+def test_growth_from_a_small_table_counts_distinct_keys_like_the_reference(cuda):
+    """A large batch with repeats into a 1024-slot map: the growth target is computed from the
+    number of distinct new keys, exactly as the reference's get + unique pre-pass does."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(21)
+    base = np.unique(rng.integers(0, 2**62, size=200_000, dtype=np.int64))
+    keys = base[rng.integers(0, base.shape[0], size=400_000)][:, None]      # many repeats
+    n_distinct = np.unique(keys).shape[0]
+    for coord in (False, True):
+        if coord:
+            k = np.stack([keys[:, 0] % 100_003, (keys[:, 0] >> 20) % 99_991], axis=1)
+            n_distinct = np.unique(k, axis=0).shape[0]
+            hm = CudaClosedHashmap(n_buckets=1024, device=cuda, coord_dims=(100_003, 99_991))
+        else:
+            k = keys
+            hm = CudaClosedHashmap(n_buckets=1024, device=cuda)
+        vals = np.zeros((k.shape[0], 1), dtype=np.float32)
+        hm.set(torch.from_numpy(k).to(cuda), torch.from_numpy(vals).to(cuda))
+        assert hm.n_elements == n_distinct
+        assert hm.n_buckets == int(n_distinct * 2.0)
+        # a second batch: half known keys, half new ones, again with repeats
+        k2 = np.concatenate([k[:50_000], k[:50_000] + 1])
+        hm.set(torch.from_numpy(k2).to(cuda), torch.from_numpy(np.ones((k2.shape[0], 1), dtype=np.float32)).to(cuda))
+        merged = np.unique(np.concatenate([k, k2]), axis=0).shape[0]
+        assert hm.n_elements == merged
