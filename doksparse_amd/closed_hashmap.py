@@ -323,6 +323,34 @@ class CudaClosedHashmap:
             assert self._key_perm.shape[0] == int(np.prod(self._key_shape, dtype=np.int64))
         return self._key_perm
 
+    @key_perm.setter
+    def key_perm(self, new):
+        if not isinstance(new, Tensor):
+            new = torch.tensor(new, device=self.device, dtype=torch.long)
+        assert new.shape == self.key_perm.shape
+        self._key_perm = new.to(device=self.device, dtype=torch.long)
+
+    def permute_keys(self, ordering):
+        """Reorder the elements of every stored key (reference: :179-191).  Keys are hashed as
+        whole rows here, so the entries are moved into a fresh table."""
+        assert self._allocated, "hashmap is empty"
+        assert len(self._key_shape) == 1, "keys are not one dimensional"
+        assert len(ordering) == self._key_shape[0]
+        assert len(set(ordering)) == len(ordering), "duplicates are not allowed"
+        keys, values = self.items()
+        ordering = list(ordering)
+        if self._coord_dims is not None:
+            self._coord_dims = tuple(self._coord_dims[o] for o in ordering)
+        for name in ("_prime1", "_prime2", "_alpha1", "_alpha2", "_beta1", "_beta2"):
+            if getattr(self, name) is not None:
+                setattr(self, name, getattr(self, name)[ordering])
+        (self._table, self._header, self._desc, self._n_phys,
+         self._slots_per_bucket, self._layout) = self._alloc_table(self._n_buckets)
+        self._n_upper = 0
+        if keys.shape[0]:
+            self._launch_set(self._prep_rows(keys[:, ordering], "keys"), values.contiguous())
+            self._n_upper = keys.shape[0]
+
     @staticmethod
     def _hash_words(keys):
         n = keys.shape[0]

@@ -116,7 +116,12 @@ template <int V> struct P8Probe {
 #ifndef DOK_P8_U
 #define DOK_P8_U 8
 #endif
-#define DOK_P8_W 4   // rows per group per phase-2 turn
+#ifndef DOK_P8_WL
+#define DOK_P8_WL 2  // rows per group per phase-2 turn of the lookup
+#endif
+#ifndef DOK_P8_WI
+#define DOK_P8_WI 4  // rows per group per phase-2 turn of the insert
+#endif
 #ifndef DOK_P8_VALUE_RELOAD
 #define DOK_P8_VALUE_RELOAD 1
 #endif
@@ -205,11 +210,11 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
     u64 t0 = (u64)home + d0, t1 = (u64)home + d1;
     const u32 b0 = (u32)(t0 >= nb ? t0 - nb : t0), b1 = (u32)(t1 >= nb ? t1 - nb : t1);
     u32 rest = L.group(pm);
-    int rr[DOK_P8_W];
-    bool hs[DOK_P8_W], h1[DOK_P8_W];
-    u64 w0[DOK_P8_W], w1[DOK_P8_W];
+    int rr[DOK_P8_WL];
+    bool hs[DOK_P8_WL], h1[DOK_P8_WL];
+    u64 w0[DOK_P8_WL], w1[DOK_P8_WL];
     #pragma unroll
-    for (int k = 0; k < DOK_P8_W; k++) {
+    for (int k = 0; k < DOK_P8_WL; k++) {
       hs[k] = rest != 0;
       rr[k] = hs[k] ? __builtin_ctz(rest) : 0;
       rest &= rest - 1;
@@ -222,7 +227,7 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
     bool act = false;
     u32 gm0 = 0, gm1 = 0;
     #pragma unroll
-    for (int k = 0; k < DOK_P8_W; k++) {
+    for (int k = 0; k < DOK_P8_WL; k++) {
       const u64 q = dok_shfl64(sk, gbase + rr[k]);
       P8Probe<V> p0, p1;
       p0.match(L, w0[k], q);
@@ -349,11 +354,11 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
   u64 pm = dok_ballot(pend);
   while (pm != 0) {
     u32 rest = L.group(pm);
-    int rr[DOK_P8_W];
-    bool hs[DOK_P8_W];
-    u64 w[DOK_P8_W];
+    int rr[DOK_P8_WI];
+    bool hs[DOK_P8_WI];
+    u64 w[DOK_P8_WI];
     #pragma unroll
-    for (int k = 0; k < DOK_P8_W; k++) {
+    for (int k = 0; k < DOK_P8_WI; k++) {
       hs[k] = rest != 0;
       rr[k] = hs[k] ? __builtin_ctz(rest) : 0;
       rest &= rest - 1;
@@ -363,7 +368,7 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
     bool act = false;
     u32 gm = 0, ge = 0, gt = 0;
     #pragma unroll
-    for (int k = 0; k < DOK_P8_W; k++) {
+    for (int k = 0; k < DOK_P8_WI; k++) {
       const u64 q = dok_shfl64(sk, gbase + rr[k]);
       P8Probe<V> pr;
       pr.match(L, w[k], q);

@@ -377,3 +377,16 @@ def test_growth_from_a_small_table_counts_distinct_keys_like_the_reference(cuda)
         hm.set(torch.from_numpy(k2).to(cuda), torch.from_numpy(np.ones((k2.shape[0], 1), dtype=np.float32)).to(cuda))
         merged = np.unique(np.concatenate([k, k2]), axis=0).shape[0]
         assert hm.n_elements == merged
+
+
+def test_permute_keys(cuda):
+    from doksparse_amd import CudaClosedHashmap
+    g = torch.Generator(device=cuda).manual_seed(5)
+    keys = torch.unique(torch.randint(0, 50, (400, 3), generator=g, device=cuda), dim=0)
+    vals = torch.arange(keys.shape[0], device=cuda, dtype=torch.float32)[:, None]
+    hm = CudaClosedHashmap(n_buckets=2048, device=cuda)
+    hm.set(keys, vals)
+    hm.permute_keys([2, 0, 1])
+    v, f = hm.get(keys[:, [2, 0, 1]])
+    assert bool(f.all()) and torch.equal(v, vals) and hm.n_elements == keys.shape[0]
+    assert not bool(hm.get(keys + 100)[1].any())
