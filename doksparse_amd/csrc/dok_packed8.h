@@ -88,17 +88,6 @@ template <int V> struct P8Probe {
   }
   // index of the matching slot, 16 if none
   __device__ __forceinline__ int slot() const { return __builtin_ctz(gm | 0x10000u); }
-  // value of slot s, fetched from the lane of the group that holds it: the holding lanes
-  // pre-shift their word so that one 32-bit shuffle suffices for values up to 4 bytes
-  __device__ __forceinline__ u64 value(const P8Lane &L, u64 w, int s) const {
-    const int vlane = L.gbase + ((P8<V>::S + ((s * V) >> 3)) & 15);
-    if (V == 8) return dok_shfl64(w, vlane);
-    u32 pre;
-    if (V == 4) pre = (s & 1) ? (u32)(w >> 32) : (u32)w;
-    else pre = (u32)(w >> (((s * V) & 7) * 8));
-    const u32 got = dok_shfl32(pre, vlane);
-    return V == 4 ? (u64)got : (u64)(got & ((1u << (8 * (V & 3))) - 1u));
-  }
 };
 
 // ---- cooperative lookup -------------------------------------------------------------------
@@ -111,8 +100,9 @@ template <int V> struct P8Probe {
 // lines in flight; everything a round decides is folded into the owner lane with selects
 // (rows that need no probe are carried through it and their outcome discarded).
 // Phase 2 serves the rows whose home bucket carries overflow marks: per turn every group takes
-// up to four of its open rows and loads the next two marked buckets of each (eight independent
-// loads per group), folds the outcomes into the owners, which then act together.
+// up to DOK_P8_WL of its open rows and loads the next two marked buckets of each (independent
+// loads), folds the outcomes into the owners, which then act together.  Two rows per turn
+// measured best: most turns have few open rows and wider turns only add instructions.
 #ifndef DOK_P8_U
 #define DOK_P8_U 8
 #endif
@@ -121,9 +111,6 @@ template <int V> struct P8Probe {
 #endif
 #ifndef DOK_P8_WI
 #define DOK_P8_WI 4  // rows per group per phase-2 turn of the insert
-#endif
-#ifndef DOK_P8_VALUE_RELOAD
-#define DOK_P8_VALUE_RELOAD 1
 #endif
 template <int V>
 __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 nb, u64 sk, u32 b,
@@ -158,28 +145,21 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
         P8Probe<V> pr;
         pr.match(L, w[u], q);
         const u32 md = dok_shfl32((u32)w[u], gbase + DOK_P8_META);
-#if !DOK_P8_VALUE_RELOAD
-        const u64 v = pr.value(L, w[u], pr.slot());
-#endif
         const bool mine = l == r;
         my_gm = mine ? pr.gm : my_gm;
         my_ge = mine ? pr.ge : my_ge;
         meta = mine ? md : meta;
-#if !DOK_P8_VALUE_RELOAD
-        my_v = mine ? v : my_v;
-#endif
         DOK_SCHED_FENCE();
       }
     }
     const bool hit1 = pend && my_gm != 0;
     const int s1 = __builtin_ctz(my_gm | 0x10000u);
-#if DOK_P8_VALUE_RELOAD
-    // the bucket line was fetched a moment ago: read the value of the matching slot from it
+    // the bucket line was fetched a moment ago: the owner reads the value of the matching slot
+    // from it (cheaper than shuffling a value out of the group in every round)
     if (hit1) {
       typedef typename ValT<V>::type T;
       my_v = *(const T *)((const char *)(buckets + (u64)home * 16) + 8 * P8<V>::S + V * s1);
     }
-#endif
     if (pend) { found = hit1; slot_s = s1; if (hit1) val = my_v; }
     open = pend && my_gm == 0 && meta != 0;
     nprobe += pend;
@@ -285,8 +265,8 @@ __device__ __forceinline__ bool p8_side_get(const DevTable &t, u64 sk, u64 &val)
 //
 // Phase 1 inspects the home bucket of all 64 rows (batched loads as in the lookup), then the
 // whole wave issues its CAS / value stores together.  Phase 2 is the general walk for rows whose
-// home bucket was full or whose claim was lost, four rows per group per turn, the owners acting
-// together.  A key placed d > 0 buckets past its home raises the home bucket's recorded largest
+// home bucket was full or whose claim was lost, DOK_P8_WI rows per group per turn, the owners
+// acting together.  A key placed d > 0 buckets past its home raises the home bucket's recorded largest
 // displacement to d.
 template <int V>
 __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val, u32 home,
