@@ -549,10 +549,8 @@ class CudaClosedHashmap:
         scratch = torch.empty(scratch_bytes // 8, device=self.device, dtype=torch.long)
         count = torch.zeros(1, device=self.device, dtype=torch.long)
         stream = _stream_ptr(self.device)
-        # pass 1: count only, to size the outputs
-        _lib.check(lib.dok_map_compact(ctypes.byref(self._desc), None, None, 0, count.data_ptr(),
-                                       scratch.data_ptr(), stream), "compact")
-        n = int(count.item())
+        # the header already holds the number of live entries: size the outputs from it
+        n = self.n_elements
         keys = values = None
         if want_keys:
             keys = torch.empty(n, *self._key_shape, device=self.device, dtype=self._key_dtype)

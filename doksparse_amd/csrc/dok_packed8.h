@@ -526,7 +526,8 @@ template <int V>
 __device__ __forceinline__ bool p8_scan_load(const DevTable &t, i64 b, u64 &w) {
   const int l = threadIdx.x & 15;
   const bool valid = b < (i64)t.nb;
-  w = valid ? t.buckets[(u64)b * 16 + l] : 0;
+  // unconditional load (clamped) so that the unrolled scan loops keep several in flight
+  w = t.buckets[(u64)(valid ? b : (i64)t.nb - 1) * 16 + l];
   return valid && l < P8<V>::S && w >= 2;
 }
 
@@ -536,6 +537,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_chunk_count_kernel(DevTable t, i64
   if (wid >= n_chunks) return;
   const int lane = threadIdx.x & 63;
   i64 cnt = 0;
+  #pragma unroll 8
   for (int s = 0; s < DOK_CHUNK / 4; s++) {
     u64 w;
     const bool live = p8_scan_load<V>(t, wid * DOK_CHUNK + s * 4 + (lane >> 4), w);
@@ -588,6 +590,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_chunk_write_kernel(DevTable t, con
   const int lane = threadIdx.x & 63;
   const int gbase = lane & 48, l = lane & 15;
   i64 base = chunk_offsets[wid];
+  #pragma unroll 8
   for (int s = 0; s < DOK_CHUNK / 4; s++) {
     u64 w;
     const bool live = p8_scan_load<V>(t, wid * DOK_CHUNK + s * 4 + (lane >> 4), w);
@@ -623,6 +626,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_rehash_kernel(DevTable src, DevTab
   const int lane = threadIdx.x & 63;
   const int gbase = lane & 48, l = lane & 15;
   int n_fresh = 0, n_full = 0;
+  #pragma unroll 8
   for (int s = 0; s < DOK_CHUNK / 4; s++) {
     u64 w;
     const bool live = p8_scan_load<V>(src, wid * DOK_CHUNK + s * 4 + (lane >> 4), w);
@@ -653,6 +657,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_to_dense_kernel(DevTable t, void *
   if (wid >= n_chunks) return;
   const int lane = threadIdx.x & 63;
   const int gbase = lane & 48, l = lane & 15;
+  #pragma unroll 8
   for (int s = 0; s < DOK_CHUNK / 4; s++) {
     u64 w;
     const bool live = p8_scan_load<V>(t, wid * DOK_CHUNK + s * 4 + (lane >> 4), w);

@@ -324,7 +324,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, c
 
 __device__ __forceinline__ bool tg_scan_load(const DevTable &t, const TgLane &L, i64 b, u64 &w) {
   const bool valid = b < (i64)t.nb;
-  w = valid ? t.buckets[(u64)b * 16 + L.l] : 0;
+  w = t.buckets[(u64)(valid ? b : (i64)t.nb - 1) * 16 + L.l];
   return valid && L.is_tag && (w & 3ULL) == 3ULL;
 }
 
@@ -333,6 +333,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_chunk_count_kernel(DevTable t, TgG
   if (wid >= n_chunks) return;
   const TgLane L(g);
   i64 cnt = 0;
+  #pragma unroll 8
   for (int s = 0; s < DOK_CHUNK / 4; s++) {
     u64 w;
     const bool live = tg_scan_load(t, L, wid * DOK_CHUNK + s * 4 + (L.lane >> 4), w);
@@ -347,6 +348,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_chunk_write_kernel(DevTable t, TgG
   if (wid >= n_chunks) return;
   const TgLane L(g);
   i64 base = chunk_offsets[wid];
+  #pragma unroll 8
   for (int s = 0; s < DOK_CHUNK / 4; s++) {
     u64 w;
     const bool live_tag = tg_scan_load(t, L, wid * DOK_CHUNK + s * 4 + (L.lane >> 4), w);
