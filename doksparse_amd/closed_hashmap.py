@@ -459,6 +459,72 @@ class CudaClosedHashmap:
         self._launch_set(keys, values)
         self._n_upper = n_old + n_new
 
+    def set_coo(self, indices, values):
+        """`set` for a coordinate-keyed map with the coordinates laid out as a COO tensor holds
+        them: ``indices`` is [ndim, n] int64, ``values`` [n, *value_shape].  Saves the transpose
+        copy that `set(indices.T, ...)` needs (reference: sparse_dok_tensor.py:66-69)."""
+        assert self._coord_dims is not None, "set_coo needs a coordinate-keyed map"
+        assert indices.dim() == 2 and indices.shape[0] == len(self._coord_dims)
+        assert indices.shape[1] == values.shape[0]
+        if not self._allocated:
+            assert indices.device == values.device == self.device and indices.dtype == torch.long
+            self._init_storage(indices[:, :0].T, values)
+        else:
+            assert indices.dtype == torch.long and indices.device == self.device
+            assert values.dtype == self._value_dtype and values.device == self.device
+            assert tuple(values.shape[1:]) == self._value_shape
+        n = indices.shape[1]
+        if n == 0:
+            return
+        if self._layout != _lib.DOK_LAYOUT_PACKED8:
+            return self.set(indices.T, values)
+        indices = self._prep_rows(indices, "indices")
+        values = self._prep_rows(values, "values")
+        lib = _lib.load()
+
+        def launch():
+            _lib.check(lib.dok_coo_set(ctypes.byref(self._desc), indices.data_ptr(), values.data_ptr(), n,
+                                       _stream_ptr(self.device)), "set_coo")
+
+        limit = int(self._rehash_threshold * self._n_buckets)
+        if self._n_upper + n <= limit:
+            launch()
+            self._n_upper += n
+            return
+        n_old = self.n_elements
+        if n_old + n <= limit:
+            launch()
+            self._n_upper = n_old + n
+        elif n_old + n <= int(0.9 * self._physical_slots()):
+            launch()
+            n_now = self.n_elements
+            if n_now > limit:
+                self.rehash(int(n_now * self._rehash_factor))
+        else:
+            self.set(indices.T, values)       # the exact-count path works on key rows
+
+    def items_coo(self):
+        """(indices [ndim, n], values [n, *value_shape]) of a coordinate-keyed map, from one pass,
+        in slot order (reference: SparseDOKTensor.indices()/values(), sparse_dok_tensor.py:156-169)."""
+        assert self._coord_dims is not None
+        if not self._allocated:
+            return None, None
+        if self._layout != _lib.DOK_LAYOUT_PACKED8:
+            keys, values = self.items()
+            return keys.T.contiguous(), values
+        lib = _lib.load()
+        scratch = torch.empty(int(lib.dok_compact_scratch_bytes(ctypes.byref(self._desc))) // 8,
+                              device=self.device, dtype=torch.long)
+        count = torch.zeros(1, device=self.device, dtype=torch.long)
+        n = self.n_elements
+        indices = torch.empty(len(self._coord_dims), n, device=self.device, dtype=torch.long)
+        values = torch.empty(n, *self._value_shape, device=self.device, dtype=self._value_dtype)
+        if n:
+            _lib.check(lib.dok_coo_compact(ctypes.byref(self._desc), indices.data_ptr(), values.data_ptr(), n,
+                                           count.data_ptr(), scratch.data_ptr(), _stream_ptr(self.device)),
+                       "items_coo")
+        return indices, values
+
     def _count_distinct(self, keys):
         """Number of distinct rows of `keys` (the reference's `unique(dim=0).shape[0]`,
         cuda_closed_hashmap.py:363).  For the packed layout the rows are inserted into a scratch

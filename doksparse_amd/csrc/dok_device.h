@@ -120,12 +120,28 @@ __device__ __forceinline__ bool dok_linearise(const DevTable &t, const i64 *row,
   return ok;
 }
 
-// Key of batch row i as an 8-byte integer (packed layout): narrower keys are zero-extended.
-// LIN selects the coordinate-keyed form at compile time, so that kernels of plain tables never
-// touch (or hold in scalar registers) the sixteen dimension / stride words of the descriptor.
-template <bool LIN>
-__device__ __forceinline__ bool dok_load_key8(const DevTable &t, const void *keys, i64 i, u64 &key) {
-  if (LIN) return dok_linearise(t, (const i64 *)keys + i * t.lin_ndim, key);
+// Key formats of the batch buffers handed to the packed-layout kernels.  The format is a
+// template argument so that kernels of plain tables never touch (or hold in scalar registers)
+// the sixteen dimension / stride words of the descriptor.
+#define DOK_KF_RAW  0   // key_bytes (1, 2, 4, 8) raw bytes per row, zero-extended to 8
+#define DOK_KF_ROWS 1   // coordinate table, row-major:    keys[i * ndim + d]
+#define DOK_KF_COLS 2   // coordinate table, column-major: keys[d * n + i]   (COO "indices")
+
+// Key of batch row i (of n) as an 8-byte integer; false if a coordinate is out of range.
+template <int KF>
+__device__ __forceinline__ bool dok_load_key8(const DevTable &t, const void *keys, i64 i, i64 n, u64 &key) {
+  if (KF == DOK_KF_ROWS) return dok_linearise(t, (const i64 *)keys + i * t.lin_ndim, key);
+  if (KF == DOK_KF_COLS) {
+    bool ok = true;
+    u64 k = 0;
+    for (int d = 0; d < t.lin_ndim; d++) {
+      const i64 c = ((const i64 *)keys)[(i64)d * n + i];
+      ok = ok && ((u64)c < (u64)t.lin_dims[d]);
+      k += (u64)c * (u64)t.lin_strides[d];
+    }
+    key = k;
+    return ok;
+  }
   switch (t.key_bytes) {
     case 8: key = ((const u64 *)keys)[i]; break;
     case 4: key = ((const u32 *)keys)[i]; break;
@@ -135,16 +151,17 @@ __device__ __forceinline__ bool dok_load_key8(const DevTable &t, const void *key
   return true;
 }
 
-template <bool LIN>
-__device__ __forceinline__ void dok_store_key8(const DevTable &t, void *keys_out, i64 i, u64 key) {
-  if (LIN) {
-    i64 *row = (i64 *)keys_out + i * t.lin_ndim;
+// The inverse, for the read-out: row i of an output holding `cap` rows.
+template <int KF>
+__device__ __forceinline__ void dok_store_key8(const DevTable &t, void *keys_out, i64 i, i64 cap, u64 key) {
+  if (KF != DOK_KF_RAW) {
     u64 rem = key;
     for (int d = 0; d < t.lin_ndim; d++) {
-      u64 s = (u64)t.lin_strides[d];
-      u64 c = rem / s;
+      const u64 s = (u64)t.lin_strides[d];
+      const u64 c = rem / s;
       rem -= c * s;
-      row[d] = (i64)c;
+      if (KF == DOK_KF_ROWS) ((i64 *)keys_out)[i * t.lin_ndim + d] = (i64)c;
+      else ((i64 *)keys_out)[(i64)d * cap + i] = (i64)c;
     }
     return;
   }

@@ -412,7 +412,7 @@ __device__ __forceinline__ int p8_side_set(const DevTable &t, u64 sk, u64 val) {
 }
 
 // ---- kernels ------------------------------------------------------------------------------
-template <int V, bool STATS, bool LIN>
+template <int V, bool STATS, int KF>
 __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                          void *__restrict__ values, u8 *__restrict__ found_out,
                                                          u64 fallback) {
@@ -421,7 +421,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
     const i64 i = DOK_TILE_ROW();
     const bool active = i < n;
     u64 key = 0;
-    const bool ok = active && dok_load_key8<LIN>(t, keys, i, key);
+    const bool ok = active && dok_load_key8<KF>(t, keys, i, n, key);
     const u64 sk = key ^ DOK_P8_XOR;
     bool found = false;
     u64 val = fallback;
@@ -442,7 +442,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
   }
 }
 
-template <int V, bool LIN>
+template <int V, int KF>
 __global__ __launch_bounds__(DOK_TPB) void p8_set_kernel(DevTable t, const void *__restrict__ keys,
                                                          const void *__restrict__ values, i64 n,
                                                          u8 *__restrict__ stored) {
@@ -451,7 +451,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_set_kernel(DevTable t, const void 
     const i64 i = DOK_TILE_ROW();
     const bool active = i < n;
     u64 key = 0;
-    const bool ok = active && dok_load_key8<LIN>(t, keys, i, key);
+    const bool ok = active && dok_load_key8<KF>(t, keys, i, n, key);
     const u64 sk = key ^ DOK_P8_XOR;
     const u64 val = ok ? dok_load_val<V>(values, i) : 0;
     int st = 0, fresh = 0;
@@ -469,7 +469,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_set_kernel(DevTable t, const void 
 }
 
 // Tombstone the matching slot with a CAS so that equal keys in one batch remove it once.
-template <int V, bool LIN>
+template <int V, int KF>
 __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                             u8 *__restrict__ removed_out) {
   int n_removed = 0;
@@ -477,7 +477,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const vo
     const i64 i = DOK_TILE_ROW();
     const bool active = i < n;
     u64 key = 0;
-    const bool ok = active && dok_load_key8<LIN>(t, keys, i, key);
+    const bool ok = active && dok_load_key8<KF>(t, keys, i, n, key);
     const u64 sk = key ^ DOK_P8_XOR;
     bool found = false, removed = false;
     u64 val = 0;
@@ -495,7 +495,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const vo
   dok_wave_add_n(&t.header[DOK_H_NELEM], -n_removed);
 }
 
-template <int V, bool LIN>
+template <int V, int KF>
 __global__ __launch_bounds__(DOK_TPB) void p8_count_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                            i64 *count) {
   int n_found = 0;
@@ -503,7 +503,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_count_kernel(DevTable t, const voi
     const i64 i = DOK_TILE_ROW();
     const bool active = i < n;
     u64 key = 0;
-    const bool ok = active && dok_load_key8<LIN>(t, keys, i, key);
+    const bool ok = active && dok_load_key8<KF>(t, keys, i, n, key);
     const u64 sk = key ^ DOK_P8_XOR;
     bool found = false;
     u64 val = 0;
@@ -582,7 +582,7 @@ __global__ __launch_bounds__(1024) void dok_scan_kernel(i64 *counts, i64 n, cons
   }
 }
 
-template <int V, bool LIN>
+template <int V, int KF>
 __global__ __launch_bounds__(DOK_TPB) void p8_chunk_write_kernel(DevTable t, const i64 *chunk_offsets, i64 n_chunks,
                                                                  void *keys_out, void *values_out, i64 cap) {
   const i64 wid = (i64)blockIdx.x * (DOK_TPB / 64) + (threadIdx.x >> 6);
@@ -599,18 +599,18 @@ __global__ __launch_bounds__(DOK_TPB) void p8_chunk_write_kernel(DevTable t, con
     const u64 vword = dok_shfl64(w, gbase + vw);
     const i64 row = base + __popcll(m & ((1ULL << lane) - 1ULL));
     if (live && row < cap) {
-      if (keys_out) dok_store_key8<LIN>(t, keys_out, row, w ^ DOK_P8_XOR);
+      if (keys_out) dok_store_key8<KF>(t, keys_out, row, cap, w ^ DOK_P8_XOR);
       if (values_out) dok_store_val<V>(values_out, row, P8<V>::extract(vword, l));
     }
     base += __popcll(m);
   }
   // the two side slots come last
-  if (!LIN && wid == 0 && lane == 0) {
+  if (KF == DOK_KF_RAW && wid == 0 && lane == 0) {
     i64 row = chunk_offsets[n_chunks];
     for (u64 k = 0; k < 2; k++) {
       if (t.header[DOK_H_SIDE_STATE + k] != 0) {
         if (row < cap) {
-          if (keys_out) dok_store_key8<LIN>(t, keys_out, row, k ^ DOK_P8_XOR);
+          if (keys_out) dok_store_key8<KF>(t, keys_out, row, cap, k ^ DOK_P8_XOR);
           if (values_out) dok_store_val<V>(values_out, row, (u64)t.header[DOK_H_SIDE_VALUE + k]);
         }
         row++;

@@ -138,10 +138,10 @@ const i64 kMaxRows = (i64)0x7fffffff * DOK_TPB;
     case 4: { constexpr int V = 4; CALL; } break; \
     default: { constexpr int V = 8; CALL; } break; \
   }
-// the same, also binding LIN (coordinate-keyed table) for the kernels that read key rows
-#define P8_DISPATCH_LIN(vb, lin, CALL)                                   \
-  if (lin) { constexpr bool LIN = true; P8_DISPATCH(vb, CALL) }          \
-  else { constexpr bool LIN = false; P8_DISPATCH(vb, CALL) }
+// the same, also binding KF (key format of the batch buffer) for the kernels that read key rows
+#define P8_DISPATCH_LIN(vb, lin, CALL)                                          \
+  if (lin) { constexpr int KF = DOK_KF_ROWS; P8_DISPATCH(vb, CALL) }            \
+  else { constexpr int KF = DOK_KF_RAW; P8_DISPATCH(vb, CALL) }
 
 }  // namespace
 
@@ -183,7 +183,7 @@ int dok_map_get(const dok_table_t *t, const void *keys, int64_t n, void *values_
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
     const u64 fb = fallback_word(fallback, d.value_bytes);
-    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, false, LIN><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, false, KF><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
   } else {
     rc = tg_launch_get(d, keys, n, values_out, fallback, found, false, s);
     if (rc) return rc;
@@ -202,7 +202,7 @@ int dok_map_get_stats(const dok_table_t *t, const void *keys, int64_t n, void *v
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
     const u64 fb = fallback_word(fallback, d.value_bytes);
-    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, true, LIN><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, true, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
   } else {
     rc = tg_launch_get(d, keys, n, values_out, fallback, found, true, s);
     if (rc) return rc;
@@ -220,11 +220,25 @@ int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int6
   if (!keys || !values) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
-    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_set_kernel<V, LIN><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, values, n, stored)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_set_kernel<V, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, values, n, stored)));
   } else {
     rc = tg_launch_set(d, keys, values, n, stored, s);
     if (rc) return rc;
   }
+  return note_launch();
+}
+
+int dok_coo_set(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (d.lin_ndim == 0) return DOK_EINVAL;
+  if (n < 0 || n > kMaxRows) return DOK_EINVAL;
+  if (n == 0) return DOK_OK;
+  if (!indices || !values) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  { constexpr int KF = DOK_KF_COLS;
+    P8_DISPATCH(d.value_bytes, (p8_set_kernel<V, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, indices, values, n, nullptr))); }
   return note_launch();
 }
 
@@ -237,7 +251,7 @@ int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t *r
   if (!keys) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
-    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_remove_kernel<V, LIN><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_remove_kernel<V, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
   } else {
     rc = tg_launch_remove(d, keys, n, removed, s);
     if (rc) return rc;
@@ -254,7 +268,7 @@ int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n, in
   if (!keys || !count) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
-    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_count_kernel<V, LIN><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, (i64 *)count)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_count_kernel<V, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, (i64 *)count)));
   } else {
     rc = tg_launch_count(d, keys, n, (i64 *)count, s);
     if (rc) return rc;
@@ -282,11 +296,31 @@ int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out, int6
     P8_DISPATCH(d.value_bytes, (p8_chunk_count_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks)));
     dok_scan_kernel<<<1, 1024, 0, s>>>(offs, n_chunks, d.lin_ndim == 0 ? d.header : nullptr, (i64 *)count_out);
     if (keys_out || values_out) {
-      P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_chunk_write_kernel<V, LIN><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks, keys_out, values_out, capacity_rows)));
+      P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_chunk_write_kernel<V, KF><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks, keys_out, values_out, capacity_rows)));
     }
   } else {
     rc = tg_launch_compact(d, offs, n_chunks, keys_out, values_out, capacity_rows, (i64 *)count_out, s);
     if (rc) return rc;
+  }
+  return note_launch();
+}
+
+int dok_coo_compact(const dok_table_t *t, int64_t *indices_out, void *values_out, int64_t capacity,
+                    int64_t *count_out, void *scratch, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (d.lin_ndim == 0) return DOK_EINVAL;
+  if (!count_out || !scratch || capacity < 0) return DOK_EINVAL;
+  if (((uintptr_t)scratch & 7) != 0) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  const i64 n_chunks = chunks_of(d);
+  i64 *offs = (i64 *)scratch;
+  P8_DISPATCH(d.value_bytes, (p8_chunk_count_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks)));
+  dok_scan_kernel<<<1, 1024, 0, s>>>(offs, n_chunks, nullptr, (i64 *)count_out);
+  if (indices_out || values_out) {
+    constexpr int KF = DOK_KF_COLS;
+    P8_DISPATCH(d.value_bytes, (p8_chunk_write_kernel<V, KF><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks, indices_out, values_out, capacity)));
   }
   return note_launch();
 }

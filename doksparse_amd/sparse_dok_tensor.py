@@ -67,10 +67,11 @@ class SparseDOKTensor(object):
             assert len(values.shape) == 1
             assert indices.shape[1] == values.shape[0]
             assert indices.shape[0] == self.ndim
-            self._hashmap.set(
-                indices.T.to(self.device),
-                values.to(device=self.device, dtype=self.dtype)[:, None],
-            )
+            vals = values.to(device=self.device, dtype=self.dtype)[:, None]
+            if self._hashmap._coord_dims == tuple(self._size):
+                self._hashmap.set_coo(indices.to(self.device), vals)
+            else:
+                self._hashmap.set(indices.T.to(self.device), vals)
 
     def _adopt_storage(self, storage):
         """Use `storage` directly if it is keyed by coordinates of this size; otherwise move its
@@ -183,10 +184,10 @@ class SparseDOKTensor(object):
 
     # ------------------------------------------------------------------ read-out
     def indices(self):
-        keys = self._hashmap.keys()
-        if keys is None:
+        idx, _ = self._hashmap.items_coo()
+        if idx is None:
             return torch.empty(self.ndim, 0, device=self.device, dtype=torch.long)
-        return keys.T[list(self._perm)] if self._is_permuted() else keys.T
+        return idx[list(self._perm)] if self._is_permuted() else idx
 
     def values(self):
         values = self._hashmap.values()
@@ -204,11 +205,12 @@ class SparseDOKTensor(object):
         self._hashmap.set_values(selectors=selectors, new_values=new_values[:, None])
 
     def to_sparse_coo(self):
-        keys, values = self._hashmap.items()
-        if keys is None:
-            keys = torch.empty(0, self.ndim, device=self.device, dtype=torch.long)
+        idx, values = self._hashmap.items_coo()
+        if idx is None:
+            idx = torch.empty(self.ndim, 0, device=self.device, dtype=torch.long)
             values = torch.empty(0, 1, device=self.device, dtype=self.dtype)
-        idx = keys.T[list(self._perm)] if self._is_permuted() else keys.T
+        if self._is_permuted():
+            idx = idx[list(self._perm)]
         return torch.sparse_coo_tensor(indices=idx, values=values.flatten(), size=tuple(self.shape),
                                        device=self.device)
 

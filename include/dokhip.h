@@ -155,6 +155,21 @@ int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out,
  * Reference: CudaClosedHashmap.rehash (cuda_closed_hashmap.py:456-468). */
 int dok_map_rehash(const dok_table_t *src, const dok_table_t *dst, void *stream);
 
+/* ---- COO bridge (tables with lin_ndim > 0) -------------------------------------------------- */
+
+/* dok_map_set for coordinates given the way a COO tensor holds them: indices is
+ * [lin_ndim][n] int64 (coordinate d of entry i at indices[d*n + i]).  No per-row flag.
+ * Reference: SparseDOKTensor.__init__ / from_sparse_coo, which transpose and copy the indices
+ * before the set (sparse_dok_tensor.py:66-69, 71-84). */
+int dok_coo_set(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
+                void *stream);
+
+/* dok_map_compact emitting COO layout: indices_out is [lin_ndim][capacity] int64, values_out
+ * [capacity].  Either output may be NULL; count_out[0] receives the number of live entries.
+ * Reference: SparseDOKTensor.indices()/values()/to_sparse_coo (sparse_dok_tensor.py:156-203). */
+int dok_coo_compact(const dok_table_t *t, int64_t *indices_out, void *values_out, int64_t capacity,
+                    int64_t *count_out, void *scratch, void *stream);
+
 /* ---- DOK indexing (tables with lin_ndim > 0) ------------------------------------------------ */
 
 /* out[e] = value stored at the coordinate the selectors give for element e of the broadcast
