@@ -390,3 +390,46 @@ def test_permute_keys(cuda):
     v, f = hm.get(keys[:, [2, 0, 1]])
     assert bool(f.all()) and torch.equal(v, vals) and hm.n_elements == keys.shape[0]
     assert not bool(hm.get(keys + 100)[1].any())
+
+
+@pytest.mark.parametrize("vdtype", [np.float32, np.int64, np.float16])
+def test_completely_full_tables_exercise_far_displacements(cuda, vdtype):
+    """Tables filled to the last physical slot: the last keys land dozens of buckets past their
+    home, beyond the 31 displacements the home bucket's map can name, so lookups take the far
+    walk.  Then tombstone churn at 100 % load."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(31)
+    probe = CudaClosedHashmap(n_buckets=1, device=cuda)
+    probe.set(torch.zeros(1, 1, dtype=torch.long, device=cuda), torch.zeros(1, 1, device=cuda).to(torch.from_numpy(np.zeros(1, vdtype)).dtype))
+    slots = probe._slots_per_bucket
+    for n_phys in (40, 64, 200):
+        cap = n_phys * slots                                   # every physical slot
+        keys = np.unique(rng.integers(0, 2**62, size=cap + 64, dtype=np.int64))[:cap, None]
+        vals = rng.integers(-100, 100, size=(cap, 1)).astype(vdtype)
+        hm = CudaClosedHashmap(n_buckets=cap, device=cuda, rehash_threshold=1.0)
+        ref = RefClosedHashmap(n_buckets=cap, rehash_threshold=1.0, rng=np.random.default_rng(1))
+        k, v = _to(cuda, keys, vals)
+        hm.set(k, v)
+        ref.set(keys, vals)
+        assert hm.n_elements == ref.n_elements == cap
+        assert hm._n_phys == n_phys
+        meta = hm._table.view(torch.int64).reshape(n_phys, 16)[:, 15].cpu().numpy()
+        if n_phys >= 64:
+            assert (meta & 1).any(), "no far displacement was produced; the test lost its point"
+        q = np.concatenate([keys, rng.integers(0, 2**62, size=(cap, 1), dtype=np.int64)])
+        _check_get(hm, ref, q, cuda, fallback=-3)
+        assert hm.probe_stats(torch.from_numpy(q).to(cuda)) >= 1.0
+        for _ in range(3):                                      # churn at full load
+            gone = keys[rng.permutation(cap)[: cap // 3]]
+            m = hm.remove(torch.from_numpy(gone).to(cuda))
+            assert np.array_equal(m.cpu().numpy(), ref.remove(gone))
+            fresh = np.unique(rng.integers(0, 2**62, size=cap, dtype=np.int64))[: gone.shape[0], None]
+            fv = rng.integers(-100, 100, size=(fresh.shape[0], 1)).astype(vdtype)
+            a, b = _to(cuda, fresh, fv)
+            hm.set(a, b)
+            ref.set(fresh, fv)
+            keys = np.concatenate([np.setdiff1d(keys[:, 0], gone[:, 0]), fresh[:, 0]])[:, None]
+            assert hm.n_elements == ref.n_elements == cap
+            _check_get(hm, ref, q, cuda)
+            _check_get(hm, ref, keys, cuda)
+        _assert_same_map(hm, ref)
