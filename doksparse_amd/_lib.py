@@ -84,6 +84,7 @@ SIGNATURES = {
     "dok_setitem_sparse": (c_int32, [POINTER(DokTable), POINTER(DokIndex), c_void_p, c_void_p, c_int64,
                                      c_uint64, c_void_p]),
     "dok_to_dense": (c_int32, [POINTER(DokTable), c_void_p, c_void_p]),
+    "dok_line_gather": (c_int32, [POINTER(DokTable), c_int64, c_uint64, c_void_p, c_void_p]),
 }
 
 _lib = None

@@ -443,4 +443,18 @@ int dok_to_dense(const dok_table_t *t, void *dense, void *stream) {
   return note_launch();
 }
 
+int dok_line_gather(const dok_table_t *t, int64_t n, uint64_t seed, uint32_t *out, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (n < 0 || (n > 0 && !out)) return DOK_EINVAL;
+  if (n == 0) return DOK_OK;
+  const i64 groups = (n + 7) / 8;
+  i64 blocks = (groups * 16 + DOK_TPB - 1) / DOK_TPB;
+  if (blocks > 16384) blocks = 16384;
+  dok_line_gather_kernel<<<(unsigned)blocks, DOK_TPB, 0, (hipStream_t)stream>>>(
+      (const u64 *)d.buckets, d.nb, n, seed, out);
+  return note_launch();
+}
+
 }  // extern "C"

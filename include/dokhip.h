@@ -212,6 +212,12 @@ int dok_setitem_sparse(const dok_table_t *t, const dok_index_t *ix, const int64_
  * Reference: SparseDOKTensor.to_dense (sparse_dok_tensor.py:195-209). */
 int dok_to_dense(const dok_table_t *t, void *dense, void *stream);
 
+/* Measurement aid with no counterpart in the reference: out[i] = a checksum of one
+ * pseudo-randomly chosen 128-byte bucket line, for i in [0, n) - the memory access pattern of
+ * dok_map_get with the probing removed.  Its rate (lines per second) is the practical ceiling
+ * for lookups on this table; the benchmark reports it beside the published HBM peak. */
+int dok_line_gather(const dok_table_t *t, int64_t n, uint64_t seed, uint32_t *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

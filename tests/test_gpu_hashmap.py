@@ -433,3 +433,31 @@ def test_completely_full_tables_exercise_far_displacements(cuda, vdtype):
             _check_get(hm, ref, q, cuda)
             _check_get(hm, ref, keys, cuda)
         _assert_same_map(hm, ref)
+
+
+def test_line_gather_measurement_kernel_reads_the_lines_it_claims(cuda):
+    """dok_line_gather: out[i] = XOR of the sixteen 8-byte words (folded to 32 bits) of bucket
+    fmix64(i ^ seed) * n_buckets >> 64, recomputed here from a copy of the table."""
+    import ctypes
+    from doksparse_amd import CudaClosedHashmap, _lib
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    rng = np.random.default_rng(77)
+    k = _unique_i64(rng, 5000)
+    hm = CudaClosedHashmap(n_buckets=10000, device=cuda)
+    hm.set(torch.from_numpy(k[:, None]).to(cuda), torch.from_numpy(k[:, None].astype(np.float32)).to(cuda))
+    n, seed = 4099, 987654321
+    out = torch.zeros(n, device=cuda, dtype=torch.int32)
+    _lib.check(_lib.load().dok_line_gather(ctypes.byref(hm._desc), n, seed, out.data_ptr(), _stream_ptr(cuda)),
+               "line_gather")
+    table = hm._table.view(torch.int64).reshape(hm._n_phys, 16).cpu().numpy().view(np.uint64)
+    M = (1 << 64) - 1
+    expect = np.empty(n, dtype=np.uint32)
+    for i in range(n):
+        x = (i ^ seed) & M
+        x ^= x >> 33; x = (x * 0xff51afd7ed558ccd) & M
+        x ^= x >> 33; x = (x * 0xc4ceb9fe1a85ec53) & M
+        x ^= x >> 33
+        line = (x * hm._n_phys) >> 64
+        w = int(np.bitwise_xor.reduce(table[line]))
+        expect[i] = (w ^ (w >> 32)) & 0xffffffff
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), expect)
