@@ -461,3 +461,58 @@ def test_line_gather_measurement_kernel_reads_the_lines_it_claims(cuda):
         w = int(np.bitwise_xor.reduce(table[line]))
         expect[i] = (w ^ (w >> 32)) & 0xffffffff
     assert np.array_equal(out.cpu().numpy().view(np.uint32), expect)
+
+
+def test_calls_replay_inside_a_hip_graph(cuda):
+    """The library neither allocates nor synchronises, so get / set / remove can be captured in a
+    HIP graph.  Every replay (with eager work and synchronisation between replays) must equal the
+    eager result and the oracle."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(4242)
+    n = 20000
+    allk = _unique_i64(rng, 5 * n)
+    hm = CudaClosedHashmap(n_buckets=8 * n, device=cuda, rehash_threshold=1.0)
+    ref = RefClosedHashmap(n_buckets=8 * n, rng=np.random.default_rng(3), rehash_threshold=1.0)
+    k0 = allk[:n, None]
+    v0 = rng.standard_normal((n, 1)).astype(np.float32)
+    hm.set(torch.from_numpy(k0).to(cuda), torch.from_numpy(v0).to(cuda))
+    ref.set(k0, v0)
+
+    sk = torch.zeros(n, 1, device=cuda, dtype=torch.int64)      # static inputs of the graph
+    sv = torch.zeros(n, 1, device=cuda, dtype=torch.float32)
+    sq = torch.zeros(2 * n, 1, device=cuda, dtype=torch.int64)
+    sg = torch.zeros(n // 2, 1, device=cuda, dtype=torch.int64)
+    sk.copy_(torch.from_numpy(k0)); sv.copy_(torch.from_numpy(v0)); sq[:n].copy_(sk); sg.copy_(sk[: n // 2])
+    # eager warm-up of every kernel the graph will hold (module load must not happen in capture)
+    hm._launch_set(sk, sv)
+    hm.get(sq)
+    hm._remove_rows(sg)
+    hm._launch_set(sk, sv)
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        hm._launch_set(sk, sv)
+        removed = hm._remove_rows(sg)
+        values, found = hm.get(sq)
+    torch.cuda.synchronize()
+
+    for r in range(1, 4):
+        newk = allk[r * n:(r + 1) * n, None]
+        newv = rng.standard_normal((n, 1)).astype(np.float32)
+        gone = np.concatenate([allk[(r - 1) * n:(r - 1) * n + n // 4, None], newk[: n // 4]])
+        q = np.concatenate([allk[: 2 * n: 2, None], allk[3 * n:4 * n, None]])
+        sk.copy_(torch.from_numpy(newk)); sv.copy_(torch.from_numpy(newv))
+        sg.copy_(torch.from_numpy(gone)); sq.copy_(torch.from_numpy(q))
+        graph.replay()
+        torch.cuda.synchronize()
+        ref.set(newk, newv)
+        rrem = ref.remove(gone)            # unique rows: the mask is a permutation of the aligned one
+        rv, rf = ref.get(q)
+        assert int(removed.sum().item()) == int(rrem.sum())
+        assert np.array_equal(found.cpu().numpy(), rf)
+        assert np.array_equal(values.cpu().numpy()[rf], rv[rf])
+        ev, ef = hm.get(sq.clone())        # eager work between replays
+        assert torch.equal(ef, found) and torch.equal(ev[ef], values[found])
+        assert hm.n_elements == ref.n_elements
+        _assert_same_map(hm, ref)
