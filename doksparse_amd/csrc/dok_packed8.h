@@ -442,30 +442,168 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
   }
 }
 
-template <int V, int KF>
-__global__ __launch_bounds__(DOK_TPB) void p8_set_kernel(DevTable t, const void *__restrict__ keys,
-                                                         const void *__restrict__ values, i64 n,
-                                                         u8 *__restrict__ stored) {
+#ifndef DOK_STREAM_WAVES
+#define DOK_STREAM_WAVES 8   // waves per SIMD the streaming kernels are compiled for
+#endif
+// Streaming insert.  Every lane carries one row at some point of its walk (bucket home + d); a
+// pass loads the current bucket of all 64 rows (batched as in phase 1 of p8_insert), the owners
+// decide and claim together, and lanes whose row is finished take the next rows of the wave's
+// contiguous share [wave * rows_per_wave, (wave + 1) * rows_per_wave) of the n rows.  A row that
+// has to walk on therefore costs the wave one more bucket load in a later pass instead of a turn
+// of its own, and the number of bucket lines in flight does not drop when the table is nearly
+// full (at load factor 0.9 this is 1.3x faster than tile-wise p8_insert).  All loads are
+// device-coherent, so a row that lost its claim to another key simply starts over at its home
+// bucket in the next pass.  The placement rules are those of p8_insert.
+//
+// `src(i, key, val)` produces row i: 0 = insert key -> val, 1 = the row addresses nothing inside
+// the table's coordinate space (counted, reported as not stored), 2 = skip the row silently.
+// The header counters are updated once per wave at the end.
+template <int V, class Src>
+__device__ __forceinline__ void p8_stream_insert(const DevTable &t, i64 n, i64 rows_per_wave,
+                                                 u8 *__restrict__ stored, Src src) {
+  const P8Lane L;
+  const int gbase = L.gbase;
+  int l = L.l;
+  DOK_OPAQUE(l);
+  u64 *const buckets = t.buckets;
+  const u64 nb = t.nb;
+
+  const i64 wave = ((i64)blockIdx.x * DOK_TPB + threadIdx.x) >> 6;
+  i64 next = wave * rows_per_wave;
+  i64 end = next + rows_per_wave;
+  if (end > n) end = n;
+  if (next > end) next = end;
+
   int n_fresh = 0, n_full = 0, n_oob = 0;
-  DOK_TILE_LOOP(n) {
-    const i64 i = DOK_TILE_ROW();
-    const bool active = i < n;
-    u64 key = 0;
-    const bool ok = active && dok_load_key8<KF>(t, keys, i, n, key);
-    const u64 sk = key ^ DOK_P8_XOR;
-    const u64 val = ok ? dok_load_val<V>(values, i) : 0;
-    int st = 0, fresh = 0;
-    bool pend = ok;
-    if (ok && sk < 2) { fresh = p8_side_set(t, sk, val); st = 1; pend = false; }
-    p8_insert<V>(t.buckets, t.nb, sk, val, pend ? p8_home(sk, t) : 0u, pend, st, fresh);
-    if (active && stored) stored[i] = (u8)st;
-    n_fresh += fresh;
-    n_full += (ok && st == 0);
-    n_oob += (active && !ok);
+  bool act = false;
+  u64 sk = 0, val = 0;
+  i64 idx = 0;
+  u32 home = 0, d = 0, tomb_d = DOK_NONE32, md_home = 0;
+  int tomb_s = 0;
+
+  for (;;) {
+    // ---- lanes without a row take the next rows of the wave's share
+    const u64 freem = dok_ballot(!act);
+    if (!act) {
+      const int rank = __builtin_amdgcn_mbcnt_hi((u32)(freem >> 32), __builtin_amdgcn_mbcnt_lo((u32)freem, 0u));
+      const i64 i = next + rank;
+      if (i < end) {
+        u64 key = 0;
+        const int code = src(i, key, val);
+        sk = key ^ DOK_P8_XOR;
+        if (code == 1) {
+          n_oob++;
+          if (stored) stored[i] = 0;
+        } else if (code == 0) {
+          if (sk < 2) {
+            n_fresh += p8_side_set(t, sk, val);
+            if (stored) stored[i] = 1;
+          } else {
+            act = true; idx = i; home = p8_home(sk, t); d = 0; tomb_d = DOK_NONE32;
+          }
+        }
+      }
+    }
+    next += __popcll(freem);
+    if (next > end) next = end;
+    if (dok_ballot(act) == 0) {
+      if (next >= end) break;
+      continue;
+    }
+
+    // ---- one pass: the current bucket of every row
+    u32 b = 0;
+    if (act) {
+      const u64 bb = (u64)home + d;
+      b = (u32)(bb >= nb ? bb - nb : bb);
+    }
+    u32 gm = 0, ge = 0, gt = 0, md = 0;
+    #pragma unroll
+    for (int r0 = 0; r0 < 16; r0 += DOK_P8_U) {
+      u64 w[DOK_P8_U];
+      #pragma unroll
+      for (int u = 0; u < DOK_P8_U; u++) {
+        const u32 qb = dok_shfl32(b, gbase + r0 + u);
+        w[u] = dok_load_coherent(buckets + (u64)qb * 16 + l);
+      }
+      #pragma unroll
+      for (int u = 0; u < DOK_P8_U; u++) {
+        const int r = r0 + u;
+        const u64 q = dok_shfl64(sk, gbase + r);
+        P8Probe<V> pr;
+        pr.match(L, w[u], q);
+        pr.tombs(L, w[u]);
+        const u32 m = dok_shfl32((u32)w[u], gbase + DOK_P8_META);
+        const bool mine = l == r;
+        gm = mine ? pr.gm : gm;
+        ge = mine ? pr.ge : ge;
+        gt = mine ? pr.gt : gt;
+        md = mine ? m : md;
+        DOK_SCHED_FENCE();
+      }
+    }
+
+    // ---- the owners act together
+    if (act) {
+      int st = -1;                                   // -1 the row walks on, 0 failed, 1 stored
+      if (d == 0) md_home = md;
+      if (gm) {
+        P8<V>::store(buckets + (u64)b * 16, __builtin_ctz(gm), val);
+        st = 1;
+      } else {
+        if (tomb_d == DOK_NONE32 && gt) { tomb_d = d; tomb_s = __builtin_ctz(gt); }
+        const bool ring_done = (ge == 0) && ((u64)d + 1 >= nb);
+        if (ge || ring_done) {
+          if (tomb_d == DOK_NONE32 && ge == 0) {
+            st = 0;                                  // no free slot anywhere
+          } else {
+            u32 td; int ts; u64 expect;
+            if (tomb_d != DOK_NONE32) { td = tomb_d; ts = tomb_s; expect = DOK_P8_TOMB; }
+            else { td = d; ts = __builtin_ctz(ge); expect = DOK_P8_EMPTY; }
+            const u64 tbb = (u64)home + td;
+            u64 *tp = buckets + (tbb >= nb ? tbb - nb : tbb) * 16;
+            const u64 old = atomicCAS(tp + ts, expect, sk);
+            if (old == expect) {
+              P8<V>::store(tp, ts, val);
+              u64 *hb = buckets + (u64)home * 16;
+              if (td >= 32) {
+                atomicMax((u32 *)(hb + DOK_P8_META) + 1, td);
+                if (!(md_home & 1u)) atomicOr((u32 *)(hb + DOK_P8_META), 1u);
+              } else if (td > 0 && !((md_home >> td) & 1u)) {
+                atomicOr((u32 *)(hb + DOK_P8_META), 1u << td);
+              }
+              st = 1; n_fresh++;
+            } else if (old == sk) {
+              st = 1;                                // an equal key of this batch won the slot
+            } else {
+              d = 0; tomb_d = DOK_NONE32;            // somebody else's key: look again
+            }
+          }
+        } else {
+          d++;
+        }
+      }
+      if (st >= 0) {
+        if (stored) stored[idx] = (u8)st;
+        n_full += (st == 0);
+        act = false;
+      }
+    }
   }
   dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
   dok_wave_add_n(&t.header[DOK_H_NFULL], n_full);
   dok_wave_add_n(&t.header[DOK_H_NOOB], n_oob);
+}
+
+template <int V, int KF>
+__global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void p8_set_kernel(DevTable t, const void *__restrict__ keys,
+                                                         const void *__restrict__ values, i64 n,
+                                                         u8 *__restrict__ stored, i64 rows_per_wave) {
+  p8_stream_insert<V>(t, n, rows_per_wave, stored, [&](i64 i, u64 &key, u64 &val) -> int {
+    if (!dok_load_key8<KF>(t, keys, i, n, key)) return 1;
+    val = dok_load_val<V>(values, i);
+    return 0;
+  });
 }
 
 // Tombstone the matching slot with a CAS so that equal keys in one batch remove it once.
@@ -687,24 +825,13 @@ __global__ __launch_bounds__(DOK_TPB) void p8_getitem_kernel(DevTable t, DevInde
 }
 
 template <int V>
-__global__ __launch_bounds__(DOK_TPB) void p8_setitem_kernel(DevTable t, DevIndex ix) {
-  int n_fresh = 0, n_full = 0, n_oob = 0;
-  DOK_TILE_LOOP(ix.n_elems) {
-    const i64 e = DOK_TILE_ROW();
-    const bool active = e < ix.n_elems;
-    u64 key = 0; i64 voff = 0;
-    const bool ok = active && dok_gather_key(t, ix, e, key, voff);
-    const u64 sk = key ^ DOK_P8_XOR;
-    const u64 val = ok ? dok_load_val<V>(ix.src, voff) : 0;
-    int st = 0, fresh = 0;
-    p8_insert<V>(t.buckets, t.nb, sk, val, ok ? p8_home(sk, t) : 0u, ok, st, fresh);
-    n_fresh += fresh;
-    n_full += (ok && st == 0);
-    n_oob += (active && !ok);
-  }
-  dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
-  dok_wave_add_n(&t.header[DOK_H_NFULL], n_full);
-  dok_wave_add_n(&t.header[DOK_H_NOOB], n_oob);
+__global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void p8_setitem_kernel(DevTable t, DevIndex ix, i64 rows_per_wave) {
+  p8_stream_insert<V>(t, ix.n_elems, rows_per_wave, nullptr, [&](i64 e, u64 &key, u64 &val) -> int {
+    i64 voff = 0;
+    if (!dok_gather_key(t, ix, e, key, voff)) return 1;
+    val = dok_load_val<V>(ix.src, voff);
+    return 0;
+  });
 }
 
 template <int V>
@@ -773,36 +900,25 @@ __global__ __launch_bounds__(DOK_TPB) void p8_getitem_sparse_kernel(DevTable t, 
 // axes of the index space) and value src_values[k]; entries whose value is zero under
 // `nonzero_mask` (all ones for integers, sign bit cleared for floating values) are skipped.
 template <int V>
-__global__ __launch_bounds__(DOK_TPB) void p8_setitem_sparse_kernel(DevTable t, DevIndex ix,
+__global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void p8_setitem_sparse_kernel(DevTable t, DevIndex ix,
                                                                     const i64 *__restrict__ src_indices,
                                                                     const void *__restrict__ src_values,
-                                                                    i64 n_src, u64 nonzero_mask) {
-  int n_fresh = 0, n_full = 0, n_oob = 0;
-  DOK_TILE_LOOP(n_src) {
-    const i64 k = DOK_TILE_ROW();
-    const bool active = k < n_src;
+                                                                    i64 n_src, u64 nonzero_mask,
+                                                                    i64 rows_per_wave) {
+  p8_stream_insert<V>(t, n_src, rows_per_wave, nullptr, [&](i64 k, u64 &key, u64 &val) -> int {
     i64 idx[DOK_MAX_DIMS];
-    bool inside = active;
+    bool inside = true;
     #pragma unroll
     for (int j = 0; j < DOK_MAX_DIMS; j++) {
       idx[j] = 0;
-      if (j < ix.sel_ndim && active) {
+      if (j < ix.sel_ndim) {
         idx[j] = src_indices[(i64)j * n_src + k];
         inside = inside && ((u64)idx[j] < (u64)ix.shape[j]);
       }
     }
-    const u64 val = active ? dok_load_val<V>(src_values, k) : 0;
-    const bool nonzero = (val & nonzero_mask) != 0;
-    u64 key = 0; i64 voff = 0;
-    const bool ok = inside && nonzero && dok_gather_at(t, ix, idx, key, voff);
-    const u64 sk = key ^ DOK_P8_XOR;
-    int st = 0, fresh = 0;
-    p8_insert<V>(t.buckets, t.nb, sk, val, ok ? p8_home(sk, t) : 0u, ok, st, fresh);
-    n_fresh += fresh;
-    n_full += (ok && st == 0);
-    n_oob += (active && nonzero && !ok);
-  }
-  dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
-  dok_wave_add_n(&t.header[DOK_H_NFULL], n_full);
-  dok_wave_add_n(&t.header[DOK_H_NOOB], n_oob);
+    val = dok_load_val<V>(src_values, k);
+    if ((val & nonzero_mask) == 0) return 2;
+    i64 voff = 0;
+    return (inside && dok_gather_at(t, ix, idx, key, voff)) ? 0 : 1;
+  });
 }

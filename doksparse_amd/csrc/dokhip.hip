@@ -115,9 +115,17 @@ inline unsigned grid_for(i64 n) {
 }
 // ... or a fixed grid that fills the machine (8 workgroups on each of 256 CUs) and loops over the
 // tiles, for kernels that end with per-wave atomics on the table header.
+#ifndef DOK_COUNT_GRID
+#define DOK_COUNT_GRID 2048
+#endif
 inline unsigned grid_counting(i64 n) {
   const i64 tiles = (n + DOK_TPB - 1) / DOK_TPB;
-  return (unsigned)(tiles < 2048 ? tiles : 2048);
+  return (unsigned)(tiles < DOK_COUNT_GRID ? tiles : DOK_COUNT_GRID);
+}
+// Contiguous share of a batch that each wave of a streaming kernel works through.
+inline i64 rows_per_wave(i64 n, unsigned grid) {
+  const i64 waves = (i64)grid * (DOK_TPB / 64);
+  return (n + waves - 1) / waves;
 }
 inline i64 chunks_of(const DevTable &d) { return ((i64)d.nb + DOK_CHUNK - 1) / DOK_CHUNK; }
 inline unsigned chunk_grid(i64 n_chunks) { return (unsigned)((n_chunks + 3) / 4); }
@@ -220,7 +228,8 @@ int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int6
   if (!keys || !values) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
-    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_set_kernel<V, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, values, n, stored)));
+    const unsigned grid = grid_counting(n);
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_set_kernel<V, KF><<<grid, DOK_TPB, 0, s>>>(d, keys, values, n, stored, rows_per_wave(n, grid))));
   } else {
     rc = tg_launch_set(d, keys, values, n, stored, s);
     if (rc) return rc;
@@ -238,7 +247,8 @@ int dok_coo_set(const dok_table_t *t, const int64_t *indices, const void *values
   if (!indices || !values) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   { constexpr int KF = DOK_KF_COLS;
-    P8_DISPATCH(d.value_bytes, (p8_set_kernel<V, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, indices, values, n, nullptr))); }
+    const unsigned grid = grid_counting(n);
+    P8_DISPATCH(d.value_bytes, (p8_set_kernel<V, KF><<<grid, DOK_TPB, 0, s>>>(d, indices, values, n, nullptr, rows_per_wave(n, grid)))); }
   return note_launch();
 }
 
@@ -364,7 +374,8 @@ int dok_setitem_dense(const dok_table_t *t, const dok_index_t *ix, const dok_vie
   if (di.n_elems == 0) return DOK_OK;
   if (di.n_elems > kMaxRows) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
-  P8_DISPATCH(d.value_bytes, (p8_setitem_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di)));
+  const unsigned grid = grid_counting(di.n_elems);
+  P8_DISPATCH(d.value_bytes, (p8_setitem_kernel<V><<<grid, DOK_TPB, 0, s>>>(d, di, rows_per_wave(di.n_elems, grid))));
   return note_launch();
 }
 
@@ -424,8 +435,9 @@ int dok_setitem_sparse(const dok_table_t *t, const dok_index_t *ix, const int64_
   if (n_src == 0) return DOK_OK;
   if (!src_values || (!src_indices && di.sel_ndim > 0)) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
-  P8_DISPATCH(d.value_bytes, (p8_setitem_sparse_kernel<V><<<grid_counting(n_src), DOK_TPB, 0, s>>>(
-      d, di, (const i64 *)src_indices, src_values, n_src, nonzero_mask)));
+  const unsigned grid = grid_counting(n_src);
+  P8_DISPATCH(d.value_bytes, (p8_setitem_sparse_kernel<V><<<grid, DOK_TPB, 0, s>>>(
+      d, di, (const i64 *)src_indices, src_values, n_src, nonzero_mask, rows_per_wave(n_src, grid))));
   return note_launch();
 }
 
