@@ -90,6 +90,21 @@ template <int V> struct P8Probe {
   __device__ __forceinline__ int slot() const { return __builtin_ctz(gm | 0x10000u); }
 };
 
+// Which free slot of a bucket a key claims.  Each key scans the slots in a cyclic order of its
+// own (start = a cheap hash of the key), so that rows racing for one bucket mostly claim
+// different slots.  Equal keys share the order, and because free slots only become fewer while
+// an insert kernel runs, the first free slot in a fixed order is the same for every view that
+// still shows it free: equal keys of one batch always end up competing for one slot, never
+// claiming two.
+template <int V> __device__ __forceinline__ int p8_slot_start(u64 sk) {
+  const u32 x = ((u32)sk ^ (u32)(sk >> 32)) * 0x9E3779B1u;
+  return (int)(((x >> 16) * (u32)P8<V>::S) >> 16);
+}
+__device__ __forceinline__ int p8_pick(u32 free_mask, int start) {   // free_mask != 0
+  const u32 from = free_mask >> start;
+  return from ? start + __builtin_ctz(from) : __builtin_ctz(free_mask);
+}
+
 // ---- cooperative lookup -------------------------------------------------------------------
 // In: per-lane stored key `sk`, home bucket `b` (0 for rows that need no probe), `pend` (row
 // needs a table probe).  Out: found / value for the lane's own row; slot_b / slot_s locate the
@@ -278,6 +293,7 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
 
   int act1 = 0;                 // 0 walk on, 1 overwrite slot, 2 claim slot
   int slot = 0;
+  u32 my_pick = 0;              // match mask, else tombstone mask, else empty mask of the home bucket
   bool tomb_here = false;       // the chosen slot of the home bucket is a tombstone
   u32 md_home = 0;
 
@@ -302,7 +318,7 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
         const int a = pr.gm ? 1 : (pr.ge ? 2 : 0);
         const u32 pick = pr.gm ? pr.gm : (pr.gt ? pr.gt : pr.ge);
         act1 = mine ? a : act1;
-        slot = mine ? __builtin_ctz(pick | 0x10000u) : slot;
+        my_pick = mine ? pick : my_pick;
         tomb_here = mine ? (pr.gm == 0 && pr.gt != 0) : tomb_here;
         md_home = mine ? md : md_home;
         DOK_SCHED_FENCE();
@@ -310,6 +326,9 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
     }
   }
 
+  const int start = p8_slot_start<V>(sk);
+  if (act1 == 1) slot = __builtin_ctz(my_pick);
+  else if (my_pick) slot = p8_pick(my_pick, start);
   u64 *hb = buckets + (u64)home * 16;
   u32 b = home, d = 0;
   u32 tomb_b = DOK_NONE32, tomb_d = 0;
@@ -365,7 +384,7 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
         P8<V>::store(buckets + (u64)b * 16, __builtin_ctz(gm), val);
         st = 1; pend = false;
       } else {
-        if (tomb_b == DOK_NONE32 && gt) { tomb_b = b; tomb_s = __builtin_ctz(gt); tomb_d = d; }
+        if (tomb_b == DOK_NONE32 && gt) { tomb_b = b; tomb_s = p8_pick(gt, start); tomb_d = d; }
         const bool ring_done = (ge == 0) && (++iters >= nb);
         if (ge || ring_done) {
           // chain end: the key is absent
@@ -374,7 +393,7 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
           } else {
             u32 tb, td; int ts; u64 expect;
             if (tomb_b != DOK_NONE32) { tb = tomb_b; ts = tomb_s; td = tomb_d; expect = DOK_P8_TOMB; }
-            else { tb = b; ts = __builtin_ctz(ge); td = d; expect = DOK_P8_EMPTY; }
+            else { tb = b; ts = p8_pick(ge, start); td = d; expect = DOK_P8_EMPTY; }
             u64 *tp = buckets + (u64)tb * 16;
             const u64 old = atomicCAS(tp + ts, expect, sk);
             if (old == expect) {
@@ -518,17 +537,25 @@ __device__ __forceinline__ void p8_stream_insert(const DevTable &t, i64 n, i64 r
       b = (u32)(bb >= nb ? bb - nb : bb);
     }
     u32 gm = 0, ge = 0, gt = 0, md = 0;
+    const u64 actm = dok_ballot(act);
+    const u32 rows_on = L.group(actm);               // lanes without a row load nothing
+    u32 rounds_on = (u32)actm | (u32)(actm >> 32);   // rounds in which no group has a row are skipped
+    rounds_on = (rounds_on | (rounds_on >> 16)) & 0xffffu;
     #pragma unroll
     for (int r0 = 0; r0 < 16; r0 += DOK_P8_U) {
       u64 w[DOK_P8_U];
       #pragma unroll
       for (int u = 0; u < DOK_P8_U; u++) {
-        const u32 qb = dok_shfl32(b, gbase + r0 + u);
-        w[u] = dok_load_coherent(buckets + (u64)qb * 16 + l);
+        w[u] = 0;
+        if ((rounds_on >> (r0 + u)) & 1u) {
+          const u32 qb = dok_shfl32(b, gbase + r0 + u);
+          if ((rows_on >> (r0 + u)) & 1u) w[u] = dok_load_coherent(buckets + (u64)qb * 16 + l);
+        }
       }
       #pragma unroll
       for (int u = 0; u < DOK_P8_U; u++) {
         const int r = r0 + u;
+        if (!((rounds_on >> r) & 1u)) continue;
         const u64 q = dok_shfl64(sk, gbase + r);
         P8Probe<V> pr;
         pr.match(L, w[u], q);
@@ -546,12 +573,13 @@ __device__ __forceinline__ void p8_stream_insert(const DevTable &t, i64 n, i64 r
     // ---- the owners act together
     if (act) {
       int st = -1;                                   // -1 the row walks on, 0 failed, 1 stored
+      const int start = p8_slot_start<V>(sk);
       if (d == 0) md_home = md;
       if (gm) {
         P8<V>::store(buckets + (u64)b * 16, __builtin_ctz(gm), val);
         st = 1;
       } else {
-        if (tomb_d == DOK_NONE32 && gt) { tomb_d = d; tomb_s = __builtin_ctz(gt); }
+        if (tomb_d == DOK_NONE32 && gt) { tomb_d = d; tomb_s = p8_pick(gt, start); }
         const bool ring_done = (ge == 0) && ((u64)d + 1 >= nb);
         if (ge || ring_done) {
           if (tomb_d == DOK_NONE32 && ge == 0) {
@@ -559,7 +587,7 @@ __device__ __forceinline__ void p8_stream_insert(const DevTable &t, i64 n, i64 r
           } else {
             u32 td; int ts; u64 expect;
             if (tomb_d != DOK_NONE32) { td = tomb_d; ts = tomb_s; expect = DOK_P8_TOMB; }
-            else { td = d; ts = __builtin_ctz(ge); expect = DOK_P8_EMPTY; }
+            else { td = d; ts = p8_pick(ge, start); expect = DOK_P8_EMPTY; }
             const u64 tbb = (u64)home + td;
             u64 *tp = buckets + (tbb >= nb ? tbb - nb : tbb) * 16;
             const u64 old = atomicCAS(tp + ts, expect, sk);
