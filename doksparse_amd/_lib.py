@@ -69,6 +69,9 @@ SIGNATURES = {
     "dok_map_get": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "dok_map_get_stats": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "dok_map_set": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
+    "dok_bulk_workspace_bytes": (c_int64, [POINTER(DokTable), c_int64]),
+    "dok_map_set_bulk": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
+    "dok_coo_set_bulk": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "dok_map_remove": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p]),
     "dok_map_count_existing": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p]),
     "dok_compact_scratch_bytes": (c_int64, [POINTER(DokTable)]),

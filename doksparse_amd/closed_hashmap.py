@@ -33,6 +33,14 @@ def _stream_ptr(device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
+# A batch goes through the bulk insert (partition by table range, merge each range in LDS)
+# instead of the per-row compare-and-swap kernel when it is large in absolute terms and holds at
+# least this many rows per physical bucket: the bulk path streams the whole table once, which
+# pays off only then.
+BULK_MIN_ROWS = 1 << 20
+BULK_MIN_ROWS_PER_BUCKET = 1.5
+
+
 def _next_prime(n):
     """Smallest prime > n (deterministic Miller-Rabin, exact below 3.3e24)."""
     def is_prime(m):
@@ -400,10 +408,34 @@ class CudaClosedHashmap:
         assert tuple(keys.shape[1:]) == self._key_shape
 
     # ------------------------------------------------------------------ set / get / remove
-    def _launch_set(self, keys, values):
+    def _bulk_workspace(self, n):
+        """Workspace tensor for a bulk insert of n rows, or None if the batch should take the
+        per-row kernel."""
+        if self._layout != _lib.DOK_LAYOUT_PACKED8:
+            return None
+        if n < BULK_MIN_ROWS or n < BULK_MIN_ROWS_PER_BUCKET * self._n_phys:
+            return None
+        nbytes = int(_lib.load().dok_bulk_workspace_bytes(ctypes.byref(self._desc), n))
+        if nbytes <= 0:
+            return None
+        ws = torch.empty(nbytes, device=self.device, dtype=torch.uint8)
+        assert ws.data_ptr() % 256 == 0
+        return ws
+
+    def _launch_set(self, keys, values, coo=False):
+        """Enqueue one insert of the batch.  coo=True: `keys` is the [ndim, n] coordinate matrix
+        of a coordinate-keyed map instead of [n, ...] key rows."""
         lib = _lib.load()
-        _lib.check(lib.dok_map_set(ctypes.byref(self._desc), keys.data_ptr(), values.data_ptr(),
-                                   keys.shape[0], None, _stream_ptr(self.device)), "set")
+        n = keys.shape[1] if coo else keys.shape[0]
+        desc, stream = ctypes.byref(self._desc), _stream_ptr(self.device)
+        ws = self._bulk_workspace(n)
+        if ws is not None:
+            fn = lib.dok_coo_set_bulk if coo else lib.dok_map_set_bulk
+            _lib.check(fn(desc, keys.data_ptr(), values.data_ptr(), n, ws.data_ptr(), ws.numel(), stream), "set")
+        elif coo:
+            _lib.check(lib.dok_coo_set(desc, keys.data_ptr(), values.data_ptr(), n, stream), "set_coo")
+        else:
+            _lib.check(lib.dok_map_set(desc, keys.data_ptr(), values.data_ptr(), n, None, stream), "set")
 
     def _physical_slots(self):
         return self._n_phys * self._slots_per_bucket
@@ -480,11 +512,9 @@ class CudaClosedHashmap:
             return self.set(indices.T, values)
         indices = self._prep_rows(indices, "indices")
         values = self._prep_rows(values, "values")
-        lib = _lib.load()
 
         def launch():
-            _lib.check(lib.dok_coo_set(ctypes.byref(self._desc), indices.data_ptr(), values.data_ptr(), n,
-                                       _stream_ptr(self.device)), "set_coo")
+            self._launch_set(indices, values, coo=True)
 
         limit = int(self._rehash_threshold * self._n_buckets)
         if self._n_upper + n <= limit:

@@ -1,0 +1,704 @@
+// Bulk insert for the packed layout: partition the batch by table range, then merge each range
+// in LDS.
+//
+// The ordinary insert (p8_set_kernel) pays one returning 64-bit atomic in HBM per row, and the
+// rate of those atomics - not memory bandwidth - is what bounds it.  When a batch holds more
+// than about one row per bucket of the table it is cheaper to stream the whole table through
+// the LDS once:
+//
+//   1. the table is cut into ranges of DOK_BULK_R consecutive buckets; the range of a row is
+//      (home bucket) / DOK_BULK_R;
+//   2. two count + scan + scatter passes (first by range / DOK_BULK_SUB, then by range inside
+//      each first-level bin) move every (key, value) row next to the other rows of its range.
+//      Every workgroup of a scatter owns a fixed stretch of the input; the count pass records how
+//      many of that stretch's rows go to each bin, a prefix sum over the workgroups turns the
+//      counts into the workgroup's private write cursors, and the scatter therefore needs no
+//      atomic on global memory.  A scatter tile is staged in LDS ordered by bin, so the global
+//      writes are runs of consecutive addresses;
+//   3. one workgroup per range copies the range's buckets into LDS, places the range's rows
+//      there and streams the buckets back;
+//   4. rows the merge cannot place by looking at their home bucket alone are handed, packed, to
+//      the ordinary insert, which runs last.
+//
+// Every step is exact for any input: bin sizes are counted, not estimated, and a batch whose
+// rows all fall into one range merely degrades to step 4's ordinary insert.
+#pragma once
+#include "dok_packed8.h"
+
+#ifndef DOK_BULK_RLOG
+#define DOK_BULK_RLOG 8                     // log2 of the buckets per range: 256 buckets = 32 KiB
+#endif
+#define DOK_BULK_R (1 << DOK_BULK_RLOG)
+#define DOK_BULK_SUBLOG 8
+#define DOK_BULK_SUB (1 << DOK_BULK_SUBLOG) // ranges per first-level bin
+#define DOK_BULK_MAXBIG 1024                // first-level bins at most
+#define DOK_BULK_TPB 256
+#ifndef DOK_BULK_T
+#define DOK_BULK_T 2048                     // rows per scatter tile
+#endif
+#define DOK_BULK_RPT (DOK_BULK_T / DOK_BULK_TPB)
+#ifndef DOK_BULK_GRID
+#define DOK_BULK_GRID 1024                  // workgroups of the first pass and of the merge
+#endif
+
+#ifdef DOK_BULK_TIMING
+#define BULK_TICK(k) do { if (threadIdx.x == 0) { const u64 now_ = wall_clock64(); tacc[k] += now_ - tlast; tlast = now_; } } while (0)
+#else
+#define BULK_TICK(k) do { } while (0)
+#endif
+
+// Device view of the caller's workspace.
+struct BulkWs {
+  u64 *keysA, *keysB;       // [n] each: rows after the first / second scatter
+  void *valsA, *valsB;      // [n] values of value_bytes each
+  u32 *wg_hist;             // [n_big][GRID]: rows of workgroup w's stretch that go to first-level bin b;
+                            //                after the scan, the exclusive prefix sum over w
+  u32 *big_off;             // [n_big + 1]    start of every first-level bin in keysA
+  u32 *sub_hist;            // [n_big][SUB][ch]: the same for the ch stretches of a first-level bin
+  u32 *part_off;            // [n_big * SUB + 1]  start of every range in keysB
+  u32 *def_cnt;             // [GRID] rows each merge workgroup handed to the ordinary insert
+  u32 n_big, n_part;
+  u32 ch;                   // stretches (workgroups) per first-level bin in the second pass
+  i64 share;                // rows per workgroup in the first pass
+};
+
+// Exclusive prefix sum of one value per thread over the workgroup (blockDim.x a multiple of 64,
+// at most 1024).  `wsum` is LDS scratch of 16 words.  Ends with a barrier.
+__device__ __forceinline__ u32 bulk_block_scan(u32 v, u32 *wsum, u32 &total) {
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  u32 inc = v;
+  #pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const u32 up = __shfl_up(inc, o, 64);
+    if (lane >= o) inc += up;
+  }
+  if (lane == 63) wsum[wv] = inc;
+  __syncthreads();
+  u32 pre = 0, tot = 0;
+  for (int k = 0; k < nw; k++) {
+    const u32 s = wsum[k];
+    if (k < wv) pre += s;
+    tot += s;
+  }
+  total = tot;
+  __syncthreads();
+  return pre + inc - v;
+}
+
+__device__ __forceinline__ u32 bulk_range_of(u64 key, const DevTable &t) {
+  return p8_home(key ^ DOK_P8_XOR, t) >> DOK_BULK_RLOG;
+}
+
+// The stretch of rows that workgroup `w` of a pass owns.
+__device__ __forceinline__ void bulk_stretch1(const BulkWs &ws, i64 n, u32 w, i64 &lo, i64 &hi) {
+  lo = (i64)w * ws.share;
+  hi = lo + ws.share;
+  if (hi > n) hi = n;
+  if (lo > hi) lo = hi;
+}
+__device__ __forceinline__ void bulk_stretch2(const BulkWs &ws, u32 b, u32 c, i64 &lo, i64 &hi) {
+  const i64 lo0 = ws.big_off[b], hi0 = ws.big_off[b + 1];
+  const i64 len = (hi0 - lo0 + ws.ch - 1) / ws.ch;
+  lo = lo0 + (i64)c * len;
+  hi = lo + len;
+  if (hi > hi0) hi = hi0;
+  if (lo > hi) lo = hi;
+}
+
+// ---- pass 1, count: rows of every workgroup's stretch per first-level bin ------------------------
+template <int KF>
+__global__ __launch_bounds__(DOK_BULK_TPB) void bulk_count1_kernel(DevTable t, const void *__restrict__ keys, i64 n,
+                                                                   BulkWs ws) {
+  __shared__ u32 cnt[DOK_BULK_MAXBIG];
+  for (int b = threadIdx.x; b < DOK_BULK_MAXBIG; b += DOK_BULK_TPB) cnt[b] = 0;
+  __syncthreads();
+  i64 lo, hi;
+  bulk_stretch1(ws, n, blockIdx.x, lo, hi);
+  for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += 4 * DOK_BULK_TPB) {
+    u64 key[4];
+    bool ok[4];
+    #pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const i64 i = i0 + u * DOK_BULK_TPB;
+      key[u] = 0;
+      ok[u] = i < hi && dok_load_key8<KF>(t, keys, i, n, key[u]);
+    }
+    #pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (ok[u] && (key[u] ^ DOK_P8_XOR) >= 2) atomicAdd(&cnt[bulk_range_of(key[u], t) >> DOK_BULK_SUBLOG], 1u);
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < (int)ws.n_big; b += DOK_BULK_TPB)
+    ws.wg_hist[(size_t)b * DOK_BULK_GRID + blockIdx.x] = cnt[b];
+}
+
+// ---- pass 1, scan: per bin over the workgroups, then over the bins ---------------------------------
+__global__ __launch_bounds__(DOK_BULK_GRID) void bulk_scan1a_kernel(BulkWs ws) {
+  __shared__ u32 wsum[16];
+  u32 *row = ws.wg_hist + (size_t)blockIdx.x * DOK_BULK_GRID;
+  const u32 c = row[threadIdx.x];
+  u32 total;
+  row[threadIdx.x] = bulk_block_scan(c, wsum, total);
+  if (threadIdx.x == 0) ws.big_off[blockIdx.x] = total;      // the bin's size; scan1b turns it into a start
+}
+__global__ __launch_bounds__(DOK_BULK_MAXBIG) void bulk_scan1b_kernel(BulkWs ws) {
+  __shared__ u32 wsum[16];
+  const u32 b = threadIdx.x;
+  const u32 c = b < ws.n_big ? ws.big_off[b] : 0u;
+  u32 total;
+  const u32 off = bulk_block_scan(c, wsum, total);
+  if (b < ws.n_big) ws.big_off[b] = off;
+  if (b == 0) ws.big_off[ws.n_big] = total;
+}
+
+// ---- pass 2, count: rows of every stretch of a first-level bin per range -----------------------------
+__global__ __launch_bounds__(DOK_BULK_TPB) void bulk_count2_kernel(DevTable t, BulkWs ws) {
+  __shared__ u32 cnt[DOK_BULK_SUB];
+  const u32 b = blockIdx.x / ws.ch, c = blockIdx.x % ws.ch;
+  for (int s = threadIdx.x; s < DOK_BULK_SUB; s += DOK_BULK_TPB) cnt[s] = 0;
+  __syncthreads();
+  i64 lo, hi;
+  bulk_stretch2(ws, b, c, lo, hi);
+  for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += 4 * DOK_BULK_TPB) {
+    u64 key[4];
+    #pragma unroll
+    for (int u = 0; u < 4; u++) {
+      const i64 i = i0 + u * DOK_BULK_TPB;
+      key[u] = i < hi ? ws.keysA[i] : 0;
+    }
+    #pragma unroll
+    for (int u = 0; u < 4; u++)
+      if (i0 + u * DOK_BULK_TPB < hi) atomicAdd(&cnt[bulk_range_of(key[u], t) & (DOK_BULK_SUB - 1)], 1u);
+  }
+  __syncthreads();
+  for (int s = threadIdx.x; s < DOK_BULK_SUB; s += DOK_BULK_TPB)
+    ws.sub_hist[((size_t)b * DOK_BULK_SUB + s) * ws.ch + c] = cnt[s];
+}
+
+// ---- pass 2, scan: per range over the stretches, then over the ranges of the bin ---------------------
+__global__ __launch_bounds__(DOK_BULK_SUB) void bulk_scan2_kernel(BulkWs ws) {
+  __shared__ u32 wsum[16];
+  const u32 b = blockIdx.x;
+  const size_t idx = (size_t)b * DOK_BULK_SUB + threadIdx.x;
+  u32 *row = ws.sub_hist + idx * ws.ch;
+  u32 run = 0;
+  for (u32 c = 0; c < ws.ch; c++) {
+    const u32 x = row[c];
+    row[c] = run;
+    run += x;
+  }
+  u32 total;
+  const u32 ex = bulk_block_scan(run, wsum, total);
+  const u32 base = ws.big_off[b];
+  ws.part_off[idx] = base + ex;
+  if (b == ws.n_big - 1 && threadIdx.x == DOK_BULK_SUB - 1) ws.part_off[idx + 1] = base + ex + run;
+}
+
+// ---- scatter: LEVEL 1 moves the caller's rows into first-level bins (keysA/valsA), LEVEL 2 moves
+// the rows of each first-level bin into their ranges (keysB/valsB) ---------------------------------
+template <int V, int KF, int LEVEL>
+__global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, const void *__restrict__ keys_in,
+                                                                    const void *__restrict__ vals_in, i64 n, BulkWs ws) {
+  typedef typename ValT<V>::type VT;
+  constexpr int NB = LEVEL == 1 ? DOK_BULK_MAXBIG : DOK_BULK_SUB;
+  constexpr int BPT = NB / DOK_BULK_TPB;             // consecutive bins per thread
+  __shared__ u32 cnt[NB], off[NB], gbase[NB];
+  __shared__ u64 skeys[DOK_BULK_T];
+  __shared__ VT svals[DOK_BULK_T];
+  __shared__ u32 wsum[16];
+  const int tid = threadIdx.x;
+  int n_fresh = 0, n_oob = 0;
+#ifdef DOK_BULK_TIMING
+  u64 tacc[6] = {0, 0, 0, 0, 0, 0};
+  u64 tlast = wall_clock64();
+#endif
+
+  // this workgroup's stretch of the input and its private write cursor of every bin
+  i64 lo0, hi0;
+  const void *kin = keys_in, *vin = vals_in;
+  u64 *out_keys;
+  VT *out_vals;
+  u32 cursor[BPT];
+  if (LEVEL == 1) {
+    bulk_stretch1(ws, n, blockIdx.x, lo0, hi0);
+    out_keys = ws.keysA;
+    out_vals = (VT *)ws.valsA;
+    #pragma unroll
+    for (int q = 0; q < BPT; q++) {
+      const u32 b = tid * BPT + q;
+      cursor[q] = b < ws.n_big ? ws.big_off[b] + ws.wg_hist[(size_t)b * DOK_BULK_GRID + blockIdx.x] : 0u;
+    }
+  } else {
+    const u32 b = blockIdx.x / ws.ch, c = blockIdx.x % ws.ch;
+    bulk_stretch2(ws, b, c, lo0, hi0);
+    kin = ws.keysA;
+    vin = ws.valsA;
+    out_keys = ws.keysB;
+    out_vals = (VT *)ws.valsB;
+    #pragma unroll
+    for (int q = 0; q < BPT; q++) {
+      const size_t idx = (size_t)b * DOK_BULK_SUB + tid * BPT + q;
+      cursor[q] = ws.part_off[idx] + ws.sub_hist[idx * ws.ch + c];
+    }
+  }
+
+  for (i64 lo = lo0; lo < hi0; lo += DOK_BULK_T) {
+    const i64 hi = lo + DOK_BULK_T < hi0 ? lo + DOK_BULK_T : hi0;
+    #pragma unroll
+    for (int q = 0; q < BPT; q++) cnt[tid * BPT + q] = 0;
+    __syncthreads();
+    BULK_TICK(0);
+
+    // the tile's rows, their bins, and their ranks inside the bins
+    u64 k[DOK_BULK_RPT], v[DOK_BULK_RPT];
+    int bn[DOK_BULK_RPT];
+    u32 rk[DOK_BULK_RPT];
+    #pragma unroll
+    for (int j = 0; j < DOK_BULK_RPT; j++) {
+      const i64 i = lo + j * DOK_BULK_TPB + tid;
+      bn[j] = -1; k[j] = 0; v[j] = 0; rk[j] = 0;
+      if (i < hi) {
+        u64 key = 0;
+        if (dok_load_key8<KF>(t, kin, i, n, key)) {
+          v[j] = dok_load_val<V>(vin, i);
+          if (LEVEL == 1 && (key ^ DOK_P8_XOR) < 2) {
+            n_fresh += p8_side_set(t, key ^ DOK_P8_XOR, v[j]);
+          } else {
+            k[j] = key;
+            const u32 r = bulk_range_of(key, t);
+            bn[j] = LEVEL == 1 ? (int)(r >> DOK_BULK_SUBLOG) : (int)(r & (DOK_BULK_SUB - 1));
+          }
+        } else {
+          n_oob++;
+        }
+      }
+    }
+    #pragma unroll
+    for (int j = 0; j < DOK_BULK_RPT; j++)
+      if (bn[j] >= 0) rk[j] = atomicAdd(&cnt[bn[j]], 1u);
+    __syncthreads();
+    BULK_TICK(1);
+
+    // bin offsets inside the tile, and where in global memory each bin's run goes
+    u32 c[BPT], csum = 0;
+    #pragma unroll
+    for (int q = 0; q < BPT; q++) {
+      c[q] = cnt[tid * BPT + q];
+      csum += c[q];
+    }
+    u32 total;
+    u32 ex = bulk_block_scan(csum, wsum, total);
+    #pragma unroll
+    for (int q = 0; q < BPT; q++) {
+      off[tid * BPT + q] = ex;
+      gbase[tid * BPT + q] = cursor[q];
+      cursor[q] += c[q];
+      ex += c[q];
+    }
+    __syncthreads();
+    BULK_TICK(2);
+
+    #pragma unroll
+    for (int j = 0; j < DOK_BULK_RPT; j++) {
+      if (bn[j] >= 0) {
+        const u32 pos = off[bn[j]] + rk[j];
+        skeys[pos] = k[j];
+        svals[pos] = (VT)v[j];
+      }
+    }
+    __syncthreads();
+    BULK_TICK(3);
+
+    for (u32 pos = tid; pos < total; pos += DOK_BULK_TPB) {
+      const u64 key = skeys[pos];
+      const u32 r = bulk_range_of(key, t);
+      const u32 b = LEVEL == 1 ? (r >> DOK_BULK_SUBLOG) : (r & (DOK_BULK_SUB - 1));
+      const u32 dst = gbase[b] + (pos - off[b]);
+      out_keys[dst] = key;
+      out_vals[dst] = svals[pos];
+    }
+    BULK_TICK(4);
+    // the barriers at the top of the next tile order these reads before the next writes
+  }
+#ifdef DOK_BULK_TIMING
+  if (threadIdx.x == 0 && LEVEL == DOK_BULK_TIMING) {
+    const int hslot[6] = {5, 6, 7, 12, 13, 14};
+    for (int q = 0; q < 6; q++) atomicAdd((u64 *)&t.header[hslot[q]], tacc[q]);
+  }
+#endif
+  if (LEVEL == 1) {
+    dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
+    dok_wave_add_n(&t.header[DOK_H_NOOB], n_oob);
+  }
+}
+
+// ---- merge: one workgroup per range -----------------------------------------------------------
+// The range's buckets sit in LDS word-major (word w of local bucket lb at tb[w * LD + lb], LD odd),
+// so that threads reading one word of scattered buckets spread over the banks.  The range's rows
+// are taken in chunks of DOK_BULK_C, every thread keeping its DOK_BULK_C / R rows in registers.
+// Per chunk, first every row LOOKS at its home bucket, then (after a barrier) the rows WRITE:
+//   - the key is in the bucket: the value is overwritten (values are never read here, so this
+//     needs no barrier);
+//   - otherwise the row marks a fingerprint of its key in a per-bucket bitmap that lives as long
+//     as the range.  If the mark was already there, an equal key may be among the range's rows,
+//     and the row goes on the range's list;
+//   - if the bucket has an EMPTY slot, the probe chain of every key whose home it is ends right
+//     here, so the key is new: the new rows of a bucket (their keys are distinct, thanks to the
+//     marks) draw a rank and the r-th of them takes the r-th free slot, tombstones first, with
+//     plain stores;
+//   - rows whose rank lies beyond the free slots, and rows whose home bucket has no EMPTY slot,
+//     go on the list as well.
+// After the last chunk the listed rows (a few per cent of a nearly full table's rows) walk their
+// chains from the home bucket, all at once, with the compare-and-swap protocol of p8_insert on
+// the LDS copy, which copes with equal keys and tombstones.  Rows whose chain runs past the
+// range's last bucket, and rows that found no room on the list, are handed to the ordinary insert.
+#ifndef DOK_BULK_C
+#define DOK_BULK_C (8 * DOK_BULK_R)
+#endif
+#define DOK_BULK_FPW 8                          // 32-bit fingerprint words per bucket
+#define DOK_BULK_LIST (2 * DOK_BULK_R)          // capacity of a range's list
+
+// n-th (0-based) set bit of m (m has more than n set bits).
+__device__ __forceinline__ int bulk_nth_bit(u32 m, u32 n) {
+  for (u32 i = 0; i < n; i++) m &= m - 1;
+  return __builtin_ctz(m);
+}
+
+template <int V>
+__global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, BulkWs ws) {
+#ifdef DOK_BULK_TIMING
+  u64 tacc[6] = {0, 0, 0, 0, 0, 0};
+  u64 tlast = wall_clock64();
+#endif
+  typedef typename ValT<V>::type VT;
+  constexpr int S = P8<V>::S;
+  constexpr int R = DOK_BULK_R;
+  constexpr int LD = R + 1;
+  constexpr int C = DOK_BULK_C;
+  constexpr int RPT = C / R;
+  __shared__ u64 tb[16 * LD];
+  __shared__ u32 fresh_cnt[R];
+  __shared__ u32 marks[R * DOK_BULK_FPW];
+  __shared__ u64 lkey[DOK_BULK_LIST];
+  __shared__ VT lval[DOK_BULK_LIST];
+  __shared__ int red[R / 64];
+  __shared__ u32 n_def;             // rows this workgroup has deferred so far
+  __shared__ u32 n_list;            // rows on the list of the current range
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  int n_fresh = 0;
+  // A workgroup merges a block of consecutive ranges; their rows are one contiguous stretch of
+  // keysB, and the rows it defers go, packed, to the same stretch of keysA - no shared cursor.
+  const u32 per = (ws.n_part + gridDim.x - 1) / gridDim.x;
+  const u32 p_lo = blockIdx.x * per < ws.n_part ? blockIdx.x * per : ws.n_part;
+  const u32 p_hi = p_lo + per < ws.n_part ? p_lo + per : ws.n_part;
+  const u32 def_base = ws.part_off[p_lo];
+  if (tid == 0) n_def = 0;
+  __syncthreads();
+
+  for (u32 p = p_lo; p < p_hi; p++) {
+    BULK_TICK(5);
+    const u32 lo = ws.part_off[p], hi = ws.part_off[p + 1];
+    if (lo == hi) continue;                          // no row of the batch lives in this range
+    const u64 b0 = (u64)p << DOK_BULK_RLOG;
+    const u64 left = t.nb - b0;
+    const u32 nbk = left < (u64)R ? (u32)left : (u32)R;
+    ulonglong2 *g = (ulonglong2 *)(t.buckets + b0 * 16);
+    ulonglong2 x[8];                                 // this thread's share of the range: 8 x 16 bytes
+    #pragma unroll
+    for (int q = 0; q < 8; q++) {
+      x[q].x = 0; x[q].y = 0;
+      if ((u32)(tid + q * R) < nbk * 8) x[q] = g[tid + q * R];
+    }
+    for (u32 c0 = lo; c0 < hi; c0 += C) {
+      const u32 c1 = c0 + C < hi ? c0 + C : hi;
+      u64 k[RPT], v[RPT];
+      bool on[RPT];
+      #pragma unroll
+      for (int j = 0; j < RPT; j++) {
+        const u32 i = c0 + j * R + tid;
+        on[j] = i < c1;
+        k[j] = 0; v[j] = 0;
+        if (on[j]) {
+          k[j] = ws.keysB[i];
+          v[j] = dok_load_val<V>(ws.valsB, i);
+        }
+      }
+      if (c0 == lo) {
+        // the bucket loads were issued before the row loads: both are in flight together
+        #pragma unroll
+        for (int q = 0; q < 8; q++) {
+          const u32 u = tid + q * R, lb = u >> 3, w = (u & 7) * 2;
+          if (u < nbk * 8) { tb[w * LD + lb] = x[q].x; tb[(w + 1) * LD + lb] = x[q].y; }
+        }
+        #pragma unroll
+        for (int q = 0; q < DOK_BULK_FPW; q++) marks[q * R + tid] = 0;
+        if (tid == 0) n_list = 0;
+      }
+      fresh_cnt[tid] = 0;
+      __syncthreads();                               // the bucket copy / the last chunk's writes are complete
+      BULK_TICK(0);
+
+      // look: act[j] = 0 nothing left to do, 1 write key and value into `slot`, 2 defer
+      int act[RPT], slot[RPT];
+      u32 lh[RPT];
+      #pragma unroll
+      for (int j = 0; j < RPT; j++) {
+        act[j] = 0; slot[j] = 0; lh[j] = 0;
+        if (on[j]) {
+          const u64 sk = k[j] ^ DOK_P8_XOR;
+          const u64 h = dok_fmix64(sk ^ t.seed);
+          lh[j] = dok_reduce(h, t.nb) - (u32)b0;
+          u32 gm = 0, ge = 0, gt = 0;
+          #pragma unroll
+          for (int s = 0; s < S; s++) {
+            const u64 w = tb[s * LD + lh[j]];
+            gm |= (u32)(w == sk) << s;
+            ge |= (u32)(w == DOK_P8_EMPTY) << s;
+            gt |= (u32)(w == DOK_P8_TOMB) << s;
+          }
+          if (gm) {
+            const int s = __builtin_ctz(gm);
+            *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lh[j]) + ((s * V) & 7)) = (VT)v[j];
+          } else {
+            bool listed = true;
+            const u32 fp = (u32)h & (32 * DOK_BULK_FPW - 1), bit = 1u << (fp & 31);
+            const u32 seen = atomicOr(&marks[lh[j] * DOK_BULK_FPW + (fp >> 5)], bit);
+            if (!(seen & bit) && ge) {
+              const u32 r = atomicAdd(&fresh_cnt[lh[j]], 1u);
+              const u32 nt = __popc(gt);
+              if (r < nt + __popc(ge)) {
+                listed = false;
+                act[j] = 1;
+                slot[j] = r < nt ? bulk_nth_bit(gt, r) : bulk_nth_bit(ge, r - nt);
+              }
+            }
+            if (listed) {
+              // onto the range's list while there is room, else to the ordinary insert
+              const u32 e = atomicAdd(&n_list, 1u);
+              if (e < DOK_BULK_LIST) { lkey[e] = k[j]; lval[e] = (VT)v[j]; }
+              else act[j] = 2;
+            }
+          }
+        }
+      }
+      __syncthreads();
+      BULK_TICK(1);
+      // write
+      #pragma unroll
+      for (int j = 0; j < RPT; j++) {
+        if (act[j] == 1) {
+          const int s = slot[j];
+          tb[s * LD + lh[j]] = k[j] ^ DOK_P8_XOR;
+          *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lh[j]) + ((s * V) & 7)) = (VT)v[j];
+          n_fresh++;
+        }
+        // deferred rows: one LDS atomic per wave, then a packed global write
+        const u64 dm = dok_ballot(act[j] == 2);
+        if (dm) {
+          u32 base = 0;
+          if (lane == 0) base = atomicAdd(&n_def, (u32)__popcll(dm));
+          base = dok_shfl32(base, 0);
+          if (act[j] == 2) {
+            const u32 at = def_base + base + (u32)__popcll(dm & ((1ULL << lane) - 1ULL));
+            ws.keysA[at] = k[j];
+            dok_store_val<V>(ws.valsA, (i64)at, v[j]);
+          }
+        }
+      }
+      BULK_TICK(2);
+    }
+    __syncthreads();
+
+    // the listed rows walk their chains, all at once
+    {
+      const u32 total = n_list < (u32)DOK_BULK_LIST ? n_list : (u32)DOK_BULK_LIST;
+      for (u32 e = tid; e < total; e += R) {
+        const u64 key = lkey[e];
+        const VT val = lval[e];
+        const u64 sk = key ^ DOK_P8_XOR;
+        const u32 lhome = p8_home(sk, t) - (u32)b0;
+        const int start = p8_slot_start<V>(sk);
+        u32 d = 0, tomb_d = DOK_NONE32;
+        int tomb_s = 0;
+        int st = -1;                                  // -1 walking, 1 placed, 2 chain leaves the range
+        while (st < 0) {
+          const u32 lb = lhome + d;
+          if (lb >= nbk) { st = 2; break; }
+          asm volatile("" ::: "memory");              // read the bucket afresh in every turn
+          u64 w[S];
+          #pragma unroll
+          for (int s = 0; s < S; s++) w[s] = tb[s * LD + lb];
+          u32 gm = 0, ge = 0, gt = 0;
+          #pragma unroll
+          for (int s = 0; s < S; s++) {
+            gm |= (u32)(w[s] == sk) << s;
+            ge |= (u32)(w[s] == DOK_P8_EMPTY) << s;
+            gt |= (u32)(w[s] == DOK_P8_TOMB) << s;
+          }
+          if (gm) {
+            const int s = __builtin_ctz(gm);
+            *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lb) + ((s * V) & 7)) = val;
+            st = 1;
+          } else {
+            if (tomb_d == DOK_NONE32 && gt) { tomb_d = d; tomb_s = p8_pick(gt, start); }
+            if (ge) {
+              u32 td; int ts; u64 expect;
+              if (tomb_d != DOK_NONE32) { td = tomb_d; ts = tomb_s; expect = DOK_P8_TOMB; }
+              else { td = d; ts = p8_pick(ge, start); expect = DOK_P8_EMPTY; }
+              const u32 tl = lhome + td;
+              const u64 old = atomicCAS(&tb[ts * LD + tl], expect, sk);
+              if (old == expect) {
+                *(VT *)((char *)(tb + (S + ((ts * V) >> 3)) * LD + tl) + ((ts * V) & 7)) = val;
+                if (td > 0) {
+                  u32 *meta = (u32 *)(tb + DOK_P8_META * LD + lhome);
+                  if (td >= 32) { atomicMax(meta + 1, td); atomicOr(meta, 1u); }
+                  else atomicOr(meta, 1u << td);
+                }
+                n_fresh++;
+                st = 1;
+              } else if (old == sk) {
+                st = 1;                               // an equal key won the slot: its value stands
+              } else {
+                d = td; tomb_d = DOK_NONE32;          // another key took it: look again from that bucket
+              }
+            } else {
+              d++;
+            }
+          }
+        }
+        if (st == 2) {
+          const u32 at = def_base + atomicAdd(&n_def, 1u);
+          ws.keysA[at] = key;
+          dok_store_val<V>(ws.valsA, (i64)at, (u64)val);
+        }
+      }
+    }
+    __syncthreads();
+    BULK_TICK(3);
+
+    for (u32 u = tid; u < nbk * 8; u += R) {
+      const u32 lb = u >> 3, w = (u & 7) * 2;
+      ulonglong2 y;
+      y.x = tb[w * LD + lb];
+      y.y = tb[(w + 1) * LD + lb];
+      g[u] = y;
+    }
+    __syncthreads();
+    BULK_TICK(4);
+  }
+#if defined(DOK_BULK_TIMING) && DOK_BULK_TIMING == 3
+  if (threadIdx.x == 0) {
+    const int hslot[6] = {5, 6, 7, 12, 13, 14};
+    for (int q = 0; q < 6; q++) atomicAdd((u64 *)&t.header[hslot[q]], tacc[q]);
+  }
+#endif
+
+  // one header update per workgroup
+  #pragma unroll
+  for (int o = 32; o > 0; o >>= 1) n_fresh += __shfl_xor(n_fresh, o, 64);
+  if ((tid & 63) == 0) red[tid >> 6] = n_fresh;
+  __syncthreads();
+  if (tid == 0) {
+    int sum = 0;
+    for (int w = 0; w < R / 64; w++) sum += red[w];
+    if (sum) atomicAdd((u64 *)&t.header[DOK_H_NELEM], (u64)(i64)sum);
+    ws.def_cnt[blockIdx.x] = n_def;
+  }
+}
+
+// ---- the rows the merge handed back: ordinary insert ---------------------------------------------
+// Launched with the merge kernel's grid: workgroup w inserts the rows merge workgroup w deferred.
+template <int V>
+__global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kernel(DevTable t, BulkWs ws) {
+  const u32 per = (ws.n_part + gridDim.x - 1) / gridDim.x;
+  const u32 p_lo = blockIdx.x * per < ws.n_part ? blockIdx.x * per : ws.n_part;
+  const i64 base = ws.part_off[p_lo];
+  const i64 n = ws.def_cnt[blockIdx.x];
+  const i64 waves = DOK_TPB / 64, wave = threadIdx.x >> 6;
+  const i64 share = (n + waves - 1) / waves;
+  i64 lo = wave * share, hi = lo + share;
+  if (hi > n) hi = n;
+  if (lo > hi) lo = hi;
+  const u64 *keys = ws.keysA;
+  const void *vals = ws.valsA;
+  p8_stream_insert_rows<V>(t, base + lo, base + hi, nullptr, [&](i64 i, u64 &key, u64 &val) -> int {
+    key = keys[i];
+    val = dok_load_val<V>(vals, i);
+    return 0;
+  });
+}
+
+// ---- host side -----------------------------------------------------------------------------------
+struct BulkPlan {
+  u32 n_part, n_big, ch;
+  i64 share;
+  size_t o_keysA, o_keysB, o_valsA, o_valsB, o_wg_hist, o_big_off, o_sub_hist, o_part_off, o_def_cnt, bytes;
+};
+
+static inline size_t bulk_align(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// False when the bulk path cannot take this table / batch (the caller then uses the ordinary
+// insert).
+static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p) {
+  if (n < 1 || n > 0x7fff0000LL) return false;
+  const u64 n_part = (d.nb + DOK_BULK_R - 1) >> DOK_BULK_RLOG;
+  const u64 n_big = (n_part + DOK_BULK_SUB - 1) >> DOK_BULK_SUBLOG;
+  if (n_big > DOK_BULK_MAXBIG) return false;
+  p.n_part = (u32)n_part;
+  p.n_big = (u32)n_big;
+  // second pass: about 4096 workgroups in all, 16 to 256 per first-level bin
+  u32 ch = 16;
+  while (ch < 256 && (u64)ch * n_big < 4096) ch *= 2;
+  p.ch = ch;
+  // first pass: equal stretches, whole tiles
+  const i64 tiles = (n + DOK_BULK_T - 1) / DOK_BULK_T;
+  p.share = ((tiles + DOK_BULK_GRID - 1) / DOK_BULK_GRID) * DOK_BULK_T;
+  const size_t parts = (size_t)n_big * DOK_BULK_SUB;
+  size_t o = 0;
+  p.o_keysA = o; o = bulk_align(o + 8 * (size_t)n);
+  p.o_keysB = o; o = bulk_align(o + 8 * (size_t)n);
+  p.o_valsA = o; o = bulk_align(o + (size_t)d.value_bytes * (size_t)n);
+  p.o_valsB = o; o = bulk_align(o + (size_t)d.value_bytes * (size_t)n);
+  p.o_wg_hist = o; o = bulk_align(o + 4 * (size_t)n_big * DOK_BULK_GRID);
+  p.o_big_off = o; o = bulk_align(o + 4 * (DOK_BULK_MAXBIG + 1));
+  p.o_sub_hist = o; o = bulk_align(o + 4 * parts * ch);
+  p.o_part_off = o; o = bulk_align(o + 4 * (parts + 1));
+  p.o_def_cnt = o; o = bulk_align(o + 4 * DOK_BULK_GRID);
+  p.bytes = o;
+  return true;
+}
+
+static void bulk_bind(const BulkPlan &p, void *workspace, BulkWs &ws) {
+  char *w = (char *)workspace;
+  ws.keysA = (u64 *)(w + p.o_keysA);
+  ws.keysB = (u64 *)(w + p.o_keysB);
+  ws.valsA = w + p.o_valsA;
+  ws.valsB = w + p.o_valsB;
+  ws.wg_hist = (u32 *)(w + p.o_wg_hist);
+  ws.big_off = (u32 *)(w + p.o_big_off);
+  ws.sub_hist = (u32 *)(w + p.o_sub_hist);
+  ws.part_off = (u32 *)(w + p.o_part_off);
+  ws.def_cnt = (u32 *)(w + p.o_def_cnt);
+  ws.n_big = p.n_big;
+  ws.n_part = p.n_part;
+  ws.ch = p.ch;
+  ws.share = p.share;
+}
+
+template <int V, int KF>
+static void bulk_launch(const DevTable &d, const void *keys, const void *values, i64 n, const BulkPlan &p,
+                        void *workspace, hipStream_t s) {
+  BulkWs ws;
+  bulk_bind(p, workspace, ws);
+  bulk_count1_kernel<KF><<<DOK_BULK_GRID, DOK_BULK_TPB, 0, s>>>(d, keys, n, ws);
+  bulk_scan1a_kernel<<<p.n_big, DOK_BULK_GRID, 0, s>>>(ws);
+  bulk_scan1b_kernel<<<1, DOK_BULK_MAXBIG, 0, s>>>(ws);
+  bulk_scatter_kernel<V, KF, 1><<<DOK_BULK_GRID, DOK_BULK_TPB, 0, s>>>(d, keys, values, n, ws);
+  bulk_count2_kernel<<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, ws);
+  bulk_scan2_kernel<<<p.n_big, DOK_BULK_SUB, 0, s>>>(ws);
+  bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
+  const unsigned gm = p.n_part < DOK_BULK_GRID ? p.n_part : DOK_BULK_GRID;
+  bulk_merge_kernel<V><<<gm, DOK_BULK_R, 0, s>>>(d, ws);
+  bulk_deferred_kernel<V><<<gm, DOK_TPB, 0, s>>>(d, ws);
+}

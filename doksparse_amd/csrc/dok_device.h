@@ -152,11 +152,13 @@ __device__ __forceinline__ bool dok_linearise(const DevTable &t, const i64 *row,
 #define DOK_KF_RAW  0   // key_bytes (1, 2, 4, 8) raw bytes per row, zero-extended to 8
 #define DOK_KF_ROWS 1   // coordinate table, row-major:    keys[i * ndim + d]
 #define DOK_KF_COLS 2   // coordinate table, column-major: keys[d * n + i]   (COO "indices")
+#define DOK_KF_U64  3   // keys already in table form: one 8-byte word per row, whatever key_bytes is
 
 // Key of batch row i (of n) as an 8-byte integer; false if a coordinate is out of range.
 template <int KF>
 __device__ __forceinline__ bool dok_load_key8(const DevTable &t, const void *keys, i64 i, i64 n, u64 &key) {
   if (KF == DOK_KF_ROWS) return dok_linearise(t, (const i64 *)keys + i * t.lin_ndim, key);
+  if (KF == DOK_KF_U64) { key = ((const u64 *)keys)[i]; return true; }
   if (KF == DOK_KF_COLS) {
     bool ok = true;
     u64 k = 0;

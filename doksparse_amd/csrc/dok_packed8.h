@@ -471,27 +471,22 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
 // has to walk on therefore costs the wave one more bucket load in a later pass instead of a turn
 // of its own, and the number of bucket lines in flight does not drop when the table is nearly
 // full (at load factor 0.9 this is 1.3x faster than tile-wise p8_insert).  All loads are
-// device-coherent, so a row that lost its claim to another key simply starts over at its home
-// bucket in the next pass.  The placement rules are those of p8_insert.
+// device-coherent, so a row that lost its claim to another key simply looks again, from the
+// bucket of the slot it lost, in the next pass.  The placement rules are those of p8_insert.
 //
 // `src(i, key, val)` produces row i: 0 = insert key -> val, 1 = the row addresses nothing inside
 // the table's coordinate space (counted, reported as not stored), 2 = skip the row silently.
 // The header counters are updated once per wave at the end.
+// The core works through the rows [next, end) that the caller assigns to this wave.
 template <int V, class Src>
-__device__ __forceinline__ void p8_stream_insert(const DevTable &t, i64 n, i64 rows_per_wave,
-                                                 u8 *__restrict__ stored, Src src) {
+__device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 next, i64 end,
+                                                      u8 *__restrict__ stored, Src src) {
   const P8Lane L;
   const int gbase = L.gbase;
   int l = L.l;
   DOK_OPAQUE(l);
   u64 *const buckets = t.buckets;
   const u64 nb = t.nb;
-
-  const i64 wave = ((i64)blockIdx.x * DOK_TPB + threadIdx.x) >> 6;
-  i64 next = wave * rows_per_wave;
-  i64 end = next + rows_per_wave;
-  if (end > n) end = n;
-  if (next > end) next = end;
 
   int n_fresh = 0, n_full = 0, n_oob = 0;
   bool act = false;
@@ -604,7 +599,10 @@ __device__ __forceinline__ void p8_stream_insert(const DevTable &t, i64 n, i64 r
             } else if (old == sk) {
               st = 1;                                // an equal key of this batch won the slot
             } else {
-              d = 0; tomb_d = DOK_NONE32;            // somebody else's key: look again
+              // somebody else's key took the slot.  Every bucket before the slot's own held
+              // neither a free slot nor this key when the row passed it, and buckets only fill up,
+              // so the row need not go back further than that bucket
+              d = td; tomb_d = DOK_NONE32;
             }
           }
         } else {
@@ -621,6 +619,18 @@ __device__ __forceinline__ void p8_stream_insert(const DevTable &t, i64 n, i64 r
   dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
   dok_wave_add_n(&t.header[DOK_H_NFULL], n_full);
   dok_wave_add_n(&t.header[DOK_H_NOOB], n_oob);
+}
+
+// Rows [0, n) split into one contiguous share per wave of the grid.
+template <int V, class Src>
+__device__ __forceinline__ void p8_stream_insert(const DevTable &t, i64 n, i64 rows_per_wave,
+                                                 u8 *__restrict__ stored, Src src) {
+  const i64 wave = ((i64)blockIdx.x * DOK_TPB + threadIdx.x) >> 6;
+  i64 next = wave * rows_per_wave;
+  i64 end = next + rows_per_wave;
+  if (end > n) end = n;
+  if (next > end) next = end;
+  p8_stream_insert_rows<V>(t, next, end, stored, src);
 }
 
 template <int V, int KF>

@@ -7,6 +7,7 @@
 #include "dok_device.h"
 #include "dok_packed8.h"
 #include "dok_tagged.h"
+#include "dok_bulk.h"
 
 namespace {
 
@@ -250,6 +251,48 @@ int dok_coo_set(const dok_table_t *t, const int64_t *indices, const void *values
     const unsigned grid = grid_counting(n);
     P8_DISPATCH(d.value_bytes, (p8_set_kernel<V, KF><<<grid, DOK_TPB, 0, s>>>(d, indices, values, n, nullptr, rows_per_wave(n, grid)))); }
   return note_launch();
+}
+
+int64_t dok_bulk_workspace_bytes(const dok_table_t *t, int64_t n) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  BulkPlan p;
+  if (layout != DOK_LAYOUT_PACKED8 || !bulk_plan(d, n, p)) return 0;
+  return (int64_t)p.bytes;
+}
+
+// Shared body of the two bulk entry points; `cols` selects the column-major coordinate format.
+static int set_bulk(const dok_table_t *t, const void *keys, const void *values, int64_t n, bool cols,
+                    void *workspace, int64_t workspace_bytes, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (cols && d.lin_ndim == 0) return DOK_EINVAL;
+  if (n < 0) return DOK_EINVAL;
+  if (n == 0) return DOK_OK;
+  if (!keys || !values || !workspace) return DOK_EINVAL;
+  BulkPlan p;
+  if (layout != DOK_LAYOUT_PACKED8 || !bulk_plan(d, n, p)) return DOK_EUNSUPPORTED;
+  if (((uintptr_t)workspace & 255) != 0 || workspace_bytes < (int64_t)p.bytes) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (cols) {
+    constexpr int KF = DOK_KF_COLS;
+    P8_DISPATCH(d.value_bytes, (bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
+  } else {
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
+  }
+  return note_launch();
+}
+
+int dok_map_set_bulk(const dok_table_t *t, const void *keys, const void *values, int64_t n,
+                     void *workspace, int64_t workspace_bytes, void *stream) {
+  return set_bulk(t, keys, values, n, false, workspace, workspace_bytes, stream);
+}
+
+int dok_coo_set_bulk(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
+                     void *workspace, int64_t workspace_bytes, void *stream) {
+  return set_bulk(t, indices, values, n, true, workspace, workspace_bytes, stream);
 }
 
 int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t *removed, void *stream) {

@@ -125,6 +125,22 @@ int dok_map_get_stats(const dok_table_t *t, const void *keys, int64_t n,
 int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int64_t n,
                 uint8_t *stored, void *stream);
 
+/* Bulk upsert: the same result as dok_map_set (stored == NULL) for a batch that is large
+ * against the table - rule of thumb: more than one row per physical bucket.  Instead of one
+ * compare-and-swap in HBM per row, the batch is partitioned by table range (two counting
+ * scatter passes through `workspace`) and every range of buckets is merged in LDS, so the
+ * table is streamed through the GPU once.  Packed layout only.
+ *   dok_bulk_workspace_bytes: device bytes dok_map_set_bulk / dok_coo_set_bulk need for n rows;
+ *     0 if the bulk path cannot take this table or n (use dok_map_set), negative on a bad table.
+ *   workspace: device, 256-byte aligned, at least that many bytes; contents need no
+ *     initialisation and are garbage afterwards.  Calls sharing one workspace must be ordered.
+ * Reference: the same closed_hashmap_set launch as dok_map_set, at the batch sizes of
+ * SparseDOKTensor.__init__ / from_sparse_coo (sparse_dok_tensor.py:59-69) and of
+ * CudaClosedHashmap.rehash (cuda_closed_hashmap.py:456-468). */
+int64_t dok_bulk_workspace_bytes(const dok_table_t *t, int64_t n);
+int dok_map_set_bulk(const dok_table_t *t, const void *keys, const void *values, int64_t n,
+                     void *workspace, int64_t workspace_bytes, void *stream);
+
 /* Tombstone each present key; header[DOK_H_NELEM] shrinks by the number removed.  Equal keys
  * in one batch: exactly one row reports 1.
  * Reference: closed_hashmap_remove (closed_hashmap_impl.cu:159-220, ClosedHashmap::remove
@@ -163,6 +179,10 @@ int dok_map_rehash(const dok_table_t *src, const dok_table_t *dst, void *stream)
  * before the set (sparse_dok_tensor.py:66-69, 71-84). */
 int dok_coo_set(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
                 void *stream);
+
+/* dok_coo_set through the bulk path (see dok_map_set_bulk). */
+int dok_coo_set_bulk(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
+                     void *workspace, int64_t workspace_bytes, void *stream);
 
 /* dok_map_compact emitting COO layout: indices_out is [lin_ndim][capacity] int64, values_out
  * [capacity].  Either output may be NULL; count_out[0] receives the number of live entries.

@@ -1,0 +1,179 @@
+"""GPU parity of the bulk insert (partition by table range + merge in LDS) against the CPU oracle.
+
+The bulk path is normally chosen only for batches of a million rows and more; the tests lower
+the thresholds so that every `set` below goes through it, at sizes the oracle finishes in
+seconds, and compare the resulting map - not the slot placement - with the oracle's."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle.ref_hashmap import RefClosedHashmap
+from test_gpu_hashmap import _assert_same_map, _check_get, _to, _unique_i64
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def bulk_always(monkeypatch):
+    from doksparse_amd import closed_hashmap as ch
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS", 0)
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS_PER_BUCKET", 0.0)
+    return ch
+
+
+def _bulk_never(monkeypatch):
+    from doksparse_amd import closed_hashmap as ch
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS", 1 << 62)
+
+
+@pytest.mark.parametrize("key_dtype,value_dtype", [
+    (np.int64, np.float32), (np.int64, np.int64), (np.int64, np.float16), (np.int64, np.int8),
+    (np.int32, np.int32), (np.int16, np.float64),
+])
+@pytest.mark.parametrize("n,capacity", [(5000, 16384), (20000, 22300), (300, 330), (60000, 2_000_000), (7, 8)])
+def test_bulk_upsert_matches_oracle(cuda, monkeypatch, key_dtype, value_dtype, n, capacity):
+    """Pre-populated table with tombstones, then one bulk batch mixing overwrites and new keys;
+    load factors up to 0.9, tables smaller and larger than one merge range."""
+    from doksparse_amd import CudaClosedHashmap, closed_hashmap as ch
+    rng = np.random.default_rng(n + capacity)
+    hi = min(2**62, int(np.iinfo(key_dtype).max))
+    if hi < 2**20:
+        n = min(n, hi // 8)
+        keys = rng.permutation(hi)[: 2 * n].astype(key_dtype)
+    else:
+        keys = _unique_i64(rng, 2 * n, hi=hi).astype(key_dtype)
+    vmax = 100 if np.dtype(value_dtype).itemsize == 1 else 30000
+    hm = CudaClosedHashmap(n_buckets=capacity, device=cuda, rehash_threshold=1.0)
+    ref = RefClosedHashmap(n_buckets=capacity, rehash_threshold=1.0, rng=np.random.default_rng(1))
+
+    _bulk_never(monkeypatch)
+    first = keys[: n // 3, None]
+    v1 = rng.integers(-vmax, vmax, size=(first.shape[0], 1)).astype(value_dtype)
+    hm.set(*_to(cuda, first, v1)); ref.set(first, v1)
+    gone = keys[: n // 6, None]
+    if gone.shape[0]:
+        hm.remove(torch.from_numpy(gone).to(cuda)); ref.remove(gone)
+
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS", 0)
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS_PER_BUCKET", 0.0)
+    batch = keys[n // 8: n, None]
+    batch = batch[rng.permutation(batch.shape[0])]
+    v2 = rng.integers(-vmax, vmax, size=(batch.shape[0], 1)).astype(value_dtype)
+    hm.set(*_to(cuda, batch, v2)); ref.set(batch, v2)
+    assert hm.n_elements == ref.n_elements
+    _assert_same_map(hm, ref)
+    _check_get(hm, ref, keys[:, None], cuda, fallback=3)
+    # and a second bulk batch on top: all overwrites
+    v3 = rng.integers(-vmax, vmax, size=(batch.shape[0], 1)).astype(value_dtype)
+    hm.set(*_to(cuda, batch, v3)); ref.set(batch, v3)
+    assert hm.n_elements == ref.n_elements
+    _assert_same_map(hm, ref)
+
+
+def test_bulk_equal_keys_inside_one_batch(cuda, bulk_always):
+    """Every key 32 times in one bulk batch: one slot per key, holding one of its values."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(11)
+    base = _unique_i64(rng, 3000)
+    keys = np.repeat(base, 32)
+    perm = rng.permutation(keys.shape[0])
+    keys = keys[perm]
+    ids = np.repeat(np.arange(base.shape[0]), 32)[perm]
+    copy = rng.integers(0, 2**30, size=keys.shape[0])
+    vals = (ids * 2**32 + copy).astype(np.int64)
+    for capacity in (3400, 8192, 200_000):
+        hm = CudaClosedHashmap(n_buckets=capacity, device=cuda, rehash_threshold=1.0)
+        hm.set(*_to(cuda, keys[:, None], vals[:, None]))
+        assert hm.n_elements == base.shape[0]
+        gk, _ = hm.items()
+        assert gk.shape[0] == base.shape[0] and np.unique(gk.cpu().numpy()).shape[0] == base.shape[0]
+        out, found = hm.get(torch.from_numpy(base[:, None]).to(cuda))
+        assert bool(found.all())
+        out = out.cpu().numpy().reshape(-1)
+        written = {}
+        for i_, c_ in zip(ids, copy):
+            written.setdefault(int(i_), set()).add(int(c_))
+        for i_ in range(base.shape[0]):
+            assert out[i_] >> 32 == i_ and int(out[i_] & (2**32 - 1)) in written[i_]
+
+
+def test_bulk_reserved_patterns_and_full_table(cuda, bulk_always):
+    from doksparse_amd import CudaClosedHashmap
+    X = np.uint64(0x9E3779B97F4A7C15)
+    special = np.array([X, X ^ np.uint64(1), 0, 1, np.uint64(2**64 - 1), np.uint64(2**63)],
+                       dtype=np.uint64).view(np.int64)[:, None]
+    vals = np.arange(1, special.shape[0] + 1, dtype=np.float32)[:, None]
+    hm = CudaClosedHashmap(n_buckets=64, device=cuda)
+    ref = RefClosedHashmap(n_buckets=64)
+    hm.set(*_to(cuda, special, vals)); ref.set(special, vals)
+    assert hm.n_elements == ref.n_elements == special.shape[0]
+    _check_get(hm, ref, special, cuda)
+    _assert_same_map(hm, ref)
+
+    # more distinct keys than physical slots: the surplus is reported, nothing is lost silently
+    hm = CudaClosedHashmap(n_buckets=100, device=cuda, rehash_threshold=1e9)
+    keys = _unique_i64(np.random.default_rng(2), 400)[:, None]
+    v = np.arange(400, dtype=np.float32)[:, None]
+    hm.set(*_to(cuda, keys, v))
+    with pytest.raises(RuntimeError):
+        hm.n_elements
+    slots = hm._n_phys * hm._slots_per_bucket
+    h = hm._header.cpu()
+    assert int(h[0]) == slots and int(h[1]) == 400 - slots
+    out, found = hm.get(torch.from_numpy(keys).to(cuda))
+    assert int(found.sum().item()) == slots
+    assert torch.equal(out[found].cpu(), torch.from_numpy(v)[found.cpu()])
+
+
+def test_bulk_coordinate_keys_and_coo_constructor(cuda, bulk_always):
+    """Coordinate-keyed maps: row-major key rows and the [ndim, n] COO layout both go through the
+    bulk path; rows outside the size are skipped and counted."""
+    from doksparse_amd import CudaClosedHashmap, SparseDOKTensor
+    rng = np.random.default_rng(21)
+    size = (300, 77, 5)
+    lin = rng.permutation(int(np.prod(size)))[:40000]
+    coords = np.stack(np.unravel_index(lin, size))
+    vals = rng.standard_normal(lin.shape[0]).astype(np.float32)
+    dok = SparseDOKTensor(size, torch.from_numpy(coords).to(cuda), torch.from_numpy(vals).to(cuda), device=cuda)
+    dense = torch.zeros(size)
+    dense[tuple(torch.from_numpy(coords))] = torch.from_numpy(vals)
+    assert dok._nnz() == lin.shape[0]
+    assert torch.equal(dok.to_dense().cpu(), dense)
+    rows = torch.arange(0, 300, 7, device=cuda)
+    assert torch.equal(dok[rows[:, None], 3:60, 2].cpu(), dense[rows.cpu()[:, None], 3:60, 2])
+
+    hm = CudaClosedHashmap(n_buckets=50000, device=cuda, coord_dims=size, rehash_threshold=1.0)
+    bad = coords.T.copy()
+    bad[::100, 1] = 77                                   # out of range in dimension 1
+    hm.set(torch.from_numpy(bad).to(cuda), torch.from_numpy(vals[:, None]).to(cuda))
+    h = hm._header.cpu()
+    n_bad = bad[::100].shape[0]
+    assert int(h[3]) == n_bad and int(h[0]) == lin.shape[0] - n_bad
+
+
+def test_bulk_entry_point_rejects_bad_arguments(cuda):
+    from doksparse_amd import CudaClosedHashmap, _lib
+    lib = _lib.load()
+    hm = CudaClosedHashmap(n_buckets=4096, device=cuda)
+    k = torch.arange(100, device=cuda)[:, None]
+    v = torch.ones(100, 1, device=cuda)
+    hm.set(k, v)
+    desc = ctypes.byref(hm._desc)
+    need = int(lib.dok_bulk_workspace_bytes(desc, 100))
+    assert need > 0
+    ws = torch.empty(need, device=cuda, dtype=torch.uint8)
+    assert lib.dok_map_set_bulk(desc, k.data_ptr(), v.data_ptr(), 100, ws.data_ptr(), need - 1, None) == _lib.DOK_EINVAL
+    assert lib.dok_map_set_bulk(desc, k.data_ptr(), v.data_ptr(), 100, ws.data_ptr() + 8, need, None) == _lib.DOK_EINVAL
+    assert lib.dok_map_set_bulk(desc, None, v.data_ptr(), 100, ws.data_ptr(), need, None) == _lib.DOK_EINVAL
+    assert lib.dok_map_set_bulk(desc, k.data_ptr(), v.data_ptr(), 0, ws.data_ptr(), need, None) == _lib.DOK_OK
+    assert lib.dok_coo_set_bulk(desc, k.data_ptr(), v.data_ptr(), 100, ws.data_ptr(), need, None) == _lib.DOK_EINVAL
+    # the tagged layout has no bulk path
+    hm2 = CudaClosedHashmap(n_buckets=256, device=cuda)
+    hm2.set(torch.rand(10, 3, device=cuda), torch.zeros(10, 5, device=cuda, dtype=torch.long))
+    assert int(lib.dok_bulk_workspace_bytes(ctypes.byref(hm2._desc), 10)) == 0
+    assert lib.dok_map_set_bulk(ctypes.byref(hm2._desc), k.data_ptr(), v.data_ptr(), 10, ws.data_ptr(), need, None) \
+        == _lib.DOK_EUNSUPPORTED
+    torch.cuda.synchronize()
+    assert hm.n_elements == 100
