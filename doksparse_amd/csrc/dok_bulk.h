@@ -37,8 +37,11 @@
 #define DOK_BULK_T 2048                     // rows per scatter tile
 #endif
 #define DOK_BULK_RPT (DOK_BULK_T / DOK_BULK_TPB)
+#ifndef DOK_BULK_CTPB
+#define DOK_BULK_CTPB 1024                  // threads per workgroup of the count kernels: they only stream
+#endif                                      // keys, and the bytes in flight per CU bound their rate
 #ifndef DOK_BULK_GRID
-#define DOK_BULK_GRID 1024                  // workgroups of the first pass and of the merge
+#define DOK_BULK_GRID 1024                  // most workgroups the first pass and the merge are given
 #endif
 
 #ifdef DOK_BULK_TIMING
@@ -58,6 +61,7 @@ struct BulkWs {
   u32 *part_off;            // [n_big * SUB + 1]  start of every range in keysB
   u32 *def_cnt;             // [GRID] rows each merge workgroup handed to the ordinary insert
   u32 n_big, n_part;
+  u32 g1;                   // workgroups of the first pass (a multiple of 64, at most DOK_BULK_GRID)
   u32 ch;                   // stretches (workgroups) per first-level bin in the second pass
   i64 share;                // rows per workgroup in the first pass
 };
@@ -107,35 +111,35 @@ __device__ __forceinline__ void bulk_stretch2(const BulkWs &ws, u32 b, u32 c, i6
 
 // ---- pass 1, count: rows of every workgroup's stretch per first-level bin ------------------------
 template <int KF>
-__global__ __launch_bounds__(DOK_BULK_TPB) void bulk_count1_kernel(DevTable t, const void *__restrict__ keys, i64 n,
+__global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count1_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                                    BulkWs ws) {
   __shared__ u32 cnt[DOK_BULK_MAXBIG];
-  for (int b = threadIdx.x; b < DOK_BULK_MAXBIG; b += DOK_BULK_TPB) cnt[b] = 0;
+  for (int b = threadIdx.x; b < DOK_BULK_MAXBIG; b += DOK_BULK_CTPB) cnt[b] = 0;
   __syncthreads();
   i64 lo, hi;
   bulk_stretch1(ws, n, blockIdx.x, lo, hi);
-  for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += 4 * DOK_BULK_TPB) {
-    u64 key[4];
-    bool ok[4];
+  for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += 8 * DOK_BULK_CTPB) {
+    u64 key[8];
+    bool ok[8];
     #pragma unroll
-    for (int u = 0; u < 4; u++) {
-      const i64 i = i0 + u * DOK_BULK_TPB;
+    for (int u = 0; u < 8; u++) {
+      const i64 i = i0 + u * DOK_BULK_CTPB;
       key[u] = 0;
       ok[u] = i < hi && dok_load_key8<KF>(t, keys, i, n, key[u]);
     }
     #pragma unroll
-    for (int u = 0; u < 4; u++)
+    for (int u = 0; u < 8; u++)
       if (ok[u] && (key[u] ^ DOK_P8_XOR) >= 2) atomicAdd(&cnt[bulk_range_of(key[u], t) >> DOK_BULK_SUBLOG], 1u);
   }
   __syncthreads();
-  for (int b = threadIdx.x; b < (int)ws.n_big; b += DOK_BULK_TPB)
-    ws.wg_hist[(size_t)b * DOK_BULK_GRID + blockIdx.x] = cnt[b];
+  for (int b = threadIdx.x; b < (int)ws.n_big; b += DOK_BULK_CTPB)
+    ws.wg_hist[(size_t)b * ws.g1 + blockIdx.x] = cnt[b];
 }
 
 // ---- pass 1, scan: per bin over the workgroups, then over the bins ---------------------------------
 __global__ __launch_bounds__(DOK_BULK_GRID) void bulk_scan1a_kernel(BulkWs ws) {
   __shared__ u32 wsum[16];
-  u32 *row = ws.wg_hist + (size_t)blockIdx.x * DOK_BULK_GRID;
+  u32 *row = ws.wg_hist + (size_t)blockIdx.x * ws.g1;
   const u32 c = row[threadIdx.x];
   u32 total;
   row[threadIdx.x] = bulk_block_scan(c, wsum, total);
@@ -152,26 +156,26 @@ __global__ __launch_bounds__(DOK_BULK_MAXBIG) void bulk_scan1b_kernel(BulkWs ws)
 }
 
 // ---- pass 2, count: rows of every stretch of a first-level bin per range -----------------------------
-__global__ __launch_bounds__(DOK_BULK_TPB) void bulk_count2_kernel(DevTable t, BulkWs ws) {
+__global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count2_kernel(DevTable t, BulkWs ws) {
   __shared__ u32 cnt[DOK_BULK_SUB];
   const u32 b = blockIdx.x / ws.ch, c = blockIdx.x % ws.ch;
-  for (int s = threadIdx.x; s < DOK_BULK_SUB; s += DOK_BULK_TPB) cnt[s] = 0;
+  for (int s = threadIdx.x; s < DOK_BULK_SUB; s += DOK_BULK_CTPB) cnt[s] = 0;
   __syncthreads();
   i64 lo, hi;
   bulk_stretch2(ws, b, c, lo, hi);
-  for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += 4 * DOK_BULK_TPB) {
-    u64 key[4];
+  for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += 8 * DOK_BULK_CTPB) {
+    u64 key[8];
     #pragma unroll
-    for (int u = 0; u < 4; u++) {
-      const i64 i = i0 + u * DOK_BULK_TPB;
+    for (int u = 0; u < 8; u++) {
+      const i64 i = i0 + u * DOK_BULK_CTPB;
       key[u] = i < hi ? ws.keysA[i] : 0;
     }
     #pragma unroll
-    for (int u = 0; u < 4; u++)
-      if (i0 + u * DOK_BULK_TPB < hi) atomicAdd(&cnt[bulk_range_of(key[u], t) & (DOK_BULK_SUB - 1)], 1u);
+    for (int u = 0; u < 8; u++)
+      if (i0 + u * DOK_BULK_CTPB < hi) atomicAdd(&cnt[bulk_range_of(key[u], t) & (DOK_BULK_SUB - 1)], 1u);
   }
   __syncthreads();
-  for (int s = threadIdx.x; s < DOK_BULK_SUB; s += DOK_BULK_TPB)
+  for (int s = threadIdx.x; s < DOK_BULK_SUB; s += DOK_BULK_CTPB)
     ws.sub_hist[((size_t)b * DOK_BULK_SUB + s) * ws.ch + c] = cnt[s];
 }
 
@@ -205,6 +209,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
   __shared__ u32 cnt[NB], off[NB], gbase[NB];
   __shared__ u64 skeys[DOK_BULK_T];
   __shared__ VT svals[DOK_BULK_T];
+  __shared__ u16 sbins[DOK_BULK_T];                  // bin of every staged row (saves a second hash)
   __shared__ u32 wsum[16];
   const int tid = threadIdx.x;
   int n_fresh = 0, n_oob = 0;
@@ -226,7 +231,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     #pragma unroll
     for (int q = 0; q < BPT; q++) {
       const u32 b = tid * BPT + q;
-      cursor[q] = b < ws.n_big ? ws.big_off[b] + ws.wg_hist[(size_t)b * DOK_BULK_GRID + blockIdx.x] : 0u;
+      cursor[q] = b < ws.n_big ? ws.big_off[b] + ws.wg_hist[(size_t)b * ws.g1 + blockIdx.x] : 0u;
     }
   } else {
     const u32 b = blockIdx.x / ws.ch, c = blockIdx.x % ws.ch;
@@ -242,34 +247,45 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     }
   }
 
-  for (i64 lo = lo0; lo < hi0; lo += DOK_BULK_T) {
+  // The rows of a tile sit in registers from their load to their place in the LDS staging area;
+  // the next tile's loads are issued as soon as the registers are free, so that they are in
+  // flight during the write-out of this tile.  st[j]: 0 no row, 1 row, 2 row outside the table's
+  // coordinate space.
+  u64 k[DOK_BULK_RPT], v[DOK_BULK_RPT];
+  int st[DOK_BULK_RPT];
+  auto load_tile = [&](i64 lo) {
     const i64 hi = lo + DOK_BULK_T < hi0 ? lo + DOK_BULK_T : hi0;
+    #pragma unroll
+    for (int j = 0; j < DOK_BULK_RPT; j++) {
+      const i64 i = lo + j * DOK_BULK_TPB + tid;
+      st[j] = 0; k[j] = 0; v[j] = 0;
+      if (i < hi) {
+        if (dok_load_key8<KF>(t, kin, i, n, k[j])) { v[j] = dok_load_val<V>(vin, i); st[j] = 1; }
+        else st[j] = 2;
+      }
+    }
+  };
+  if (lo0 < hi0) load_tile(lo0);
+
+  for (i64 lo = lo0; lo < hi0; lo += DOK_BULK_T) {
     #pragma unroll
     for (int q = 0; q < BPT; q++) cnt[tid * BPT + q] = 0;
     __syncthreads();
     BULK_TICK(0);
 
-    // the tile's rows, their bins, and their ranks inside the bins
-    u64 k[DOK_BULK_RPT], v[DOK_BULK_RPT];
+    // bins of the tile's rows and their ranks inside the bins
     int bn[DOK_BULK_RPT];
     u32 rk[DOK_BULK_RPT];
     #pragma unroll
     for (int j = 0; j < DOK_BULK_RPT; j++) {
-      const i64 i = lo + j * DOK_BULK_TPB + tid;
-      bn[j] = -1; k[j] = 0; v[j] = 0; rk[j] = 0;
-      if (i < hi) {
-        u64 key = 0;
-        if (dok_load_key8<KF>(t, kin, i, n, key)) {
-          v[j] = dok_load_val<V>(vin, i);
-          if (LEVEL == 1 && (key ^ DOK_P8_XOR) < 2) {
-            n_fresh += p8_side_set(t, key ^ DOK_P8_XOR, v[j]);
-          } else {
-            k[j] = key;
-            const u32 r = bulk_range_of(key, t);
-            bn[j] = LEVEL == 1 ? (int)(r >> DOK_BULK_SUBLOG) : (int)(r & (DOK_BULK_SUB - 1));
-          }
+      bn[j] = -1; rk[j] = 0;
+      if (st[j] == 2) n_oob++;
+      if (st[j] == 1) {
+        if (LEVEL == 1 && (k[j] ^ DOK_P8_XOR) < 2) {
+          n_fresh += p8_side_set(t, k[j] ^ DOK_P8_XOR, v[j]);
         } else {
-          n_oob++;
+          const u32 r = bulk_range_of(k[j], t);
+          bn[j] = LEVEL == 1 ? (int)(r >> DOK_BULK_SUBLOG) : (int)(r & (DOK_BULK_SUB - 1));
         }
       }
     }
@@ -304,18 +320,22 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
         const u32 pos = off[bn[j]] + rk[j];
         skeys[pos] = k[j];
         svals[pos] = (VT)v[j];
+        sbins[pos] = (u16)bn[j];
       }
     }
+    if (lo + DOK_BULK_T < hi0) load_tile(lo + DOK_BULK_T);
     __syncthreads();
     BULK_TICK(3);
 
-    for (u32 pos = tid; pos < total; pos += DOK_BULK_TPB) {
-      const u64 key = skeys[pos];
-      const u32 r = bulk_range_of(key, t);
-      const u32 b = LEVEL == 1 ? (r >> DOK_BULK_SUBLOG) : (r & (DOK_BULK_SUB - 1));
-      const u32 dst = gbase[b] + (pos - off[b]);
-      out_keys[dst] = key;
-      out_vals[dst] = svals[pos];
+    #pragma unroll
+    for (int j = 0; j < DOK_BULK_RPT; j++) {
+      const u32 pos = tid + j * DOK_BULK_TPB;
+      if (pos < total) {
+        const u32 b = sbins[pos];
+        const u32 dst = gbase[b] + (pos - off[b]);
+        out_keys[dst] = skeys[pos];
+        out_vals[dst] = svals[pos];
+      }
     }
     BULK_TICK(4);
     // the barriers at the top of the next tile order these reads before the next writes
@@ -631,7 +651,7 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
 
 // ---- host side -----------------------------------------------------------------------------------
 struct BulkPlan {
-  u32 n_part, n_big, ch;
+  u32 n_part, n_big, ch, g1, gm;
   i64 share;
   size_t o_keysA, o_keysB, o_valsA, o_valsB, o_wg_hist, o_big_off, o_sub_hist, o_part_off, o_def_cnt, bytes;
 };
@@ -640,8 +660,9 @@ static inline size_t bulk_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // False when the bulk path cannot take this table / batch (the caller then uses the ordinary
 // insert).
-static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p) {
+static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p, u32 g1 = DOK_BULK_GRID, u32 gm = DOK_BULK_GRID) {
   if (n < 1 || n > 0x7fff0000LL) return false;
+  p.g1 = g1;
   const u64 n_part = (d.nb + DOK_BULK_R - 1) >> DOK_BULK_RLOG;
   const u64 n_big = (n_part + DOK_BULK_SUB - 1) >> DOK_BULK_SUBLOG;
   if (n_big > DOK_BULK_MAXBIG) return false;
@@ -653,7 +674,8 @@ static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p) {
   p.ch = ch;
   // first pass: equal stretches, whole tiles
   const i64 tiles = (n + DOK_BULK_T - 1) / DOK_BULK_T;
-  p.share = ((tiles + DOK_BULK_GRID - 1) / DOK_BULK_GRID) * DOK_BULK_T;
+  p.share = ((tiles + g1 - 1) / g1) * DOK_BULK_T;
+  p.gm = p.n_part < gm ? p.n_part : gm;
   const size_t parts = (size_t)n_big * DOK_BULK_SUB;
   size_t o = 0;
   p.o_keysA = o; o = bulk_align(o + 8 * (size_t)n);
@@ -682,8 +704,41 @@ static void bulk_bind(const BulkPlan &p, void *workspace, BulkWs &ws) {
   ws.def_cnt = (u32 *)(w + p.o_def_cnt);
   ws.n_big = p.n_big;
   ws.n_part = p.n_part;
+  ws.g1 = p.g1;
   ws.ch = p.ch;
   ws.share = p.share;
+}
+
+// Persistent kernels get exactly as many workgroups as the device holds at once, so that no
+// workgroup waits for a slot while others have already finished their share.
+static int bulk_cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+    else cus = 256;
+  }
+  return cus;
+}
+template <class K>
+static u32 bulk_resident(K kernel, int block, u32 limit, u32 multiple) {
+  int occ = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, block, 0) != hipSuccess || occ < 1) occ = 1;
+  u64 g = (u64)occ * (u64)bulk_cu_count();
+  if (g > limit) g = limit;
+  g -= g % multiple;
+  return g < multiple ? multiple : (u32)g;
+}
+
+template <int V, int KF>
+static bool bulk_plan_for(const DevTable &d, i64 n, BulkPlan &p) {
+  static u32 g1 = 0, gm = 0;
+  if (g1 == 0) {
+    g1 = bulk_resident(bulk_scatter_kernel<V, KF, 1>, DOK_BULK_TPB, DOK_BULK_GRID, 64);
+    gm = bulk_resident(bulk_merge_kernel<V>, DOK_BULK_R, DOK_BULK_GRID, 1);
+  }
+  return bulk_plan(d, n, p, g1, gm);
 }
 
 template <int V, int KF>
@@ -691,14 +746,13 @@ static void bulk_launch(const DevTable &d, const void *keys, const void *values,
                         void *workspace, hipStream_t s) {
   BulkWs ws;
   bulk_bind(p, workspace, ws);
-  bulk_count1_kernel<KF><<<DOK_BULK_GRID, DOK_BULK_TPB, 0, s>>>(d, keys, n, ws);
-  bulk_scan1a_kernel<<<p.n_big, DOK_BULK_GRID, 0, s>>>(ws);
+  bulk_count1_kernel<KF><<<p.g1, DOK_BULK_CTPB, 0, s>>>(d, keys, n, ws);
+  bulk_scan1a_kernel<<<p.n_big, p.g1, 0, s>>>(ws);
   bulk_scan1b_kernel<<<1, DOK_BULK_MAXBIG, 0, s>>>(ws);
-  bulk_scatter_kernel<V, KF, 1><<<DOK_BULK_GRID, DOK_BULK_TPB, 0, s>>>(d, keys, values, n, ws);
-  bulk_count2_kernel<<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, ws);
+  bulk_scatter_kernel<V, KF, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, keys, values, n, ws);
+  bulk_count2_kernel<<<p.n_big * p.ch, DOK_BULK_CTPB, 0, s>>>(d, ws);
   bulk_scan2_kernel<<<p.n_big, DOK_BULK_SUB, 0, s>>>(ws);
   bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
-  const unsigned gm = p.n_part < DOK_BULK_GRID ? p.n_part : DOK_BULK_GRID;
-  bulk_merge_kernel<V><<<gm, DOK_BULK_R, 0, s>>>(d, ws);
-  bulk_deferred_kernel<V><<<gm, DOK_TPB, 0, s>>>(d, ws);
+  bulk_merge_kernel<V><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
+  bulk_deferred_kernel<V><<<p.gm, DOK_TPB, 0, s>>>(d, ws);
 }

@@ -66,8 +66,9 @@ __device__ __forceinline__ u64 dok_fmix64(u64 x) {
   return x;
 }
 
-// Multiply-high range reduction: maps a 64-bit hash uniformly onto [0, nb) without division.
-__device__ __forceinline__ u32 dok_reduce(u64 h, u64 nb) { return (u32)__umul64hi(h, nb); }
+// Multiply-high range reduction: maps a hash uniformly onto [0, nb) without division.  A table
+// has fewer than 2^32 buckets, so the upper half of the hash and one 32 x 32 -> 64 bit multiply do.
+__device__ __forceinline__ u32 dok_reduce(u64 h, u64 nb) { return (u32)(((h >> 32) * (u64)(u32)nb) >> 32); }
 
 __device__ __forceinline__ u64 dok_ballot(bool p) { return __ballot(p); }
 

@@ -276,11 +276,12 @@ static int set_bulk(const dok_table_t *t, const void *keys, const void *values, 
   if (layout != DOK_LAYOUT_PACKED8 || !bulk_plan(d, n, p)) return DOK_EUNSUPPORTED;
   if (((uintptr_t)workspace & 255) != 0 || workspace_bytes < (int64_t)p.bytes) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  // the launch plan shares the workspace layout of the sizing plan above and only narrows the grids
   if (cols) {
     constexpr int KF = DOK_KF_COLS;
-    P8_DISPATCH(d.value_bytes, (bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
+    P8_DISPATCH(d.value_bytes, (bulk_plan_for<V, KF>(d, n, p), bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
   } else {
-    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (bulk_plan_for<V, KF>(d, n, p), bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
   }
   return note_launch();
 }

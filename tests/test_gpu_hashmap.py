@@ -437,7 +437,7 @@ def test_completely_full_tables_exercise_far_displacements(cuda, vdtype):
 
 def test_line_gather_measurement_kernel_reads_the_lines_it_claims(cuda):
     """dok_line_gather: out[i] = XOR of the sixteen 8-byte words (folded to 32 bits) of bucket
-    fmix64(i ^ seed) * n_buckets >> 64, recomputed here from a copy of the table."""
+    (fmix64(i ^ seed) >> 32) * n_buckets >> 32, recomputed here from a copy of the table."""
     import ctypes
     from doksparse_amd import CudaClosedHashmap, _lib
     from doksparse_amd.closed_hashmap import _stream_ptr
@@ -457,7 +457,7 @@ def test_line_gather_measurement_kernel_reads_the_lines_it_claims(cuda):
         x ^= x >> 33; x = (x * 0xff51afd7ed558ccd) & M
         x ^= x >> 33; x = (x * 0xc4ceb9fe1a85ec53) & M
         x ^= x >> 33
-        line = (x * hm._n_phys) >> 64
+        line = ((x >> 32) * hm._n_phys) >> 32
         w = int(np.bitwise_xor.reduce(table[line]))
         expect[i] = (w ^ (w >> 32)) & 0xffffffff
     assert np.array_equal(out.cpu().numpy().view(np.uint32), expect)
