@@ -32,11 +32,12 @@
 #define DOK_BULK_SUBLOG 8
 #define DOK_BULK_SUB (1 << DOK_BULK_SUBLOG) // ranges per first-level bin
 #define DOK_BULK_MAXBIG 1024                // first-level bins at most
-#define DOK_BULK_TPB 256
-#ifndef DOK_BULK_T
-#define DOK_BULK_T 2048                     // rows per scatter tile
+#ifndef DOK_BULK_TPB
+#define DOK_BULK_TPB 512
 #endif
-#define DOK_BULK_RPT (DOK_BULK_T / DOK_BULK_TPB)
+#ifndef DOK_BULK_T
+#define DOK_BULK_T 4096                     // rows per scatter tile (half of it for 8-byte values, so
+#endif                                      // that two workgroups still share a CU's LDS)
 #ifndef DOK_BULK_CTPB
 #define DOK_BULK_CTPB 1024                  // threads per workgroup of the count kernels: they only stream
 #endif                                      // keys, and the bytes in flight per CU bound their rate
@@ -113,9 +114,12 @@ __device__ __forceinline__ void bulk_stretch2(const BulkWs &ws, u32 b, u32 c, i6
 template <int KF>
 __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count1_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                                    BulkWs ws) {
-  __shared__ u32 cnt[DOK_BULK_MAXBIG];
-  for (int b = threadIdx.x; b < DOK_BULK_MAXBIG; b += DOK_BULK_CTPB) cnt[b] = 0;
+  // Few bins and 64 lanes per atomic instruction mean many lanes on one address, which the LDS
+  // serialises; four copies of the histogram, picked by the lane, thin that out.
+  __shared__ u32 cnt[4 * DOK_BULK_MAXBIG];
+  for (int b = threadIdx.x; b < 4 * DOK_BULK_MAXBIG; b += DOK_BULK_CTPB) cnt[b] = 0;
   __syncthreads();
+  const u32 copy = (threadIdx.x & 3) * DOK_BULK_MAXBIG;
   i64 lo, hi;
   bulk_stretch1(ws, n, blockIdx.x, lo, hi);
   for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += 8 * DOK_BULK_CTPB) {
@@ -129,11 +133,13 @@ __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count1_kernel(DevTable t, 
     }
     #pragma unroll
     for (int u = 0; u < 8; u++)
-      if (ok[u] && (key[u] ^ DOK_P8_XOR) >= 2) atomicAdd(&cnt[bulk_range_of(key[u], t) >> DOK_BULK_SUBLOG], 1u);
+      if (ok[u] && (key[u] ^ DOK_P8_XOR) >= 2)
+        atomicAdd(&cnt[copy + (bulk_range_of(key[u], t) >> DOK_BULK_SUBLOG)], 1u);
   }
   __syncthreads();
   for (int b = threadIdx.x; b < (int)ws.n_big; b += DOK_BULK_CTPB)
-    ws.wg_hist[(size_t)b * ws.g1 + blockIdx.x] = cnt[b];
+    ws.wg_hist[(size_t)b * ws.g1 + blockIdx.x] =
+        cnt[b] + cnt[DOK_BULK_MAXBIG + b] + cnt[2 * DOK_BULK_MAXBIG + b] + cnt[3 * DOK_BULK_MAXBIG + b];
 }
 
 // ---- pass 1, scan: per bin over the workgroups, then over the bins ---------------------------------
@@ -157,10 +163,11 @@ __global__ __launch_bounds__(DOK_BULK_MAXBIG) void bulk_scan1b_kernel(BulkWs ws)
 
 // ---- pass 2, count: rows of every stretch of a first-level bin per range -----------------------------
 __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count2_kernel(DevTable t, BulkWs ws) {
-  __shared__ u32 cnt[DOK_BULK_SUB];
+  __shared__ u32 cnt[4 * DOK_BULK_SUB];              // four copies, as in the first count
   const u32 b = blockIdx.x / ws.ch, c = blockIdx.x % ws.ch;
-  for (int s = threadIdx.x; s < DOK_BULK_SUB; s += DOK_BULK_CTPB) cnt[s] = 0;
+  for (int s = threadIdx.x; s < 4 * DOK_BULK_SUB; s += DOK_BULK_CTPB) cnt[s] = 0;
   __syncthreads();
+  const u32 copy = (threadIdx.x & 3) * DOK_BULK_SUB;
   i64 lo, hi;
   bulk_stretch2(ws, b, c, lo, hi);
   for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += 8 * DOK_BULK_CTPB) {
@@ -172,11 +179,12 @@ __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count2_kernel(DevTable t, 
     }
     #pragma unroll
     for (int u = 0; u < 8; u++)
-      if (i0 + u * DOK_BULK_CTPB < hi) atomicAdd(&cnt[bulk_range_of(key[u], t) & (DOK_BULK_SUB - 1)], 1u);
+      if (i0 + u * DOK_BULK_CTPB < hi) atomicAdd(&cnt[copy + (bulk_range_of(key[u], t) & (DOK_BULK_SUB - 1))], 1u);
   }
   __syncthreads();
   for (int s = threadIdx.x; s < DOK_BULK_SUB; s += DOK_BULK_CTPB)
-    ws.sub_hist[((size_t)b * DOK_BULK_SUB + s) * ws.ch + c] = cnt[s];
+    ws.sub_hist[((size_t)b * DOK_BULK_SUB + s) * ws.ch + c] =
+        cnt[s] + cnt[DOK_BULK_SUB + s] + cnt[2 * DOK_BULK_SUB + s] + cnt[3 * DOK_BULK_SUB + s];
 }
 
 // ---- pass 2, scan: per range over the stretches, then over the ranges of the bin ---------------------
@@ -204,12 +212,14 @@ template <int V, int KF, int LEVEL>
 __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, const void *__restrict__ keys_in,
                                                                     const void *__restrict__ vals_in, i64 n, BulkWs ws) {
   typedef typename ValT<V>::type VT;
+  constexpr int T = V == 8 ? DOK_BULK_T / 2 : DOK_BULK_T;
+  constexpr int RPT = T / DOK_BULK_TPB;
   constexpr int NB = LEVEL == 1 ? DOK_BULK_MAXBIG : DOK_BULK_SUB;
-  constexpr int BPT = NB / DOK_BULK_TPB;             // consecutive bins per thread
+  constexpr int BPT = NB >= DOK_BULK_TPB ? NB / DOK_BULK_TPB : 1;   // consecutive bins per thread
   __shared__ u32 cnt[NB], off[NB], gbase[NB];
-  __shared__ u64 skeys[DOK_BULK_T];
-  __shared__ VT svals[DOK_BULK_T];
-  __shared__ u16 sbins[DOK_BULK_T];                  // bin of every staged row (saves a second hash)
+  __shared__ u64 skeys[T];
+  __shared__ VT svals[T];
+  __shared__ u16 sbins[T];                  // bin of every staged row (saves a second hash)
   __shared__ u32 wsum[16];
   const int tid = threadIdx.x;
   int n_fresh = 0, n_oob = 0;
@@ -243,7 +253,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     #pragma unroll
     for (int q = 0; q < BPT; q++) {
       const size_t idx = (size_t)b * DOK_BULK_SUB + tid * BPT + q;
-      cursor[q] = ws.part_off[idx] + ws.sub_hist[idx * ws.ch + c];
+      cursor[q] = tid * BPT + q < NB ? ws.part_off[idx] + ws.sub_hist[idx * ws.ch + c] : 0u;
     }
   }
 
@@ -251,12 +261,12 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
   // the next tile's loads are issued as soon as the registers are free, so that they are in
   // flight during the write-out of this tile.  st[j]: 0 no row, 1 row, 2 row outside the table's
   // coordinate space.
-  u64 k[DOK_BULK_RPT], v[DOK_BULK_RPT];
-  int st[DOK_BULK_RPT];
+  u64 k[RPT], v[RPT];
+  int st[RPT];
   auto load_tile = [&](i64 lo) {
-    const i64 hi = lo + DOK_BULK_T < hi0 ? lo + DOK_BULK_T : hi0;
+    const i64 hi = lo + T < hi0 ? lo + T : hi0;
     #pragma unroll
-    for (int j = 0; j < DOK_BULK_RPT; j++) {
+    for (int j = 0; j < RPT; j++) {
       const i64 i = lo + j * DOK_BULK_TPB + tid;
       st[j] = 0; k[j] = 0; v[j] = 0;
       if (i < hi) {
@@ -267,17 +277,18 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
   };
   if (lo0 < hi0) load_tile(lo0);
 
-  for (i64 lo = lo0; lo < hi0; lo += DOK_BULK_T) {
+  for (i64 lo = lo0; lo < hi0; lo += T) {
     #pragma unroll
-    for (int q = 0; q < BPT; q++) cnt[tid * BPT + q] = 0;
+    for (int q = 0; q < BPT; q++)
+      if (tid * BPT + q < NB) cnt[tid * BPT + q] = 0;
     __syncthreads();
     BULK_TICK(0);
 
     // bins of the tile's rows and their ranks inside the bins
-    int bn[DOK_BULK_RPT];
-    u32 rk[DOK_BULK_RPT];
+    int bn[RPT];
+    u32 rk[RPT];
     #pragma unroll
-    for (int j = 0; j < DOK_BULK_RPT; j++) {
+    for (int j = 0; j < RPT; j++) {
       bn[j] = -1; rk[j] = 0;
       if (st[j] == 2) n_oob++;
       if (st[j] == 1) {
@@ -290,7 +301,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
       }
     }
     #pragma unroll
-    for (int j = 0; j < DOK_BULK_RPT; j++)
+    for (int j = 0; j < RPT; j++)
       if (bn[j] >= 0) rk[j] = atomicAdd(&cnt[bn[j]], 1u);
     __syncthreads();
     BULK_TICK(1);
@@ -299,15 +310,17 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     u32 c[BPT], csum = 0;
     #pragma unroll
     for (int q = 0; q < BPT; q++) {
-      c[q] = cnt[tid * BPT + q];
+      c[q] = tid * BPT + q < NB ? cnt[tid * BPT + q] : 0u;
       csum += c[q];
     }
     u32 total;
     u32 ex = bulk_block_scan(csum, wsum, total);
     #pragma unroll
     for (int q = 0; q < BPT; q++) {
-      off[tid * BPT + q] = ex;
-      gbase[tid * BPT + q] = cursor[q];
+      if (tid * BPT + q < NB) {
+        off[tid * BPT + q] = ex;
+        gbase[tid * BPT + q] = cursor[q];
+      }
       cursor[q] += c[q];
       ex += c[q];
     }
@@ -315,7 +328,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     BULK_TICK(2);
 
     #pragma unroll
-    for (int j = 0; j < DOK_BULK_RPT; j++) {
+    for (int j = 0; j < RPT; j++) {
       if (bn[j] >= 0) {
         const u32 pos = off[bn[j]] + rk[j];
         skeys[pos] = k[j];
@@ -323,12 +336,12 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
         sbins[pos] = (u16)bn[j];
       }
     }
-    if (lo + DOK_BULK_T < hi0) load_tile(lo + DOK_BULK_T);
+    if (lo + T < hi0) load_tile(lo + T);
     __syncthreads();
     BULK_TICK(3);
 
     #pragma unroll
-    for (int j = 0; j < DOK_BULK_RPT; j++) {
+    for (int j = 0; j < RPT; j++) {
       const u32 pos = tid + j * DOK_BULK_TPB;
       if (pos < total) {
         const u32 b = sbins[pos];

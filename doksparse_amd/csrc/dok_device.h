@@ -135,13 +135,18 @@ __global__ __launch_bounds__(DOK_TPB) void dok_line_gather_kernel(const u64 *__r
 
 // Row-major linearisation of an int64 coordinate row; false if any coordinate is outside
 // [0, dim).  Negative coordinates are not wrapped (the reference does not wrap them either).
+// The loop runs to the compile-time maximum under a uniform guard, so that it unrolls and the
+// coordinate loads of several rows can be in flight together.
 __device__ __forceinline__ bool dok_linearise(const DevTable &t, const i64 *row, u64 &key) {
   bool ok = true;
   u64 k = 0;
-  for (int d = 0; d < t.lin_ndim; d++) {
-    i64 c = row[d];
-    ok = ok && ((u64)c < (u64)t.lin_dims[d]);
-    k += (u64)c * (u64)t.lin_strides[d];
+  #pragma unroll
+  for (int d = 0; d < DOK_MAX_DIMS; d++) {
+    if (d < t.lin_ndim) {
+      const i64 c = row[d];
+      ok = ok && ((u64)c < (u64)t.lin_dims[d]);
+      k += (u64)c * (u64)t.lin_strides[d];
+    }
   }
   key = k;
   return ok;
@@ -163,10 +168,13 @@ __device__ __forceinline__ bool dok_load_key8(const DevTable &t, const void *key
   if (KF == DOK_KF_COLS) {
     bool ok = true;
     u64 k = 0;
-    for (int d = 0; d < t.lin_ndim; d++) {
-      const i64 c = ((const i64 *)keys)[(i64)d * n + i];
-      ok = ok && ((u64)c < (u64)t.lin_dims[d]);
-      k += (u64)c * (u64)t.lin_strides[d];
+    #pragma unroll
+    for (int d = 0; d < DOK_MAX_DIMS; d++) {
+      if (d < t.lin_ndim) {
+        const i64 c = ((const i64 *)keys)[(i64)d * n + i];
+        ok = ok && ((u64)c < (u64)t.lin_dims[d]);
+        k += (u64)c * (u64)t.lin_strides[d];
+      }
     }
     key = k;
     return ok;

@@ -280,6 +280,11 @@ static int set_bulk(const dok_table_t *t, const void *keys, const void *values, 
   if (cols) {
     constexpr int KF = DOK_KF_COLS;
     P8_DISPATCH(d.value_bytes, (bulk_plan_for<V, KF>(d, n, p), bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
+  } else if (d.lin_ndim == 0 && d.key_bytes == 8) {
+    // 8-byte raw keys are already in table form: the loader without the width switch lets the
+    // compiler keep a whole tile's loads in flight
+    constexpr int KF = DOK_KF_U64;
+    P8_DISPATCH(d.value_bytes, (bulk_plan_for<V, KF>(d, n, p), bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
   } else {
     P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (bulk_plan_for<V, KF>(d, n, p), bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
   }
