@@ -61,6 +61,7 @@ struct BulkWs {
   u32 *sub_hist;            // [n_big][SUB][ch]: the same for the ch stretches of a first-level bin
   u32 *part_off;            // [n_big * SUB + 1]  start of every range in keysB
   u32 *def_cnt;             // [GRID] rows each merge workgroup handed to the ordinary insert
+  u32 *meta_cnt;            // [GRID] displacement marks each merge workgroup left to be applied
   u32 n_big, n_part;
   u32 g1;                   // workgroups of the first pass (a multiple of 64, at most DOK_BULK_GRID)
   u32 ch;                   // stretches (workgroups) per first-level bin in the second pass
@@ -417,6 +418,8 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   __shared__ int red[R / 64];
   __shared__ u32 n_def;             // rows this workgroup has deferred so far
   __shared__ u32 n_list;            // rows on the list of the current range
+  __shared__ u32 n_carry;           // listed rows whose chain ran on into the next range
+  __shared__ u32 n_meta;            // displacement marks noted down for the kernel after the merge
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   int n_fresh = 0;
@@ -426,13 +429,15 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   const u32 p_lo = blockIdx.x * per < ws.n_part ? blockIdx.x * per : ws.n_part;
   const u32 p_hi = p_lo + per < ws.n_part ? p_lo + per : ws.n_part;
   const u32 def_base = ws.part_off[p_lo];
-  if (tid == 0) n_def = 0;
+  if (tid == 0) { n_def = 0; n_carry = 0; n_meta = 0; }
   __syncthreads();
 
   for (u32 p = p_lo; p < p_hi; p++) {
     BULK_TICK(5);
     const u32 lo = ws.part_off[p], hi = ws.part_off[p + 1];
-    if (lo == hi) continue;                          // no row of the batch lives in this range
+    const u32 carried = n_carry;                     // rows handed on by the range before (they sit
+                                                     // at the head of the list already)
+    if (lo == hi && carried == 0) continue;          // nothing to do in this range
     const u64 b0 = (u64)p << DOK_BULK_RLOG;
     const u64 left = t.nb - b0;
     const u32 nbk = left < (u64)R ? (u32)left : (u32)R;
@@ -442,6 +447,15 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
     for (int q = 0; q < 8; q++) {
       x[q].x = 0; x[q].y = 0;
       if ((u32)(tid + q * R) < nbk * 8) x[q] = g[tid + q * R];
+    }
+    if (lo == hi) {
+      // only carried rows: the chunk loop below, which otherwise stores the bucket copy, is empty
+      #pragma unroll
+      for (int q = 0; q < 8; q++) {
+        const u32 u = tid + q * R, lb = u >> 3, w = (u & 7) * 2;
+        if (u < nbk * 8) { tb[w * LD + lb] = x[q].x; tb[(w + 1) * LD + lb] = x[q].y; }
+      }
+      if (tid == 0) n_list = carried;
     }
     for (u32 c0 = lo; c0 < hi; c0 += C) {
       const u32 c1 = c0 + C < hi ? c0 + C : hi;
@@ -466,7 +480,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
         }
         #pragma unroll
         for (int q = 0; q < DOK_BULK_FPW; q++) marks[q * R + tid] = 0;
-        if (tid == 0) n_list = 0;
+        if (tid == 0) n_list = carried;
       }
       fresh_cnt[tid] = 0;
       __syncthreads();                               // the bucket copy / the last chunk's writes are complete
@@ -543,20 +557,27 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
     }
     __syncthreads();
 
-    // the listed rows walk their chains, all at once
+    // The listed rows walk their chains, all at once.  A row whose chain runs past the range's
+    // last bucket is handed on to the next range, which this workgroup merges next: there it
+    // continues at the first bucket (its home then lies before the range: lhome < 0).  Rows of
+    // the block's last range, rows that passed a tombstone (its slot is no longer in LDS), and
+    // rows that run through a whole range are left to the ordinary insert instead.
+    if (tid == 0) n_carry = 0;                       // every thread has read it at the top of the range
+    __syncthreads();
+    const u32 total = n_list < (u32)DOK_BULK_LIST ? n_list : (u32)DOK_BULK_LIST;
     {
-      const u32 total = n_list < (u32)DOK_BULK_LIST ? n_list : (u32)DOK_BULK_LIST;
       for (u32 e = tid; e < total; e += R) {
         const u64 key = lkey[e];
         const VT val = lval[e];
         const u64 sk = key ^ DOK_P8_XOR;
-        const u32 lhome = p8_home(sk, t) - (u32)b0;
+        const i64 home = (i64)p8_home(sk, t);
+        const int lhome = (int)(home - (i64)b0);      // negative for a carried row
         const int start = p8_slot_start<V>(sk);
-        u32 d = 0, tomb_d = DOK_NONE32;
+        u32 d = lhome < 0 ? (u32)(-lhome) : 0u, tomb_d = DOK_NONE32;
         int tomb_s = 0;
         int st = -1;                                  // -1 walking, 1 placed, 2 chain leaves the range
         while (st < 0) {
-          const u32 lb = lhome + d;
+          const u32 lb = (u32)(lhome + (int)d);
           if (lb >= nbk) { st = 2; break; }
           asm volatile("" ::: "memory");              // read the bucket afresh in every turn
           u64 w[S];
@@ -579,14 +600,21 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
               u32 td; int ts; u64 expect;
               if (tomb_d != DOK_NONE32) { td = tomb_d; ts = tomb_s; expect = DOK_P8_TOMB; }
               else { td = d; ts = p8_pick(ge, start); expect = DOK_P8_EMPTY; }
-              const u32 tl = lhome + td;
+              const u32 tl = (u32)(lhome + (int)td);
               const u64 old = atomicCAS(&tb[ts * LD + tl], expect, sk);
               if (old == expect) {
                 *(VT *)((char *)(tb + (S + ((ts * V) >> 3)) * LD + tl) + ((ts * V) & 7)) = val;
-                if (td > 0) {
+                if (td > 0 && lhome >= 0) {
                   u32 *meta = (u32 *)(tb + DOK_P8_META * LD + lhome);
                   if (td >= 32) { atomicMax(meta + 1, td); atomicOr(meta, 1u); }
                   else atomicOr(meta, 1u << td);
+                } else if (td > 0) {
+                  // A carried row: its home bucket went back to HBM with plain stores a moment ago,
+                  // and an atomic on that line from inside this kernel is not ordered against
+                  // them.  The mark is noted down (in the part of keysB this workgroup has consumed)
+                  // and applied by the kernel that runs after the merge.
+                  const u32 mi = atomicAdd(&n_meta, 1u);
+                  ws.keysB[def_base + mi] = ((u64)home << 32) | (u64)td;
                 }
                 n_fresh++;
                 st = 1;
@@ -601,11 +629,32 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           }
         }
         if (st == 2) {
-          const u32 at = def_base + atomicAdd(&n_def, 1u);
-          ws.keysA[at] = key;
-          dok_store_val<V>(ws.valsA, (i64)at, (u64)val);
+          bool carry = p + 1 < p_hi && tomb_d == DOK_NONE32 && lhome >= 0;
+          if (carry) {
+            const u32 c = atomicAdd(&n_carry, 1u);
+            if (c < (u32)R && total + c < (u32)DOK_BULK_LIST) { lkey[total + c] = key; lval[total + c] = val; }
+            else carry = false;                       // n_carry is clamped below
+          }
+          if (!carry) {
+            const u32 at = def_base + atomicAdd(&n_def, 1u);
+            ws.keysA[at] = key;
+            dok_store_val<V>(ws.valsA, (i64)at, (u64)val);
+          }
         }
       }
+    }
+    __syncthreads();
+    {
+      // the carried rows move to the head of the list, where the next range expects them
+      u32 nc = n_carry;
+      if (nc > (u32)R) nc = R;
+      if (total + nc > (u32)DOK_BULK_LIST) nc = DOK_BULK_LIST - total;
+      u64 ck = 0; VT cv = 0;
+      if ((u32)tid < nc) { ck = lkey[total + tid]; cv = lval[total + tid]; }
+      __syncthreads();
+      if ((u32)tid < nc) { lkey[tid] = ck; lval[tid] = cv; }
+      __syncthreads();
+      if (tid == 0) n_carry = nc;
     }
     __syncthreads();
     BULK_TICK(3);
@@ -637,6 +686,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
     for (int w = 0; w < R / 64; w++) sum += red[w];
     if (sum) atomicAdd((u64 *)&t.header[DOK_H_NELEM], (u64)(i64)sum);
     ws.def_cnt[blockIdx.x] = n_def;
+    ws.meta_cnt[blockIdx.x] = n_meta;
   }
 }
 
@@ -647,6 +697,15 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
   const u32 per = (ws.n_part + gridDim.x - 1) / gridDim.x;
   const u32 p_lo = blockIdx.x * per < ws.n_part ? blockIdx.x * per : ws.n_part;
   const i64 base = ws.part_off[p_lo];
+  // displacement marks the merge could not set itself (see there)
+  const u32 n_marks = ws.meta_cnt[blockIdx.x];
+  for (u32 i = threadIdx.x; i < n_marks; i += DOK_TPB) {
+    const u64 note = ws.keysB[base + i];
+    const u32 td = (u32)note;
+    u32 *meta = (u32 *)(t.buckets + (note >> 32) * 16 + DOK_P8_META);
+    if (td >= 32) { atomicMax(meta + 1, td); atomicOr(meta, 1u); }
+    else atomicOr(meta, 1u << td);
+  }
   const i64 n = ws.def_cnt[blockIdx.x];
   const i64 waves = DOK_TPB / 64, wave = threadIdx.x >> 6;
   const i64 share = (n + waves - 1) / waves;
@@ -666,7 +725,7 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
 struct BulkPlan {
   u32 n_part, n_big, ch, g1, gm;
   i64 share;
-  size_t o_keysA, o_keysB, o_valsA, o_valsB, o_wg_hist, o_big_off, o_sub_hist, o_part_off, o_def_cnt, bytes;
+  size_t o_keysA, o_keysB, o_valsA, o_valsB, o_wg_hist, o_big_off, o_sub_hist, o_part_off, o_def_cnt, o_meta_cnt, bytes;
 };
 
 static inline size_t bulk_align(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -700,6 +759,7 @@ static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p, u32 g1 = DOK_BULK_G
   p.o_sub_hist = o; o = bulk_align(o + 4 * parts * ch);
   p.o_part_off = o; o = bulk_align(o + 4 * (parts + 1));
   p.o_def_cnt = o; o = bulk_align(o + 4 * DOK_BULK_GRID);
+  p.o_meta_cnt = o; o = bulk_align(o + 4 * DOK_BULK_GRID);
   p.bytes = o;
   return true;
 }
@@ -715,6 +775,7 @@ static void bulk_bind(const BulkPlan &p, void *workspace, BulkWs &ws) {
   ws.sub_hist = (u32 *)(w + p.o_sub_hist);
   ws.part_off = (u32 *)(w + p.o_part_off);
   ws.def_cnt = (u32 *)(w + p.o_def_cnt);
+  ws.meta_cnt = (u32 *)(w + p.o_meta_cnt);
   ws.n_big = p.n_big;
   ws.n_part = p.n_part;
   ws.g1 = p.g1;

@@ -72,6 +72,45 @@ def test_bulk_upsert_matches_oracle(cuda, monkeypatch, key_dtype, value_dtype, n
     _assert_same_map(hm, ref)
 
 
+def test_bulk_nearly_full_table_larger_than_one_pass_of_workgroups(cuda, bulk_always):
+    """2.7M keys into 3M slots (load factor 0.9, ~1170 merge ranges): workgroups merge several
+    consecutive ranges each, probe chains cross range boundaries, and the rows that do are handed
+    from one range to the next.  Then a second batch of the same size: overwrites plus the keys
+    that fill the table to 97 %.  Keys are unique inside each batch, so the expected map is known
+    without the oracle (whose slot-by-slot probing takes minutes at this load): the last value
+    written to each key."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(31)
+    n, extra, capacity = 2_700_000, 210_000, 3_000_000
+    keys = _unique_i64(rng, n + extra)
+    vals = rng.standard_normal((keys.shape[0], 1)).astype(np.float32)
+    hm = CudaClosedHashmap(n_buckets=capacity, device=cuda, rehash_threshold=1.0)
+    hm.set(*_to(cuda, keys[:n, None], vals[:n]))
+    assert hm.n_elements == n
+    got, found = hm.get(torch.from_numpy(keys[:, None]).to(cuda))
+    found = found.cpu().numpy()
+    assert found[:n].all() and not found[n:].any()
+    assert np.array_equal(got.cpu().numpy()[:n], vals[:n])
+
+    again = np.concatenate([keys[n:], keys[: n - extra]])
+    v2 = rng.standard_normal((again.shape[0], 1)).astype(np.float32)
+    hm.set(*_to(cuda, again[:, None], v2))
+    assert hm.n_elements == n + extra
+    expect = vals.copy()
+    expect[n:] = v2[:extra]
+    expect[: n - extra] = v2[extra:]
+    absent = _unique_i64(rng, 100_000) | (1 << 62)
+    got, found = hm.get(torch.from_numpy(np.concatenate([keys, absent])[:, None]).to(cuda), fallback_value=-1.0)
+    found, got = found.cpu().numpy(), got.cpu().numpy()
+    assert found[: keys.shape[0]].all() and not found[keys.shape[0]:].any()
+    assert np.array_equal(got[: keys.shape[0]], expect) and (got[keys.shape[0]:] == -1.0).all()
+    k_out, v_out = hm.items()
+    order = np.argsort(k_out.cpu().numpy().reshape(-1))
+    ref_order = np.argsort(keys)
+    assert np.array_equal(k_out.cpu().numpy().reshape(-1)[order], keys[ref_order])
+    assert np.array_equal(v_out.cpu().numpy()[order], expect[ref_order])
+
+
 def test_bulk_equal_keys_inside_one_batch(cuda, bulk_always):
     """Every key 32 times in one bulk batch: one slot per key, holding one of its values."""
     from doksparse_amd import CudaClosedHashmap
