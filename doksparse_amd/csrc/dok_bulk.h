@@ -387,7 +387,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
 // the LDS copy, which copes with equal keys and tombstones.  Rows whose chain runs past the
 // range's last bucket, and rows that found no room on the list, are handed to the ordinary insert.
 #ifndef DOK_BULK_C
-#define DOK_BULK_C (8 * DOK_BULK_R)
+#define DOK_BULK_C (6 * DOK_BULK_R)
 #endif
 #define DOK_BULK_FPW 8                          // 32-bit fingerprint words per bucket
 #define DOK_BULK_LIST (2 * DOK_BULK_R)          // capacity of a range's list

@@ -253,6 +253,60 @@ __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, c
     u64 iters = 0;
     const u8 *vrow = values + (size_t)i * g.V;
 
+    // Phase 1: the home bucket of all 64 rows is inspected first (the loads of eight rows per
+    // group in flight together), then every owner lane whose row can be decided there acts at
+    // once - the claims, the slot writes and the publishing stores of a whole wave overlap
+    // instead of following one another row by row.  Rows that need more (home bucket full, a
+    // lost claim, a slot that is being written, a tag collision) go through the general loop
+    // below, which starts over at the home bucket.
+    {
+      TgView my;
+      my.hit = my.tagonly = my.busy = my.empty = my.tomb = 0;
+      #pragma unroll
+      for (int r0 = 0; r0 < 16; r0 += 8) {
+        u64 w[8];
+        #pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const u32 qb = dok_shfl32(home, L.gbase + r0 + u);
+          w[u] = dok_load_coherent(t.buckets + (u64)qb * 16 + L.l);
+        }
+        #pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const int j = L.gbase + r0 + u;
+          const u64 qfull = dok_shfl64(tag_full, j);
+          const TgView v = tg_inspect(g, L, true, w[u], qfull, lds_keys + (wave_row0 + j) * g.KW);
+          if (L.l == r0 + u) my = v;
+        }
+      }
+      if (pend) {
+        u64 *bucket = t.buckets + (u64)home * 16;
+        const u64 qbusy = tag_full & ~1ULL;
+        if (my.hit) {
+          u64 *slot = bucket + __builtin_ctz(my.hit);
+          if (atomicCAS(slot, tag_full, qbusy) == tag_full) {
+            for (int k = 0; k < g.VW; k++)
+              dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
+            DOK_TG_RELEASE();
+            dok_store_coherent(slot, tag_full);
+          }
+          st = 1; pend = false;
+        } else if (my.busy == 0 && (my.tagonly & ~my.hit) == 0 && my.empty) {
+          // the chain ends in the home bucket and the key is not there: first tombstone, else
+          // first empty slot
+          u64 *slot = bucket + __builtin_ctz(my.tomb ? my.tomb : my.empty);
+          const u64 expect = my.tomb ? DOK_TG_TOMB : DOK_TG_EMPTY;
+          if (atomicCAS(slot, expect, qbusy) == expect) {
+            for (int k = 0; k < g.KW; k++) dok_store_coherent(slot + 1 + k, krow[k]);
+            for (int k = 0; k < g.VW; k++)
+              dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
+            DOK_TG_RELEASE();
+            dok_store_coherent(slot, tag_full);
+            st = 1; fresh = 1; pend = false;
+          }
+        }
+      }
+    }
+
     u64 pm = dok_ballot(pend);
     while (pm != 0) {
       if (dok_ballot(confirm) != 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
