@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one get launch of the default workload moves, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE scaled against a table scan and a table clear of known size
 # (profiles/hashmap_get_64M_int64_f32_lf05.txt); reported only for that exact workload.
-TRAFFIC_DEFAULT_WORKLOAD = 6.694e9
+TRAFFIC_DEFAULT_WORKLOAD = 6.721e9
 # algorithmic bytes per op for 8-byte keys and 4-byte values: one 128-byte bucket line per op,
 # plus the batch row and the outputs
 B_GET = 8 + 128 + 4 + 1           # key in, bucket line, value out, flag out
