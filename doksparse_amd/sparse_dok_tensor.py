@@ -20,6 +20,7 @@ selectors, a scalar selector behind a slice) the intended result is returned ins
 step other than 1, which the reference silently ignores, raises ``ValueError``.
 """
 import ctypes
+import weakref
 
 import numpy as np
 import torch
@@ -31,6 +32,26 @@ from .closed_hashmap import CudaClosedHashmap, _stream_ptr
 from .util import str2dtype, next_power_of_2, shape_to_stride
 
 _INT_DTYPES = {torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8}
+
+
+# `nonzero` of a boolean mask needs a device-to-host synchronisation (its result's shape). Code
+# that indexes with the same mask tensor again and again pays that every time, so the index
+# tensors of the last few masks are kept, keyed by the mask OBJECT (a weak reference, never an
+# address that could be reused) and its version counter, which every in-place write bumps.
+_MASK_CACHE = {}
+_MASK_CACHE_SIZE = 8
+
+
+def _mask_indices(mask, device):
+    key = id(mask)
+    hit = _MASK_CACHE.get(key)
+    if hit is not None and hit[0]() is mask and hit[1] == mask._version and hit[2] == device:
+        return hit[3]
+    idx = mask.to(device).nonzero(as_tuple=True)
+    if len(_MASK_CACHE) >= _MASK_CACHE_SIZE:
+        _MASK_CACHE.pop(next(iter(_MASK_CACHE)))
+    _MASK_CACHE[key] = (weakref.ref(mask), mask._version, device, idx)
+    return idx
 
 
 class SparseDOKTensor(object):
@@ -278,7 +299,7 @@ class SparseDOKTensor(object):
             if isinstance(sel, np.ndarray):
                 sel = torch.from_numpy(sel)
             if isinstance(sel, Tensor) and sel.dtype == torch.bool:
-                flat.extend(sel.to(self.device).nonzero(as_tuple=True))
+                flat.extend(_mask_indices(sel, self.device))
             elif isinstance(sel, Tensor) and sel.dtype in _INT_DTYPES:
                 flat.append(sel.to(self.device).long())
             elif isinstance(sel, (bool, np.bool_)):

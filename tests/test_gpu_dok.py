@@ -383,3 +383,27 @@ def test_views_share_storage(cuda):
     assert torch.equal(v.flatten().to_dense().cpu(), dense.permute(2, 0, 1).reshape(-1))
     assert torch.equal(v.reshape(30, 7).to_dense().cpu(), dense.permute(2, 0, 1).reshape(30, 7))
     assert torch.equal(v.abs().to_dense().cpu(), dense.permute(2, 0, 1).abs())
+
+
+def test_repeated_mask_selectors_follow_in_place_changes(cuda):
+    """The index tensors of a boolean mask are kept between calls; an in-place write to the mask
+    and a different mask object must both be seen."""
+    from doksparse_amd import SparseDOKTensor
+    g = torch.Generator().manual_seed(8)
+    dense = torch.zeros(40, 16)
+    flat = torch.randperm(40 * 16, generator=g)[:200]
+    dense.view(-1)[flat] = torch.randn(200, generator=g)
+    dok = SparseDOKTensor.from_dense(dense.to(cuda))
+    mask = torch.zeros(16, dtype=torch.bool, device=cuda)
+    mask[[1, 4, 9]] = True
+    rows = torch.arange(0, 40, 3, device=cuda)
+    for _ in range(3):
+        assert torch.equal(dok[rows[:, None], mask].cpu(), dense[rows.cpu()[:, None], mask.cpu()])
+    mask[4] = False                                   # in-place change: the version counter moves
+    mask[12] = True
+    assert torch.equal(dok[rows[:, None], mask].cpu(), dense[rows.cpu()[:, None], mask.cpu()])
+    for k in range(12):                                # fresh mask objects, more than the cache holds
+        m2 = torch.zeros(16, dtype=torch.bool, device=cuda)
+        m2[[k, (k + 5) % 16]] = True
+        assert torch.equal(dok[rows[:, None], m2].cpu(), dense[rows.cpu()[:, None], m2.cpu()])
+        del m2
