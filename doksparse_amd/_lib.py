@@ -79,6 +79,8 @@ SIGNATURES = {
     "dok_coo_set": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p]),
     "dok_coo_compact": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "dok_map_rehash": (c_int32, [POINTER(DokTable), POINTER(DokTable), c_void_p]),
+    "dok_rehash_bulk_workspace_bytes": (c_int64, [POINTER(DokTable), POINTER(DokTable)]),
+    "dok_map_rehash_bulk": (c_int32, [POINTER(DokTable), POINTER(DokTable), c_void_p, c_int64, c_void_p]),
     "dok_getitem_dense": (c_int32, [POINTER(DokTable), POINTER(DokIndex), c_void_p, c_void_p]),
     "dok_setitem_dense": (c_int32, [POINTER(DokTable), POINTER(DokIndex), POINTER(DokView), c_void_p]),
     "dok_count_items": (c_int32, [POINTER(DokTable), POINTER(DokIndex), c_void_p, c_void_p]),

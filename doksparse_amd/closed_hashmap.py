@@ -700,7 +700,18 @@ class CudaClosedHashmap:
         self._seed = int(np.random.randint(1, 2**62, dtype=np.int64))
         table, header, desc, n_phys, slots, layout = self._alloc_table(n_buckets)
         if layout == _lib.DOK_LAYOUT_PACKED8:
-            _lib.check(lib.dok_map_rehash(ctypes.byref(old[2]), ctypes.byref(desc), _stream_ptr(self.device)), "rehash")
+            ws = None
+            if self._n_upper >= BULK_MIN_ROWS and self._n_upper >= BULK_MIN_ROWS_PER_BUCKET * n_phys:
+                # (the upper bound is only a hint for picking the path; both give the same table)
+                nbytes = int(lib.dok_rehash_bulk_workspace_bytes(ctypes.byref(old[2]), ctypes.byref(desc)))
+                if nbytes > 0:
+                    ws = torch.empty(nbytes, device=self.device, dtype=torch.uint8)
+            if ws is not None:
+                _lib.check(lib.dok_map_rehash_bulk(ctypes.byref(old[2]), ctypes.byref(desc), ws.data_ptr(),
+                                                   ws.numel(), _stream_ptr(self.device)), "rehash")
+            else:
+                _lib.check(lib.dok_map_rehash(ctypes.byref(old[2]), ctypes.byref(desc),
+                                              _stream_ptr(self.device)), "rehash")
             self._table, self._header, self._desc, self._n_phys = table, header, desc, n_phys
             self._n_buckets = n_buckets
         else:

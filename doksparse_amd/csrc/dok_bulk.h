@@ -95,6 +95,21 @@ __device__ __forceinline__ u32 bulk_range_of(u64 key, const DevTable &t) {
   return p8_home(key ^ DOK_P8_XOR, t) >> DOK_BULK_RLOG;
 }
 
+// Row i of the batch: its key (and, for a table source, whether word i is a live key slot at all).
+// Returns 1 = row, 0 = no row here, 2 = the row's coordinates lie outside the table.
+template <int KF>
+__device__ __forceinline__ int bulk_load_key(const DevTable &t, const void *keys, i64 i, i64 n, u64 &key) {
+  if (KF == DOK_KF_TABLE) {
+    const int S = 120 / (8 + t.value_bytes);         // slots per bucket of the source (same widths)
+    key = 0;
+    if ((int)(i & 15) >= S) return 0;
+    const u64 w = ((const u64 *)keys)[i];
+    key = w ^ DOK_P8_XOR;
+    return w >= 2 ? 1 : 0;
+  }
+  return dok_load_key8<KF>(t, keys, i, n, key) ? 1 : 2;
+}
+
 // The stretch of rows that workgroup `w` of a pass owns.
 __device__ __forceinline__ void bulk_stretch1(const BulkWs &ws, i64 n, u32 w, i64 &lo, i64 &hi) {
   lo = (i64)w * ws.share;
@@ -130,7 +145,7 @@ __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count1_kernel(DevTable t, 
     for (int u = 0; u < 8; u++) {
       const i64 i = i0 + u * DOK_BULK_CTPB;
       key[u] = 0;
-      ok[u] = i < hi && dok_load_key8<KF>(t, keys, i, n, key[u]);
+      ok[u] = i < hi && bulk_load_key<KF>(t, keys, i, n, key[u]) == 1;
     }
     #pragma unroll
     for (int u = 0; u < 8; u++)
@@ -271,8 +286,13 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
       const i64 i = lo + j * DOK_BULK_TPB + tid;
       st[j] = 0; k[j] = 0; v[j] = 0;
       if (i < hi) {
-        if (dok_load_key8<KF>(t, kin, i, n, k[j])) { v[j] = dok_load_val<V>(vin, i); st[j] = 1; }
-        else st[j] = 2;
+        st[j] = bulk_load_key<KF>(t, kin, i, n, k[j]);
+        if (st[j] == 1) {
+          if (KF == DOK_KF_TABLE)                     // value i & 15 of bucket i >> 4 of the source
+            v[j] = *(const VT *)((const char *)kin + (i >> 4) * 128 + 8 * P8<V>::S + V * (i & 15));
+          else
+            v[j] = dok_load_val<V>(vin, i);
+        }
       }
     }
   };
@@ -732,7 +752,11 @@ static inline size_t bulk_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // False when the bulk path cannot take this table / batch (the caller then uses the ordinary
 // insert).
-static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p, u32 g1 = DOK_BULK_GRID, u32 gm = DOK_BULK_GRID) {
+// n = rows of the input that are looked at, n_cap = most rows that can turn out to be real (the
+// two differ for a table source, where most words are not key slots).
+static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p, u32 g1 = DOK_BULK_GRID, u32 gm = DOK_BULK_GRID,
+                      i64 n_cap = -1) {
+  if (n_cap < 0) n_cap = n;
   if (n < 1 || n > 0x7fff0000LL) return false;
   p.g1 = g1;
   const u64 n_part = (d.nb + DOK_BULK_R - 1) >> DOK_BULK_RLOG;
@@ -750,10 +774,10 @@ static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p, u32 g1 = DOK_BULK_G
   p.gm = p.n_part < gm ? p.n_part : gm;
   const size_t parts = (size_t)n_big * DOK_BULK_SUB;
   size_t o = 0;
-  p.o_keysA = o; o = bulk_align(o + 8 * (size_t)n);
-  p.o_keysB = o; o = bulk_align(o + 8 * (size_t)n);
-  p.o_valsA = o; o = bulk_align(o + (size_t)d.value_bytes * (size_t)n);
-  p.o_valsB = o; o = bulk_align(o + (size_t)d.value_bytes * (size_t)n);
+  p.o_keysA = o; o = bulk_align(o + 8 * (size_t)n_cap);
+  p.o_keysB = o; o = bulk_align(o + 8 * (size_t)n_cap);
+  p.o_valsA = o; o = bulk_align(o + (size_t)d.value_bytes * (size_t)n_cap);
+  p.o_valsB = o; o = bulk_align(o + (size_t)d.value_bytes * (size_t)n_cap);
   p.o_wg_hist = o; o = bulk_align(o + 4 * (size_t)n_big * DOK_BULK_GRID);
   p.o_big_off = o; o = bulk_align(o + 4 * (DOK_BULK_MAXBIG + 1));
   p.o_sub_hist = o; o = bulk_align(o + 4 * parts * ch);
@@ -806,13 +830,22 @@ static u32 bulk_resident(K kernel, int block, u32 limit, u32 multiple) {
 }
 
 template <int V, int KF>
-static bool bulk_plan_for(const DevTable &d, i64 n, BulkPlan &p) {
+static bool bulk_plan_for(const DevTable &d, i64 n, BulkPlan &p, i64 n_cap = -1) {
   static u32 g1 = 0, gm = 0;
   if (g1 == 0) {
     g1 = bulk_resident(bulk_scatter_kernel<V, KF, 1>, DOK_BULK_TPB, DOK_BULK_GRID, 64);
     gm = bulk_resident(bulk_merge_kernel<V>, DOK_BULK_R, DOK_BULK_GRID, 1);
   }
-  return bulk_plan(d, n, p, g1, gm);
+  return bulk_plan(d, n, p, g1, gm, n_cap);
+}
+
+// The two reserved key patterns live in the table header, not in a bucket.
+__global__ void bulk_side_slots_kernel(DevTable src, DevTable dst) {
+  if (threadIdx.x < 2 && src.header[DOK_H_SIDE_STATE + threadIdx.x] != 0) {
+    dst.header[DOK_H_SIDE_STATE + threadIdx.x] = 1;
+    dst.header[DOK_H_SIDE_VALUE + threadIdx.x] = src.header[DOK_H_SIDE_VALUE + threadIdx.x];
+    atomicAdd((u64 *)&dst.header[DOK_H_NELEM], 1ULL);
+  }
 }
 
 template <int V, int KF>

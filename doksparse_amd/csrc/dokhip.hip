@@ -400,6 +400,51 @@ int dok_map_rehash(const dok_table_t *src, const dok_table_t *dst, void *stream)
   return note_launch();
 }
 
+// Rows the source of a bulk rehash is scanned as (every 8-byte word of its buckets) and the most
+// of them that can be live entries.
+static void rehash_rows(const DevTable &a, i64 &n_in, i64 &n_cap) {
+  n_in = (i64)a.nb * 16;
+  n_cap = (i64)a.nb * (120 / (8 + a.value_bytes));
+}
+
+int64_t dok_rehash_bulk_workspace_bytes(const dok_table_t *src, const dok_table_t *dst) {
+  DevTable a, b; int la, lb;
+  int rc = make_dev_table(src, a, la);
+  if (rc) return rc;
+  rc = make_dev_table(dst, b, lb);
+  if (rc) return rc;
+  if (la != DOK_LAYOUT_PACKED8 || lb != DOK_LAYOUT_PACKED8) return 0;
+  i64 n_in, n_cap;
+  rehash_rows(a, n_in, n_cap);
+  BulkPlan p;
+  if (!bulk_plan(b, n_in, p, DOK_BULK_GRID, DOK_BULK_GRID, n_cap)) return 0;
+  return (int64_t)p.bytes;
+}
+
+int dok_map_rehash_bulk(const dok_table_t *src, const dok_table_t *dst, void *workspace,
+                        int64_t workspace_bytes, void *stream) {
+  DevTable a, b; int la, lb;
+  int rc = make_dev_table(src, a, la);
+  if (rc) return rc;
+  rc = make_dev_table(dst, b, lb);
+  if (rc) return rc;
+  if (a.key_bytes != b.key_bytes || a.value_bytes != b.value_bytes || a.lin_ndim != b.lin_ndim) return DOK_EINVAL;
+  if (a.buckets == b.buckets || !workspace) return DOK_EINVAL;
+  for (int k = 0; k < a.lin_ndim; k++) if (a.lin_dims[k] != b.lin_dims[k]) return DOK_EINVAL;
+  if (la != DOK_LAYOUT_PACKED8) return DOK_EUNSUPPORTED;
+  i64 n_in, n_cap;
+  rehash_rows(a, n_in, n_cap);
+  BulkPlan p;
+  if (!bulk_plan(b, n_in, p, DOK_BULK_GRID, DOK_BULK_GRID, n_cap)) return DOK_EUNSUPPORTED;
+  if (((uintptr_t)workspace & 255) != 0 || workspace_bytes < (int64_t)p.bytes) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  constexpr int KF = DOK_KF_TABLE;
+  P8_DISPATCH(b.value_bytes, (bulk_plan_for<V, KF>(b, n_in, p, n_cap),
+                              bulk_launch<V, KF>(b, a.buckets, nullptr, n_in, p, workspace, s)));
+  bulk_side_slots_kernel<<<1, 64, 0, s>>>(a, b);
+  return note_launch();
+}
+
 int dok_getitem_dense(const dok_table_t *t, const dok_index_t *ix, void *out, void *stream) {
   DevTable d; int layout; DevIndex di;
   int rc = make_dev_table(t, d, layout);

@@ -171,6 +171,16 @@ int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out,
  * Reference: CudaClosedHashmap.rehash (cuda_closed_hashmap.py:456-468). */
 int dok_map_rehash(const dok_table_t *src, const dok_table_t *dst, void *stream);
 
+/* dok_map_rehash through the bulk path (see dok_map_set_bulk): the live entries of src are
+ * partitioned by range of dst and merged in LDS.  Same contract as dok_map_rehash plus a
+ * caller-owned workspace of dok_rehash_bulk_workspace_bytes(src, dst) bytes (0 = not available
+ * for these tables, use dok_map_rehash).  Worth it when src holds several entries per bucket of
+ * dst and millions of them.
+ * Reference: CudaClosedHashmap.rehash (cuda_closed_hashmap.py:456-468). */
+int64_t dok_rehash_bulk_workspace_bytes(const dok_table_t *src, const dok_table_t *dst);
+int dok_map_rehash_bulk(const dok_table_t *src, const dok_table_t *dst, void *workspace,
+                        int64_t workspace_bytes, void *stream);
+
 /* ---- COO bridge (tables with lin_ndim > 0) -------------------------------------------------- */
 
 /* dok_map_set for coordinates given the way a COO tensor holds them: indices is

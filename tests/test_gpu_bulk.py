@@ -258,3 +258,53 @@ def test_bulk_call_replays_inside_a_hip_graph(cuda):
         assert hm.n_elements == ref.n_elements
         _check_get(hm, ref, allk[:, None], cuda)             # eager work between replays
         _assert_same_map(hm, ref)
+
+
+@pytest.mark.parametrize("value_dtype", [np.float32, np.int64, np.float16, np.int8])
+def test_bulk_rehash_keeps_the_map(cuda, bulk_always, value_dtype):
+    """rehash through the bulk path (the old table is the batch): live entries move, tombstones
+    and empty slots do not, the two reserved key patterns survive; growing and shrinking."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(17)
+    X = np.uint64(0x9E3779B97F4A7C15)
+    special = np.array([X, X ^ np.uint64(1)], dtype=np.uint64).view(np.int64)
+    keys = np.concatenate([_unique_i64(rng, 60000), special])[:, None]
+    vals = rng.integers(-100, 100, size=(keys.shape[0], 1)).astype(value_dtype)
+    hm = CudaClosedHashmap(n_buckets=70000, device=cuda, rehash_threshold=1.0)
+    ref = RefClosedHashmap(n_buckets=70000, rehash_threshold=1.0, rng=np.random.default_rng(1))
+    hm.set(*_to(cuda, keys, vals)); ref.set(keys, vals)
+    gone = keys[::3]
+    hm.remove(torch.from_numpy(gone).to(cuda)); ref.remove(gone)
+    for new_size in (300_000, 45_000, 1_000_000):
+        hm.rehash(new_size); ref.rehash(new_size)
+        assert hm.n_buckets == ref.n_buckets == new_size
+        assert hm.n_elements == ref.n_elements
+        _assert_same_map(hm, ref)
+        _check_get(hm, ref, keys, cuda, fallback=5)
+    # the rehashed table is an ordinary table: per-row set, remove and get keep working on it
+    more = (_unique_i64(rng, 5000) | (1 << 62))[:, None]
+    mv = rng.integers(-100, 100, size=(5000, 1)).astype(value_dtype)
+    hm.set(*_to(cuda, more, mv)); ref.set(more, mv)
+    hm.remove(torch.from_numpy(keys[1::3]).to(cuda)); ref.remove(keys[1::3])
+    assert hm.n_elements == ref.n_elements
+    _assert_same_map(hm, ref)
+
+
+def test_bulk_rehash_of_a_coordinate_keyed_tensor(cuda, bulk_always):
+    from doksparse_amd import SparseDOKTensor
+    g = torch.Generator().manual_seed(4)
+    size = (500, 300)
+    lin = torch.randperm(size[0] * size[1], generator=g)[:30000]
+    coords = torch.stack([lin // size[1], lin % size[1]])
+    vals = torch.randn(30000, generator=g)
+    dok = SparseDOKTensor(size, coords.to(cuda), vals.to(cuda), device=cuda)
+    dense = torch.zeros(size)
+    dense[coords[0], coords[1]] = vals
+    dok.storage().rehash(200_000)
+    assert dok._nnz() == 30000
+    assert torch.equal(dok.to_dense().cpu(), dense)
+    more = torch.randperm(size[0] * size[1], generator=g)[:40000]
+    mv = torch.randn(40000, generator=g)
+    dok[(more // size[1]).to(cuda), (more % size[1]).to(cuda)] = mv.to(cuda)       # grows again
+    dense[more // size[1], more % size[1]] = mv
+    assert torch.equal(dok.to_dense().cpu(), dense)
