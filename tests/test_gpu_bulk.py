@@ -308,3 +308,48 @@ def test_bulk_rehash_of_a_coordinate_keyed_tensor(cuda, bulk_always):
     dok[(more // size[1]).to(cuda), (more % size[1]).to(cuda)] = mv.to(cuda)       # grows again
     dense[more // size[1], more % size[1]] = mv
     assert torch.equal(dok.to_dense().cpu(), dense)
+
+
+def test_bulk_and_per_row_insert_agree_on_random_configurations(cuda, monkeypatch):
+    """Twelve random configurations (size, load factor up to 0.97, share of repeated keys, value
+    width): three batches each with removals in between, once through the per-row kernel and once
+    through the bulk path.  Values are a function of key and batch number, so the resulting map
+    is unique and must be the same (which the oracle pins for the per-row path elsewhere)."""
+    from doksparse_amd import CudaClosedHashmap, closed_hashmap as ch
+    rng = np.random.default_rng(2024)
+
+    def val_of(keys, rnd, dt):
+        x = (keys * 2654435761 + rnd * 97) >> 7
+        if dt.is_floating_point:
+            return ((x % 2001) - 1000).to(dt)
+        if dt == torch.int8:
+            return ((x % 201) - 100).to(dt)
+        return x.to(dt)
+
+    for case in range(12):
+        n = int(10 ** rng.uniform(3, 6.2))
+        lf = float(rng.uniform(0.2, 0.97))
+        dt = [torch.float32, torch.int64, torch.float16, torch.int8][case % 4]
+        universe = int(n * rng.uniform(0.6, 1.5)) + 10
+        cap = int(universe / lf) + 16
+        g = torch.Generator(device=cuda); g.manual_seed(case)
+        keyspace = torch.randint(-2**62, 2**62, (universe,), generator=g, device=cuda)
+        maps = []
+        for bulk in (False, True):
+            monkeypatch.setattr(ch, "BULK_MIN_ROWS", 0 if bulk else 1 << 62)
+            monkeypatch.setattr(ch, "BULK_MIN_ROWS_PER_BUCKET", 0.0)
+            hm = CudaClosedHashmap(n_buckets=cap, device=cuda, rehash_threshold=1e9, seed=77 + case)
+            gg = torch.Generator(device=cuda); gg.manual_seed(1000 + case)
+            for rnd in range(3):
+                k = keyspace[torch.randint(0, universe, (n,), generator=gg, device=cuda)]
+                hm.set(k[:, None], val_of(k, rnd, dt)[:, None])
+                if rnd == 0:
+                    gone = keyspace[torch.randint(0, universe, (n // 5,), generator=gg, device=cuda)]
+                    hm._remove_rows(gone[:, None].contiguous())
+            h = hm._header.cpu()
+            keys, vals = hm.items()
+            order = torch.argsort(keys.reshape(-1))
+            maps.append((keys.reshape(-1)[order], vals.reshape(-1)[order], int(h[0]), int(h[1])))
+        a, b = maps
+        assert a[2] == b[2] == a[0].shape[0] and a[3] == b[3] == 0, (case, a[2:], b[2:])
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]), f"case {case}: maps differ"
