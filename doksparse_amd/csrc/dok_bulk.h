@@ -402,10 +402,12 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
 //     plain stores;
 //   - rows whose rank lies beyond the free slots, and rows whose home bucket has no EMPTY slot,
 //     go on the list as well.
-// After the last chunk the listed rows (a few per cent of a nearly full table's rows) walk their
-// chains from the home bucket, all at once, with the compare-and-swap protocol of p8_insert on
-// the LDS copy, which copes with equal keys and tombstones.  Rows whose chain runs past the
-// range's last bucket, and rows that found no room on the list, are handed to the ordinary insert.
+// After the last chunk the listed rows (a tenth of the rows at load factor 0.9) are placed all at
+// once, without walking their chains: lookup through the home bucket's displacement map, one row
+// per key through a small hash set, free slots through a bitmap and per-bucket tickets (see
+// there).  Rows that find no room up to the range's last bucket move on to the next range of the
+// same workgroup; rows that found no room on the list, and a few awkward cases, are handed to the
+// ordinary insert.
 #ifndef DOK_BULK_C
 #define DOK_BULK_C (6 * DOK_BULK_R)
 #endif
@@ -432,9 +434,11 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   constexpr int RPT = C / R;
   __shared__ u64 tb[16 * LD];
   __shared__ u32 fresh_cnt[R];
-  __shared__ u32 marks[R * DOK_BULK_FPW];
+  __shared__ __align__(8) u32 marks[R * DOK_BULK_FPW];
   __shared__ u64 lkey[DOK_BULK_LIST];
   __shared__ VT lval[DOK_BULK_LIST];
+  __shared__ u8 lflag[DOK_BULK_LIST];       // 1: the row met a fingerprint mark (an equal key may be around)
+  __shared__ u32 freemap[DOK_BULK_R / 32];  // buckets that still have an unclaimed free slot
   __shared__ int red[R / 64];
   __shared__ u32 n_def;             // rows this workgroup has deferred so far
   __shared__ u32 n_list;            // rows on the list of the current range
@@ -453,7 +457,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   __syncthreads();
 
   for (u32 p = p_lo; p < p_hi; p++) {
-    BULK_TICK(5);
+    BULK_TICK(4);
     const u32 lo = ws.part_off[p], hi = ws.part_off[p + 1];
     const u32 carried = n_carry;                     // rows handed on by the range before (they sit
                                                      // at the head of the list already)
@@ -543,7 +547,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
             if (listed) {
               // onto the range's list while there is room, else to the ordinary insert
               const u32 e = atomicAdd(&n_list, 1u);
-              if (e < DOK_BULK_LIST) { lkey[e] = k[j]; lval[e] = (VT)v[j]; }
+              if (e < DOK_BULK_LIST) { lkey[e] = k[j]; lval[e] = (VT)v[j]; lflag[e] = (seen & bit) ? 1 : 0; }
               else act[j] = 2;
             }
           }
@@ -577,92 +581,149 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
     }
     __syncthreads();
 
-    // The listed rows walk their chains, all at once.  A row whose chain runs past the range's
-    // last bucket is handed on to the next range, which this workgroup merges next: there it
-    // continues at the first bucket (its home then lies before the range: lhome < 0).  Rows of
-    // the block's last range, rows that passed a tombstone (its slot is no longer in LDS), and
-    // rows that run through a whole range are left to the ordinary insert instead.
-    if (tid == 0) n_carry = 0;                       // every thread has read it at the top of the range
-    __syncthreads();
-    const u32 total = n_list < (u32)DOK_BULK_LIST ? n_list : (u32)DOK_BULK_LIST;
+    // The listed rows, one thread each, all at once.  They do not walk their chains:
+    //   - where the key can sit is on record: besides the home bucket, at the displacements the
+    //     home bucket's map marks (the rows placed so far have set their marks in the LDS copy);
+    //   - rows that do not find their key pass a small hash set (in the memory of the fingerprint
+    //     marks, which are done with) that lets one row per key through - the value of that row
+    //     stands for the equal keys of the batch;
+    //   - what is left are distinct new keys, which fight over free slots only.  A new key
+    //     belongs into the first bucket from its home on that has a free slot (a tombstone, else
+    //     an EMPTY slot; every bucket before it then has no EMPTY slot, which is the placement
+    //     rule).  A bitmap of the buckets with free slots left finds that bucket, and a ticket
+    //     counter per bucket hands out exactly as many tickets as it has free slots, so failed
+    //     claims do not pile up and every bucket whose tickets are gone ends up full.
+    // A row that finds no free bucket up to the range's end is handed on to the next range, which
+    // this workgroup merges next (it is then known to be new and the only one of its key: its home
+    // lies before the range, lhome < 0, and it takes the first free slot from bucket 0 on).  Rows
+    // of the block's last range, carried rows that cross a second range and rows whose key may
+    // sit beyond the range's end go to the ordinary insert instead.
+    u64 *hset = (u64 *)marks;
+    constexpr u32 HSET = R * DOK_BULK_FPW / 2;
     {
-      for (u32 e = tid; e < total; e += R) {
-        const u64 key = lkey[e];
-        const VT val = lval[e];
-        const u64 sk = key ^ DOK_P8_XOR;
-        const i64 home = (i64)p8_home(sk, t);
-        const int lhome = (int)(home - (i64)b0);      // negative for a carried row
-        const int start = p8_slot_start<V>(sk);
-        u32 d = lhome < 0 ? (u32)(-lhome) : 0u, tomb_d = DOK_NONE32;
-        int tomb_s = 0;
-        int st = -1;                                  // -1 walking, 1 placed, 2 chain leaves the range
-        while (st < 0) {
-          const u32 lb = (u32)(lhome + (int)d);
-          if (lb >= nbk) { st = 2; break; }
-          asm volatile("" ::: "memory");              // read the bucket afresh in every turn
-          u64 w[S];
+      int nfree = 0;
+      if ((u32)tid < nbk) {
+        #pragma unroll
+        for (int s = 0; s < S; s++) nfree += tb[s * LD + tid] < 2 ? 1 : 0;
+      }
+      fresh_cnt[tid] = (u32)nfree;                   // from here on: tickets for the bucket's free slots
+      const u64 fm = dok_ballot(nfree != 0);
+      if (lane == 0) { freemap[(tid >> 6) * 2] = (u32)fm; freemap[(tid >> 6) * 2 + 1] = (u32)(fm >> 32); }
+      #pragma unroll
+      for (u32 q = 0; q < HSET / R; q++) hset[q * R + tid] = 0;
+      if (tid == 0) n_carry = 0;                     // every thread has read it at the top of the range
+    }
+    __syncthreads();
+    BULK_TICK(3);
+    const u32 total = n_list < (u32)DOK_BULK_LIST ? n_list : (u32)DOK_BULK_LIST;
+    for (u32 e = tid; e < total; e += R) {
+      const u64 key = lkey[e];
+      const VT val = lval[e];
+      const u64 sk = key ^ DOK_P8_XOR;
+      const u64 h = dok_fmix64(sk ^ t.seed);
+      const i64 home = (i64)dok_reduce(h, t.nb);
+      const int lhome = (int)(home - (i64)b0);        // negative for a carried row
+      const int start = p8_slot_start<V>(sk);
+      bool done = false, beyond = false;
+      if (lhome >= 0) {
+        const u64 mw = ((volatile u64 *)tb)[DOK_P8_META * LD + lhome];
+        // bit 0 stands for the home bucket here: the look has checked it, but a row that met a
+        // fingerprint mark may find the key there by now
+        u32 mk = ((u32)mw & ~1u) | (u32)lflag[e];
+        const u32 far_hi = ((u32)mw & 1u) ? (u32)(mw >> 32) : 0u;
+        u32 d = 0;
+        while (true) {
+          if (mk) { d = (u32)__builtin_ctz(mk); mk &= mk - 1; }
+          else if (d < 32 && far_hi >= 32) d = 32;
+          else if (d >= 32 && d < far_hi) d++;
+          else break;
+          const u32 lb = (u32)lhome + d;
+          if (lb >= nbk) { beyond = true; break; }
+          u32 gm = 0;
           #pragma unroll
-          for (int s = 0; s < S; s++) w[s] = tb[s * LD + lb];
-          u32 gm = 0, ge = 0, gt = 0;
-          #pragma unroll
-          for (int s = 0; s < S; s++) {
-            gm |= (u32)(w[s] == sk) << s;
-            ge |= (u32)(w[s] == DOK_P8_EMPTY) << s;
-            gt |= (u32)(w[s] == DOK_P8_TOMB) << s;
-          }
+          for (int s = 0; s < S; s++) gm |= (u32)(tb[s * LD + lb] == sk) << s;
           if (gm) {
             const int s = __builtin_ctz(gm);
             *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lb) + ((s * V) & 7)) = val;
-            st = 1;
-          } else {
-            if (tomb_d == DOK_NONE32 && gt) { tomb_d = d; tomb_s = p8_pick(gt, start); }
-            if (ge) {
-              u32 td; int ts; u64 expect;
-              if (tomb_d != DOK_NONE32) { td = tomb_d; ts = tomb_s; expect = DOK_P8_TOMB; }
-              else { td = d; ts = p8_pick(ge, start); expect = DOK_P8_EMPTY; }
-              const u32 tl = (u32)(lhome + (int)td);
-              const u64 old = atomicCAS(&tb[ts * LD + tl], expect, sk);
-              if (old == expect) {
-                *(VT *)((char *)(tb + (S + ((ts * V) >> 3)) * LD + tl) + ((ts * V) & 7)) = val;
-                if (td > 0 && lhome >= 0) {
-                  u32 *meta = (u32 *)(tb + DOK_P8_META * LD + lhome);
-                  if (td >= 32) { atomicMax(meta + 1, td); atomicOr(meta, 1u); }
-                  else atomicOr(meta, 1u << td);
-                } else if (td > 0) {
-                  // A carried row: its home bucket went back to HBM with plain stores a moment ago,
-                  // and an atomic on that line from inside this kernel is not ordered against
-                  // them.  The mark is noted down (in the part of keysB this workgroup has consumed)
-                  // and applied by the kernel that runs after the merge.
-                  const u32 mi = atomicAdd(&n_meta, 1u);
-                  ws.keysB[def_base + mi] = ((u64)home << 32) | (u64)td;
-                }
-                n_fresh++;
-                st = 1;
-              } else if (old == sk) {
-                st = 1;                               // an equal key won the slot: its value stands
-              } else {
-                d = td; tomb_d = DOK_NONE32;          // another key took it: look again from that bucket
-              }
-            } else {
-              d++;
-            }
+            done = true;
+            break;
           }
         }
-        if (st == 2) {
-          bool carry = p + 1 < p_hi && tomb_d == DOK_NONE32 && lhome >= 0;
-          if (carry) {
-            const u32 c = atomicAdd(&n_carry, 1u);
-            if (c < (u32)R && total + c < (u32)DOK_BULK_LIST) { lkey[total + c] = key; lval[total + c] = val; }
-            else carry = false;                       // n_carry is clamped below
-          }
-          if (!carry) {
-            const u32 at = def_base + atomicAdd(&n_def, 1u);
-            ws.keysA[at] = key;
-            dok_store_val<V>(ws.valsA, (i64)at, (u64)val);
+        if (!done && !beyond) {
+          // one row per key goes on
+          u32 i = (u32)(h >> 8) & (HSET - 1);
+          while (true) {
+            const u64 old = atomicCAS(&hset[i], 0ULL, sk);
+            if (old == 0) break;
+            if (old == sk) { done = true; break; }
+            i = (i + 1) & (HSET - 1);
           }
         }
       }
+      if (done) continue;
+      u32 from = lhome < 0 ? 0u : (u32)lhome;
+      while (!beyond) {
+        // first bucket at or after `from` with a free slot left
+        u32 T = DOK_NONE32;
+        for (u32 wi = from >> 5; wi < (u32)(R / 32); wi++) {
+          u32 m = ((volatile u32 *)freemap)[wi];
+          if (wi == (from >> 5)) m &= ~0u << (from & 31);
+          if (m) { T = wi * 32 + (u32)__builtin_ctz(m); break; }
+        }
+        if (T == DOK_NONE32) break;                   // the chain leaves the range
+        const int ticket = atomicSub((int *)&fresh_cnt[T], 1);
+        if (ticket <= 1) atomicAnd(&freemap[T >> 5], ~(1u << (T & 31)));   // the last one is out
+        if (ticket <= 0) { from = T + 1; continue; }
+        // the ticket stands for one of the bucket's free slots; the other ticket holders may
+        // take the one tried first, but not all of them
+        while (!done) {
+          asm volatile("" ::: "memory");              // read the bucket afresh in every turn
+          u32 ge = 0, gt = 0;
+          #pragma unroll
+          for (int s = 0; s < S; s++) {
+            const u64 w = tb[s * LD + T];
+            ge |= (u32)(w == DOK_P8_EMPTY) << s;
+            gt |= (u32)(w == DOK_P8_TOMB) << s;
+          }
+          if ((ge | gt) == 0) break;                  // cannot happen
+          const int ts = gt ? p8_pick(gt, start) : p8_pick(ge, start);
+          const u64 expect = gt ? DOK_P8_TOMB : DOK_P8_EMPTY;
+          done = atomicCAS(&tb[ts * LD + T], expect, sk) == expect;
+          if (done) {
+            *(VT *)((char *)(tb + (S + ((ts * V) >> 3)) * LD + T) + ((ts * V) & 7)) = val;
+            const u32 td = (u32)((int)T - lhome);
+            if (td > 0 && lhome >= 0) {
+              u32 *meta = (u32 *)(tb + DOK_P8_META * LD + lhome);
+              if (td >= 32) { atomicMax(meta + 1, td); atomicOr(meta, 1u); }
+              else atomicOr(meta, 1u << td);
+            } else if (td > 0) {
+              // A carried row: its home bucket went back to HBM with plain stores a moment ago,
+              // and an atomic on that line from inside this kernel is not ordered against
+              // them.  The mark is noted down (in the part of keysB this workgroup has consumed)
+              // and applied by the kernel that runs after the merge.
+              const u32 mi = atomicAdd(&n_meta, 1u);
+              ws.keysB[def_base + mi] = ((u64)home << 32) | (u64)td;
+            }
+            n_fresh++;
+          }
+        }
+        break;
+      }
+      if (!done) {
+        bool carry = !beyond && p + 1 < p_hi && lhome >= 0;
+        if (carry) {
+          const u32 c = atomicAdd(&n_carry, 1u);
+          if (c < (u32)R && total + c < (u32)DOK_BULK_LIST) { lkey[total + c] = key; lval[total + c] = val; }
+          else carry = false;                         // n_carry is clamped below
+        }
+        if (!carry) {
+          const u32 at = def_base + atomicAdd(&n_def, 1u);
+          ws.keysA[at] = key;
+          dok_store_val<V>(ws.valsA, (i64)at, (u64)val);
+        }
+      }
     }
+    BULK_TICK(5);
     __syncthreads();
     {
       // the carried rows move to the head of the list, where the next range expects them
@@ -677,7 +738,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
       if (tid == 0) n_carry = nc;
     }
     __syncthreads();
-    BULK_TICK(3);
+    BULK_TICK(4);
 
     for (u32 u = tid; u < nbk * 8; u += R) {
       const u32 lb = u >> 3, w = (u & 7) * 2;
@@ -687,7 +748,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
       g[u] = y;
     }
     __syncthreads();
-    BULK_TICK(4);
+    BULK_TICK(0);
   }
 #if defined(DOK_BULK_TIMING) && DOK_BULK_TIMING == 3
   if (threadIdx.x == 0) {
