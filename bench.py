@@ -387,6 +387,19 @@ def main():
         # overwrite pass (every key present)
         o_avg, _ = time_kernel(lambda: raw_set(keys, values), 5)
         results["overwrite_mops_lf05"] = round(n / o_avg / 1e3, 1)
+        # remove of a random half of the keys (the keys are in random order); the removed rows
+        # are stored again outside the timed region
+        half = keys[: n // 2]
+        rem_f = torch.empty(n // 2, device=device, dtype=torch.uint8)
+        def raw_remove():
+            _dl.check(_dl.load().dok_map_remove(ctypes.byref(hm._desc), half.data_ptr(), n // 2, rem_f.data_ptr(),
+                                                _stream_ptr(device)), "remove")
+        raw_remove()
+        assert bool(rem_f.all()) and hm.n_elements == n - n // 2
+        r_avg, _ = time_kernel(raw_remove, 5, prep=lambda: raw_set(half, values[: n // 2]))
+        results["remove_ms_lf05"] = round(r_avg, 4)
+        results["remove_mops_lf05"] = round((n // 2) / r_avg / 1e3, 1)
+        del half, rem_f
         del hm
         torch.cuda.empty_cache()
 

@@ -439,6 +439,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   __shared__ VT lval[DOK_BULK_LIST];
   __shared__ u8 lflag[DOK_BULK_LIST];       // 1: the row met a fingerprint mark (an equal key may be around)
   __shared__ u32 freemap[DOK_BULK_R / 32];  // buckets that still have an unclaimed free slot
+  __shared__ u32 fmask[DOK_BULK_R];         // per bucket: EMPTY slots (low half), tombstones (high half)
   __shared__ int red[R / 64];
   __shared__ u32 n_def;             // rows this workgroup has deferred so far
   __shared__ u32 n_list;            // rows on the list of the current range
@@ -601,11 +602,17 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
     u64 *hset = (u64 *)marks;
     constexpr u32 HSET = R * DOK_BULK_FPW / 2;
     {
-      int nfree = 0;
+      u32 ge = 0, gt = 0;
       if ((u32)tid < nbk) {
         #pragma unroll
-        for (int s = 0; s < S; s++) nfree += tb[s * LD + tid] < 2 ? 1 : 0;
+        for (int s = 0; s < S; s++) {
+          const u64 w = tb[s * LD + tid];
+          ge |= (u32)(w == DOK_P8_EMPTY) << s;
+          gt |= (u32)(w == DOK_P8_TOMB) << s;
+        }
       }
+      fmask[tid] = ge | (gt << 16);
+      const int nfree = __popc(ge) + __popc(gt);
       fresh_cnt[tid] = (u32)nfree;                   // from here on: tickets for the bucket's free slots
       const u64 fm = dok_ballot(nfree != 0);
       if (lane == 0) { freemap[(tid >> 6) * 2] = (u32)fm; freemap[(tid >> 6) * 2 + 1] = (u32)(fm >> 32); }
@@ -623,7 +630,6 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
       const u64 h = dok_fmix64(sk ^ t.seed);
       const i64 home = (i64)dok_reduce(h, t.nb);
       const int lhome = (int)(home - (i64)b0);        // negative for a carried row
-      const int start = p8_slot_start<V>(sk);
       bool done = false, beyond = false;
       if (lhome >= 0) {
         const u64 mw = ((volatile u64 *)tb)[DOK_P8_META * LD + lhome];
@@ -674,38 +680,32 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
         const int ticket = atomicSub((int *)&fresh_cnt[T], 1);
         if (ticket <= 1) atomicAnd(&freemap[T >> 5], ~(1u << (T & 31)));   // the last one is out
         if (ticket <= 0) { from = T + 1; continue; }
-        // the ticket stands for one of the bucket's free slots; the other ticket holders may
-        // take the one tried first, but not all of them
-        while (!done) {
-          asm volatile("" ::: "memory");              // read the bucket afresh in every turn
-          u32 ge = 0, gt = 0;
-          #pragma unroll
-          for (int s = 0; s < S; s++) {
-            const u64 w = tb[s * LD + T];
-            ge |= (u32)(w == DOK_P8_EMPTY) << s;
-            gt |= (u32)(w == DOK_P8_TOMB) << s;
+        // The ticket stands for one of the free slots the bucket had when the tickets were
+        // counted: the k-th row to arrive takes the k-th of them, tombstones first.  Nobody else
+        // writes that slot, so a store does (rows checking this bucket for their own, different
+        // key may read it before or after).
+        {
+          const u32 fm = fmask[T], ge = fm & 0xffffu, gt = fm >> 16;
+          const u32 nt = __popc(gt);
+          const u32 k = nt + __popc(ge) - (u32)ticket;
+          const int ts = k < nt ? bulk_nth_bit(gt, k) : bulk_nth_bit(ge, k - nt);
+          __hip_atomic_store(&tb[ts * LD + T], sk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          *(VT *)((char *)(tb + (S + ((ts * V) >> 3)) * LD + T) + ((ts * V) & 7)) = val;
+          const u32 td = (u32)((int)T - lhome);
+          if (td > 0 && lhome >= 0) {
+            u32 *meta = (u32 *)(tb + DOK_P8_META * LD + lhome);
+            if (td >= 32) { atomicMax(meta + 1, td); atomicOr(meta, 1u); }
+            else atomicOr(meta, 1u << td);
+          } else if (td > 0) {
+            // A carried row: its home bucket went back to HBM with plain stores a moment ago,
+            // and an atomic on that line from inside this kernel is not ordered against
+            // them.  The mark is noted down (in the part of keysB this workgroup has consumed)
+            // and applied by the kernel that runs after the merge.
+            const u32 mi = atomicAdd(&n_meta, 1u);
+            ws.keysB[def_base + mi] = ((u64)home << 32) | (u64)td;
           }
-          if ((ge | gt) == 0) break;                  // cannot happen
-          const int ts = gt ? p8_pick(gt, start) : p8_pick(ge, start);
-          const u64 expect = gt ? DOK_P8_TOMB : DOK_P8_EMPTY;
-          done = atomicCAS(&tb[ts * LD + T], expect, sk) == expect;
-          if (done) {
-            *(VT *)((char *)(tb + (S + ((ts * V) >> 3)) * LD + T) + ((ts * V) & 7)) = val;
-            const u32 td = (u32)((int)T - lhome);
-            if (td > 0 && lhome >= 0) {
-              u32 *meta = (u32 *)(tb + DOK_P8_META * LD + lhome);
-              if (td >= 32) { atomicMax(meta + 1, td); atomicOr(meta, 1u); }
-              else atomicOr(meta, 1u << td);
-            } else if (td > 0) {
-              // A carried row: its home bucket went back to HBM with plain stores a moment ago,
-              // and an atomic on that line from inside this kernel is not ordered against
-              // them.  The mark is noted down (in the part of keysB this workgroup has consumed)
-              // and applied by the kernel that runs after the merge.
-              const u32 mi = atomicAdd(&n_meta, 1u);
-              ws.keysB[def_base + mi] = ((u64)home << 32) | (u64)td;
-            }
-            n_fresh++;
-          }
+          n_fresh++;
+          done = true;
         }
         break;
       }
