@@ -108,9 +108,10 @@ def raw_calls(hm):
     return get, set_, clear
 
 
-def raw_bulk_set(hm, n):
+def raw_bulk_set(hm, n, build=False):
     """Closure launching the bulk insert (partition + merge) of n rows on a preallocated
-    workspace; None if the library has no bulk path for this table."""
+    workspace; None if the library has no bulk path for this table.  build=True: the variant
+    that takes the table as uninitialised memory (clear + insert in one pass)."""
     from doksparse_amd import _lib
     from doksparse_amd.closed_hashmap import _stream_ptr
     lib = _lib.load()
@@ -120,9 +121,11 @@ def raw_bulk_set(hm, n):
         return None
     ws = torch.empty(nbytes, device=hm.device, dtype=torch.uint8)
 
+    fn = lib.dok_map_build_bulk if build else lib.dok_map_set_bulk
+
     def bulk(k, v):
-        _lib.check(lib.dok_map_set_bulk(desc, k.data_ptr(), v.data_ptr(), k.shape[0], ws.data_ptr(), nbytes,
-                                        _stream_ptr(hm.device)), "set_bulk")
+        _lib.check(fn(desc, k.data_ptr(), v.data_ptr(), k.shape[0], ws.data_ptr(), nbytes,
+                      _stream_ptr(hm.device)), "set_bulk")
 
     return bulk
 
@@ -379,6 +382,15 @@ def main():
             b_avg, _ = time_kernel(lambda: bulk(keys, values), 5, prep=raw_clear)
             results["set_bulk_ms_lf05"] = round(b_avg, 4)
             s_avg = min(s_avg, b_avg)
+            # the same rows into a table taken as uninitialised memory (what the first set of a
+            # new map and a rehash run): no clear before, no read of the table
+            del bulk
+            bulk = raw_bulk_set(hm, n, build=True)
+            bulk(keys, values)
+            assert hm.n_elements == n
+            bb_avg, _ = time_kernel(lambda: bulk(keys, values), 5)
+            results["build_ms_lf05"] = round(bb_avg, 4)
+            results["build_mops_lf05"] = round(n / bb_avg / 1e3, 1)
         results["set_ms_lf05"] = round(s_avg, 4)
         results["set_mops_lf05"] = round(n / s_avg / 1e3, 1)
         results["set_algo_gbs_lf05"] = round(n * B_SET / s_avg / 1e6, 1)
@@ -419,6 +431,11 @@ def main():
             assert hm9.n_elements == n
             results["set_bulk_ms_lf09"] = round(b9, 4)
             s9 = min(s9, b9)
+            del bulk9
+            bulk9 = raw_bulk_set(hm9, n, build=True)
+            bb9, _ = time_kernel(lambda: bulk9(keys, values), 3)
+            assert hm9.n_elements == n
+            results["build_ms_lf09"] = round(bb9, 4)
         del bulk9
         results["get_kernel_ms_lf09"] = round(g9, 4)
         results["get_mops_lf09"] = round(n / g9 / 1e3, 1)

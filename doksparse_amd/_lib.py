@@ -72,6 +72,8 @@ SIGNATURES = {
     "dok_bulk_workspace_bytes": (c_int64, [POINTER(DokTable), c_int64]),
     "dok_map_set_bulk": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "dok_coo_set_bulk": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
+    "dok_map_build_bulk": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
+    "dok_coo_build_bulk": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "dok_map_remove": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p]),
     "dok_map_count_existing": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p]),
     "dok_compact_scratch_bytes": (c_int64, [POINTER(DokTable)]),

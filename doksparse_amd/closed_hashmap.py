@@ -80,7 +80,7 @@ class _TableState:
 
 _SHARED = ("_table", "_header", "_desc", "_n_phys", "_slots_per_bucket", "_layout", "_n_buckets",
            "_key_shape", "_key_dtype", "_value_shape", "_value_dtype", "_key_bytes", "_value_bytes",
-           "_n_upper", "_seed")
+           "_n_upper", "_seed", "_pending_clear")
 
 
 def _forward(name):
@@ -145,6 +145,9 @@ class CudaClosedHashmap:
         self._value_bytes = 0
         # host-side upper bound of n_elements; lets set() skip the device read-back
         self._n_upper = 0
+        # True only inside set()/set_coo(), between the allocation of the table and its first
+        # insert: the bucket memory is still uninitialised (a bulk build writes all of it)
+        self._pending_clear = False
 
     # ------------------------------------------------------------------ physical table
     for _name in _SHARED:
@@ -171,7 +174,9 @@ class CudaClosedHashmap:
             d.lin_ndim = 0
         return d
 
-    def _alloc_table(self, n_buckets):
+    def _alloc_table(self, n_buckets, clear=True):
+        """New table tensors and their descriptor.  clear=False leaves the memory uninitialised:
+        only for a caller that clears it (_clear_table) or builds it in bulk right away."""
         lib = _lib.load()
         kb = 8 if self._coord_dims is not None else self._key_bytes
         slots = ctypes.c_int32(0)
@@ -183,8 +188,17 @@ class CudaClosedHashmap:
         assert table.data_ptr() % DOK_BUCKET_BYTES == 0
         header = torch.empty(DOK_HEADER_WORDS, device=self.device, dtype=torch.long)
         desc = self._make_desc(table, header, n_phys)
-        _lib.check(lib.dok_table_clear(ctypes.byref(desc), _stream_ptr(self.device)), "clear")
+        if clear:
+            self._clear_table(desc)
         return table, header, desc, n_phys, int(slots.value), int(layout)
+
+    def _clear_table(self, desc):
+        _lib.check(_lib.load().dok_table_clear(ctypes.byref(desc), _stream_ptr(self.device)), "clear")
+
+    def _ensure_cleared(self):
+        if self._pending_clear:
+            self._pending_clear = False
+            self._clear_table(self._desc)
 
     def _init_storage(self, keys, values):
         self._key_shape = tuple(keys.shape[1:])
@@ -197,7 +211,8 @@ class CudaClosedHashmap:
             assert keys.dtype == torch.long and self._key_shape == (len(self._coord_dims),), \
                 "a coordinate-keyed map takes int64 key rows of one coordinate per dimension"
         (self._table, self._header, self._desc, self._n_phys,
-         self._slots_per_bucket, self._layout) = self._alloc_table(self._n_buckets)
+         self._slots_per_bucket, self._layout) = self._alloc_table(self._n_buckets, clear=False)
+        self._pending_clear = True
         self._n_upper = 0
 
     def _read_header(self):
@@ -430,6 +445,13 @@ class CudaClosedHashmap:
         n = keys.shape[1] if coo else keys.shape[0]
         desc, stream = ctypes.byref(self._desc), _stream_ptr(self.device)
         ws = self._bulk_workspace(n)
+        if ws is not None and self._pending_clear:
+            # first insert into a new table: the build writes every bucket, no clear needed
+            self._pending_clear = False
+            fn = lib.dok_coo_build_bulk if coo else lib.dok_map_build_bulk
+            _lib.check(fn(desc, keys.data_ptr(), values.data_ptr(), n, ws.data_ptr(), ws.numel(), stream), "set")
+            return
+        self._ensure_cleared()
         if ws is not None:
             fn = lib.dok_coo_set_bulk if coo else lib.dok_map_set_bulk
             _lib.check(fn(desc, keys.data_ptr(), values.data_ptr(), n, ws.data_ptr(), ws.numel(), stream), "set")
@@ -453,17 +475,21 @@ class CudaClosedHashmap:
             assert new_values.device == self.device
             assert tuple(new_values.shape[1:]) == self._value_shape
         n = new_keys.shape[0]
-        if n == 0:
-            return
-        keys = self._prep_rows(new_keys, "keys")
-        values = self._prep_rows(new_values, "values")
+        try:
+            if n:
+                self._set_rows(self._prep_rows(new_keys, "keys"), self._prep_rows(new_values, "values"))
+        finally:
+            self._ensure_cleared()      # a new table never leaves this call uninitialised
 
+    def _set_rows(self, keys, values):
+        n = keys.shape[0]
         limit = int(self._rehash_threshold * self._n_buckets)
         if self._n_upper + n <= limit:
             # cannot cross the threshold whatever the batch holds: no read-back, no sync
             self._launch_set(keys, values)
             self._n_upper += n
             return
+        self._ensure_cleared()
         n_old = self.n_elements
         if n_old + n <= limit:
             self._launch_set(keys, values)
@@ -507,9 +533,16 @@ class CudaClosedHashmap:
             assert values.dtype == self._value_dtype and values.device == self.device
             assert tuple(values.shape[1:]) == self._value_shape
         n = indices.shape[1]
-        if n == 0:
-            return
+        try:
+            if n:
+                self._set_coo_rows(indices, values)
+        finally:
+            self._ensure_cleared()      # a new table never leaves this call uninitialised
+
+    def _set_coo_rows(self, indices, values):
+        n = indices.shape[1]
         if self._layout != _lib.DOK_LAYOUT_PACKED8:
+            self._ensure_cleared()
             return self.set(indices.T, values)
         indices = self._prep_rows(indices, "indices")
         values = self._prep_rows(values, "values")
@@ -522,6 +555,7 @@ class CudaClosedHashmap:
             launch()
             self._n_upper += n
             return
+        self._ensure_cleared()
         n_old = self.n_elements
         if n_old + n <= limit:
             launch()
@@ -698,7 +732,7 @@ class CudaClosedHashmap:
         lib = _lib.load()
         old = (self._table, self._header, self._desc)
         self._seed = int(np.random.randint(1, 2**62, dtype=np.int64))
-        table, header, desc, n_phys, slots, layout = self._alloc_table(n_buckets)
+        table, header, desc, n_phys, slots, layout = self._alloc_table(n_buckets, clear=False)
         if layout == _lib.DOK_LAYOUT_PACKED8:
             ws = None
             if self._n_upper >= BULK_MIN_ROWS and self._n_upper >= BULK_MIN_ROWS_PER_BUCKET * n_phys:
@@ -707,14 +741,17 @@ class CudaClosedHashmap:
                 if nbytes > 0:
                     ws = torch.empty(nbytes, device=self.device, dtype=torch.uint8)
             if ws is not None:
+                # writes every bucket of the new table: no clear
                 _lib.check(lib.dok_map_rehash_bulk(ctypes.byref(old[2]), ctypes.byref(desc), ws.data_ptr(),
                                                    ws.numel(), _stream_ptr(self.device)), "rehash")
             else:
+                self._clear_table(desc)
                 _lib.check(lib.dok_map_rehash(ctypes.byref(old[2]), ctypes.byref(desc),
                                               _stream_ptr(self.device)), "rehash")
             self._table, self._header, self._desc, self._n_phys = table, header, desc, n_phys
             self._n_buckets = n_buckets
         else:
+            self._clear_table(desc)
             keys, values = self.items()
             self._table, self._header, self._desc, self._n_phys = table, header, desc, n_phys
             self._n_buckets = n_buckets

@@ -420,7 +420,10 @@ __device__ __forceinline__ int bulk_nth_bit(u32 m, u32 n) {
   return __builtin_ctz(m);
 }
 
-template <int V>
+// FRESH: the table's buckets hold nothing yet, not even the EMPTY pattern.  The merge then takes
+// every range as empty instead of reading it and writes every range, also those without rows, so
+// neither a clear of the table nor its read is paid for.
+template <int V, bool FRESH>
 __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, BulkWs ws) {
 #ifdef DOK_BULK_TIMING
   u64 tacc[6] = {0, 0, 0, 0, 0, 0};
@@ -462,16 +465,21 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
     const u32 lo = ws.part_off[p], hi = ws.part_off[p + 1];
     const u32 carried = n_carry;                     // rows handed on by the range before (they sit
                                                      // at the head of the list already)
-    if (lo == hi && carried == 0) continue;          // nothing to do in this range
+    if (!FRESH && lo == hi && carried == 0) continue;   // nothing to do in this range
     const u64 b0 = (u64)p << DOK_BULK_RLOG;
     const u64 left = t.nb - b0;
     const u32 nbk = left < (u64)R ? (u32)left : (u32)R;
     ulonglong2 *g = (ulonglong2 *)(t.buckets + b0 * 16);
+    if (FRESH && lo == hi && carried == 0) {
+      ulonglong2 z; z.x = 0; z.y = 0;
+      for (u32 u = tid; u < nbk * 8; u += R) g[u] = z;
+      continue;
+    }
     ulonglong2 x[8];                                 // this thread's share of the range: 8 x 16 bytes
     #pragma unroll
     for (int q = 0; q < 8; q++) {
       x[q].x = 0; x[q].y = 0;
-      if ((u32)(tid + q * R) < nbk * 8) x[q] = g[tid + q * R];
+      if (!FRESH && (u32)(tid + q * R) < nbk * 8) x[q] = g[tid + q * R];
     }
     if (lo == hi) {
       // only carried rows: the chunk loop below, which otherwise stores the bucket copy, is empty
@@ -895,7 +903,7 @@ static bool bulk_plan_for(const DevTable &d, i64 n, BulkPlan &p, i64 n_cap = -1)
   static u32 g1 = 0, gm = 0;
   if (g1 == 0) {
     g1 = bulk_resident(bulk_scatter_kernel<V, KF, 1>, DOK_BULK_TPB, DOK_BULK_GRID, 64);
-    gm = bulk_resident(bulk_merge_kernel<V>, DOK_BULK_R, DOK_BULK_GRID, 1);
+    gm = bulk_resident(bulk_merge_kernel<V, false>, DOK_BULK_R, DOK_BULK_GRID, 1);
   }
   return bulk_plan(d, n, p, g1, gm, n_cap);
 }
@@ -909,11 +917,13 @@ __global__ void bulk_side_slots_kernel(DevTable src, DevTable dst) {
   }
 }
 
-template <int V, int KF>
+// FRESH: the table's memory is uninitialised (see bulk_merge_kernel); the header is zeroed here.
+template <int V, int KF, bool FRESH = false>
 static void bulk_launch(const DevTable &d, const void *keys, const void *values, i64 n, const BulkPlan &p,
                         void *workspace, hipStream_t s) {
   BulkWs ws;
   bulk_bind(p, workspace, ws);
+  if (FRESH) dok_fill_kernel<<<1, DOK_TPB, 0, s>>>(d.buckets, 0, d.header);
   bulk_count1_kernel<KF><<<p.g1, DOK_BULK_CTPB, 0, s>>>(d, keys, n, ws);
   bulk_scan1a_kernel<<<p.n_big, p.g1, 0, s>>>(ws);
   bulk_scan1b_kernel<<<1, DOK_BULK_MAXBIG, 0, s>>>(ws);
@@ -921,6 +931,6 @@ static void bulk_launch(const DevTable &d, const void *keys, const void *values,
   bulk_count2_kernel<<<p.n_big * p.ch, DOK_BULK_CTPB, 0, s>>>(d, ws);
   bulk_scan2_kernel<<<p.n_big, DOK_BULK_SUB, 0, s>>>(ws);
   bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
-  bulk_merge_kernel<V><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
+  bulk_merge_kernel<V, FRESH><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
   bulk_deferred_kernel<V><<<p.gm, DOK_TPB, 0, s>>>(d, ws);
 }

@@ -262,43 +262,58 @@ int64_t dok_bulk_workspace_bytes(const dok_table_t *t, int64_t n) {
   return (int64_t)p.bytes;
 }
 
-// Shared body of the two bulk entry points; `cols` selects the column-major coordinate format.
-static int set_bulk(const dok_table_t *t, const void *keys, const void *values, int64_t n, bool cols,
+// Shared body of the bulk entry points; `cols` selects the column-major coordinate format,
+// `fresh` the build into uninitialised table memory.
+static int set_bulk(const dok_table_t *t, const void *keys, const void *values, int64_t n, bool cols, bool fresh,
                     void *workspace, int64_t workspace_bytes, void *stream) {
   DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
   if (cols && d.lin_ndim == 0) return DOK_EINVAL;
   if (n < 0) return DOK_EINVAL;
-  if (n == 0) return DOK_OK;
+  if (n == 0) return fresh ? DOK_EINVAL : DOK_OK;      // a build writes the table: it needs rows
   if (!keys || !values || !workspace) return DOK_EINVAL;
   BulkPlan p;
   if (layout != DOK_LAYOUT_PACKED8 || !bulk_plan(d, n, p)) return DOK_EUNSUPPORTED;
   if (((uintptr_t)workspace & 255) != 0 || workspace_bytes < (int64_t)p.bytes) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   // the launch plan shares the workspace layout of the sizing plan above and only narrows the grids
+#define BULK_GO (bulk_plan_for<V, KF>(d, n, p),                                                    \
+                 fresh ? bulk_launch<V, KF, true>(d, keys, values, n, p, workspace, s)             \
+                       : bulk_launch<V, KF, false>(d, keys, values, n, p, workspace, s))
   if (cols) {
     constexpr int KF = DOK_KF_COLS;
-    P8_DISPATCH(d.value_bytes, (bulk_plan_for<V, KF>(d, n, p), bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
+    P8_DISPATCH(d.value_bytes, BULK_GO);
   } else if (d.lin_ndim == 0 && d.key_bytes == 8) {
     // 8-byte raw keys are already in table form: the loader without the width switch lets the
     // compiler keep a whole tile's loads in flight
     constexpr int KF = DOK_KF_U64;
-    P8_DISPATCH(d.value_bytes, (bulk_plan_for<V, KF>(d, n, p), bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
+    P8_DISPATCH(d.value_bytes, BULK_GO);
   } else {
-    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (bulk_plan_for<V, KF>(d, n, p), bulk_launch<V, KF>(d, keys, values, n, p, workspace, s)));
+    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, BULK_GO);
   }
+#undef BULK_GO
   return note_launch();
 }
 
 int dok_map_set_bulk(const dok_table_t *t, const void *keys, const void *values, int64_t n,
                      void *workspace, int64_t workspace_bytes, void *stream) {
-  return set_bulk(t, keys, values, n, false, workspace, workspace_bytes, stream);
+  return set_bulk(t, keys, values, n, false, false, workspace, workspace_bytes, stream);
 }
 
 int dok_coo_set_bulk(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
                      void *workspace, int64_t workspace_bytes, void *stream) {
-  return set_bulk(t, indices, values, n, true, workspace, workspace_bytes, stream);
+  return set_bulk(t, indices, values, n, true, false, workspace, workspace_bytes, stream);
+}
+
+int dok_map_build_bulk(const dok_table_t *t, const void *keys, const void *values, int64_t n,
+                       void *workspace, int64_t workspace_bytes, void *stream) {
+  return set_bulk(t, keys, values, n, false, true, workspace, workspace_bytes, stream);
+}
+
+int dok_coo_build_bulk(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
+                       void *workspace, int64_t workspace_bytes, void *stream) {
+  return set_bulk(t, indices, values, n, true, true, workspace, workspace_bytes, stream);
 }
 
 int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t *removed, void *stream) {
@@ -440,7 +455,7 @@ int dok_map_rehash_bulk(const dok_table_t *src, const dok_table_t *dst, void *wo
   hipStream_t s = (hipStream_t)stream;
   constexpr int KF = DOK_KF_TABLE;
   P8_DISPATCH(b.value_bytes, (bulk_plan_for<V, KF>(b, n_in, p, n_cap),
-                              bulk_launch<V, KF>(b, a.buckets, nullptr, n_in, p, workspace, s)));
+                              bulk_launch<V, KF, true>(b, a.buckets, nullptr, n_in, p, workspace, s)));
   bulk_side_slots_kernel<<<1, 64, 0, s>>>(a, b);
   return note_launch();
 }

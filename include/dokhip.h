@@ -141,6 +141,17 @@ int64_t dok_bulk_workspace_bytes(const dok_table_t *t, int64_t n);
 int dok_map_set_bulk(const dok_table_t *t, const void *keys, const void *values, int64_t n,
                      void *workspace, int64_t workspace_bytes, void *stream);
 
+/* dok_table_clear followed by dok_map_set_bulk, in one pass: the bucket memory and the header
+ * of t need no initialisation, every bucket and header word is written (n >= 1).  The merge takes
+ * each range of buckets as empty instead of reading it, so neither the clear nor the read of the
+ * table is paid for.
+ * Reference: the first set after the table allocation - CudaClosedHashmap.set on a new map
+ * fills uuid with the EMPTY marker and then launches closed_hashmap_set
+ * (cuda_closed_hashmap.py:36-53, 321-384), as SparseDOKTensor.__init__ does for a COO source
+ * (sparse_dok_tensor.py:59-69). */
+int dok_map_build_bulk(const dok_table_t *t, const void *keys, const void *values, int64_t n,
+                       void *workspace, int64_t workspace_bytes, void *stream);
+
 /* Tombstone each present key; header[DOK_H_NELEM] shrinks by the number removed.  Equal keys
  * in one batch: exactly one row reports 1.
  * Reference: closed_hashmap_remove (closed_hashmap_impl.cu:159-220, ClosedHashmap::remove
@@ -171,11 +182,13 @@ int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out,
  * Reference: CudaClosedHashmap.rehash (cuda_closed_hashmap.py:456-468). */
 int dok_map_rehash(const dok_table_t *src, const dok_table_t *dst, void *stream);
 
-/* dok_map_rehash through the bulk path (see dok_map_set_bulk): the live entries of src are
- * partitioned by range of dst and merged in LDS.  Same contract as dok_map_rehash plus a
- * caller-owned workspace of dok_rehash_bulk_workspace_bytes(src, dst) bytes (0 = not available
- * for these tables, use dok_map_rehash).  Worth it when src holds several entries per bucket of
- * dst and millions of them.
+/* dok_map_rehash through the bulk path (see dok_map_build_bulk): the live entries of src are
+ * partitioned by range of dst and merged in LDS.  Unlike dok_map_rehash, dst need NOT be
+ * cleared: its bucket memory and header may be uninitialised and are overwritten in full
+ * (whatever dst held is gone).  Needs a caller-owned workspace of
+ * dok_rehash_bulk_workspace_bytes(src, dst) bytes (0 = not available for these tables, use
+ * dok_map_rehash).  Worth it when src holds several entries per bucket of dst and millions of
+ * them.
  * Reference: CudaClosedHashmap.rehash (cuda_closed_hashmap.py:456-468). */
 int64_t dok_rehash_bulk_workspace_bytes(const dok_table_t *src, const dok_table_t *dst);
 int dok_map_rehash_bulk(const dok_table_t *src, const dok_table_t *dst, void *workspace,
@@ -193,6 +206,10 @@ int dok_coo_set(const dok_table_t *t, const int64_t *indices, const void *values
 /* dok_coo_set through the bulk path (see dok_map_set_bulk). */
 int dok_coo_set_bulk(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
                      void *workspace, int64_t workspace_bytes, void *stream);
+
+/* dok_coo_set into uninitialised table memory (see dok_map_build_bulk). */
+int dok_coo_build_bulk(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
+                       void *workspace, int64_t workspace_bytes, void *stream);
 
 /* dok_map_compact emitting COO layout: indices_out is [lin_ndim][capacity] int64, values_out
  * [capacity].  Either output may be NULL; count_out[0] receives the number of live entries.

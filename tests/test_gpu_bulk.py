@@ -353,3 +353,128 @@ def test_bulk_and_per_row_insert_agree_on_random_configurations(cuda, monkeypatc
         a, b = maps
         assert a[2] == b[2] == a[0].shape[0] and a[3] == b[3] == 0, (case, a[2:], b[2:])
         assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]), f"case {case}: maps differ"
+
+
+def _garbage(hm):
+    """Overwrite the table's bucket memory and header with a pattern no kernel writes."""
+    hm._table.fill_(0xA5)
+    hm._header.fill_(-0x0123456789ABCDEF)
+
+
+@pytest.mark.parametrize("value_dtype", [np.float32, np.int64, np.float16, np.int8])
+@pytest.mark.parametrize("n,capacity", [(5000, 16384), (20000, 22300), (300, 400), (3000, 2_000_000), (7, 8)])
+def test_build_into_uninitialised_table_matches_oracle(cuda, value_dtype, n, capacity):
+    """dok_map_build_bulk = clear + bulk insert in one pass: table memory and header are filled
+    with garbage first, ranges with and without rows (the sparse 2M-slot table), equal keys in the
+    batch, the reserved key patterns.  Afterwards the table must behave like any other: lookups,
+    read-out, count, a removal and a per-row insert on top."""
+    from doksparse_amd import CudaClosedHashmap, _lib
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    lib = _lib.load()
+    rng = np.random.default_rng(n + capacity + np.dtype(value_dtype).itemsize)
+    XOR = np.uint64(0x9E3779B97F4A7C15).astype(np.int64)
+    keys = _unique_i64(rng, 2 * n, hi=2**62)
+    keys[0], keys[1] = XOR, XOR ^ np.int64(1)                   # the two reserved stored patterns
+    vmax = 100 if np.dtype(value_dtype).itemsize == 1 else 30000
+    hm = CudaClosedHashmap(n_buckets=capacity, device=cuda, rehash_threshold=1.0)
+    ref = RefClosedHashmap(n_buckets=capacity, rehash_threshold=1.0, rng=np.random.default_rng(1))
+    # allocate through a tiny first set, then throw the contents away
+    seed_v = np.zeros((1, 1), dtype=value_dtype)
+    hm.set(*_to(cuda, keys[-1:, None], seed_v))
+    _garbage(hm)
+    batch = np.concatenate([keys[:n], keys[: n // 10]])[:, None]      # a tenth of the keys twice
+    vals = rng.integers(-vmax, vmax, size=(batch.shape[0], 1)).astype(value_dtype)
+    tk, tv = _to(cuda, batch, vals)
+    desc = ctypes.byref(hm._desc)
+    nbytes = int(lib.dok_bulk_workspace_bytes(desc, batch.shape[0]))
+    assert nbytes > 0
+    ws = torch.empty(nbytes, device=cuda, dtype=torch.uint8)
+    _lib.check(lib.dok_map_build_bulk(desc, tk.data_ptr(), tv.data_ptr(), batch.shape[0], ws.data_ptr(), nbytes,
+                                      _stream_ptr(cuda)), "build")
+    # the oracle: unique keys first, then the repeated ones (either value of an equal key is allowed)
+    ref.set(batch[:n], vals[:n])
+    assert hm.n_elements == ref.n_elements == n
+    got_v, got_f = hm.get(tk)
+    assert bool(got_f.all())
+    got = got_v.cpu().numpy()
+    first = {int(k): v for k, v in zip(batch[:n, 0], vals[:n, 0])}
+    second = {int(k): v for k, v in zip(batch[n:, 0], vals[n:, 0])}
+    for k, g in zip(batch[:, 0], got[:, 0]):
+        assert g == first[int(k)] or (int(k) in second and g == second[int(k)])
+    ks, vs = hm.items()
+    assert sorted(ks.cpu().numpy().reshape(-1).tolist()) == sorted(batch[:n, 0].tolist())
+    _, miss = hm.get(torch.from_numpy(keys[n:, None]).to(cuda))
+    assert not bool(miss.any())
+    # ordinary operations on the built table
+    ref2 = RefClosedHashmap(n_buckets=capacity, rehash_threshold=1.0, rng=np.random.default_rng(2))
+    ref2.set(ks.cpu().numpy().reshape(-1, 1), vs.cpu().numpy().reshape(-1, 1))
+    gone = keys[: n // 2, None]
+    hm.remove(torch.from_numpy(gone).to(cuda)); ref2.remove(gone)
+    more = keys[n: n + n // 4, None]
+    mv = rng.integers(-vmax, vmax, size=(more.shape[0], 1)).astype(value_dtype)
+    if more.shape[0]:
+        hm.set(*_to(cuda, more, mv)); ref2.set(more, mv)
+    assert hm.n_elements == ref2.n_elements
+    _assert_same_map(hm, ref2)
+    _check_get(hm, ref2, keys[:, None], cuda, fallback=5)
+
+
+def test_first_set_of_a_new_map_builds_without_clear(cuda, bulk_always):
+    """CudaClosedHashmap.set on a new map: the table is allocated uninitialised and built in one
+    pass when the batch takes the bulk path, cleared first otherwise; either way it is complete
+    when set returns, also for an empty first batch."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(11)
+    keys = _unique_i64(rng, 40000, hi=2**62)
+    vals = rng.integers(-1000, 1000, size=(40000, 1)).astype(np.int32)
+    hm = CudaClosedHashmap(n_buckets=60000, device=cuda)
+    hm.set(*_to(cuda, keys[:30000, None], vals[:30000]))
+    assert not hm._pending_clear and hm.n_elements == 30000
+    ref = RefClosedHashmap(n_buckets=60000, rng=np.random.default_rng(1))
+    ref.set(keys[:30000, None], vals[:30000])
+    _assert_same_map(hm, ref)
+    _check_get(hm, ref, keys[:, None], cuda, fallback=-1)
+    # empty first batch: the table must still come out cleared
+    hm2 = CudaClosedHashmap(n_buckets=1000, device=cuda)
+    hm2.set(torch.empty(0, 1, dtype=torch.long, device=cuda), torch.empty(0, 1, dtype=torch.int32, device=cuda))
+    assert not hm2._pending_clear and hm2.n_elements == 0
+    assert hm2.items()[0].shape[0] == 0
+    _, f = hm2.get(torch.from_numpy(keys[:100, None]).to(cuda))
+    assert not bool(f.any())
+    # first batch above the growth threshold: the count is read before the insert
+    hm3 = CudaClosedHashmap(n_buckets=1000, device=cuda)
+    hm3.set(*_to(cuda, keys[:5000, None], vals[:5000]))
+    assert hm3.n_elements == 5000 and hm3.n_buckets >= 5000
+    ref3 = RefClosedHashmap(n_buckets=1000, rng=np.random.default_rng(1))
+    ref3.set(keys[:5000, None], vals[:5000])
+    assert hm3.n_buckets == ref3.n_buckets
+    _assert_same_map(hm3, ref3)
+
+
+def test_bulk_rehash_overwrites_an_uninitialised_destination(cuda):
+    """dok_map_rehash_bulk needs no cleared destination: garbage in, the source's entries out."""
+    from doksparse_amd import CudaClosedHashmap, _lib
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    lib = _lib.load()
+    rng = np.random.default_rng(21)
+    n = 50000
+    keys = _unique_i64(rng, n + 1000, hi=2**62)
+    vals = rng.standard_normal((n, 1)).astype(np.float32)
+    src = CudaClosedHashmap(n_buckets=70000, device=cuda, rehash_threshold=1.0)
+    src.set(*_to(cuda, keys[:n, None], vals))
+    src.remove(torch.from_numpy(keys[:5000, None]).to(cuda))
+    dst = CudaClosedHashmap(n_buckets=400000, device=cuda, rehash_threshold=1.0, seed=99)
+    dst.set(*_to(cuda, keys[n:, None], vals[:1000]))          # allocates; these entries must vanish
+    _garbage(dst)
+    a, b = ctypes.byref(src._desc), ctypes.byref(dst._desc)
+    nbytes = int(lib.dok_rehash_bulk_workspace_bytes(a, b))
+    assert nbytes > 0
+    ws = torch.empty(nbytes, device=cuda, dtype=torch.uint8)
+    _lib.check(lib.dok_map_rehash_bulk(a, b, ws.data_ptr(), nbytes, _stream_ptr(cuda)), "rehash")
+    assert dst.n_elements == n - 5000
+    v, f = dst.get(torch.from_numpy(keys[:, None]).to(cuda))
+    f = f.cpu().numpy()
+    assert not f[:5000].any() and f[5000:n].all() and not f[n:].any()
+    assert np.array_equal(v.cpu().numpy()[5000:n], vals[5000:])
+    ks, _ = dst.items()
+    assert sorted(ks.cpu().numpy().reshape(-1).tolist()) == sorted(keys[5000:n].tolist())
