@@ -241,7 +241,7 @@ def other_configs(device):
     # cfg5: 4-D (4096, 4096, 64, 8) float16, 100M entries at load factor 0.85
     gen.manual_seed(1005)
     size, strides = (4096, 4096, 64, 8), (4096 * 64 * 8, 64 * 8, 8, 1)
-    lin = uniq_lin(100_000_000, 2**39)
+    lin = uniq_lin(100_000_000, 2**33)
     coords = torch.stack([(lin // st) % s for st, s in zip(strides, size)])
     vals = torch.randn(lin.numel(), generator=gen, device=device).half()
     store = CudaClosedHashmap(n_buckets=int(np.ceil(lin.numel() / 0.85)), device=device, rehash_threshold=0.9,

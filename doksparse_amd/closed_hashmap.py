@@ -38,8 +38,13 @@ def _stream_ptr(device):
 # least this many rows per physical bucket.  The bulk path costs about 35 us per million rows
 # plus 59 us per million buckets (it streams the whole table once) plus ~0.13 ms of launches;
 # the per-row kernel about 66 us per million rows (MI355X, 8-byte keys, 4-byte values).
+# In a table that ends up nearly full the per-row kernel walks longer chains (about 150 us per
+# million rows into a table at 85 % with tombstones), so there the bulk path pays from fewer
+# rows per bucket on.
 BULK_MIN_ROWS = 1 << 23
 BULK_MIN_ROWS_PER_BUCKET = 2.5
+BULK_MIN_ROWS_PER_BUCKET_LOADED = 1.5
+BULK_LOADED_FILL = 0.7
 
 
 def _next_prime(n):
@@ -429,7 +434,13 @@ class CudaClosedHashmap:
         per-row kernel."""
         if self._layout != _lib.DOK_LAYOUT_PACKED8:
             return None
-        if n < BULK_MIN_ROWS or n < BULK_MIN_ROWS_PER_BUCKET * self._n_phys:
+        if n < BULK_MIN_ROWS:
+            return None
+        # (_n_upper is not lowered by removals, so it also counts tombstones - which is what the
+        # length of the probe chains depends on)
+        loaded = self._n_upper + n >= BULK_LOADED_FILL * self._physical_slots()
+        if n < (min(BULK_MIN_ROWS_PER_BUCKET, BULK_MIN_ROWS_PER_BUCKET_LOADED) if loaded
+                else BULK_MIN_ROWS_PER_BUCKET) * self._n_phys:
             return None
         nbytes = int(_lib.load().dok_bulk_workspace_bytes(ctypes.byref(self._desc), n))
         if nbytes <= 0:
