@@ -137,3 +137,70 @@ def test_cfg5_full_size_churn(cuda):
     v, f = dok.storage().get(qc)
     assert not bool(f[:1_000_000].any()) and bool(f[1_000_000:].all())
     assert torch.equal(v[1_000_000:, 0], fv[:1_000_000])
+
+
+@pytest.mark.parametrize("load_factor", [0.5, 0.9])
+def test_cfg3_full_size_int64_to_float32(cuda, load_factor):
+    """The headline configuration: 2^26 unique int64 keys -> float32 at load factor 0.5 and 0.9.
+    Build (bulk path, uninitialised table), bulk upsert on top, get of 2^26 queries (half hits, half
+    misses), read-out round trip, removal of a random half, per-row re-insert of a quarter.  Every
+    result is compared with the sorted-array map."""
+    from doksparse_amd import CudaClosedHashmap
+    gen = torch.Generator(device=cuda); gen.manual_seed(1003)
+    n = 1 << 26
+    draw = torch.unique(torch.randint(0, 2**62, (2 * n + (1 << 20),), generator=gen, device=cuda))
+    draw = draw[torch.randperm(draw.numel(), generator=gen, device=cuda)]
+    assert draw.numel() >= 2 * n
+    keys, absent = draw[:n].contiguous(), draw[n: 2 * n].contiguous()
+    del draw
+    values = torch.randn(n, generator=gen, device=cuda)
+    capacity = 2 * n if load_factor == 0.5 else int(np.ceil(n / 0.9))
+    hm = CudaClosedHashmap(n_buckets=capacity, device=cuda, rehash_threshold=1.0)
+
+    hm.set(keys[:, None], values[:, None])                       # first set: build
+    assert hm.n_elements == n and hm.n_buckets == capacity
+    model = SortedMap(keys, values)
+
+    def check(queries):
+        got_v, got_f = hm.get(queries[:, None])
+        exp_v, exp_f = model.get(queries)
+        assert torch.equal(got_f, exp_f)
+        assert torch.equal(got_v[:, 0], exp_v)
+        return int(exp_f.sum())
+
+    mixed = torch.cat([keys[: n // 2], absent[: n // 2]])
+    mixed = mixed[torch.randperm(n, generator=gen, device=cuda)]
+    assert check(mixed) == n // 2
+    del mixed
+
+    # bulk upsert into the populated table: a quarter overwritten, nothing new
+    values[: n // 4] += 1.0
+    hm.set(keys[: n // 4, None], values[: n // 4, None])
+    assert hm.n_elements == n
+    model = SortedMap(keys, values)
+    assert check(keys) == n
+
+    # read-out: exactly the stored pairs, each once
+    ks, vs = hm.items()
+    assert ks.shape[0] == n
+    order = torch.argsort(ks[:, 0])
+    assert torch.equal(ks[order, 0], model.keys) and torch.equal(vs[order, 0], model.values)
+    del ks, vs, order
+
+    # removal of a random half (the keys are in random order), then a per-row re-insert of a quarter
+    gone = hm._remove_rows(keys[: n // 2, None].contiguous())
+    assert bool(gone.all()) and hm.n_elements == n - n // 2
+    model = SortedMap(keys[n // 2:], values[n // 2:])
+    assert check(keys) == n - n // 2
+    assert check(absent[: n // 4]) == 0
+    back = keys[: n // 4]
+    from doksparse_amd import closed_hashmap as ch
+    old = ch.BULK_MIN_ROWS
+    ch.BULK_MIN_ROWS = 1 << 62
+    try:
+        hm.set(back[:, None], values[: n // 4, None])
+    finally:
+        ch.BULK_MIN_ROWS = old
+    assert hm.n_elements == n - n // 2 + n // 4
+    model = SortedMap(torch.cat([keys[n // 2:], back]), torch.cat([values[n // 2:], values[: n // 4]]))
+    assert check(keys) == n - n // 2 + n // 4
