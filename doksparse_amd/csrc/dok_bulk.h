@@ -488,6 +488,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
         const u32 u = tid + q * R, lb = u >> 3, w = (u & 7) * 2;
         if (u < nbk * 8) { tb[w * LD + lb] = x[q].x; tb[(w + 1) * LD + lb] = x[q].y; }
       }
+      if (FRESH) fmask[tid] = 0;
       if (tid == 0) n_list = carried;
     }
     for (u32 c0 = lo; c0 < hi; c0 += C) {
@@ -513,10 +514,14 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
         }
         #pragma unroll
         for (int q = 0; q < DOK_BULK_FPW; q++) marks[q * R + tid] = 0;
+        if (FRESH) fmask[tid] = 0;                   // slots filled so far, per bucket
         if (tid == 0) n_list = carried;
       }
-      fresh_cnt[tid] = 0;
-      __syncthreads();                               // the bucket copy / the last chunk's writes are complete
+      if (!FRESH) fresh_cnt[tid] = 0;
+      // the bucket copy / the last chunk's writes are complete (a fresh table's slots are only
+      // written in the chunks, never read, so there only the first chunk has to wait - for the
+      // zeroes of the empty copy)
+      if (!FRESH || c0 == lo) __syncthreads();
       BULK_TICK(0);
 
       // look: act[j] = 0 nothing left to do, 1 write key and value into `slot`, 2 defer
@@ -529,6 +534,29 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           const u64 sk = k[j] ^ DOK_P8_XOR;
           const u64 h = dok_fmix64(sk ^ t.seed);
           lh[j] = dok_reduce(h, t.nb) - (u32)b0;
+          if (FRESH) {
+            // Nothing is in the table yet: a row that sets a new fingerprint mark carries a key
+            // no earlier row of the range has, and takes the next slot of its bucket - no slot
+            // is read or compared.  Rows that meet a mark, or a full bucket, go on the list.
+            const u32 fp = (u32)h & (32 * DOK_BULK_FPW - 1), bit = 1u << (fp & 31);
+            const u32 seen = atomicOr(&marks[lh[j] * DOK_BULK_FPW + (fp >> 5)], bit);
+            bool listed = true;
+            if (!(seen & bit)) {
+              const u32 r = atomicAdd(&fmask[lh[j]], 1u);
+              if (r < (u32)S) {
+                tb[r * LD + lh[j]] = sk;
+                *(VT *)((char *)(tb + (S + ((r * V) >> 3)) * LD + lh[j]) + ((r * V) & 7)) = (VT)v[j];
+                n_fresh++;
+                listed = false;
+              }
+            }
+            if (listed) {
+              const u32 e = atomicAdd(&n_list, 1u);
+              if (e < DOK_BULK_LIST) { lkey[e] = k[j]; lval[e] = (VT)v[j]; lflag[e] = (seen & bit) ? 1 : 0; }
+              else act[j] = 2;
+            }
+            continue;
+          }
           u32 gm = 0, ge = 0, gt = 0;
           #pragma unroll
           for (int s = 0; s < S; s++) {
@@ -562,7 +590,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           }
         }
       }
-      __syncthreads();
+      if (!FRESH) __syncthreads();
       BULK_TICK(1);
       // write
       #pragma unroll
@@ -611,7 +639,11 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
     constexpr u32 HSET = R * DOK_BULK_FPW / 2;
     {
       u32 ge = 0, gt = 0;
-      if ((u32)tid < nbk) {
+      if (FRESH) {
+        // slots 0 .. filled-1 hold keys, the rest is EMPTY (the count may have run past S)
+        const u32 f = fmask[tid] < (u32)S ? fmask[tid] : (u32)S;
+        if ((u32)tid < nbk) ge = ((1u << S) - 1u) & ~((1u << f) - 1u);
+      } else if ((u32)tid < nbk) {
         #pragma unroll
         for (int s = 0; s < S; s++) {
           const u64 w = tb[s * LD + tid];
