@@ -441,6 +441,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   __shared__ u64 lkey[DOK_BULK_LIST];
   __shared__ VT lval[DOK_BULK_LIST];
   __shared__ u8 lflag[DOK_BULK_LIST];       // 1: the row met a fingerprint mark (an equal key may be around)
+  __shared__ u32 lpend[DOK_BULK_LIST];      // carried rows: marked displacements still to be looked at
   __shared__ u32 freemap[DOK_BULK_R / 32];  // buckets that still have an unclaimed free slot
   __shared__ u32 fmask[DOK_BULK_R];         // per bucket: EMPTY slots (low half), tombstones (high half)
   __shared__ int red[R / 64];
@@ -671,6 +672,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
       const i64 home = (i64)dok_reduce(h, t.nb);
       const int lhome = (int)(home - (i64)b0);        // negative for a carried row
       bool done = false, beyond = false;
+      u32 pend = 0;                                   // marked displacements that lie past this range
       if (lhome >= 0) {
         const u64 mw = ((volatile u64 *)tb)[DOK_P8_META * LD + lhome];
         // bit 0 stands for the home bucket here: the look has checked it, but a row that met a
@@ -684,7 +686,13 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           else if (d >= 32 && d < far_hi) d++;
           else break;
           const u32 lb = (u32)lhome + d;
-          if (lb >= nbk) { beyond = true; break; }
+          if (lb >= nbk) {
+            // the key may sit in the next range: the row goes there with the marks left to check
+            // (far displacements are left to the ordinary insert)
+            if (d < 32 && far_hi == 0) pend = mk | (1u << d);
+            else beyond = true;
+            break;
+          }
           u32 gm = 0;
           #pragma unroll
           for (int s = 0; s < S; s++) gm |= (u32)(tb[s * LD + lb] == sk) << s;
@@ -705,10 +713,34 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
             i = (i + 1) & (HSET - 1);
           }
         }
+      } else {
+        // a carried row: the buckets its home marks and the range before did not hold
+        u32 mk = lpend[e];
+        while (mk) {
+          const u32 d = (u32)__builtin_ctz(mk);
+          mk &= mk - 1;
+          const int lbs = lhome + (int)d;
+          if (lbs < 0) continue;
+          const u32 lb = (u32)lbs;
+          if (lb >= nbk) { beyond = true; break; }
+          u32 gm = 0;
+          #pragma unroll
+          for (int s = 0; s < S; s++) gm |= (u32)(tb[s * LD + lb] == sk) << s;
+          if (gm) {
+            const int s = __builtin_ctz(gm);
+            *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lb) + ((s * V) & 7)) = val;
+            done = true;
+            break;
+          }
+        }
       }
       if (done) continue;
+      // (A row with marks left to check is not placed here even if the range has room: its key
+      // may sit further on.  Its home marks a bucket past the range's end, so no bucket from its
+      // home to that end has an EMPTY slot, then or now, and a place in the next range keeps
+      // its chain whole.)
       u32 from = lhome < 0 ? 0u : (u32)lhome;
-      while (!beyond) {
+      while (!beyond && pend == 0) {
         // first bucket at or after `from` with a free slot left
         u32 T = DOK_NONE32;
         for (u32 wi = from >> 5; wi < (u32)(R / 32); wi++) {
@@ -753,7 +785,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
         bool carry = !beyond && p + 1 < p_hi && lhome >= 0;
         if (carry) {
           const u32 c = atomicAdd(&n_carry, 1u);
-          if (c < (u32)R && total + c < (u32)DOK_BULK_LIST) { lkey[total + c] = key; lval[total + c] = val; }
+          if (c < (u32)R && total + c < (u32)DOK_BULK_LIST) { lkey[total + c] = key; lval[total + c] = val; lpend[total + c] = pend; }
           else carry = false;                         // n_carry is clamped below
         }
         if (!carry) {
@@ -770,10 +802,10 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
       u32 nc = n_carry;
       if (nc > (u32)R) nc = R;
       if (total + nc > (u32)DOK_BULK_LIST) nc = DOK_BULK_LIST - total;
-      u64 ck = 0; VT cv = 0;
-      if ((u32)tid < nc) { ck = lkey[total + tid]; cv = lval[total + tid]; }
+      u64 ck = 0; VT cv = 0; u32 cp = 0;
+      if ((u32)tid < nc) { ck = lkey[total + tid]; cv = lval[total + tid]; cp = lpend[total + tid]; }
       __syncthreads();
-      if ((u32)tid < nc) { lkey[tid] = ck; lval[tid] = cv; }
+      if ((u32)tid < nc) { lkey[tid] = ck; lval[tid] = cv; lpend[tid] = cp; }
       __syncthreads();
       if (tid == 0) n_carry = nc;
     }

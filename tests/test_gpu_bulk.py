@@ -478,3 +478,39 @@ def test_bulk_rehash_overwrites_an_uninitialised_destination(cuda):
     assert np.array_equal(v.cpu().numpy()[5000:n], vals[5000:])
     ks, _ = dst.items()
     assert sorted(ks.cpu().numpy().reshape(-1).tolist()) == sorted(keys[5000:n].tolist())
+
+
+def test_bulk_upsert_into_a_populated_table_with_tombstones(cuda, bulk_always):
+    """1.5M keys at load factor 0.88, a fifth removed (tombstones), then one bulk batch of
+    overwrites (also of keys that sit in the range after their home's - their rows follow the
+    home bucket's displacement marks across the range boundary), re-inserts of removed keys and
+    new keys.  Keys are unique inside each batch, so the expected map is known in closed form."""
+    from doksparse_amd import CudaClosedHashmap
+    from test_gpu_fullsize import SortedMap
+    gen = torch.Generator(device=cuda); gen.manual_seed(77)
+    n = 1_500_000
+    draw = torch.unique(torch.randint(0, 2**62, (2 * n + 50_000,), generator=gen, device=cuda))
+    draw = draw[torch.randperm(draw.numel(), generator=gen, device=cuda)]
+    keys, extra = draw[:n].contiguous(), draw[n: n + n // 4].contiguous()
+    vals = torch.randint(-2**31, 2**31 - 1, (n,), generator=gen, device=cuda, dtype=torch.int64).to(torch.int32)
+    hm = CudaClosedHashmap(n_buckets=int(n / 0.88), device=cuda, rehash_threshold=1.0)
+    hm.set(keys[:, None], vals[:, None])
+    assert hm.n_elements == n
+    gone = keys[: n // 5]
+    assert bool(hm._remove_rows(gone[:, None].contiguous()).all())
+    # the batch: half of the surviving keys, half of the removed ones, and new keys
+    batch = torch.cat([keys[n // 5:][: 2 * n // 5], gone[: n // 10], extra[: n // 8]])
+    batch = batch[torch.randperm(batch.numel(), generator=gen, device=cuda)].contiguous()
+    bvals = torch.randint(-2**31, 2**31 - 1, (batch.numel(),), generator=gen, device=cuda, dtype=torch.int64).to(torch.int32)
+    hm.set(batch[:, None], bvals[:, None])
+    untouched = keys[n // 5:][2 * n // 5:]
+    model = SortedMap(torch.cat([untouched, batch]),
+                      torch.cat([vals[n // 5:][2 * n // 5:], bvals]))
+    assert hm.n_elements == model.keys.numel()
+    probe = torch.cat([keys, extra])
+    got_v, got_f = hm.get(probe[:, None])
+    exp_v, exp_f = model.get(probe)
+    assert torch.equal(got_f, exp_f) and torch.equal(got_v[:, 0], exp_v)
+    ks, vs = hm.items()
+    order = torch.argsort(ks[:, 0])
+    assert torch.equal(ks[order, 0], model.keys) and torch.equal(vs[order, 0], model.values)
