@@ -107,6 +107,10 @@ __device__ __forceinline__ int bulk_load_key(const DevTable &t, const void *keys
     key = w ^ DOK_P8_XOR;
     return w >= 2 ? 1 : 0;
   }
+  if (KF == DOK_KF_LIN) {
+    key = ((const u64 *)keys)[i];
+    return key == ~0ULL ? 2 : 1;
+  }
   return dok_load_key8<KF>(t, keys, i, n, key) ? 1 : 2;
 }
 
@@ -127,7 +131,10 @@ __device__ __forceinline__ void bulk_stretch2(const BulkWs &ws, u32 b, u32 c, i6
 }
 
 // ---- pass 1, count: rows of every workgroup's stretch per first-level bin ------------------------
-template <int KF>
+// EMIT: the keys are coordinate rows of several words each; their linearised form is written to
+// keysB (free until the second scatter) so that the first scatter reads 8 bytes per row instead
+// of the coordinates a second time.
+template <int KF, bool EMIT>
 __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count1_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                                    BulkWs ws) {
   // Few bins and 64 lanes per atomic instruction mean many lanes on one address, which the LDS
@@ -146,6 +153,7 @@ __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count1_kernel(DevTable t, 
       const i64 i = i0 + u * DOK_BULK_CTPB;
       key[u] = 0;
       ok[u] = i < hi && bulk_load_key<KF>(t, keys, i, n, key[u]) == 1;
+      if (EMIT && i < hi) ws.keysB[i] = ok[u] ? key[u] : ~0ULL;
     }
     #pragma unroll
     for (int u = 0; u < 8; u++)
@@ -988,10 +996,15 @@ static void bulk_launch(const DevTable &d, const void *keys, const void *values,
   BulkWs ws;
   bulk_bind(p, workspace, ws);
   if (FRESH) dok_fill_kernel<<<1, DOK_TPB, 0, s>>>(d.buckets, 0, d.header);
-  bulk_count1_kernel<KF><<<p.g1, DOK_BULK_CTPB, 0, s>>>(d, keys, n, ws);
+  // coordinate rows of three and more dimensions are linearised once, by the count
+  constexpr bool COORDS = KF == DOK_KF_COLS || KF == DOK_KF_ROWS;
+  const bool emit = COORDS && d.lin_ndim >= 3;
+  if (emit) bulk_count1_kernel<KF, COORDS><<<p.g1, DOK_BULK_CTPB, 0, s>>>(d, keys, n, ws);
+  else bulk_count1_kernel<KF, false><<<p.g1, DOK_BULK_CTPB, 0, s>>>(d, keys, n, ws);
   bulk_scan1a_kernel<<<p.n_big, p.g1, 0, s>>>(ws);
   bulk_scan1b_kernel<<<1, DOK_BULK_MAXBIG, 0, s>>>(ws);
-  bulk_scatter_kernel<V, KF, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, keys, values, n, ws);
+  if (emit) bulk_scatter_kernel<V, COORDS ? DOK_KF_LIN : KF, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, ws.keysB, values, n, ws);
+  else bulk_scatter_kernel<V, KF, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, keys, values, n, ws);
   bulk_count2_kernel<<<p.n_big * p.ch, DOK_BULK_CTPB, 0, s>>>(d, ws);
   bulk_scan2_kernel<<<p.n_big, DOK_BULK_SUB, 0, s>>>(ws);
   bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);

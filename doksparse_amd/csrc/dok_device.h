@@ -161,6 +161,8 @@ __device__ __forceinline__ bool dok_linearise(const DevTable &t, const i64 *row,
 #define DOK_KF_U64  3   // keys already in table form: one 8-byte word per row, whatever key_bytes is
 #define DOK_KF_TABLE 4  // (bulk rehash only) the "batch" is another packed table: row i is word i of
                         // its bucket array; the words that are live key slots are the rows
+#define DOK_KF_LIN  5   // (bulk path only) linearised coordinates, one 8-byte word per row; all ones =
+                        // a row whose coordinates lie outside the table
 
 // Key of batch row i (of n) as an 8-byte integer; false if a coordinate is out of range.
 template <int KF>
