@@ -16,9 +16,11 @@
 //      atomic on global memory.  A scatter tile is staged in LDS ordered by bin, so the global
 //      writes are runs of consecutive addresses;
 //   3. one workgroup per range copies the range's buckets into LDS, places the range's rows
-//      there and streams the buckets back;
-//   4. rows the merge cannot place by looking at their home bucket alone are handed, packed, to
-//      the ordinary insert, which runs last.
+//      there and streams the buckets back (a table that holds nothing yet is not read: the
+//      copy starts empty, and the clear of the table is saved as well);
+//   4. the few rows the merge cannot place within the ranges of one workgroup (chains that run
+//      into a range another workgroup owns, overflow of the per-range lists) are handed,
+//      packed, to the ordinary insert, which runs last.
 //
 // Every step is exact for any input: bin sizes are counted, not estimated, and a batch whose
 // rows all fall into one range merely degrades to step 4's ordinary insert.
