@@ -560,6 +560,18 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
                 n_fresh++;
                 listed = false;
               }
+            } else {
+              // An equal key may be among the earlier rows: if it is in the bucket by now, its
+              // value is overwritten here (a batch with many equal keys would otherwise flood
+              // the list); if not (yet), the row goes on the list and is sorted out there.
+              u32 gm = 0;
+              #pragma unroll
+              for (int s = 0; s < S; s++) gm |= (u32)(((volatile u64 *)tb)[s * LD + lh[j]] == sk) << s;
+              if (gm) {
+                const int s = __builtin_ctz(gm);
+                *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lh[j]) + ((s * V) & 7)) = (VT)v[j];
+                listed = false;
+              }
             }
             if (listed) {
               const u32 e = atomicAdd(&n_list, 1u);

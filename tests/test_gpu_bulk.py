@@ -514,3 +514,23 @@ def test_bulk_upsert_into_a_populated_table_with_tombstones(cuda, bulk_always):
     ks, vs = hm.items()
     order = torch.argsort(ks[:, 0])
     assert torch.equal(ks[order, 0], model.keys) and torch.equal(vs[order, 0], model.values)
+
+
+@pytest.mark.parametrize("distinct", [1, 300, 20000])
+def test_build_with_many_equal_keys(cuda, bulk_always, distinct):
+    """First set of a new map (fresh-table merge) with every key repeated many times: each key is
+    stored once and holds the value of one of its rows."""
+    from doksparse_amd import CudaClosedHashmap
+    gen = torch.Generator(device=cuda); gen.manual_seed(distinct)
+    n = 400_000
+    base = torch.unique(torch.randint(0, 2**62, (distinct + 16,), generator=gen, device=cuda))[:distinct]
+    keys = base[torch.randint(0, distinct, (n,), generator=gen, device=cuda)].contiguous()
+    vals = torch.arange(n, device=cuda, dtype=torch.int32)
+    hm = CudaClosedHashmap(n_buckets=max(2 * distinct, 64), device=cuda, rehash_threshold=1.0)
+    hm.set(keys[:, None], vals[:, None])
+    assert hm.n_elements == int(torch.unique(keys).numel())
+    v, f = hm.get(keys[:, None])
+    assert bool(f.all())
+    assert bool((keys[v[:, 0].long()] == keys).all())      # the value is the index of a row with this key
+    ks, _ = hm.items()
+    assert torch.equal(torch.sort(ks[:, 0]).values, torch.unique(keys))
