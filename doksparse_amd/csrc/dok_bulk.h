@@ -37,9 +37,29 @@
 #ifndef DOK_BULK_TPB
 #define DOK_BULK_TPB 512
 #endif
+// Rows per scatter tile.  A tile is staged in LDS whole (8 + V + 2 bytes per row), and the larger
+// it is, the longer the runs of rows that leave for one bin: for 8-byte keys with 4-byte values
+// one workgroup per CU with a tile that nearly fills the LDS beats two with half the tile
+// (scatter of 64M rows: 0.57 -> 0.47 ms).  Where it does not, the sizes below say so; all of
+// them are measured choices.
 #ifndef DOK_BULK_T
-#define DOK_BULK_T 4096                     // rows per scatter tile (half of it for 8-byte values, so
-#endif                                      // that two workgroups still share a CU's LDS)
+#define DOK_BULK_T 8192                     // first pass (up to 1024 bins: 12 KiB of bin arrays)
+#endif
+#ifndef DOK_BULK_T1C
+#define DOK_BULK_T1C 4096                   //   ... from coordinate rows or a table: the loads weigh more
+#endif                                      //   than the writes there, and two workgroups per CU hide them
+#ifndef DOK_BULK_T1V8
+#define DOK_BULK_T1V8 6144                  //   ... with 8-byte values
+#endif
+#ifndef DOK_BULK_T2
+#define DOK_BULK_T2 10240                   // second pass (256 bins)
+#endif
+#ifndef DOK_BULK_T2S
+#define DOK_BULK_T2S 4096                   //   ... with 1- and 2-byte values (measured: three workgroups
+#endif                                      //   per CU with small tiles are faster there)
+#ifndef DOK_BULK_T2V8
+#define DOK_BULK_T2V8 8192                  //   ... with 8-byte values
+#endif
 #ifndef DOK_BULK_CTPB
 #define DOK_BULK_CTPB 1024                  // threads per workgroup of the count kernels: they only stream
 #endif                                      // keys, and the bytes in flight per CU bound their rate
@@ -238,7 +258,10 @@ template <int V, int KF, int LEVEL>
 __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, const void *__restrict__ keys_in,
                                                                     const void *__restrict__ vals_in, i64 n, BulkWs ws) {
   typedef typename ValT<V>::type VT;
-  constexpr int T = V == 8 ? DOK_BULK_T / 2 : DOK_BULK_T;
+  constexpr bool CHEAP = KF == DOK_KF_U64 || KF == DOK_KF_RAW;      // one load per row
+  constexpr int T = LEVEL == 1 ? (!CHEAP ? DOK_BULK_T1C : V == 8 ? DOK_BULK_T1V8 : DOK_BULK_T)
+                               : (V == 8 ? DOK_BULK_T2V8 : V == 4 ? DOK_BULK_T2 : DOK_BULK_T2S);
+  static_assert(T % DOK_BULK_TPB == 0, "every thread stages the same number of rows");
   constexpr int RPT = T / DOK_BULK_TPB;
   constexpr int NB = LEVEL == 1 ? DOK_BULK_MAXBIG : DOK_BULK_SUB;
   constexpr int BPT = NB >= DOK_BULK_TPB ? NB / DOK_BULK_TPB : 1;   // consecutive bins per thread
@@ -560,10 +583,14 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
                 n_fresh++;
                 listed = false;
               }
-            } else {
-              // An equal key may be among the earlier rows: if it is in the bucket by now, its
-              // value is overwritten here (a batch with many equal keys would otherwise flood
-              // the list); if not (yet), the row goes on the list and is sorted out there.
+            }
+            // A row that met a mark may repeat the key of an earlier row.  A few such rows per wave
+            // are the normal case (fingerprints collide) and go on the list, whose pass sorts
+            // them out.  Many of them mean a batch with many equal keys, which would flood the
+            // list: then they look into their bucket right here and, where the key is in it by
+            // now, overwrite its value.  (The test is per wave, so the usual batch does not pay
+            // for the reads of this branch.)
+            if (__popcll(dok_ballot((seen & bit) != 0)) >= 8 && (seen & bit)) {
               u32 gm = 0;
               #pragma unroll
               for (int s = 0; s < S; s++) gm |= (u32)(((volatile u64 *)tb)[s * LD + lh[j]] == sk) << s;
