@@ -47,6 +47,17 @@ BULK_MIN_ROWS_PER_BUCKET_LOADED = 1.5
 BULK_LOADED_FILL = 0.7
 
 
+def bulk_pays(n, n_phys, slots_per_bucket, n_upper):
+    """Whether a batch of n rows into a table of n_phys buckets should take the bulk path.
+    n_upper: upper bound of the slots in use before the batch; it is not lowered by removals,
+    so it also counts tombstones - which is what the length of the probe chains depends on."""
+    if n < BULK_MIN_ROWS:
+        return False
+    loaded = n_upper + n >= BULK_LOADED_FILL * n_phys * slots_per_bucket
+    per_bucket = min(BULK_MIN_ROWS_PER_BUCKET, BULK_MIN_ROWS_PER_BUCKET_LOADED) if loaded else BULK_MIN_ROWS_PER_BUCKET
+    return n >= per_bucket * n_phys
+
+
 def _next_prime(n):
     """Smallest prime > n (deterministic Miller-Rabin, exact below 3.3e24)."""
     def is_prime(m):
@@ -434,13 +445,7 @@ class CudaClosedHashmap:
         per-row kernel."""
         if self._layout != _lib.DOK_LAYOUT_PACKED8:
             return None
-        if n < BULK_MIN_ROWS:
-            return None
-        # (_n_upper is not lowered by removals, so it also counts tombstones - which is what the
-        # length of the probe chains depends on)
-        loaded = self._n_upper + n >= BULK_LOADED_FILL * self._physical_slots()
-        if n < (min(BULK_MIN_ROWS_PER_BUCKET, BULK_MIN_ROWS_PER_BUCKET_LOADED) if loaded
-                else BULK_MIN_ROWS_PER_BUCKET) * self._n_phys:
+        if not bulk_pays(n, self._n_phys, self._slots_per_bucket, self._n_upper):
             return None
         nbytes = int(_lib.load().dok_bulk_workspace_bytes(ctypes.byref(self._desc), n))
         if nbytes <= 0:

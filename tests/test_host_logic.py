@@ -240,3 +240,23 @@ def test_affine_plan_4d_and_views():
     assert out_shape == (6, 3)
     assert ix.sel[2].base == 1 and ix.sel[3].base == 2          # view dims 0, 2 -> storage dims 2, 3
     assert list(ix.sel[0].strides)[:2] == [1, 0] and list(ix.sel[1].strides)[:2] == [0, 1]
+
+
+def test_bulk_path_decision():
+    """The host rule that sends a batch through the bulk insert: large batches with enough rows
+    per bucket, fewer rows per bucket when the table ends up nearly full."""
+    from doksparse_amd.closed_hashmap import bulk_pays
+    M = 1 << 20
+    S = 10                                        # slots per bucket of int64 -> float32
+    # the headline build: 64M rows into 2^27 slots
+    assert bulk_pays(64 * M, 128 * M // S, S, 0)
+    # small batches never
+    assert not bulk_pays(4 * M, 4 * M // S, S, 0)
+    # a large batch that is thin against the table (1.25 rows per bucket, table stays empty)
+    assert not bulk_pays(16 * M, int(16 * M / 1.25), S, 0)
+    # the same density pays once the table ends up more than 70 % full ...
+    nb = 10 * M
+    assert not bulk_pays(16 * M, nb, S, 0)                    # 1.6 rows per bucket, ends 16 % full
+    assert bulk_pays(16 * M, nb, S, int(0.6 * nb * S))        # ends 76 % full
+    # ... but not below 1.5 rows per bucket
+    assert not bulk_pays(12 * M, nb, S, int(0.8 * nb * S))
