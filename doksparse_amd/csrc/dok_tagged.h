@@ -253,74 +253,42 @@ __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, c
     u64 iters = 0;
     const u8 *vrow = values + (size_t)i * g.V;
 
-    // Phase 1: the home bucket of all 64 rows is inspected first (the loads of eight rows per
-    // group in flight together), then every owner lane whose row can be decided there acts at
-    // once - the claims, the slot writes and the publishing stores of a whole wave overlap
-    // instead of following one another row by row.  Rows that need more (home bucket full, a
-    // lost claim, a slot that is being written, a tag collision) go through the general loop
-    // below, which starts over at the home bucket.
-    {
-      TgView my;
-      my.hit = my.tagonly = my.busy = my.empty = my.tomb = 0;
-      #pragma unroll
-      for (int r0 = 0; r0 < 16; r0 += 8) {
-        u64 w[8];
-        #pragma unroll
-        for (int u = 0; u < 8; u++) {
-          const u32 qb = dok_shfl32(home, L.gbase + r0 + u);
-          w[u] = dok_load_coherent(t.buckets + (u64)qb * 16 + L.l);
-        }
-        #pragma unroll
-        for (int u = 0; u < 8; u++) {
-          const int j = L.gbase + r0 + u;
-          const u64 qfull = dok_shfl64(tag_full, j);
-          const TgView v = tg_inspect(g, L, true, w[u], qfull, lds_keys + (wave_row0 + j) * g.KW);
-          if (L.l == r0 + u) my = v;
-        }
-      }
-      if (pend) {
-        u64 *bucket = t.buckets + (u64)home * 16;
-        const u64 qbusy = tag_full & ~1ULL;
-        if (my.hit) {
-          u64 *slot = bucket + __builtin_ctz(my.hit);
-          if (atomicCAS(slot, tag_full, qbusy) == tag_full) {
-            for (int k = 0; k < g.VW; k++)
-              dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
-            DOK_TG_RELEASE();
-            dok_store_coherent(slot, tag_full);
-          }
-          st = 1; pend = false;
-        } else if (my.busy == 0 && (my.tagonly & ~my.hit) == 0 && my.empty) {
-          // the chain ends in the home bucket and the key is not there: first tombstone, else
-          // first empty slot
-          u64 *slot = bucket + __builtin_ctz(my.tomb ? my.tomb : my.empty);
-          const u64 expect = my.tomb ? DOK_TG_TOMB : DOK_TG_EMPTY;
-          if (atomicCAS(slot, expect, qbusy) == expect) {
-            for (int k = 0; k < g.KW; k++) dok_store_coherent(slot + 1 + k, krow[k]);
-            for (int k = 0; k < g.VW; k++)
-              dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
-            DOK_TG_RELEASE();
-            dok_store_coherent(slot, tag_full);
-            st = 1; fresh = 1; pend = false;
-          }
-        }
-      }
-    }
-
+    // Turns: in every turn the current bucket of EVERY pending row of the wave is inspected (the
+    // loads of eight rows per group in flight together), then all owner lanes act at once - the
+    // claims, the slot writes and the publishing stores of a whole wave overlap instead of
+    // following one another row by row.  The first turn looks at the home buckets and settles
+    // most rows; rows that walk on (bucket full, a lost claim, a slot that is being written, a
+    // tag collision) stay pending for the next turn.
     u64 pm = dok_ballot(pend);
     while (pm != 0) {
       if (dok_ballot(confirm) != 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-      const u32 sub = (u32)(pm >> L.gbase) & 0xffffu;
-      const bool has = sub != 0;
-      const int r = has ? __builtin_ctz(sub) : 0;
-      const int j = L.gbase + r;
-      const u32 qb = dok_shfl32(b, j);
-      const u64 qfull = dok_shfl64(tag_full, j);
-      const u64 w = dok_load_coherent(t.buckets + (u64)(has ? qb : 0u) * 16 + L.l);
-      const TgView v = tg_inspect(g, L, has, w, qfull, lds_keys + (wave_row0 + j) * g.KW);
-      if (has && L.l == r) {
+      const u32 sub = (u32)(pm >> L.gbase) & 0xffffu;          // this group's pending rows
+      u32 any = (u32)pm | (u32)(pm >> 32);
+      any = (any | (any >> 16)) & 0xffffu;                      // row numbers pending in some group
+      TgView v;
+      v.hit = v.tagonly = v.busy = v.empty = v.tomb = 0;
+      #pragma unroll
+      for (int r0 = 0; r0 < 16; r0 += 8) {
+        if (((any >> r0) & 0xffu) == 0) continue;
+        u64 w[8];
+        #pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const u32 qb = dok_shfl32(b, L.gbase + r0 + u);
+          w[u] = 0;
+          if ((sub >> (r0 + u)) & 1u) w[u] = dok_load_coherent(t.buckets + (u64)qb * 16 + L.l);
+        }
+        #pragma unroll
+        for (int u = 0; u < 8; u++) {
+          if (!((any >> (r0 + u)) & 1u)) continue;
+          const int j = L.gbase + r0 + u;
+          const u64 qfull = dok_shfl64(tag_full, j);
+          const TgView x = tg_inspect(g, L, ((sub >> (r0 + u)) & 1u) != 0, w[u], qfull, lds_keys + (wave_row0 + j) * g.KW);
+          if (L.l == r0 + u) v = x;
+        }
+      }
+      if (pend) {
         u64 *bucket = t.buckets + (u64)b * 16;
-        const u64 qbusy = qfull & ~1ULL;
+        const u64 qfull = tag_full, qbusy = tag_full & ~1ULL;
         if (v.hit) {
           u64 *slot = bucket + __builtin_ctz(v.hit);
           if (atomicCAS(slot, qfull, qbusy) == qfull) {
