@@ -482,6 +482,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   __shared__ u32 n_list;            // rows on the list of the current range
   __shared__ u32 n_carry;           // listed rows whose chain ran on into the next range
   __shared__ u32 n_meta;            // displacement marks noted down for the kernel after the merge
+  __shared__ u32 range_live;        // the current range's buckets hold something (a key, a tombstone, a mark)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   int n_fresh = 0;
@@ -491,7 +492,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   const u32 p_lo = blockIdx.x * per < ws.n_part ? blockIdx.x * per : ws.n_part;
   const u32 p_hi = p_lo + per < ws.n_part ? p_lo + per : ws.n_part;
   const u32 def_base = ws.part_off[p_lo];
-  if (tid == 0) { n_def = 0; n_carry = 0; n_meta = 0; }
+  if (tid == 0) { n_def = 0; n_carry = 0; n_meta = 0; range_live = 0; }
   __syncthreads();
 
   for (u32 p = p_lo; p < p_hi; p++) {
@@ -525,6 +526,10 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
       if (FRESH) fmask[tid] = 0;
       if (tid == 0) n_list = carried;
     }
+    // `fr`: the range holds nothing, so its rows need not look at slots (see the look below).  Known
+    // at compile time for a fresh table, found out while the copy is staged otherwise (upserts
+    // into a cleared or sparsely filled table).
+    bool fr = FRESH;
     for (u32 c0 = lo; c0 < hi; c0 += C) {
       const u32 c1 = c0 + C < hi ? c0 + C : hi;
       u64 k[RPT], v[RPT];
@@ -546,16 +551,23 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           const u32 u = tid + q * R, lb = u >> 3, w = (u & 7) * 2;
           if (u < nbk * 8) { tb[w * LD + lb] = x[q].x; tb[(w + 1) * LD + lb] = x[q].y; }
         }
+        if (!FRESH) {
+          u64 nz = 0;
+          #pragma unroll
+          for (int q = 0; q < 8; q++) nz |= x[q].x | x[q].y;
+          if (nz) range_live = 1;
+        }
         #pragma unroll
         for (int q = 0; q < DOK_BULK_FPW; q++) marks[q * R + tid] = 0;
-        if (FRESH) fmask[tid] = 0;                   // slots filled so far, per bucket
+        fmask[tid] = 0;                              // (empty range) slots filled so far, per bucket
         if (tid == 0) n_list = carried;
       }
       if (!FRESH) fresh_cnt[tid] = 0;
-      // the bucket copy / the last chunk's writes are complete (a fresh table's slots are only
+      // the bucket copy / the last chunk's writes are complete (an empty range's slots are only
       // written in the chunks, never read, so there only the first chunk has to wait - for the
       // zeroes of the empty copy)
-      if (!FRESH || c0 == lo) __syncthreads();
+      if (!fr || c0 == lo) __syncthreads();
+      if (!FRESH && c0 == lo) fr = range_live == 0;
       BULK_TICK(0);
 
       // look: act[j] = 0 nothing left to do, 1 write key and value into `slot`, 2 defer
@@ -568,8 +580,8 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           const u64 sk = k[j] ^ DOK_P8_XOR;
           const u64 h = dok_fmix64(sk ^ t.seed);
           lh[j] = dok_reduce(h, t.nb) - (u32)b0;
-          if (FRESH) {
-            // Nothing is in the table yet: a row that sets a new fingerprint mark carries a key
+          if (fr) {
+            // Nothing is in the range yet: a row that sets a new fingerprint mark carries a key
             // no earlier row of the range has, and takes the next slot of its bucket - no slot
             // is read or compared.  Rows that meet a mark, or a full bucket, go on the list.
             const u32 fp = (u32)h & (32 * DOK_BULK_FPW - 1), bit = 1u << (fp & 31);
@@ -640,7 +652,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           }
         }
       }
-      if (!FRESH) __syncthreads();
+      if (!fr) __syncthreads();
       BULK_TICK(1);
       // write
       #pragma unroll
@@ -689,7 +701,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
     constexpr u32 HSET = R * DOK_BULK_FPW / 2;
     {
       u32 ge = 0, gt = 0;
-      if (FRESH) {
+      if (fr) {
         // slots 0 .. filled-1 hold keys, the rest is EMPTY (the count may have run past S)
         const u32 f = fmask[tid] < (u32)S ? fmask[tid] : (u32)S;
         if ((u32)tid < nbk) ge = ((1u << S) - 1u) & ~((1u << f) - 1u);
@@ -856,7 +868,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
       __syncthreads();
       if ((u32)tid < nc) { lkey[tid] = ck; lval[tid] = cv; lpend[tid] = cp; }
       __syncthreads();
-      if (tid == 0) n_carry = nc;
+      if (tid == 0) { n_carry = nc; range_live = 0; }
     }
     __syncthreads();
     BULK_TICK(4);
