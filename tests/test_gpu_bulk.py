@@ -534,3 +534,56 @@ def test_build_with_many_equal_keys(cuda, bulk_always, distinct):
     assert bool((keys[v[:, 0].long()] == keys).all())      # the value is the index of a row with this key
     ks, _ = hm.items()
     assert torch.equal(torch.sort(ks[:, 0]).values, torch.unique(keys))
+
+
+@pytest.mark.parametrize("size", [(5000, 3000), (300, 77, 50), (40, 30, 20, 16), (9, 8, 7, 6, 5, 4)])
+def test_bulk_and_per_row_agree_on_coordinate_batches(cuda, monkeypatch, size):
+    """Coordinate keys in both layouts ([n, ndim] rows and [ndim, n] COO columns; three and more
+    dimensions are linearised by the bulk path's first count), repeated coordinates, coordinates
+    outside the size, a removal in between and a second batch: the per-row kernels and the bulk
+    path must leave the same map and the same counters."""
+    from doksparse_amd import CudaClosedHashmap, closed_hashmap as ch
+    gen = torch.Generator(device=cuda); gen.manual_seed(len(size))
+    vol = int(np.prod(size))
+    n = min(200_000, vol // 3)
+
+    def batch(rnd):
+        c = torch.stack([torch.randint(0, s, (n,), generator=gen, device=cuda) for s in size])      # [ndim, n]
+        c[0, ::97] = size[0] + rnd                                       # rows outside the size
+        lin = torch.zeros(n, dtype=torch.long, device=cuda)
+        for d, s in enumerate(size):
+            lin = lin * s + c[d]
+        return c, ((lin * 31 + rnd) % 1000).to(torch.float32)           # equal coordinates carry equal values
+
+    b1, b2 = batch(0), batch(1)
+    gone = b1[0][:, 5:n // 4:3].T.contiguous()
+    gone = gone[(gone[:, 0] < size[0])]
+    results = []
+    for bulk in (False, True):
+        monkeypatch.setattr(ch, "BULK_MIN_ROWS", 0 if bulk else 1 << 62)
+        monkeypatch.setattr(ch, "BULK_MIN_ROWS_PER_BUCKET", 0.0)
+        per_layout = []
+        for coo in (False, True):
+            hm = CudaClosedHashmap(n_buckets=int(1.3 * 2 * n), device=cuda, coord_dims=size, rehash_threshold=1.0,
+                                   seed=4242)
+            for c, v in (b1, b2):
+                if coo:
+                    hm.set_coo(c.contiguous(), v[:, None].contiguous())
+                else:
+                    hm.set(c.T.contiguous(), v[:, None].contiguous())
+                if c is b1[0]:
+                    hm._remove_rows(gone)
+            idx, vals = hm.items_coo()
+            lin = torch.zeros(idx.shape[1], dtype=torch.long, device=cuda)
+            for d, s in enumerate(size):
+                lin = lin * s + idx[d]
+            order = torch.argsort(lin)
+            h = hm._header.cpu()
+            per_layout.append((lin[order], vals.reshape(-1)[order], int(h[0]), int(h[1]), int(h[3])))
+        results.append(per_layout)
+    ref = results[0][0]
+    assert ref[2] == ref[0].shape[0] and ref[3] == 0 and ref[4] == 2 * len(range(0, n, 97))
+    for per_layout in results:
+        for got in per_layout:
+            assert got[2:] == ref[2:]
+            assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
