@@ -38,7 +38,7 @@ def _stream_ptr(device):
 # least this many rows per physical bucket.  The bulk path costs about 35 us per million rows
 # plus 59 us per million buckets (it streams the whole table once) plus ~0.13 ms of launches;
 # the per-row kernel about 66 us per million rows (MI355X, 8-byte keys, 4-byte values).
-# In a table that ends up nearly full the per-row kernel walks longer chains (about 150 us per
+# In a table that ends up nearly full the per-row kernel walks longer chains (about 100 us per
 # million rows into a table at 85 % with tombstones), so there the bulk path pays from fewer
 # rows per bucket on.
 BULK_MIN_ROWS = 1 << 23

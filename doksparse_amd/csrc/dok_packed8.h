@@ -472,7 +472,13 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
 // of its own, and the number of bucket lines in flight does not drop when the table is nearly
 // full (at load factor 0.9 this is 1.3x faster than tile-wise p8_insert).  All loads are
 // device-coherent, so a row that lost its claim to another key simply looks again, from the
-// bucket of the slot it lost, in the next pass.  The placement rules are those of p8_insert.
+// bucket of the slot it lost, in the next pass.
+// A row's place is the first free slot of its walk (a tombstone of that bucket before an EMPTY
+// slot), as in p8_insert.  That the key is not in the table further on is not established by
+// walking to the chain's end - in a table with many tombstones that end is far away - but
+// through the home bucket's displacement map: a key with this home can only sit at a marked
+// displacement, so the marked buckets beyond the chosen slot are looked at and then the slot is
+// claimed.  (Without removals there are none: the first free slot is the chain's end.)
 //
 // `src(i, key, val)` produces row i: 0 = insert key -> val, 1 = the row addresses nothing inside
 // the table's coordinate space (counted, reported as not stored), 2 = skip the row silently.
@@ -492,8 +498,11 @@ __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 nex
   bool act = false;
   u64 sk = 0, val = 0;
   i64 idx = 0;
-  u32 home = 0, d = 0, tomb_d = DOK_NONE32, md_home = 0;
-  int tomb_s = 0;
+  u32 home = 0, d = 0, md_home = 0, far_home = 0;
+  // once the walk has met a free slot: the slot, and what is left to look at before the claim
+  bool chosen = false, slot_tomb = false;
+  u32 slot_d = 0, cd = 0, chk = 0, far_next = 0, far_to = 0;
+  int slot_s = 0;
 
   for (;;) {
     // ---- lanes without a row take the next rows of the wave's share
@@ -513,7 +522,7 @@ __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 nex
             n_fresh += p8_side_set(t, sk, val);
             if (stored) stored[i] = 1;
           } else {
-            act = true; idx = i; home = p8_home(sk, t); d = 0; tomb_d = DOK_NONE32;
+            act = true; idx = i; home = p8_home(sk, t); d = 0; chosen = false;
           }
         }
       }
@@ -525,13 +534,15 @@ __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 nex
       continue;
     }
 
-    // ---- one pass: the current bucket of every row
+    // ---- one pass: the current bucket of every row (the next bucket of its walk, or - once it
+    // has chosen a slot - the next bucket its home marks beyond that slot)
+    const u32 dcur = chosen ? cd : d;
     u32 b = 0;
     if (act) {
-      const u64 bb = (u64)home + d;
+      const u64 bb = (u64)home + dcur;
       b = (u32)(bb >= nb ? bb - nb : bb);
     }
-    u32 gm = 0, ge = 0, gt = 0, md = 0;
+    u32 gm = 0, ge = 0, gt = 0, md = 0, mh = 0;
     const u64 actm = dok_ballot(act);
     const u32 rows_on = L.group(actm);               // lanes without a row load nothing
     u32 rounds_on = (u32)actm | (u32)(actm >> 32);   // rounds in which no group has a row are skipped
@@ -555,58 +566,73 @@ __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 nex
         P8Probe<V> pr;
         pr.match(L, w[u], q);
         pr.tombs(L, w[u]);
-        const u32 m = dok_shfl32((u32)w[u], gbase + DOK_P8_META);
+        const u64 mw = dok_shfl64(w[u], gbase + DOK_P8_META);
         const bool mine = l == r;
         gm = mine ? pr.gm : gm;
         ge = mine ? pr.ge : ge;
         gt = mine ? pr.gt : gt;
-        md = mine ? m : md;
+        md = mine ? (u32)mw : md;
+        mh = mine ? (u32)(mw >> 32) : mh;
         DOK_SCHED_FENCE();
       }
     }
 
     // ---- the owners act together
     if (act) {
-      int st = -1;                                   // -1 the row walks on, 0 failed, 1 stored
-      const int start = p8_slot_start<V>(sk);
-      if (d == 0) md_home = md;
+      int st = -1;                                   // -1 the row goes on, 0 failed, 1 stored
+      bool claim = false;
       if (gm) {
         P8<V>::store(buckets + (u64)b * 16, __builtin_ctz(gm), val);
         st = 1;
-      } else {
-        if (tomb_d == DOK_NONE32 && gt) { tomb_d = d; tomb_s = p8_pick(gt, start); }
-        const bool ring_done = (ge == 0) && ((u64)d + 1 >= nb);
-        if (ge || ring_done) {
-          if (tomb_d == DOK_NONE32 && ge == 0) {
-            st = 0;                                  // no free slot anywhere
-          } else {
-            u32 td; int ts; u64 expect;
-            if (tomb_d != DOK_NONE32) { td = tomb_d; ts = tomb_s; expect = DOK_P8_TOMB; }
-            else { td = d; ts = p8_pick(ge, start); expect = DOK_P8_EMPTY; }
-            const u64 tbb = (u64)home + td;
-            u64 *tp = buckets + (tbb >= nb ? tbb - nb : tbb) * 16;
-            const u64 old = atomicCAS(tp + ts, expect, sk);
-            if (old == expect) {
-              P8<V>::store(tp, ts, val);
-              u64 *hb = buckets + (u64)home * 16;
-              if (td >= 32) {
-                atomicMax((u32 *)(hb + DOK_P8_META) + 1, td);
-                if (!(md_home & 1u)) atomicOr((u32 *)(hb + DOK_P8_META), 1u);
-              } else if (td > 0 && !((md_home >> td) & 1u)) {
-                atomicOr((u32 *)(hb + DOK_P8_META), 1u << td);
-              }
-              st = 1; n_fresh++;
-            } else if (old == sk) {
-              st = 1;                                // an equal key of this batch won the slot
-            } else {
-              // somebody else's key took the slot.  Every bucket before the slot's own held
-              // neither a free slot nor this key when the row passed it, and buckets only fill up,
-              // so the row need not go back further than that bucket
-              d = td; tomb_d = DOK_NONE32;
-            }
-          }
+      } else if (!chosen) {
+        if (d == 0) { md_home = md; far_home = mh; }
+        if (gt | ge) {
+          // The first free slot of the walk is the row's place (a tombstone of the bucket before
+          // an EMPTY slot).  The key may still sit further on: exactly at the displacements the
+          // home bucket marks, so those beyond this bucket are looked at before the claim.
+          const int start = p8_slot_start<V>(sk);
+          chosen = true;
+          slot_tomb = gt != 0;
+          slot_d = d;
+          slot_s = p8_pick(gt ? gt : ge, start);
+          chk = d < 31 ? (md_home & ~((2u << d) - 1u)) : 0u;
+          far_next = d + 1 > 32u ? d + 1 : 32u;
+          far_to = (md_home & 1u) ? far_home : 0u;
+        } else if ((u64)d + 1 >= nb) {
+          st = 0;                                    // no free slot anywhere
         } else {
           d++;
+        }
+      }
+      if (st < 0 && chosen) {
+        if (chk) { cd = (u32)__builtin_ctz(chk); chk &= chk - 1; }
+        else if (far_next <= far_to) cd = far_next++;
+        else claim = true;
+      }
+      if (claim) {
+        const u32 td = slot_d;
+        const u64 expect = slot_tomb ? DOK_P8_TOMB : DOK_P8_EMPTY;
+        const u64 tbb = (u64)home + td;
+        u64 *tp = buckets + (tbb >= nb ? tbb - nb : tbb) * 16;
+        const u64 old = atomicCAS(tp + slot_s, expect, sk);
+        if (old == expect) {
+          P8<V>::store(tp, slot_s, val);
+          u64 *hb = buckets + (u64)home * 16;
+          if (td >= 32) {
+            atomicMax((u32 *)(hb + DOK_P8_META) + 1, td);
+            if (!(md_home & 1u)) atomicOr((u32 *)(hb + DOK_P8_META), 1u);
+          } else if (td > 0 && !((md_home >> td) & 1u)) {
+            atomicOr((u32 *)(hb + DOK_P8_META), 1u << td);
+          }
+          st = 1; n_fresh++;
+        } else if (old == sk) {
+          st = 1;                                    // an equal key of this batch won the slot
+        } else {
+          // somebody else's key took the slot.  Every bucket before the slot's own held
+          // neither a free slot nor this key when the row passed it, and buckets only fill up,
+          // so the row need not go back further than that bucket
+          chosen = false;
+          d = td;
         }
       }
       if (st >= 0) {
