@@ -516,3 +516,33 @@ def test_calls_replay_inside_a_hip_graph(cuda):
         assert torch.equal(ef, found) and torch.equal(ev[ef], values[found])
         assert hm.n_elements == ref.n_elements
         _assert_same_map(hm, ref)
+
+
+@pytest.mark.parametrize("capacity", [150, 3000, 20000])
+def test_keys_beyond_freed_slots_are_overwritten_not_duplicated(cuda, capacity):
+    """At 95 % load many keys sit buckets past their home.  Removing other keys leaves tombstones
+    in front of them; a later set of such a key meets a free slot before it reaches the key and
+    must still find the key (through the home bucket's displacement map), not store it twice.
+    Three rounds of remove / overwrite / re-insert with equal keys in the batches."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(capacity)
+    n = int(capacity * 0.95)
+    keys = _unique_i64(rng, n)[:, None]
+    vals = rng.integers(-1000, 1000, size=(n, 1)).astype(np.int32)
+    hm = CudaClosedHashmap(n_buckets=capacity, device=cuda, rehash_threshold=1.0)
+    ref = RefClosedHashmap(n_buckets=capacity, rehash_threshold=1.0, rng=np.random.default_rng(1))
+    hm.set(*_to(cuda, keys, vals)); ref.set(keys, vals)
+    for rnd in range(3):
+        gone = keys[rng.permutation(n)[: n // 2]]
+        m = hm.remove(torch.from_numpy(gone).to(cuda))
+        assert np.array_equal(m.cpu().numpy(), ref.remove(gone))
+        # every key again, each twice with the same value: half are overwrites of keys that now
+        # have tombstones in front of them, half go back into tombstones
+        again = np.concatenate([keys, keys])[rng.permutation(2 * n)]
+        v2 = ((again * 7 + rnd) % 1000).astype(np.int32)
+        hm.set(*_to(cuda, again, v2)); ref.set(again, v2)
+        assert hm.n_elements == ref.n_elements == n
+        _assert_same_map(hm, ref)
+        ks, _ = hm.items()
+        assert np.unique(ks.cpu().numpy()).shape[0] == n       # no key in two slots
+        _check_get(hm, ref, keys, cuda, fallback=0)
