@@ -18,9 +18,10 @@
 //   3. one workgroup per range copies the range's buckets into LDS, places the range's rows
 //      there and streams the buckets back (a table that holds nothing yet is not read: the
 //      copy starts empty, and the clear of the table is saved as well);
-//   4. the few rows the merge cannot place within the ranges of one workgroup (chains that run
-//      into a range another workgroup owns, overflow of the per-range lists) are handed,
-//      packed, to the ordinary insert, which runs last.
+//   4. rows whose chain runs out of a workgroup's block of ranges are placed in the next block's
+//      first ranges by a small follow-up kernel, once those ranges are final;
+//   5. the handful of rows left (overflow of the per-range lists, keys that may sit at far
+//      displacements) are handed, packed, to the ordinary insert, which runs last.
 //
 // Every step is exact for any input: bin sizes are counted, not estimated, and a batch whose
 // rows all fall into one range merely degrades to step 4's ordinary insert.
@@ -84,6 +85,7 @@ struct BulkWs {
   u32 *part_off;            // [n_big * SUB + 1]  start of every range in keysB
   u32 *def_cnt;             // [GRID] rows each merge workgroup handed to the ordinary insert
   u32 *meta_cnt;            // [GRID] displacement marks each merge workgroup left to be applied
+  u32 *edge_cnt;            // [GRID] rows each merge workgroup could not place in the last range of its block
   u32 n_big, n_part;
   u32 g1;                   // workgroups of the first pass (a multiple of 64, at most DOK_BULK_GRID)
   u32 ch;                   // stretches (workgroups) per first-level bin in the second pass
@@ -483,6 +485,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   __shared__ u32 n_carry;           // listed rows whose chain ran on into the next range
   __shared__ u32 n_meta;            // displacement marks noted down for the kernel after the merge
   __shared__ u32 range_live;        // the current range's buckets hold something (a key, a tombstone, a mark)
+  __shared__ u32 n_edge;            // rows that leave the block's last range (see bulk_edge_kernel)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   int n_fresh = 0;
@@ -491,8 +494,8 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   const u32 per = (ws.n_part + gridDim.x - 1) / gridDim.x;
   const u32 p_lo = blockIdx.x * per < ws.n_part ? blockIdx.x * per : ws.n_part;
   const u32 p_hi = p_lo + per < ws.n_part ? p_lo + per : ws.n_part;
-  const u32 def_base = ws.part_off[p_lo];
-  if (tid == 0) { n_def = 0; n_carry = 0; n_meta = 0; range_live = 0; }
+  const u32 def_base = ws.part_off[p_lo], blk_end = ws.part_off[p_hi];
+  if (tid == 0) { n_def = 0; n_carry = 0; n_meta = 0; range_live = 0; n_edge = 0; }
   __syncthreads();
 
   for (u32 p = p_lo; p < p_hi; p++) {
@@ -850,7 +853,13 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           else carry = false;                         // n_carry is clamped below
         }
         if (!carry) {
-          const u32 at = def_base + atomicAdd(&n_def, 1u);
+          // Rows that have looked at every bucket their home marks, are the only row of their key
+          // and found no room up to the end of the block's LAST range continue in the next
+          // block's first range: bulk_edge_kernel places them there once this kernel is through.
+          // They are listed from the top of the workgroup's stretch downwards; everything else
+          // goes, from the bottom upwards, to the ordinary insert.
+          const bool edge = p + 1 == p_hi && p_hi < ws.n_part && !beyond && pend == 0 && (lhome >= 0 || lpend[e] == 0);
+          const u32 at = edge ? blk_end - 1 - atomicAdd(&n_edge, 1u) : def_base + atomicAdd(&n_def, 1u);
           ws.keysA[at] = key;
           dok_store_val<V>(ws.valsA, (i64)at, (u64)val);
         }
@@ -901,6 +910,130 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
     if (sum) atomicAdd((u64 *)&t.header[DOK_H_NELEM], (u64)(i64)sum);
     ws.def_cnt[blockIdx.x] = n_def;
     ws.meta_cnt[blockIdx.x] = n_meta;
+    ws.edge_cnt[blockIdx.x] = n_edge;
+  }
+}
+
+// ---- rows that left a block's last range ------------------------------------------------------------
+// Launched with the merge kernel's grid, after it.  Workgroup w takes the rows merge workgroup w
+// listed as leaving the last range of its block - new keys, one row each, with no free slot from
+// their home bucket to the block's end - and places them in the next block's first range (and the
+// one after, if the blocks are that long), whose buckets are final by now: the same bitmap and
+// tickets as in the merge, on an LDS copy of the range.  The workgroups touch disjoint ranges.
+// Rows that find no room there either join the rows for the ordinary insert.
+template <int V>
+__global__ __launch_bounds__(DOK_BULK_R) void bulk_edge_kernel(DevTable t, BulkWs ws) {
+  typedef typename ValT<V>::type VT;
+  constexpr int S = P8<V>::S;
+  constexpr int R = DOK_BULK_R;
+  constexpr int LD = R + 1;
+  __shared__ u64 tb[16 * LD];
+  __shared__ u32 tickets[R], fmask[R], freemap[R / 32];
+  __shared__ u32 n_left, n_note, n_a;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const u32 per = (ws.n_part + gridDim.x - 1) / gridDim.x;
+  const u32 p_lo = blockIdx.x * per < ws.n_part ? blockIdx.x * per : ws.n_part;
+  const u32 p_hi = p_lo + per < ws.n_part ? p_lo + per : ws.n_part;
+  const u32 n_rows = ws.edge_cnt[blockIdx.x];
+  // (more rows than threads: left to the ordinary insert, which reads the list as it is)
+  if (n_rows == 0 || n_rows > (u32)R || p_hi >= ws.n_part) return;
+  const u32 def_base = ws.part_off[p_lo], top = ws.part_off[p_hi];
+  const u32 note_base = def_base + ws.meta_cnt[blockIdx.x], a_base = def_base + ws.def_cnt[blockIdx.x];
+  bool have = (u32)tid < n_rows;
+  u64 key = 0, sk = 0, home = 0;
+  VT val = 0;
+  if (have) {
+    key = ws.keysA[top - 1 - tid];
+    val = (VT)dok_load_val<V>(ws.valsA, (i64)(top - 1 - tid));
+    sk = key ^ DOK_P8_XOR;
+    home = p8_home(sk, t);
+  }
+  if (tid == 0) { n_note = 0; n_a = 0; }
+  int n_fresh = 0;
+  const u32 guests = per < 2 ? per : 2;
+  for (u32 gi = 0; gi < guests && p_hi + gi < ws.n_part; gi++) {
+    const u32 p = p_hi + gi;
+    const u64 b0 = (u64)p << DOK_BULK_RLOG;
+    const u64 left = t.nb - b0;
+    const u32 nbk = left < (u64)R ? (u32)left : (u32)R;
+    ulonglong2 *g = (ulonglong2 *)(t.buckets + b0 * 16);
+    for (u32 u = tid; u < nbk * 8; u += R) {
+      const ulonglong2 x = g[u];
+      const u32 lb = u >> 3, w = (u & 7) * 2;
+      tb[w * LD + lb] = x.x; tb[(w + 1) * LD + lb] = x.y;
+    }
+    if (tid == 0) n_left = 0;
+    __syncthreads();
+    {
+      u32 ge = 0, gt = 0;
+      if ((u32)tid < nbk) {
+        #pragma unroll
+        for (int s = 0; s < S; s++) {
+          const u64 w = tb[s * LD + tid];
+          ge |= (u32)(w == DOK_P8_EMPTY) << s;
+          gt |= (u32)(w == DOK_P8_TOMB) << s;
+        }
+      }
+      fmask[tid] = ge | (gt << 16);
+      const int nfree = __popc(ge) + __popc(gt);
+      tickets[tid] = (u32)nfree;
+      const u64 fm = dok_ballot(nfree != 0);
+      if (lane == 0) { freemap[(tid >> 6) * 2] = (u32)fm; freemap[(tid >> 6) * 2 + 1] = (u32)(fm >> 32); }
+    }
+    __syncthreads();
+    if (have) {
+      u32 from = 0;
+      while (true) {
+        u32 T = DOK_NONE32;
+        for (u32 wi = from >> 5; wi < (u32)(R / 32); wi++) {
+          u32 m = ((volatile u32 *)freemap)[wi];
+          if (wi == (from >> 5)) m &= ~0u << (from & 31);
+          if (m) { T = wi * 32 + (u32)__builtin_ctz(m); break; }
+        }
+        if (T == DOK_NONE32) break;
+        const int ticket = atomicSub((int *)&tickets[T], 1);
+        if (ticket <= 1) atomicAnd(&freemap[T >> 5], ~(1u << (T & 31)));
+        if (ticket <= 0) { from = T + 1; continue; }
+        const u32 fm = fmask[T], ge = fm & 0xffffu, gt = fm >> 16;
+        const u32 nt = __popc(gt);
+        const u32 k = nt + __popc(ge) - (u32)ticket;
+        const int ts = k < nt ? bulk_nth_bit(gt, k) : bulk_nth_bit(ge, k - nt);
+        tb[ts * LD + T] = sk;
+        *(VT *)((char *)(tb + (S + ((ts * V) >> 3)) * LD + T) + ((ts * V) & 7)) = val;
+        // the displacement mark belongs to a bucket of another range: noted for the kernel that follows
+        const u64 td = b0 + T - home;
+        ws.keysB[note_base + atomicAdd(&n_note, 1u)] = (home << 32) | td;
+        n_fresh++;
+        have = false;
+        break;
+      }
+      if (have) atomicAdd(&n_left, 1u);
+    }
+    __syncthreads();
+    for (u32 u = tid; u < nbk * 8; u += R) {
+      const u32 lb = u >> 3, w = (u & 7) * 2;
+      ulonglong2 y;
+      y.x = tb[w * LD + lb];
+      y.y = tb[(w + 1) * LD + lb];
+      g[u] = y;
+    }
+    const u32 still = n_left;
+    __syncthreads();
+    if (still == 0) break;
+  }
+  // what is left joins the rows for the ordinary insert (the list above has been read in full, so
+  // its place may be written over)
+  if (have) {
+    const u32 at = a_base + atomicAdd(&n_a, 1u);
+    ws.keysA[at] = key;
+    dok_store_val<V>(ws.valsA, (i64)at, (u64)val);
+  }
+  dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
+  __syncthreads();
+  if (tid == 0) {
+    ws.def_cnt[blockIdx.x] += n_a;
+    ws.meta_cnt[blockIdx.x] += n_note;
+    ws.edge_cnt[blockIdx.x] = 0;
   }
 }
 
@@ -920,7 +1053,11 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
     if (td >= 32) { atomicMax(meta + 1, td); atomicOr(meta, 1u); }
     else atomicOr(meta, 1u << td);
   }
-  const i64 n = ws.def_cnt[blockIdx.x];
+  // the rows from the bottom of the stretch, and - if bulk_edge_kernel has not taken them - the
+  // rows listed from its top downwards
+  const u32 p_hi = p_lo + per < ws.n_part ? p_lo + per : ws.n_part;
+  const i64 top = ws.part_off[p_hi];
+  const i64 n_a = ws.def_cnt[blockIdx.x], n = n_a + ws.edge_cnt[blockIdx.x];
   const i64 waves = DOK_TPB / 64, wave = threadIdx.x >> 6;
   const i64 share = (n + waves - 1) / waves;
   i64 lo = wave * share, hi = lo + share;
@@ -928,9 +1065,10 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
   if (lo > hi) lo = hi;
   const u64 *keys = ws.keysA;
   const void *vals = ws.valsA;
-  p8_stream_insert_rows<V>(t, base + lo, base + hi, nullptr, [&](i64 i, u64 &key, u64 &val) -> int {
-    key = keys[i];
-    val = dok_load_val<V>(vals, i);
+  p8_stream_insert_rows<V>(t, lo, hi, nullptr, [&](i64 i, u64 &key, u64 &val) -> int {
+    const i64 at = i < n_a ? base + i : top - 1 - (i - n_a);
+    key = keys[at];
+    val = dok_load_val<V>(vals, at);
     return 0;
   });
 }
@@ -939,7 +1077,7 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
 struct BulkPlan {
   u32 n_part, n_big, ch, g1, gm;
   i64 share;
-  size_t o_keysA, o_keysB, o_valsA, o_valsB, o_wg_hist, o_big_off, o_sub_hist, o_part_off, o_def_cnt, o_meta_cnt, bytes;
+  size_t o_keysA, o_keysB, o_valsA, o_valsB, o_wg_hist, o_big_off, o_sub_hist, o_part_off, o_def_cnt, o_meta_cnt, o_edge_cnt, bytes;
 };
 
 static inline size_t bulk_align(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -978,6 +1116,7 @@ static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p, u32 g1 = DOK_BULK_G
   p.o_part_off = o; o = bulk_align(o + 4 * (parts + 1));
   p.o_def_cnt = o; o = bulk_align(o + 4 * DOK_BULK_GRID);
   p.o_meta_cnt = o; o = bulk_align(o + 4 * DOK_BULK_GRID);
+  p.o_edge_cnt = o; o = bulk_align(o + 4 * DOK_BULK_GRID);
   p.bytes = o;
   return true;
 }
@@ -994,6 +1133,7 @@ static void bulk_bind(const BulkPlan &p, void *workspace, BulkWs &ws) {
   ws.part_off = (u32 *)(w + p.o_part_off);
   ws.def_cnt = (u32 *)(w + p.o_def_cnt);
   ws.meta_cnt = (u32 *)(w + p.o_meta_cnt);
+  ws.edge_cnt = (u32 *)(w + p.o_edge_cnt);
   ws.n_big = p.n_big;
   ws.n_part = p.n_part;
   ws.g1 = p.g1;
@@ -1062,5 +1202,6 @@ static void bulk_launch(const DevTable &d, const void *keys, const void *values,
   bulk_scan2_kernel<<<p.n_big, DOK_BULK_SUB, 0, s>>>(ws);
   bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
   bulk_merge_kernel<V, FRESH><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
+  if (p.gm > 1) bulk_edge_kernel<V><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
   bulk_deferred_kernel<V><<<p.gm, DOK_TPB, 0, s>>>(d, ws);
 }
