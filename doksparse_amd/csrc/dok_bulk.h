@@ -441,8 +441,8 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
 // once, without walking their chains: lookup through the home bucket's displacement map, one row
 // per key through a small hash set, free slots through a bitmap and per-bucket tickets (see
 // there).  Rows that find no room up to the range's last bucket move on to the next range of the
-// same workgroup; rows that found no room on the list, and a few awkward cases, are handed to the
-// ordinary insert.
+// same workgroup, or - out of the block's last range - to bulk_edge_kernel; rows that found no
+// room on the list, and a few awkward cases, are handed to the ordinary insert.
 #ifndef DOK_BULK_C
 #define DOK_BULK_C (6 * DOK_BULK_R)
 #endif
