@@ -608,6 +608,25 @@ class SparseDOKTensor(object):
                 y = y.unsqueeze(d)
         return y.sqrt() if p == 2 else y.pow(1.0 / p) if p not in (0, 1) else y
 
+    def normalize(self, dim=-1, p=2, eps=1e-12):
+        """Stored magnitudes divided by the p-norm of their slice along `dim`, as a sparse COO
+        tensor (reference: sparse_dok_tensor.py:405-411 through functions.py:123-161, which takes
+        the softmax of log |v|^p over the stored entries - signs are not kept - and the 1/p-th
+        power of the result; entries with |v|^p below eps count as eps)."""
+        coo = self.to_sparse_coo().coalesce()
+        v = coo.values()
+        powered = v.bool().to(v.dtype) if p == 0 else v.abs() if p == 1 else v.square() if p == 2 else v.abs().pow(p)
+        logs = powered.clamp_min(eps).log()
+        t = torch.sparse_coo_tensor(coo.indices(), logs, size=tuple(self.shape), device=self.device)
+        y = torch.sparse.softmax(t, dim=dim % self.ndim)
+        return y.sqrt() if p == 2 else y.pow(1.0 / p)
+
+    def normalize_(self, dim=-1, p=2, eps=1e-12):
+        """The reference's in-place variant works on the temporary COO copy it makes of the tensor
+        (sparse_dok_tensor.py:413-419), so the DOK tensor keeps its values and the normalised COO
+        tensor is what the caller gets; the same here."""
+        return self.normalize(dim=dim, p=p, eps=eps)
+
     def softmax(self, dim=-1):
         return torch.sparse.softmax(self.to_sparse_coo().coalesce(), dim=dim % self.ndim)
 

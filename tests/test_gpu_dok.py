@@ -407,3 +407,40 @@ def test_repeated_mask_selectors_follow_in_place_changes(cuda):
         m2[[k, (k + 5) % 16]] = True
         assert torch.equal(dok[rows[:, None], m2].cpu(), dense[rows.cpu()[:, None], m2.cpu()])
         del m2
+
+
+def test_reductions_and_elementwise_glue(cuda):
+    """The methods that stay torch glue over the read-out (reference: sparse_dok_tensor.py:352-561):
+    sum, norm, normalize, softmax, log_softmax, index_select, select and the element-wise maps,
+    against the same operations on the dense tensor (softmax and normalize run over the stored
+    entries only, as torch.sparse does)."""
+    from doksparse_amd import SparseDOKTensor
+    gen = torch.Generator(device="cpu"); gen.manual_seed(9)
+    dense = torch.zeros(40, 30)
+    mask = torch.rand(40, 30, generator=gen) < 0.3
+    dense[mask] = torch.randn(int(mask.sum()), generator=gen) * 3
+    dok = SparseDOKTensor.from_dense(dense.to(cuda))
+    assert torch.allclose(dok.sum().cpu(), dense.sum(), atol=1e-4)
+    assert torch.allclose(dok.sum(dim=1).to_dense().cpu(), dense.sum(dim=1), atol=1e-4)
+    for p in (1, 2, 3):
+        assert torch.allclose(dok.norm(dim=1, p=p).cpu(), dense.norm(dim=1, p=p), atol=1e-4)
+        n = dok.normalize(dim=1, p=p).to_dense().cpu()
+        expect = dense.abs() / dense.norm(dim=1, p=p, keepdim=True).clamp_min(1e-30)
+        assert torch.allclose(n, expect, atol=1e-5)
+        assert torch.allclose(dok.normalize_(dim=1, p=p).to_dense().cpu(), expect, atol=1e-5)
+    assert torch.equal(dok.to_dense().cpu(), dense)                       # normalize_ leaves the tensor alone
+    sm = dok.softmax(dim=1).to_dense().cpu()
+    e = torch.where(mask, dense.exp(), torch.zeros(()))
+    assert torch.allclose(sm, e / e.sum(dim=1, keepdim=True).clamp_min(1e-30), atol=1e-5)
+    lsm = dok.log_softmax(dim=1).coalesce()
+    assert torch.allclose(lsm.values().cpu().exp(), sm[tuple(lsm.indices().cpu())], atol=1e-5)
+    idx = torch.tensor([3, 0, 17], device=cuda)
+    assert torch.equal(dok.index_select(0, idx).to_dense().cpu(), dense[idx.cpu()])
+    assert torch.equal(dok.select(1, 4).to_dense().cpu(), dense[:, 4])
+    assert torch.equal(dok.abs().to_dense().cpu(), dense.abs())
+    assert torch.equal(dok.ceil().to_dense().cpu(), dense.ceil())
+    assert torch.equal(dok.floor().to_dense().cpu(), dense.floor())
+    assert torch.equal(dok.round().to_dense().cpu(), dense.round())
+    assert torch.allclose(dok.abs().sqrt().to_dense().cpu(), dense.abs().sqrt())
+    assert torch.equal(dok.flatten().to_dense().cpu(), dense.flatten())
+    assert torch.equal(dok.reshape(20, 60).to_dense().cpu(), dense.reshape(20, 60))
