@@ -311,7 +311,7 @@ def test_bulk_rehash_of_a_coordinate_keyed_tensor(cuda, bulk_always):
 
 
 def test_bulk_and_per_row_insert_agree_on_random_configurations(cuda, monkeypatch):
-    """Twelve random configurations (size, load factor up to 0.97, share of repeated keys, value
+    """Twenty-four random configurations (size, load factor up to 0.97, share of repeated keys, value
     width): three batches each with removals in between, once through the per-row kernel and once
     through the bulk path.  Values are a function of key and batch number, so the resulting map
     is unique and must be the same (which the oracle pins for the per-row path elsewhere)."""
@@ -326,7 +326,7 @@ def test_bulk_and_per_row_insert_agree_on_random_configurations(cuda, monkeypatc
             return ((x % 201) - 100).to(dt)
         return x.to(dt)
 
-    for case in range(12):
+    for case in range(24):
         n = int(10 ** rng.uniform(3, 6.2))
         lf = float(rng.uniform(0.2, 0.97))
         dt = [torch.float32, torch.int64, torch.float16, torch.int8][case % 4]
