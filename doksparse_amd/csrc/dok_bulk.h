@@ -24,7 +24,7 @@
 //      displacements) are handed, packed, to the ordinary insert, which runs last.
 //
 // Every step is exact for any input: bin sizes are counted, not estimated, and a batch whose
-// rows all fall into one range merely degrades to step 4's ordinary insert.
+// rows all fall into one range merely degrades to step 5's ordinary insert.
 #pragma once
 #include "dok_packed8.h"
 

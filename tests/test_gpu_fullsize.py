@@ -204,3 +204,82 @@ def test_cfg3_full_size_int64_to_float32(cuda, load_factor):
     assert hm.n_elements == n - n // 2 + n // 4
     model = SortedMap(torch.cat([keys[n // 2:], back]), torch.cat([values[n // 2:], values[: n // 4]]))
     assert check(keys) == n - n // 2 + n // 4
+
+
+def test_table_beyond_four_gib(cuda, monkeypatch):
+    """A table of 7 GiB: bucket byte offsets pass 2^32 (the reference's kernels index with 32-bit
+    ints, closed_hashmap_impl.cu:72).  Per-row insert, bulk upsert on top, get, removal and
+    read-out are checked through closed forms: key i is i times an odd constant (a bijection of
+    the 64-bit integers, so the keys are distinct) and its value is i mod 2^24."""
+    from doksparse_amd import CudaClosedHashmap
+    from doksparse_amd import closed_hashmap as ch
+    odd = -7046029254386353131                              # 0x9E3779B97F4A7C15 as int64
+    def rows(lo, hi):
+        i = torch.arange(lo, hi, device=cuda, dtype=torch.long)
+        return (i * odd)[:, None], (i % (1 << 24)).float()[:, None]
+
+    capacity = 560_000_000
+    hm = CudaClosedHashmap(n_buckets=capacity, device=cuda, rehash_threshold=1.0)
+    n1, n2, n_miss = 30_000_000, 150_000_000, 20_000_000
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS", 1 << 62)      # first batch: the per-row kernel
+    k1, v1 = rows(0, n1)
+    hm.set(k1, v1)
+    assert hm._n_phys * 128 > 6 * 2**30
+    assert hm.n_elements == n1
+    got, found = hm.get(k1)
+    assert bool(found.all()) and torch.equal(got, v1)
+    del got, found
+
+    # second batch through the bulk path: the last third of the first batch again (new values)
+    # and n2 new keys
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS", 0)
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS_PER_BUCKET", 0.0)
+    k2, v2 = rows(n1 - n1 // 3, n1 + n2)
+    v2 += 1.0
+    assert hm._bulk_workspace(k2.shape[0]) is not None
+    hm.set(k2, v2)
+    total = n1 + n2
+    assert hm.n_elements == total
+    got, found = hm.get(k2)
+    assert bool(found.all()) and torch.equal(got, v2)
+    del got, found
+    head = n1 - n1 // 3
+    got, found = hm.get(k1[:head])
+    assert bool(found.all()) and torch.equal(got, v1[:head])
+    km, _ = rows(total, total + n_miss)
+    got, found = hm.get(km)
+    assert not bool(found.any()) and not bool(got.any())
+    del got, found, km
+
+    # read-out: every key once (the wrapped sum of the keys is a checksum of the set)
+    ks = hm.keys()
+    assert ks.shape[0] == total
+    i_sum = total * (total - 1) // 2
+    expect = (i_sum * odd) % (1 << 64)
+    assert int(ks.sum()) % (1 << 64) == expect
+    del ks
+
+    # removal of the first batch's head, then those keys are gone and the rest is there
+    gone = hm._remove_rows(k1[:head].contiguous())
+    assert bool(gone.all()) and hm.n_elements == total - head
+    assert not bool(hm.get(k1[:head])[1].any())
+    assert bool(hm.get(k2[-n_miss:])[1].all())
+
+
+def test_table_beyond_the_bulk_limit_takes_the_per_row_kernel(cuda, monkeypatch):
+    """More than 2^26 buckets: the bulk path declines (its two partition levels address at most
+    1024 x 256 ranges), and a batch that would otherwise qualify is inserted row by row."""
+    from doksparse_amd import CudaClosedHashmap
+    from doksparse_amd import closed_hashmap as ch
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS", 0)
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS_PER_BUCKET", 0.0)
+    hm = CudaClosedHashmap(n_buckets=700_000_000, device=cuda, rehash_threshold=1.0)
+    n = 20_000_000
+    i = torch.arange(n, device=cuda, dtype=torch.long)
+    keys, values = (i * -7046029254386353131)[:, None], (i % (1 << 24)).float()[:, None]
+    hm.set(keys, values)
+    assert hm._n_phys > 2**26 and hm._bulk_workspace(n) is None
+    assert hm.n_elements == n
+    got, found = hm.get(keys)
+    assert bool(found.all()) and torch.equal(got, values)
+    assert not bool(hm.get(keys + 1)[1].any())
