@@ -8,7 +8,7 @@
 //
 //   1. the table is cut into ranges of DOK_BULK_R consecutive buckets; the range of a row is
 //      (home bucket) / DOK_BULK_R;
-//   2. two count + scan + scatter passes (first by range / DOK_BULK_SUB, then by range inside
+//   2. two count + scan + scatter passes (first by range / 256 (range / 1024 for very large tables), then by range inside
 //      each first-level bin) move every (key, value) row next to the other rows of its range.
 //      Every workgroup of a scatter owns a fixed stretch of the input; the count pass records how
 //      many of that stretch's rows go to each bin, a prefix sum over the workgroups turns the
@@ -32,8 +32,8 @@
 #define DOK_BULK_RLOG 8                     // log2 of the buckets per range: 256 buckets = 32 KiB
 #endif
 #define DOK_BULK_R (1 << DOK_BULK_RLOG)
-#define DOK_BULK_SUBLOG 8
-#define DOK_BULK_SUB (1 << DOK_BULK_SUBLOG) // ranges per first-level bin
+#define DOK_BULK_SUBLOG 8                   // log2 of the ranges per first-level bin ...
+#define DOK_BULK_SUBLOG_WIDE 10             // ... and for tables of more than 1024 << 8 ranges
 #define DOK_BULK_MAXBIG 1024                // first-level bins at most
 #ifndef DOK_BULK_TPB
 #define DOK_BULK_TPB 512
@@ -81,12 +81,13 @@ struct BulkWs {
   u32 *wg_hist;             // [n_big][GRID]: rows of workgroup w's stretch that go to first-level bin b;
                             //                after the scan, the exclusive prefix sum over w
   u32 *big_off;             // [n_big + 1]    start of every first-level bin in keysA
-  u32 *sub_hist;            // [n_big][SUB][ch]: the same for the ch stretches of a first-level bin
-  u32 *part_off;            // [n_big * SUB + 1]  start of every range in keysB
+  u32 *sub_hist;            // [n_big << sublog][ch]: the same for the ch stretches of a first-level bin
+  u32 *part_off;            // [(n_big << sublog) + 1]  start of every range in keysB
   u32 *def_cnt;             // [GRID] rows each merge workgroup handed to the ordinary insert
   u32 *meta_cnt;            // [GRID] displacement marks each merge workgroup left to be applied
   u32 *edge_cnt;            // [GRID] rows each merge workgroup could not place in the last range of its block
   u32 n_big, n_part;
+  u32 sublog;               // log2 of the ranges per first-level bin
   u32 g1;                   // workgroups of the first pass (a multiple of 64, at most DOK_BULK_GRID)
   u32 ch;                   // stretches (workgroups) per first-level bin in the second pass
   i64 share;                // rows per workgroup in the first pass
@@ -182,7 +183,7 @@ __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count1_kernel(DevTable t, 
     #pragma unroll
     for (int u = 0; u < 8; u++)
       if (ok[u] && (key[u] ^ DOK_P8_XOR) >= 2)
-        atomicAdd(&cnt[copy + (bulk_range_of(key[u], t) >> DOK_BULK_SUBLOG)], 1u);
+        atomicAdd(&cnt[copy + (bulk_range_of(key[u], t) >> ws.sublog)], 1u);
   }
   __syncthreads();
   for (int b = threadIdx.x; b < (int)ws.n_big; b += DOK_BULK_CTPB)
@@ -210,12 +211,14 @@ __global__ __launch_bounds__(DOK_BULK_MAXBIG) void bulk_scan1b_kernel(BulkWs ws)
 }
 
 // ---- pass 2, count: rows of every stretch of a first-level bin per range -----------------------------
+template <int SL>
 __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count2_kernel(DevTable t, BulkWs ws) {
-  __shared__ u32 cnt[4 * DOK_BULK_SUB];              // four copies, as in the first count
+  constexpr int SUB = 1 << SL;
+  __shared__ u32 cnt[4 * SUB];                       // four copies, as in the first count
   const u32 b = blockIdx.x / ws.ch, c = blockIdx.x % ws.ch;
-  for (int s = threadIdx.x; s < 4 * DOK_BULK_SUB; s += DOK_BULK_CTPB) cnt[s] = 0;
+  for (int s = threadIdx.x; s < 4 * SUB; s += DOK_BULK_CTPB) cnt[s] = 0;
   __syncthreads();
-  const u32 copy = (threadIdx.x & 3) * DOK_BULK_SUB;
+  const u32 copy = (threadIdx.x & 3) * SUB;
   i64 lo, hi;
   bulk_stretch2(ws, b, c, lo, hi);
   for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += 8 * DOK_BULK_CTPB) {
@@ -227,19 +230,21 @@ __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count2_kernel(DevTable t, 
     }
     #pragma unroll
     for (int u = 0; u < 8; u++)
-      if (i0 + u * DOK_BULK_CTPB < hi) atomicAdd(&cnt[copy + (bulk_range_of(key[u], t) & (DOK_BULK_SUB - 1))], 1u);
+      if (i0 + u * DOK_BULK_CTPB < hi) atomicAdd(&cnt[copy + (bulk_range_of(key[u], t) & (SUB - 1))], 1u);
   }
   __syncthreads();
-  for (int s = threadIdx.x; s < DOK_BULK_SUB; s += DOK_BULK_CTPB)
-    ws.sub_hist[((size_t)b * DOK_BULK_SUB + s) * ws.ch + c] =
-        cnt[s] + cnt[DOK_BULK_SUB + s] + cnt[2 * DOK_BULK_SUB + s] + cnt[3 * DOK_BULK_SUB + s];
+  for (int s = threadIdx.x; s < SUB; s += DOK_BULK_CTPB)
+    ws.sub_hist[((size_t)b * SUB + s) * ws.ch + c] =
+        cnt[s] + cnt[SUB + s] + cnt[2 * SUB + s] + cnt[3 * SUB + s];
 }
 
 // ---- pass 2, scan: per range over the stretches, then over the ranges of the bin ---------------------
-__global__ __launch_bounds__(DOK_BULK_SUB) void bulk_scan2_kernel(BulkWs ws) {
+template <int SL>
+__global__ __launch_bounds__(1 << SL) void bulk_scan2_kernel(BulkWs ws) {
+  constexpr int SUB = 1 << SL;
   __shared__ u32 wsum[16];
   const u32 b = blockIdx.x;
-  const size_t idx = (size_t)b * DOK_BULK_SUB + threadIdx.x;
+  const size_t idx = (size_t)b * SUB + threadIdx.x;
   u32 *row = ws.sub_hist + idx * ws.ch;
   u32 run = 0;
   for (u32 c = 0; c < ws.ch; c++) {
@@ -251,12 +256,12 @@ __global__ __launch_bounds__(DOK_BULK_SUB) void bulk_scan2_kernel(BulkWs ws) {
   const u32 ex = bulk_block_scan(run, wsum, total);
   const u32 base = ws.big_off[b];
   ws.part_off[idx] = base + ex;
-  if (b == ws.n_big - 1 && threadIdx.x == DOK_BULK_SUB - 1) ws.part_off[idx + 1] = base + ex + run;
+  if (b == ws.n_big - 1 && threadIdx.x == SUB - 1) ws.part_off[idx + 1] = base + ex + run;
 }
 
 // ---- scatter: LEVEL 1 moves the caller's rows into first-level bins (keysA/valsA), LEVEL 2 moves
 // the rows of each first-level bin into their ranges (keysB/valsB) ---------------------------------
-template <int V, int KF, int LEVEL>
+template <int V, int KF, int LEVEL, int SL = DOK_BULK_SUBLOG>
 __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, const void *__restrict__ keys_in,
                                                                     const void *__restrict__ vals_in, i64 n, BulkWs ws) {
   typedef typename ValT<V>::type VT;
@@ -265,7 +270,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
                                : (V == 8 ? DOK_BULK_T2V8 : V == 4 ? DOK_BULK_T2 : DOK_BULK_T2S);
   static_assert(T % DOK_BULK_TPB == 0, "every thread stages the same number of rows");
   constexpr int RPT = T / DOK_BULK_TPB;
-  constexpr int NB = LEVEL == 1 ? DOK_BULK_MAXBIG : DOK_BULK_SUB;
+  constexpr int NB = LEVEL == 1 ? DOK_BULK_MAXBIG : (1 << SL);
   constexpr int BPT = NB >= DOK_BULK_TPB ? NB / DOK_BULK_TPB : 1;   // consecutive bins per thread
   __shared__ u32 cnt[NB], off[NB], gbase[NB];
   __shared__ u64 skeys[T];
@@ -303,7 +308,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     out_vals = (VT *)ws.valsB;
     #pragma unroll
     for (int q = 0; q < BPT; q++) {
-      const size_t idx = (size_t)b * DOK_BULK_SUB + tid * BPT + q;
+      const size_t idx = (size_t)b * NB + tid * BPT + q;
       cursor[q] = tid * BPT + q < NB ? ws.part_off[idx] + ws.sub_hist[idx * ws.ch + c] : 0u;
     }
   }
@@ -352,7 +357,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
           n_fresh += p8_side_set(t, k[j] ^ DOK_P8_XOR, v[j]);
         } else {
           const u32 r = bulk_range_of(k[j], t);
-          bn[j] = LEVEL == 1 ? (int)(r >> DOK_BULK_SUBLOG) : (int)(r & (DOK_BULK_SUB - 1));
+          bn[j] = LEVEL == 1 ? (int)(r >> ws.sublog) : (int)(r & (NB - 1));
         }
       }
     }
@@ -1075,7 +1080,7 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
 
 // ---- host side -----------------------------------------------------------------------------------
 struct BulkPlan {
-  u32 n_part, n_big, ch, g1, gm;
+  u32 n_part, n_big, sublog, ch, g1, gm;
   i64 share;
   size_t o_keysA, o_keysB, o_valsA, o_valsB, o_wg_hist, o_big_off, o_sub_hist, o_part_off, o_def_cnt, o_meta_cnt, o_edge_cnt, bytes;
 };
@@ -1092,7 +1097,8 @@ static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p, u32 g1 = DOK_BULK_G
   if (n < 1 || n > 0x7fff0000LL) return false;
   p.g1 = g1;
   const u64 n_part = (d.nb + DOK_BULK_R - 1) >> DOK_BULK_RLOG;
-  const u64 n_big = (n_part + DOK_BULK_SUB - 1) >> DOK_BULK_SUBLOG;
+  p.sublog = n_part <= ((u64)DOK_BULK_MAXBIG << DOK_BULK_SUBLOG) ? DOK_BULK_SUBLOG : DOK_BULK_SUBLOG_WIDE;
+  const u64 n_big = (n_part + (1u << p.sublog) - 1) >> p.sublog;
   if (n_big > DOK_BULK_MAXBIG) return false;
   p.n_part = (u32)n_part;
   p.n_big = (u32)n_big;
@@ -1104,7 +1110,7 @@ static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p, u32 g1 = DOK_BULK_G
   const i64 tiles = (n + DOK_BULK_T - 1) / DOK_BULK_T;
   p.share = ((tiles + g1 - 1) / g1) * DOK_BULK_T;
   p.gm = p.n_part < gm ? p.n_part : gm;
-  const size_t parts = (size_t)n_big * DOK_BULK_SUB;
+  const size_t parts = (size_t)n_big << p.sublog;
   size_t o = 0;
   p.o_keysA = o; o = bulk_align(o + 8 * (size_t)n_cap);
   p.o_keysB = o; o = bulk_align(o + 8 * (size_t)n_cap);
@@ -1136,6 +1142,7 @@ static void bulk_bind(const BulkPlan &p, void *workspace, BulkWs &ws) {
   ws.edge_cnt = (u32 *)(w + p.o_edge_cnt);
   ws.n_big = p.n_big;
   ws.n_part = p.n_part;
+  ws.sublog = p.sublog;
   ws.g1 = p.g1;
   ws.ch = p.ch;
   ws.share = p.share;
@@ -1198,9 +1205,15 @@ static void bulk_launch(const DevTable &d, const void *keys, const void *values,
   bulk_scan1b_kernel<<<1, DOK_BULK_MAXBIG, 0, s>>>(ws);
   if (emit) bulk_scatter_kernel<V, COORDS ? DOK_KF_LIN : KF, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, ws.keysB, values, n, ws);
   else bulk_scatter_kernel<V, KF, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, keys, values, n, ws);
-  bulk_count2_kernel<<<p.n_big * p.ch, DOK_BULK_CTPB, 0, s>>>(d, ws);
-  bulk_scan2_kernel<<<p.n_big, DOK_BULK_SUB, 0, s>>>(ws);
-  bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
+  if (p.sublog == DOK_BULK_SUBLOG) {
+    bulk_count2_kernel<DOK_BULK_SUBLOG><<<p.n_big * p.ch, DOK_BULK_CTPB, 0, s>>>(d, ws);
+    bulk_scan2_kernel<DOK_BULK_SUBLOG><<<p.n_big, 1 << DOK_BULK_SUBLOG, 0, s>>>(ws);
+    bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
+  } else {
+    bulk_count2_kernel<DOK_BULK_SUBLOG_WIDE><<<p.n_big * p.ch, DOK_BULK_CTPB, 0, s>>>(d, ws);
+    bulk_scan2_kernel<DOK_BULK_SUBLOG_WIDE><<<p.n_big, 1 << DOK_BULK_SUBLOG_WIDE, 0, s>>>(ws);
+    bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG_WIDE><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
+  }
   bulk_merge_kernel<V, FRESH><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
   if (p.gm > 1) bulk_edge_kernel<V><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
   bulk_deferred_kernel<V><<<p.gm, DOK_TPB, 0, s>>>(d, ws);

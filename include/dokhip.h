@@ -132,7 +132,7 @@ int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int6
  * table is streamed through the GPU once.  Packed layout only.
  *   dok_bulk_workspace_bytes: device bytes dok_map_set_bulk / dok_coo_set_bulk need for n rows;
  *     0 if the bulk path cannot take this table or n (tagged layout, n >= 2^31, more than
- *     2^26 buckets: use dok_map_set), negative on a bad table.
+ *     2^28 buckets: use dok_map_set), negative on a bad table.
  *   workspace: device, 256-byte aligned, at least that many bytes; contents need no
  *     initialisation and are garbage afterwards.  Calls sharing one workspace must be ordered.
  * Reference: the same closed_hashmap_set launch as dok_map_set, at the batch sizes of

@@ -266,19 +266,57 @@ def test_table_beyond_four_gib(cuda, monkeypatch):
     assert bool(hm.get(k2[-n_miss:])[1].all())
 
 
-def test_table_beyond_the_bulk_limit_takes_the_per_row_kernel(cuda, monkeypatch):
-    """More than 2^26 buckets: the bulk path declines (its two partition levels address at most
-    1024 x 256 ranges), and a batch that would otherwise qualify is inserted row by row."""
+def test_bulk_path_with_the_wide_second_level(cuda, monkeypatch):
+    """Between 2^26 and 2^28 buckets the bulk path partitions 1024 ranges per first-level bin
+    instead of 256.  A table of 100M buckets (12.8 GB): bulk build of 200M rows into uninitialised
+    memory, bulk upsert of 50M stored + 50M new keys, then get / read-out checksum / count."""
     from doksparse_amd import CudaClosedHashmap
     from doksparse_amd import closed_hashmap as ch
     monkeypatch.setattr(ch, "BULK_MIN_ROWS", 0)
     monkeypatch.setattr(ch, "BULK_MIN_ROWS_PER_BUCKET", 0.0)
-    hm = CudaClosedHashmap(n_buckets=700_000_000, device=cuda, rehash_threshold=1.0)
+    odd = -7046029254386353131
+    def rows(lo, hi, bump):
+        i = torch.arange(lo, hi, device=cuda, dtype=torch.long)
+        return (i * odd)[:, None], ((i % (1 << 24)).float() + bump)[:, None]
+
+    hm = CudaClosedHashmap(n_buckets=1_000_000_000, device=cuda, rehash_threshold=1.0)
+    n1 = 200_000_000
+    k1, v1 = rows(0, n1, 0.0)
+    hm.set(k1, v1)                                          # build
+    assert 2**26 < hm._n_phys <= 2**28 and hm._bulk_workspace(n1) is not None
+    assert hm.n_elements == n1
+    got, found = hm.get(k1)
+    assert bool(found.all()) and torch.equal(got, v1)
+    del got, found
+    k2, v2 = rows(n1 - 50_000_000, n1 + 50_000_000, 1.0)
+    hm.set(k2, v2)                                          # upsert into the populated table
+    total = n1 + 50_000_000
+    assert hm.n_elements == total
+    got, found = hm.get(k2)
+    assert bool(found.all()) and torch.equal(got, v2)
+    got, found = hm.get(k1[: n1 - 50_000_000])
+    assert bool(found.all()) and torch.equal(got, v1[: n1 - 50_000_000])
+    del got, found
+    assert not bool(hm.get(rows(total, total + 10_000_000, 0.0)[0])[1].any())
+    ks = hm.keys()
+    assert ks.shape[0] == total
+    assert int(ks.sum()) % (1 << 64) == (total * (total - 1) // 2 * odd) % (1 << 64)
+
+
+def test_table_beyond_the_bulk_limit_takes_the_per_row_kernel(cuda, monkeypatch):
+    """More than 2^28 buckets (a table of 36 GB): the bulk path declines (its two partition levels
+    address at most 1024 x 1024 ranges), and a batch that would otherwise qualify is inserted row
+    by row."""
+    from doksparse_amd import CudaClosedHashmap
+    from doksparse_amd import closed_hashmap as ch
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS", 0)
+    monkeypatch.setattr(ch, "BULK_MIN_ROWS_PER_BUCKET", 0.0)
+    hm = CudaClosedHashmap(n_buckets=2_800_000_000, device=cuda, rehash_threshold=1.0)
     n = 20_000_000
     i = torch.arange(n, device=cuda, dtype=torch.long)
     keys, values = (i * -7046029254386353131)[:, None], (i % (1 << 24)).float()[:, None]
     hm.set(keys, values)
-    assert hm._n_phys > 2**26 and hm._bulk_workspace(n) is None
+    assert hm._n_phys > 2**28 and hm._bulk_workspace(n) is None
     assert hm.n_elements == n
     got, found = hm.get(keys)
     assert bool(found.all()) and torch.equal(got, values)
