@@ -120,23 +120,56 @@ __device__ __forceinline__ u32 bulk_range_of(u64 key, const DevTable &t) {
   return p8_home(key ^ DOK_P8_XOR, t) >> DOK_BULK_RLOG;
 }
 
-// Row i of the batch: its key (and, for a table source, whether word i is a live key slot at all).
+// Row i of the batch, in two steps: bulk_fetch only loads, bulk_finish turns what was loaded into
+// the key.  A kernel issues the fetches of all the rows it holds before it finishes any of them,
+// so that their loads are in flight together (a load is not moved across the branch that guards
+// its row, and a use inside that branch would wait for it right there).
+// ND: the number of dimensions of a coordinate source - a compile-time constant, so that no
+// branch separates the loads of one row either; 0 for the other sources.
+template <int KF, int ND> struct BulkRaw { u64 w[ND > 0 ? ND : 1]; };
+
+template <int KF, int ND>
+__device__ __forceinline__ void bulk_fetch(const DevTable &t, const void *keys, i64 i, i64 n, BulkRaw<KF, ND> &r) {
+  if constexpr (KF == DOK_KF_ROWS) {
+    #pragma unroll
+    for (int d = 0; d < ND; d++) r.w[d] = ((const u64 *)keys)[i * ND + d];
+  } else if constexpr (KF == DOK_KF_COLS) {
+    #pragma unroll
+    for (int d = 0; d < ND; d++) r.w[d] = ((const u64 *)keys)[(i64)d * n + i];
+  } else if constexpr (KF == DOK_KF_TABLE) {
+    // word i of the source table's buckets; only the first S words of a bucket are key slots
+    r.w[0] = 0;
+    if ((int)(i & 15) < 120 / (8 + t.value_bytes)) r.w[0] = ((const u64 *)keys)[i];
+  } else if constexpr (KF == DOK_KF_RAW) {
+    dok_load_key8<DOK_KF_RAW>(t, keys, i, n, r.w[0]);
+  } else {
+    r.w[0] = ((const u64 *)keys)[i];                  // DOK_KF_U64, DOK_KF_LIN
+  }
+}
+
 // Returns 1 = row, 0 = no row here, 2 = the row's coordinates lie outside the table.
-template <int KF>
-__device__ __forceinline__ int bulk_load_key(const DevTable &t, const void *keys, i64 i, i64 n, u64 &key) {
-  if (KF == DOK_KF_TABLE) {
-    const int S = 120 / (8 + t.value_bytes);         // slots per bucket of the source (same widths)
-    key = 0;
-    if ((int)(i & 15) >= S) return 0;
-    const u64 w = ((const u64 *)keys)[i];
-    key = w ^ DOK_P8_XOR;
-    return w >= 2 ? 1 : 0;
-  }
-  if (KF == DOK_KF_LIN) {
-    key = ((const u64 *)keys)[i];
+template <int KF, int ND>
+__device__ __forceinline__ int bulk_finish(const DevTable &t, const BulkRaw<KF, ND> &r, u64 &key) {
+  if constexpr (KF == DOK_KF_ROWS || KF == DOK_KF_COLS) {
+    bool ok = true;
+    u64 k = 0;
+    #pragma unroll
+    for (int d = 0; d < ND; d++) {
+      ok &= r.w[d] < (u64)t.lin_dims[d];
+      k += r.w[d] * (u64)t.lin_strides[d];
+    }
+    key = k;
+    return ok ? 1 : 2;
+  } else if constexpr (KF == DOK_KF_TABLE) {
+    key = r.w[0] ^ DOK_P8_XOR;                        // EMPTY, TOMB and the words that are no slots: no row
+    return r.w[0] >= 2 ? 1 : 0;
+  } else if constexpr (KF == DOK_KF_LIN) {
+    key = r.w[0];
     return key == ~0ULL ? 2 : 1;
+  } else {
+    key = r.w[0];
+    return 1;
   }
-  return dok_load_key8<KF>(t, keys, i, n, key) ? 1 : 2;
 }
 
 // The stretch of rows that workgroup `w` of a pass owns.
@@ -159,7 +192,7 @@ __device__ __forceinline__ void bulk_stretch2(const BulkWs &ws, u32 b, u32 c, i6
 // EMIT: the keys are coordinate rows of several words each; their linearised form is written to
 // keysB (free until the second scatter) so that the first scatter reads 8 bytes per row instead
 // of the coordinates a second time.
-template <int KF, bool EMIT>
+template <int KF, bool EMIT, int ND>
 __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count1_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                                    BulkWs ws) {
   // Few bins and 64 lanes per atomic instruction mean many lanes on one address, which the LDS
@@ -168,20 +201,28 @@ __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count1_kernel(DevTable t, 
   for (int b = threadIdx.x; b < 4 * DOK_BULK_MAXBIG; b += DOK_BULK_CTPB) cnt[b] = 0;
   __syncthreads();
   const u32 copy = (threadIdx.x & 3) * DOK_BULK_MAXBIG;
+  // rows a thread has in flight: 8 to 16 eight-byte loads
+  constexpr int U = ND <= 2 ? 8 : ND <= 4 ? 4 : 2;
   i64 lo, hi;
   bulk_stretch1(ws, n, blockIdx.x, lo, hi);
-  for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += 8 * DOK_BULK_CTPB) {
-    u64 key[8];
-    bool ok[8];
+  for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += U * DOK_BULK_CTPB) {
+    BulkRaw<KF, ND> raw[U] = {};
     #pragma unroll
-    for (int u = 0; u < 8; u++) {
+    for (int u = 0; u < U; u++) {
+      const i64 i = i0 + u * DOK_BULK_CTPB;
+      if (i < hi) bulk_fetch<KF, ND>(t, keys, i, n, raw[u]);
+    }
+    u64 key[U];
+    bool ok[U];
+    #pragma unroll
+    for (int u = 0; u < U; u++) {
       const i64 i = i0 + u * DOK_BULK_CTPB;
       key[u] = 0;
-      ok[u] = i < hi && bulk_load_key<KF>(t, keys, i, n, key[u]) == 1;
+      ok[u] = i < hi && bulk_finish<KF, ND>(t, raw[u], key[u]) == 1;
       if (EMIT && i < hi) ws.keysB[i] = ok[u] ? key[u] : ~0ULL;
     }
     #pragma unroll
-    for (int u = 0; u < 8; u++)
+    for (int u = 0; u < U; u++)
       if (ok[u] && (key[u] ^ DOK_P8_XOR) >= 2)
         atomicAdd(&cnt[copy + (bulk_range_of(key[u], t) >> ws.sublog)], 1u);
   }
@@ -261,7 +302,7 @@ __global__ __launch_bounds__(1 << SL) void bulk_scan2_kernel(BulkWs ws) {
 
 // ---- scatter: LEVEL 1 moves the caller's rows into first-level bins (keysA/valsA), LEVEL 2 moves
 // the rows of each first-level bin into their ranges (keysB/valsB) ---------------------------------
-template <int V, int KF, int LEVEL, int SL = DOK_BULK_SUBLOG>
+template <int V, int KF, int LEVEL, int SL = DOK_BULK_SUBLOG, int ND = 0>
 __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, const void *__restrict__ keys_in,
                                                                     const void *__restrict__ vals_in, i64 n, BulkWs ws) {
   typedef typename ValT<V>::type VT;
@@ -315,23 +356,51 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
 
   // The rows of a tile sit in registers from their load to their place in the LDS staging area;
   // the next tile's loads are issued as soon as the registers are free, so that they are in
-  // flight during the write-out of this tile.  st[j]: 0 no row, 1 row, 2 row outside the table's
-  // coordinate space.
-  u64 k[RPT], v[RPT];
-  int st[RPT];
+  // flight during the write-out of this tile, and are only turned into keys (finish_tile) at the
+  // top of the next round.  st[j]: 0 no row, 1 row, 2 row outside the table's coordinate space.
+  u64 k[RPT];
+  VT v[RPT];                                // (as loaded: widening a 1- or 2-byte value would be a use,
+  int st[RPT];                              // and a use inside a row's guard waits for the load there)
+  // what was fetched and is not finished yet: the coordinates of a coordinate source; the one word
+  // of any other source waits in k[j] itself
+  constexpr bool COORDS = ND > 0;
+  BulkRaw<KF, ND> raw[COORDS ? RPT : 1];
   auto load_tile = [&](i64 lo) {
     const i64 hi = lo + T < hi0 ? lo + T : hi0;
     #pragma unroll
     for (int j = 0; j < RPT; j++) {
       const i64 i = lo + j * DOK_BULK_TPB + tid;
-      st[j] = 0; k[j] = 0; v[j] = 0;
+      k[j] = 0; v[j] = 0;
+      if (COORDS) raw[COORDS ? j : 0] = BulkRaw<KF, ND>{};
       if (i < hi) {
-        st[j] = bulk_load_key<KF>(t, kin, i, n, k[j]);
-        if (st[j] == 1) {
-          if (KF == DOK_KF_TABLE)                     // value i & 15 of bucket i >> 4 of the source
+        if constexpr (COORDS) {
+          bulk_fetch<KF, ND>(t, kin, i, n, raw[j]);
+        } else {
+          BulkRaw<KF, ND> r;
+          bulk_fetch<KF, ND>(t, kin, i, n, r);
+          k[j] = r.w[0];
+        }
+        if (KF == DOK_KF_TABLE) {                     // value i & 15 of bucket i >> 4 of the source
+          if ((int)(i & 15) < P8<V>::S)
             v[j] = *(const VT *)((const char *)kin + (i >> 4) * 128 + 8 * P8<V>::S + V * (i & 15));
-          else
-            v[j] = dok_load_val<V>(vin, i);
+        } else {
+          v[j] = ((const VT *)vin)[i];
+        }
+      }
+    }
+  };
+  auto finish_tile = [&](i64 lo) {
+    const i64 hi = lo + T < hi0 ? lo + T : hi0;
+    #pragma unroll
+    for (int j = 0; j < RPT; j++) {
+      st[j] = 0;
+      if (lo + j * DOK_BULK_TPB + tid < hi) {
+        if constexpr (COORDS) {
+          st[j] = bulk_finish<KF, ND>(t, raw[j], k[j]);
+        } else {
+          BulkRaw<KF, ND> r;
+          r.w[0] = k[j];
+          st[j] = bulk_finish<KF, ND>(t, r, k[j]);
         }
       }
     }
@@ -342,6 +411,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     #pragma unroll
     for (int q = 0; q < BPT; q++)
       if (tid * BPT + q < NB) cnt[tid * BPT + q] = 0;
+    finish_tile(lo);
     __syncthreads();
     BULK_TICK(0);
 
@@ -354,7 +424,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
       if (st[j] == 2) n_oob++;
       if (st[j] == 1) {
         if (LEVEL == 1 && (k[j] ^ DOK_P8_XOR) < 2) {
-          n_fresh += p8_side_set(t, k[j] ^ DOK_P8_XOR, v[j]);
+          n_fresh += p8_side_set(t, k[j] ^ DOK_P8_XOR, (u64)v[j]);
         } else {
           const u32 r = bulk_range_of(k[j], t);
           bn[j] = LEVEL == 1 ? (int)(r >> ws.sublog) : (int)(r & (NB - 1));
@@ -393,7 +463,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
       if (bn[j] >= 0) {
         const u32 pos = off[bn[j]] + rk[j];
         skeys[pos] = k[j];
-        svals[pos] = (VT)v[j];
+        svals[pos] = v[j];
         sbins[pos] = (u16)bn[j];
       }
     }
@@ -453,6 +523,10 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
 #endif
 #define DOK_BULK_FPW 8                          // 32-bit fingerprint words per bucket
 #define DOK_BULK_LIST (2 * DOK_BULK_R)          // capacity of a range's list
+
+// Register type of a row's value in the merge: see there.
+template <int V> struct BulkValReg { typedef u32 type; };
+template <> struct BulkValReg<8> { typedef u64 type; };
 
 // n-th (0-based) set bit of m (m has more than n set bits).
 __device__ __forceinline__ int bulk_nth_bit(u32 m, u32 n) {
@@ -540,7 +614,14 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
     bool fr = FRESH;
     for (u32 c0 = lo; c0 < hi; c0 += C) {
       const u32 c1 = c0 + C < hi ? c0 + C : hi;
-      u64 k[RPT], v[RPT];
+      u64 k[RPT];
+      // Values of one and two bytes are fetched as the aligned 32-bit word of valsB that holds
+      // them and cut out where they are used: narrowing right after the load would be a use
+      // inside the row's guard, and the loads of the chunk's rows would no longer overlap.
+      typedef typename BulkValReg<V>::type VR;
+      VR v[RPT];
+      const u32 vsh = V < 4 ? ((c0 + (u32)tid) & (4 / V - 1)) * 8 * V : 0;   // (the same for every j: R is a multiple of 4)
+#define BULK_VAL(j) ((VT)(V < 4 ? (VR)(v[j] >> vsh) : v[j]))
       bool on[RPT];
       #pragma unroll
       for (int j = 0; j < RPT; j++) {
@@ -549,7 +630,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
         k[j] = 0; v[j] = 0;
         if (on[j]) {
           k[j] = ws.keysB[i];
-          v[j] = dok_load_val<V>(ws.valsB, i);
+          v[j] = V < 4 ? (VR)((const u32 *)ws.valsB)[i / (V < 4 ? 4 / V : 1)] : (VR)((const VT *)ws.valsB)[i];
         }
       }
       if (c0 == lo) {
@@ -599,7 +680,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
               const u32 r = atomicAdd(&fmask[lh[j]], 1u);
               if (r < (u32)S) {
                 tb[r * LD + lh[j]] = sk;
-                *(VT *)((char *)(tb + (S + ((r * V) >> 3)) * LD + lh[j]) + ((r * V) & 7)) = (VT)v[j];
+                *(VT *)((char *)(tb + (S + ((r * V) >> 3)) * LD + lh[j]) + ((r * V) & 7)) = BULK_VAL(j);
                 n_fresh++;
                 listed = false;
               }
@@ -616,13 +697,13 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
               for (int s = 0; s < S; s++) gm |= (u32)(((volatile u64 *)tb)[s * LD + lh[j]] == sk) << s;
               if (gm) {
                 const int s = __builtin_ctz(gm);
-                *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lh[j]) + ((s * V) & 7)) = (VT)v[j];
+                *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lh[j]) + ((s * V) & 7)) = BULK_VAL(j);
                 listed = false;
               }
             }
             if (listed) {
               const u32 e = atomicAdd(&n_list, 1u);
-              if (e < DOK_BULK_LIST) { lkey[e] = k[j]; lval[e] = (VT)v[j]; lflag[e] = (seen & bit) ? 1 : 0; }
+              if (e < DOK_BULK_LIST) { lkey[e] = k[j]; lval[e] = BULK_VAL(j); lflag[e] = (seen & bit) ? 1 : 0; }
               else act[j] = 2;
             }
             continue;
@@ -637,7 +718,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           }
           if (gm) {
             const int s = __builtin_ctz(gm);
-            *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lh[j]) + ((s * V) & 7)) = (VT)v[j];
+            *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lh[j]) + ((s * V) & 7)) = BULK_VAL(j);
           } else {
             bool listed = true;
             const u32 fp = (u32)h & (32 * DOK_BULK_FPW - 1), bit = 1u << (fp & 31);
@@ -654,7 +735,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
             if (listed) {
               // onto the range's list while there is room, else to the ordinary insert
               const u32 e = atomicAdd(&n_list, 1u);
-              if (e < DOK_BULK_LIST) { lkey[e] = k[j]; lval[e] = (VT)v[j]; lflag[e] = (seen & bit) ? 1 : 0; }
+              if (e < DOK_BULK_LIST) { lkey[e] = k[j]; lval[e] = BULK_VAL(j); lflag[e] = (seen & bit) ? 1 : 0; }
               else act[j] = 2;
             }
           }
@@ -668,7 +749,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
         if (act[j] == 1) {
           const int s = slot[j];
           tb[s * LD + lh[j]] = k[j] ^ DOK_P8_XOR;
-          *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lh[j]) + ((s * V) & 7)) = (VT)v[j];
+          *(VT *)((char *)(tb + (S + ((s * V) >> 3)) * LD + lh[j]) + ((s * V) & 7)) = BULK_VAL(j);
           n_fresh++;
         }
         // deferred rows: one LDS atomic per wave, then a packed global write
@@ -680,11 +761,12 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           if (act[j] == 2) {
             const u32 at = def_base + base + (u32)__popcll(dm & ((1ULL << lane) - 1ULL));
             ws.keysA[at] = k[j];
-            dok_store_val<V>(ws.valsA, (i64)at, v[j]);
+            dok_store_val<V>(ws.valsA, (i64)at, (u64)BULK_VAL(j));
           }
         }
       }
       BULK_TICK(2);
+#undef BULK_VAL
     }
     __syncthreads();
 
@@ -1174,7 +1256,8 @@ template <int V, int KF>
 static bool bulk_plan_for(const DevTable &d, i64 n, BulkPlan &p, i64 n_cap = -1) {
   static u32 g1 = 0, gm = 0;
   if (g1 == 0) {
-    g1 = bulk_resident(bulk_scatter_kernel<V, KF, 1>, DOK_BULK_TPB, DOK_BULK_GRID, 64);
+    constexpr int ND = (KF == DOK_KF_COLS || KF == DOK_KF_ROWS) ? 2 : 0;   // (the dimensions do not change the LDS use)
+    g1 = bulk_resident(bulk_scatter_kernel<V, KF, 1, DOK_BULK_SUBLOG, ND>, DOK_BULK_TPB, DOK_BULK_GRID, 64);
     gm = bulk_resident(bulk_merge_kernel<V, false>, DOK_BULK_R, DOK_BULK_GRID, 1);
   }
   return bulk_plan(d, n, p, g1, gm, n_cap);
@@ -1190,21 +1273,22 @@ __global__ void bulk_side_slots_kernel(DevTable src, DevTable dst) {
 }
 
 // FRESH: the table's memory is uninitialised (see bulk_merge_kernel); the header is zeroed here.
-template <int V, int KF, bool FRESH = false>
-static void bulk_launch(const DevTable &d, const void *keys, const void *values, i64 n, const BulkPlan &p,
-                        void *workspace, hipStream_t s) {
+// ND: dimensions of a coordinate source (KF rows or columns), else 0.
+template <int V, int KF, int ND, bool FRESH>
+static void bulk_launch_nd(const DevTable &d, const void *keys, const void *values, i64 n, const BulkPlan &p,
+                           void *workspace, hipStream_t s) {
   BulkWs ws;
   bulk_bind(p, workspace, ws);
   if (FRESH) dok_fill_kernel<<<1, DOK_TPB, 0, s>>>(d.buckets, 0, d.header);
   // coordinate rows of three and more dimensions are linearised once, by the count
-  constexpr bool COORDS = KF == DOK_KF_COLS || KF == DOK_KF_ROWS;
-  const bool emit = COORDS && d.lin_ndim >= 3;
-  if (emit) bulk_count1_kernel<KF, COORDS><<<p.g1, DOK_BULK_CTPB, 0, s>>>(d, keys, n, ws);
-  else bulk_count1_kernel<KF, false><<<p.g1, DOK_BULK_CTPB, 0, s>>>(d, keys, n, ws);
+  constexpr bool EMIT = ND >= 3;
+  bulk_count1_kernel<KF, EMIT, ND><<<p.g1, DOK_BULK_CTPB, 0, s>>>(d, keys, n, ws);
   bulk_scan1a_kernel<<<p.n_big, p.g1, 0, s>>>(ws);
   bulk_scan1b_kernel<<<1, DOK_BULK_MAXBIG, 0, s>>>(ws);
-  if (emit) bulk_scatter_kernel<V, COORDS ? DOK_KF_LIN : KF, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, ws.keysB, values, n, ws);
-  else bulk_scatter_kernel<V, KF, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, keys, values, n, ws);
+  if constexpr (EMIT)
+    bulk_scatter_kernel<V, DOK_KF_LIN, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, ws.keysB, values, n, ws);
+  else
+    bulk_scatter_kernel<V, KF, 1, DOK_BULK_SUBLOG, ND><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, keys, values, n, ws);
   if (p.sublog == DOK_BULK_SUBLOG) {
     bulk_count2_kernel<DOK_BULK_SUBLOG><<<p.n_big * p.ch, DOK_BULK_CTPB, 0, s>>>(d, ws);
     bulk_scan2_kernel<DOK_BULK_SUBLOG><<<p.n_big, 1 << DOK_BULK_SUBLOG, 0, s>>>(ws);
@@ -1217,4 +1301,23 @@ static void bulk_launch(const DevTable &d, const void *keys, const void *values,
   bulk_merge_kernel<V, FRESH><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
   if (p.gm > 1) bulk_edge_kernel<V><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
   bulk_deferred_kernel<V><<<p.gm, DOK_TPB, 0, s>>>(d, ws);
+}
+
+template <int V, int KF, bool FRESH = false>
+static void bulk_launch(const DevTable &d, const void *keys, const void *values, i64 n, const BulkPlan &p,
+                        void *workspace, hipStream_t s) {
+  if constexpr (KF == DOK_KF_COLS || KF == DOK_KF_ROWS) {
+    switch (d.lin_ndim) {                              // 1 .. DOK_MAX_DIMS, checked with the descriptor
+      case 1: return bulk_launch_nd<V, KF, 1, FRESH>(d, keys, values, n, p, workspace, s);
+      case 2: return bulk_launch_nd<V, KF, 2, FRESH>(d, keys, values, n, p, workspace, s);
+      case 3: return bulk_launch_nd<V, KF, 3, FRESH>(d, keys, values, n, p, workspace, s);
+      case 4: return bulk_launch_nd<V, KF, 4, FRESH>(d, keys, values, n, p, workspace, s);
+      case 5: return bulk_launch_nd<V, KF, 5, FRESH>(d, keys, values, n, p, workspace, s);
+      case 6: return bulk_launch_nd<V, KF, 6, FRESH>(d, keys, values, n, p, workspace, s);
+      case 7: return bulk_launch_nd<V, KF, 7, FRESH>(d, keys, values, n, p, workspace, s);
+      default: return bulk_launch_nd<V, KF, 8, FRESH>(d, keys, values, n, p, workspace, s);
+    }
+  } else {
+    bulk_launch_nd<V, KF, 0, FRESH>(d, keys, values, n, p, workspace, s);
+  }
 }

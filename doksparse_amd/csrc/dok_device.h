@@ -135,8 +135,9 @@ __global__ __launch_bounds__(DOK_TPB) void dok_line_gather_kernel(const u64 *__r
 
 // Row-major linearisation of an int64 coordinate row; false if any coordinate is outside
 // [0, dim).  Negative coordinates are not wrapped (the reference does not wrap them either).
-// The loop runs to the compile-time maximum under a uniform guard, so that it unrolls and the
-// coordinate loads of several rows can be in flight together.
+// The loop runs to the compile-time maximum under a uniform guard, so that it unrolls.  (Each
+// coordinate is used right after its load; the streaming kernels of the bulk path, where the
+// loads of many rows must overlap, have a loader of their own.)
 __device__ __forceinline__ bool dok_linearise(const DevTable &t, const i64 *row, u64 &key) {
   bool ok = true;
   u64 k = 0;
