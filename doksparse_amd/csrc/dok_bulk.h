@@ -41,23 +41,20 @@
 // Rows per scatter tile.  A tile is staged in LDS whole (8 + V + 2 bytes per row), and the larger
 // it is, the longer the runs of rows that leave for one bin: for 8-byte keys with 4-byte values
 // one workgroup per CU with a tile that nearly fills the LDS beats two with half the tile
-// (scatter of 64M rows: 0.57 -> 0.47 ms).  Where it does not, the sizes below say so; all of
-// them are measured choices.
+// (scatter of 64M rows: 0.57 -> 0.47 ms).  All sizes are measured choices.
 #ifndef DOK_BULK_T
 #define DOK_BULK_T 8192                     // first pass (up to 1024 bins: 12 KiB of bin arrays)
 #endif
-#ifndef DOK_BULK_T1C
-#define DOK_BULK_T1C 4096                   //   ... from coordinate rows or a table: the loads weigh more
-#endif                                      //   than the writes there, and two workgroups per CU hide them
 #ifndef DOK_BULK_T1V8
 #define DOK_BULK_T1V8 6144                  //   ... with 8-byte values
 #endif
 #ifndef DOK_BULK_T2
-#define DOK_BULK_T2 10240                   // second pass (256 bins)
+#define DOK_BULK_T2 10240                   // second pass
 #endif
 #ifndef DOK_BULK_T2S
-#define DOK_BULK_T2S 4096                   //   ... with 1- and 2-byte values (measured: three workgroups
-#endif                                      //   per CU with small tiles are faster there)
+#define DOK_BULK_T2S 4096                   //   ... with 1- and 2-byte values when a workgroup's stretch is short
+#endif                                      //   (three workgroups per CU with small tiles are faster then)
+#define DOK_BULK_T2S_BELOW 16384            //   ... which is: fewer rows than this per workgroup
 #ifndef DOK_BULK_T2V8
 #define DOK_BULK_T2V8 8192                  //   ... with 8-byte values
 #endif
@@ -302,13 +299,12 @@ __global__ __launch_bounds__(1 << SL) void bulk_scan2_kernel(BulkWs ws) {
 
 // ---- scatter: LEVEL 1 moves the caller's rows into first-level bins (keysA/valsA), LEVEL 2 moves
 // the rows of each first-level bin into their ranges (keysB/valsB) ---------------------------------
-template <int V, int KF, int LEVEL, int SL = DOK_BULK_SUBLOG, int ND = 0>
+template <int V, int KF, int LEVEL, int SL = DOK_BULK_SUBLOG, int ND = 0, bool SMALLT = false>
 __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, const void *__restrict__ keys_in,
                                                                     const void *__restrict__ vals_in, i64 n, BulkWs ws) {
   typedef typename ValT<V>::type VT;
-  constexpr bool CHEAP = KF == DOK_KF_U64 || KF == DOK_KF_RAW;      // one load per row
-  constexpr int T = LEVEL == 1 ? (!CHEAP ? DOK_BULK_T1C : V == 8 ? DOK_BULK_T1V8 : DOK_BULK_T)
-                               : (V == 8 ? DOK_BULK_T2V8 : V == 4 ? DOK_BULK_T2 : DOK_BULK_T2S);
+  constexpr int T = LEVEL == 1 ? (V == 8 ? DOK_BULK_T1V8 : DOK_BULK_T)
+                               : (V == 8 ? DOK_BULK_T2V8 : SMALLT ? DOK_BULK_T2S : DOK_BULK_T2);
   static_assert(T % DOK_BULK_TPB == 0, "every thread stages the same number of rows");
   constexpr int RPT = T / DOK_BULK_TPB;
   constexpr int NB = LEVEL == 1 ? DOK_BULK_MAXBIG : (1 << SL);
@@ -1289,10 +1285,13 @@ static void bulk_launch_nd(const DevTable &d, const void *keys, const void *valu
     bulk_scatter_kernel<V, DOK_KF_LIN, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, ws.keysB, values, n, ws);
   else
     bulk_scatter_kernel<V, KF, 1, DOK_BULK_SUBLOG, ND><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, keys, values, n, ws);
+  // narrow values: small second-pass tiles when the workgroups' stretches are short
+  const bool smallt = V <= 2 && n / ((i64)p.n_big * p.ch) < DOK_BULK_T2S_BELOW;
   if (p.sublog == DOK_BULK_SUBLOG) {
     bulk_count2_kernel<DOK_BULK_SUBLOG><<<p.n_big * p.ch, DOK_BULK_CTPB, 0, s>>>(d, ws);
     bulk_scan2_kernel<DOK_BULK_SUBLOG><<<p.n_big, 1 << DOK_BULK_SUBLOG, 0, s>>>(ws);
-    bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
+    if (smallt) bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG, 0, V <= 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
+    else bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
   } else {
     bulk_count2_kernel<DOK_BULK_SUBLOG_WIDE><<<p.n_big * p.ch, DOK_BULK_CTPB, 0, s>>>(d, ws);
     bulk_scan2_kernel<DOK_BULK_SUBLOG_WIDE><<<p.n_big, 1 << DOK_BULK_SUBLOG_WIDE, 0, s>>>(ws);
