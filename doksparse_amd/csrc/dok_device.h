@@ -43,7 +43,18 @@ struct DevTable {
   int pad_;
   i64 lin_dims[DOK_MAX_DIMS];
   i64 lin_strides[DOK_MAX_DIMS];   // row-major strides of lin_dims
+  u64 lin_magic[DOK_MAX_DIMS];     // division by lin_strides[d] as multiply + shift (dok_div_stride);
+  int lin_shift[DOK_MAX_DIMS];     // set by the host for strides above 1
 };
+
+// n / d for the stride d that (magic, shift) were made for (host: div_magic in dokhip.hip).  The
+// round-up method of Granlund and Montgomery in its branch-free form: q = hi64(magic * n),
+// n / d = (((n - q) >> 1) + q) >> shift.  A 64-bit divide costs some 150 instructions here, and
+// the read-out of a coordinate table divides once per dimension and entry.
+__device__ __forceinline__ u64 dok_div_stride(u64 n, u64 magic, int shift) {
+  const u64 q = __umul64hi(magic, n);
+  return (((n - q) >> 1) + q) >> shift;
+}
 
 // Kernel-argument form of dok_index_t (+ optional source-value view).
 struct DevIndex {
@@ -200,7 +211,7 @@ __device__ __forceinline__ void dok_store_key8(const DevTable &t, void *keys_out
     u64 rem = key;
     for (int d = 0; d < t.lin_ndim; d++) {
       const u64 s = (u64)t.lin_strides[d];
-      const u64 c = rem / s;
+      const u64 c = s == 1 ? rem : dok_div_stride(rem, t.lin_magic[d], t.lin_shift[d]);
       rem -= c * s;
       if (KF == DOK_KF_ROWS) ((i64 *)keys_out)[i * t.lin_ndim + d] = (i64)c;
       else ((i64 *)keys_out)[(i64)d * cap + i] = (i64)c;

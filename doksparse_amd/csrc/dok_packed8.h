@@ -756,10 +756,16 @@ __global__ __launch_bounds__(1024) void dok_scan_kernel(i64 *counts, i64 n, cons
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   if (tid == 0) carry_s = 0;
   __syncthreads();
-  for (i64 base = 0; base < n; base += 1024) {
-    const i64 idx = base + tid;
-    const i64 v = idx < n ? counts[idx] : 0;
-    i64 inc = v;
+  // eight consecutive counts per thread and round: the rounds are serial (barriers, a carry), so
+  // fewer and fatter ones
+  for (i64 base = 0; base < n; base += 8 * 1024) {
+    const i64 i0 = base + (i64)tid * 8;
+    i64 v[8], sum = 0;
+    #pragma unroll
+    for (int k = 0; k < 8; k++) v[k] = i0 + k < n ? counts[i0 + k] : 0;
+    #pragma unroll
+    for (int k = 0; k < 8; k++) { const i64 x = v[k]; v[k] = sum; sum += x; }
+    i64 inc = sum;
     #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
       const i64 up = __shfl_up(inc, o, 64);
@@ -770,7 +776,10 @@ __global__ __launch_bounds__(1024) void dok_scan_kernel(i64 *counts, i64 n, cons
     i64 wpre = 0;
     for (int k = 0; k < wv; k++) wpre += wsum[k];
     const i64 carry = carry_s;
-    if (idx < n) counts[idx] = carry + wpre + inc - v;
+    const i64 excl = carry + wpre + inc - sum;
+    #pragma unroll
+    for (int k = 0; k < 8; k++)
+      if (i0 + k < n) counts[i0 + k] = excl + v[k];
     __syncthreads();
     if (tid == 1023) carry_s = carry + wpre + inc;
     __syncthreads();

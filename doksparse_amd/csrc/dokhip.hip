@@ -37,6 +37,20 @@ int layout_of(int kb, int vb, int *slots) {
   return DOK_LAYOUT_TAGGED;
 }
 
+// Multiplier and shift that divide a 64-bit integer by d >= 2 (see dok_div_stride).
+static void div_magic(u64 d, u64 &magic, int &shift) {
+  const int fl = 63 - __builtin_clzll(d);
+  if ((d & (d - 1)) == 0) { magic = 0; shift = fl - 1; return; }      // power of two: q = 0, n >> 1 >> (fl - 1)
+  const unsigned __int128 num = (unsigned __int128)1 << (64 + fl);     // d > 2^fl, so the quotient fits 64 bits
+  u64 m = (u64)(num / d);
+  const u64 rem = (u64)(num % d);
+  m += m;
+  const u64 twice = rem + rem;
+  if (twice >= d || twice < rem) m += 1;
+  magic = m + 1;
+  shift = fl;
+}
+
 // Validate a table descriptor and build its kernel-argument form.
 int make_dev_table(const dok_table_t *t, DevTable &d, int &layout) {
   if (!t || !t->buckets || !t->header) return DOK_EINVAL;
@@ -62,6 +76,7 @@ int make_dev_table(const dok_table_t *t, DevTable &d, int &layout) {
       if (t->lin_dims[k] < 0) return DOK_EINVAL;
       d.lin_dims[k] = t->lin_dims[k];
       d.lin_strides[k] = (i64)vol;
+      if (vol > 1) div_magic((u64)vol, d.lin_magic[k], d.lin_shift[k]);
       vol *= (unsigned __int128)(t->lin_dims[k] > 0 ? t->lin_dims[k] : 1);
       if (vol >> 63) return DOK_EUNSUPPORTED;
     }

@@ -44,6 +44,37 @@ def test_construct_readout_to_dense(cuda):
         assert dok.indices().shape == (2, 60) and dok.values().shape == (60,)
 
 
+@pytest.mark.parametrize("size", [
+    (7, 1, 1000003, 3, 1),                    # dimensions of 1 (strides that repeat), a prime
+    (2147483647, 2147483629),                 # two primes below 2^31: keys up to 2^62
+    (3, 5, 7, 11, 13, 17, 19, 23),            # eight dimensions, no stride a power of two
+    (4096, 4096, 64, 8),                      # every stride a power of two
+    (1, 1, 1),                                # a single cell
+    (1000000, 1000000),
+    (9223372036854775807,),                   # one dimension of 2^63 - 1
+])
+def test_readout_recovers_coordinates_for_awkward_shapes(cuda, size):
+    """indices() turns the stored linear keys back into coordinates by multiply-and-shift
+    division by the row-major strides: it must return exactly the coordinates that went in,
+    the largest coordinate of every dimension included."""
+    from doksparse_amd import SparseDOKTensor
+    g = torch.Generator().manual_seed(len(size))
+    n = 1 if all(s == 1 for s in size) else 4000
+    coords = torch.stack([torch.randint(0, s, (n,), generator=g) if s > 1 else torch.zeros(n, dtype=torch.long)
+                          for s in size])
+    coords[:, 0] = torch.tensor([s - 1 for s in size])              # the far corner
+    if n > 1:
+        coords[:, 1] = 0                                             # and the origin
+    coords = torch.unique(coords, dim=1)
+    vals = torch.arange(1, coords.shape[1] + 1, dtype=torch.float32)
+    dok = SparseDOKTensor(size, coords.to(cuda), vals.to(cuda), device=cuda)
+    idx, v = dok.indices().cpu(), dok.values().cpu()
+    assert idx.shape == coords.shape
+    order = torch.argsort(v)                                         # the values number the input columns
+    assert torch.equal(v[order], vals)
+    assert torch.equal(idx[:, order], coords)
+
+
 GET_CASES = [
     lambda r, c, m: (r, c),
     lambda r, c, m: (r[:, None], c[None, :]),
