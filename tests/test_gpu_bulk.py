@@ -536,7 +536,8 @@ def test_build_with_many_equal_keys(cuda, bulk_always, distinct):
     assert torch.equal(torch.sort(ks[:, 0]).values, torch.unique(keys))
 
 
-@pytest.mark.parametrize("size", [(5000, 3000), (300, 77, 50), (40, 30, 20, 16), (9, 8, 7, 6, 5, 4)])
+@pytest.mark.parametrize("size", [(900_000,), (5000, 3000), (300, 77, 50), (40, 30, 20, 16), (12, 9, 8, 7, 11),
+                                  (9, 8, 7, 6, 5, 4), (5, 4, 7, 3, 6, 5, 4), (3, 5, 4, 3, 6, 2, 5, 4)])
 def test_bulk_and_per_row_agree_on_coordinate_batches(cuda, monkeypatch, size):
     """Coordinate keys in both layouts ([n, ndim] rows and [ndim, n] COO columns; three and more
     dimensions are linearised by the bulk path's first count), repeated coordinates, coordinates
