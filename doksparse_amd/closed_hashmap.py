@@ -521,13 +521,14 @@ class CudaClosedHashmap:
             return
         # the batch may not fit.  Rows that miss bound the distinct new keys from above; if even
         # that bound stays under the threshold nothing can grow and no sort is needed
-        _, is_found = self.get(keys)
-        n_miss = int((~is_found).sum().item())
+        # (counted by a kernel that writes one number: no value rows, no flags)
+        n_miss = n - int(self.count_existing(keys).item())
         if n_old + n_miss <= limit:
             self._launch_set(keys, values)
             self._n_upper = n_old + n_miss
             return
         # otherwise count the distinct new keys exactly, as the reference does
+        _, is_found = self.get(keys)
         n_new = self._count_distinct(keys[~is_found])
         if n_old + n_new > limit:
             self.rehash(int((n_old + n_new) * self._rehash_factor))

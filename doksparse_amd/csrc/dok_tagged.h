@@ -423,13 +423,28 @@ static int tg_launch_get(const DevTable &d, const void *keys, i64 n, void *value
   return DOK_OK;
 }
 
+// Most workgroups of the kernels that loop over tiles and end with one atomic per wave on a
+// counter.  Few workgroups keep those atomics cheap (same-address atomics serialise at ~12 ns
+// each), many even out the long probe chains of a loaded table; measured on 32M float32[3] ->
+// int64[5] rows at load factors 0.5 / 0.9: count 1.58 / 10.2 ms with 2048 workgroups,
+// 1.46 / 5.6 ms with 8192; set 9.6 / 22.7 ms with 2048, 9.0 / 15.4 ms with 32768; remove of 8M
+// 0.68 / 1.10 ms with 2048, 1.65 / 2.35 ms with 32768.
+#ifndef DOK_TG_COUNT_GRID
+#define DOK_TG_COUNT_GRID 8192u
+#endif
+#ifndef DOK_TG_REMOVE_GRID
+#define DOK_TG_REMOVE_GRID 2048u
+#endif
+#ifndef DOK_TG_SET_GRID
+#define DOK_TG_SET_GRID 32768u
+#endif
 static int tg_launch_count(const DevTable &d, const void *keys, i64 n, i64 *count, hipStream_t s) {
   TgGeom g;
   int rc = tg_geom(d, nullptr, g);
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_lookup_kernel<1, false><<<(grid < 2048u ? grid : 2048u), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, nullptr, nullptr, count);
+  tg_lookup_kernel<1, false><<<(grid < DOK_TG_COUNT_GRID ? grid : DOK_TG_COUNT_GRID), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, nullptr, nullptr, count);
   return DOK_OK;
 }
 
@@ -439,7 +454,7 @@ static int tg_launch_remove(const DevTable &d, const void *keys, i64 n, u8 *remo
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_lookup_kernel<2, false><<<(grid < 2048u ? grid : 2048u), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, nullptr, removed, nullptr);
+  tg_lookup_kernel<2, false><<<(grid < DOK_TG_REMOVE_GRID ? grid : DOK_TG_REMOVE_GRID), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, nullptr, removed, nullptr);
   return DOK_OK;
 }
 
@@ -449,7 +464,7 @@ static int tg_launch_set(const DevTable &d, const void *keys, const void *values
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k) || !tg_aligned(values, g.unit_v)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_set_kernel<<<(grid < 2048u ? grid : 2048u), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, (const u8 *)values, n, stored);
+  tg_set_kernel<<<(grid < DOK_TG_SET_GRID ? grid : DOK_TG_SET_GRID), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, (const u8 *)values, n, stored);
   return DOK_OK;
 }
 

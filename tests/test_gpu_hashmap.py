@@ -402,19 +402,23 @@ def test_completely_full_tables_exercise_far_displacements(cuda, vdtype):
     probe = CudaClosedHashmap(n_buckets=1, device=cuda)
     probe.set(torch.zeros(1, 1, dtype=torch.long, device=cuda), torch.zeros(1, 1, device=cuda).to(torch.from_numpy(np.zeros(1, vdtype)).dtype))
     slots = probe._slots_per_bucket
-    for n_phys in (40, 64, 200):
+    # (buckets, rows per set call).  One call for all rows: the waves race, and where the last keys
+    # end up differs from run to run.  One row per call: a fixed order, the same table every
+    # time - that case must show a far displacement.
+    for n_phys, step in ((40, None), (64, None), (200, None), (120, 1)):
         cap = n_phys * slots                                   # every physical slot
         keys = np.unique(rng.integers(0, 2**62, size=cap + 64, dtype=np.int64))[:cap, None]
         vals = rng.integers(-100, 100, size=(cap, 1)).astype(vdtype)
-        hm = CudaClosedHashmap(n_buckets=cap, device=cuda, rehash_threshold=1.0)
+        hm = CudaClosedHashmap(n_buckets=cap, device=cuda, rehash_threshold=1.0, seed=77)
         ref = RefClosedHashmap(n_buckets=cap, rehash_threshold=1.0, rng=np.random.default_rng(1))
         k, v = _to(cuda, keys, vals)
-        hm.set(k, v)
+        for lo in range(0, cap, step or cap):
+            hm.set(k[lo: lo + (step or cap)], v[lo: lo + (step or cap)])
         ref.set(keys, vals)
         assert hm.n_elements == ref.n_elements == cap
         assert hm._n_phys == n_phys
         meta = hm._table.view(torch.int64).reshape(n_phys, 16)[:, 15].cpu().numpy()
-        if n_phys >= 64:
+        if step:
             assert (meta & 1).any(), "no far displacement was produced; the test lost its point"
         q = np.concatenate([keys, rng.integers(0, 2**62, size=(cap, 1), dtype=np.int64)])
         _check_get(hm, ref, q, cuda, fallback=-3)
