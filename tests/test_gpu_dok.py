@@ -475,3 +475,75 @@ def test_reductions_and_elementwise_glue(cuda):
     assert torch.allclose(dok.abs().sqrt().to_dense().cpu(), dense.abs().sqrt())
     assert torch.equal(dok.flatten().to_dense().cpu(), dense.flatten())
     assert torch.equal(dok.reshape(20, 60).to_dense().cpu(), dense.reshape(20, 60))
+
+
+def _random_selectors(rng, shape):
+    """A random indexing expression over the leading dimensions of `shape`: integers, slices,
+    index tensors that broadcast to one shape, lists, and at most one 1-D mask (kept apart
+    from the index tensors)."""
+    n_sel = int(rng.integers(1, len(shape) + 1))
+    bshape = tuple(int(x) for x in rng.integers(1, 5, size=int(rng.integers(1, 3))))
+    use_mask, mask_done, sel = rng.random() < 0.25, False, []
+    for d in range(n_sel):
+        s = shape[d]
+        kind = rng.choice(["int", "slice", "tensor", "mask", "full", "list"], p=[0.2, 0.2, 0.3, 0.1, 0.15, 0.05])
+        if kind == "mask" and (not use_mask or mask_done):
+            kind = "slice"
+        if kind in ("tensor", "list") and use_mask:
+            kind = "slice"
+        if kind == "int":
+            sel.append(int(rng.integers(0, s)))
+        elif kind == "full":
+            sel.append(slice(None))
+        elif kind == "slice":
+            a, b = sorted(int(x) for x in rng.integers(0, s + 1, size=2))
+            sel.append(slice(a if rng.random() < 0.8 else None, b if rng.random() < 0.8 else None))
+        elif kind == "tensor":
+            shp = tuple(x if rng.random() < 0.7 else 1 for x in bshape)
+            sel.append(torch.from_numpy(rng.integers(0, s, size=shp)).long())
+        elif kind == "list":
+            sel.append([int(x) for x in rng.integers(0, s, size=bshape[-1])])
+        else:
+            m = torch.from_numpy(rng.random(s) < 0.5)
+            m[0] = m[0] or not bool(m.any())
+            sel.append(m)
+            mask_done = True
+    return tuple(sel)
+
+
+def test_random_selectors_against_the_oracle(cuda):
+    """Differential test: random shapes (1 to 5 dimensions), random contents and random indexing
+    expressions; every expression the oracle accepts is read through the HIP path and compared,
+    then assigned one value through both and the tensors compared.  (Equal coordinates inside
+    one assignment: the reference over-counts its element counter, so the entry count is compared
+    with the oracle's distinct coordinates.)"""
+    from doksparse_amd import SparseDOKTensor
+    rng = np.random.default_rng(20)
+    compared = 0
+    for case in range(80):
+        shape = tuple(int(x) for x in rng.integers(1, 9, size=int(rng.integers(1, 6))))
+        vol = int(np.prod(shape))
+        nnz = max(1, int(rng.integers(0, vol + 1)))
+        idx = torch.stack(torch.unravel_index(torch.from_numpy(rng.permutation(vol)[:nnz]), shape))
+        vals = torch.from_numpy(rng.integers(1, 100, size=nnz)).float()
+        dok = SparseDOKTensor(shape, idx.to(cuda), vals.to(cuda), device=cuda)
+        ref = RefSparseDOKTensor(shape, idx, vals, rng=np.random.default_rng(case))
+        for _ in range(4):
+            sel = _random_selectors(rng, shape)
+            dsel = tuple(s.to(cuda) if isinstance(s, torch.Tensor) else s for s in sel)
+            try:
+                exp = ref[sel]
+            except Exception:
+                continue                          # rejected by the oracle, as by the reference
+            got = dok[dsel]
+            assert got.shape == exp.shape and torch.equal(got.cpu(), exp), (shape, sel)
+            val = float(rng.integers(-50, 50))
+            try:
+                ref[sel] = torch.full(exp.shape, val)
+            except Exception:
+                continue
+            dok[dsel] = torch.full(exp.shape, val, device=cuda)
+            assert torch.equal(dok.to_dense().cpu(), ref.to_dense()), (shape, sel)
+            assert dok._nnz() == np.unique(ref.indices().cpu().numpy(), axis=1).shape[1], (shape, sel)
+            compared += 1
+    assert compared > 200
