@@ -641,7 +641,10 @@ class SparseDOKTensor(object):
 
     # ------------------------------------------------------------------ views and re-layout
     def permute_(self, *ordering):
-        """Reorder the dimensions in place; nothing is moved (reference: :439-443)."""
+        """Reorder the dimensions in place; nothing is moved (reference: :439-443).  The order is
+        given as separate arguments, as in the reference, or as one sequence, as torch takes it."""
+        if len(ordering) == 1 and isinstance(ordering[0], (list, tuple)):
+            ordering = ordering[0]
         ordering = [int(o) % self.ndim for o in ordering]
         assert sorted(ordering) == list(range(self.ndim))
         self._perm = tuple(self._perm[o] for o in ordering)

@@ -547,3 +547,46 @@ def test_random_selectors_against_the_oracle(cuda):
             assert dok._nnz() == np.unique(ref.indices().cpu().numpy(), axis=1).shape[1], (shape, sel)
             compared += 1
     assert compared > 200
+
+
+def test_random_selectors_through_permuted_views(cuda):
+    """The same differential test through `permute` views: reads and writes through the view must
+    equal an oracle tensor built from the permuted coordinates, and the base tensor must see
+    the writes (the view shares its table)."""
+    from doksparse_amd import SparseDOKTensor
+    rng = np.random.default_rng(21)
+    compared = 0
+    for case in range(50):
+        nd = int(rng.integers(2, 6))
+        shape = tuple(int(x) for x in rng.integers(1, 8, size=nd))
+        vol = int(np.prod(shape))
+        nnz = max(1, int(rng.integers(0, vol + 1)))
+        idx = torch.stack(torch.unravel_index(torch.from_numpy(rng.permutation(vol)[:nnz]), shape))
+        vals = torch.from_numpy(rng.integers(1, 100, size=nnz)).float()
+        dok = SparseDOKTensor(shape, idx.to(cuda), vals.to(cuda), device=cuda)
+        perm = [int(x) for x in rng.permutation(nd)]
+        view = dok.permute(*perm) if case % 2 else dok.permute(perm)
+        pshape = tuple(shape[p] for p in perm)
+        inverse = [perm.index(d) for d in range(nd)]
+        ref = RefSparseDOKTensor(pshape, idx[perm], vals, rng=np.random.default_rng(case))
+        assert tuple(view.shape) == pshape
+        for _ in range(4):
+            sel = _random_selectors(rng, pshape)
+            dsel = tuple(s.to(cuda) if isinstance(s, torch.Tensor) else s for s in sel)
+            try:
+                exp = ref[sel]
+            except Exception:
+                continue
+            got = view[dsel]
+            assert got.shape == exp.shape and torch.equal(got.cpu(), exp), (shape, perm, sel)
+            val = float(rng.integers(-50, 50))
+            try:
+                ref[sel] = torch.full(exp.shape, val)
+            except Exception:
+                continue
+            view[dsel] = torch.full(exp.shape, val, device=cuda)
+            assert torch.equal(view.to_dense().cpu(), ref.to_dense()), (shape, perm, sel)
+            assert torch.equal(dok.to_dense().cpu(), ref.to_dense().permute(*inverse)), (shape, perm, sel)
+            assert dok._nnz() == view._nnz()
+            compared += 1
+    assert compared > 100
