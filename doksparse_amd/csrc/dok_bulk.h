@@ -503,7 +503,8 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
 //     as the range.  If the mark was already there, an equal key may be among the range's rows,
 //     and the row goes on the range's list;
 //   - if the bucket has an EMPTY slot, the probe chain of every key whose home it is ends right
-//     here, so the key is new: the new rows of a bucket (their keys are distinct, thanks to the
+//     here, so the key is new (the same holds for a bucket of keys and tombstones whose
+//     displacement map is empty): the new rows of a bucket (their keys are distinct, thanks to the
 //     marks) draw a rank and the r-th of them takes the r-th free slot, tombstones first, with
 //     plain stores;
 //   - rows whose rank lies beyond the free slots, and rows whose home bucket has no EMPTY slot,
@@ -719,7 +720,10 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
             bool listed = true;
             const u32 fp = (u32)h & (32 * DOK_BULK_FPW - 1), bit = 1u << (fp & 31);
             const u32 seen = atomicOr(&marks[lh[j] * DOK_BULK_FPW + (fp >> 5)], bit);
-            if (!(seen & bit) && ge) {
+            // The key is new if its chain ends in this bucket: the bucket has an EMPTY slot, or -
+            // in a bucket of keys and tombstones only - its displacement map is empty, so no key
+            // whose home it is lives anywhere else.
+            if (!(seen & bit) && (ge || (gt && tb[DOK_P8_META * LD + lh[j]] == 0))) {
               const u32 r = atomicAdd(&fresh_cnt[lh[j]], 1u);
               const u32 nt = __popc(gt);
               if (r < nt + __popc(ge)) {
