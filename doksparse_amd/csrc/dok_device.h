@@ -246,17 +246,28 @@ template <int V> __device__ __forceinline__ void dok_store_val(void *values, i64
 // unused axes.
 __device__ __forceinline__ bool dok_gather_at(const DevTable &t, const DevIndex &ix,
                                               const i64 (&idx)[DOK_MAX_DIMS], u64 &key, i64 &voff) {
-  bool ok = true;
-  u64 k = 0;
+  // first every dimension's selector is read, then the values are used: a use next to its load
+  // would make the loads of the dimensions wait for one another
+  i64 g[DOK_MAX_DIMS];
   #pragma unroll
   for (int d = 0; d < DOK_MAX_DIMS; d++) {
+    g[d] = 0;
     if (d < ix.ndim) {
       i64 off = 0;
       #pragma unroll
       for (int j = 0; j < DOK_MAX_DIMS; j++)
         if (j < ix.sel_ndim) off += idx[j] * ix.sstride[d][j];
       const i64 *sp = ix.sel[d];
-      const i64 c = ix.sbase[d] + (sp ? sp[off] : off);
+      g[d] = off;
+      if (sp) g[d] = sp[off];
+    }
+  }
+  bool ok = true;
+  u64 k = 0;
+  #pragma unroll
+  for (int d = 0; d < DOK_MAX_DIMS; d++) {
+    if (d < ix.ndim) {
+      const i64 c = ix.sbase[d] + g[d];
       ok = ok && ((u64)c < (u64)t.lin_dims[d]);
       k += (u64)c * (u64)t.lin_strides[d];
     }
