@@ -146,18 +146,24 @@ __global__ __launch_bounds__(DOK_TPB) void dok_line_gather_kernel(const u64 *__r
 
 // Row-major linearisation of an int64 coordinate row; false if any coordinate is outside
 // [0, dim).  Negative coordinates are not wrapped (the reference does not wrap them either).
-// The loop runs to the compile-time maximum under a uniform guard, so that it unrolls.  (Each
-// coordinate is used right after its load; the streaming kernels of the bulk path, where the
-// loads of many rows must overlap, have a loader of their own.)
+// The loops run to the compile-time maximum under a uniform guard, so that they unroll; the
+// coordinates are loaded first and used afterwards, so that the loads of a row overlap.  (The
+// streaming kernels of the bulk path, where the loads of many rows must overlap, have a loader
+// of their own.)
 __device__ __forceinline__ bool dok_linearise(const DevTable &t, const i64 *row, u64 &key) {
+  i64 c[DOK_MAX_DIMS];
+  #pragma unroll
+  for (int d = 0; d < DOK_MAX_DIMS; d++) {
+    c[d] = 0;
+    if (d < t.lin_ndim) c[d] = row[d];               // loads only: they overlap
+  }
   bool ok = true;
   u64 k = 0;
   #pragma unroll
   for (int d = 0; d < DOK_MAX_DIMS; d++) {
     if (d < t.lin_ndim) {
-      const i64 c = row[d];
-      ok = ok && ((u64)c < (u64)t.lin_dims[d]);
-      k += (u64)c * (u64)t.lin_strides[d];
+      ok = ok && ((u64)c[d] < (u64)t.lin_dims[d]);
+      k += (u64)c[d] * (u64)t.lin_strides[d];
     }
   }
   key = k;
@@ -182,14 +188,19 @@ __device__ __forceinline__ bool dok_load_key8(const DevTable &t, const void *key
   if (KF == DOK_KF_ROWS) return dok_linearise(t, (const i64 *)keys + i * t.lin_ndim, key);
   if (KF == DOK_KF_U64) { key = ((const u64 *)keys)[i]; return true; }
   if (KF == DOK_KF_COLS) {
+    i64 c[DOK_MAX_DIMS];
+    #pragma unroll
+    for (int d = 0; d < DOK_MAX_DIMS; d++) {
+      c[d] = 0;
+      if (d < t.lin_ndim) c[d] = ((const i64 *)keys)[(i64)d * n + i];
+    }
     bool ok = true;
     u64 k = 0;
     #pragma unroll
     for (int d = 0; d < DOK_MAX_DIMS; d++) {
       if (d < t.lin_ndim) {
-        const i64 c = ((const i64 *)keys)[(i64)d * n + i];
-        ok = ok && ((u64)c < (u64)t.lin_dims[d]);
-        k += (u64)c * (u64)t.lin_strides[d];
+        ok = ok && ((u64)c[d] < (u64)t.lin_dims[d]);
+        k += (u64)c[d] * (u64)t.lin_strides[d];
       }
     }
     key = k;
