@@ -235,6 +235,8 @@ class CudaClosedHashmap:
         h = self._header.cpu()
         n_full = int(h[_lib.DOK_H_NFULL])
         if n_full:
+            # reported once, by the first read after the batch that overflowed
+            self._header[_lib.DOK_H_NFULL] = 0
             raise RuntimeError(f"hashmap is full: {n_full} rows could not be stored")
         return h
 
@@ -479,6 +481,22 @@ class CudaClosedHashmap:
     def _physical_slots(self):
         return self._n_phys * self._slots_per_bucket
 
+    def _growth_limit(self):
+        """Entries beyond which `set` grows the table (reference: :365).  A threshold above 1
+        switches growth off, as in the reference; rows that then find no slot are not lost
+        silently: the `set` that overflowed raises (see _launch_checked)."""
+        return int(self._rehash_threshold * self._n_buckets)
+
+    def _launch_checked(self, launch, n):
+        """Run an insert of n rows that stays under the growth limit.  If the rows might not fit
+        physically (only possible with a threshold above 1), the header is read back right away
+        so that an overflow raises in the call that caused it."""
+        risky = self._n_upper + n > self._physical_slots()
+        launch()
+        self._n_upper += n
+        if risky:
+            self.n_elements
+
     def set(self, new_keys, new_values):
         """Upsert a batch (reference: cuda_closed_hashmap.py:321-384).  Returns None."""
         assert new_keys.shape[0] == new_values.shape[0]
@@ -499,17 +517,15 @@ class CudaClosedHashmap:
 
     def _set_rows(self, keys, values):
         n = keys.shape[0]
-        limit = int(self._rehash_threshold * self._n_buckets)
+        limit = self._growth_limit()
         if self._n_upper + n <= limit:
             # cannot cross the threshold whatever the batch holds: no read-back, no sync
-            self._launch_set(keys, values)
-            self._n_upper += n
+            self._launch_checked(lambda: self._launch_set(keys, values), n)
             return
         self._ensure_cleared()
         n_old = self.n_elements
         if n_old + n <= limit:
-            self._launch_set(keys, values)
-            self._n_upper = n_old + n
+            self._launch_checked(lambda: self._launch_set(keys, values), n)
             return
         if n_old + n <= int(0.9 * self._physical_slots()):
             # the batch fits physically: insert, then apply the reference's growth rule to the
@@ -524,16 +540,14 @@ class CudaClosedHashmap:
         # (counted by a kernel that writes one number: no value rows, no flags)
         n_miss = n - int(self.count_existing(keys).item())
         if n_old + n_miss <= limit:
-            self._launch_set(keys, values)
-            self._n_upper = n_old + n_miss
+            self._launch_checked(lambda: self._launch_set(keys, values), n_miss)
             return
         # otherwise count the distinct new keys exactly, as the reference does
         _, is_found = self.get(keys)
         n_new = self._count_distinct(keys[~is_found])
         if n_old + n_new > limit:
             self.rehash(int((n_old + n_new) * self._rehash_factor))
-        self._launch_set(keys, values)
-        self._n_upper = n_old + n_new
+        self._launch_checked(lambda: self._launch_set(keys, values), n_new)
 
     def set_coo(self, indices, values):
         """`set` for a coordinate-keyed map with the coordinates laid out as a COO tensor holds
@@ -567,16 +581,14 @@ class CudaClosedHashmap:
         def launch():
             self._launch_set(indices, values, coo=True)
 
-        limit = int(self._rehash_threshold * self._n_buckets)
+        limit = self._growth_limit()
         if self._n_upper + n <= limit:
-            launch()
-            self._n_upper += n
+            self._launch_checked(launch, n)
             return
         self._ensure_cleared()
         n_old = self.n_elements
         if n_old + n <= limit:
-            launch()
-            self._n_upper = n_old + n
+            self._launch_checked(launch, n)
         elif n_old + n <= int(0.9 * self._physical_slots()):
             launch()
             n_now = self.n_elements
@@ -750,6 +762,10 @@ class CudaClosedHashmap:
         if not self._allocated:
             self._n_buckets = n_buckets
             return
+        if n_buckets < self._n_upper:
+            n_now = self.n_elements
+            if n_buckets < n_now:
+                raise ValueError(f"rehash({n_buckets}): the map holds {n_now} entries")
         lib = _lib.load()
         old = (self._table, self._header, self._desc)
         self._seed = int(np.random.randint(1, 2**62, dtype=np.int64))

@@ -65,12 +65,6 @@
 #define DOK_BULK_GRID 1024                  // most workgroups the first pass and the merge are given
 #endif
 
-#ifdef DOK_BULK_TIMING
-#define BULK_TICK(k) do { if (threadIdx.x == 0) { const u64 now_ = wall_clock64(); tacc[k] += now_ - tlast; tlast = now_; } } while (0)
-#else
-#define BULK_TICK(k) do { } while (0)
-#endif
-
 // Device view of the caller's workspace.
 struct BulkWs {
   u64 *keysA, *keysB;       // [n] each: rows after the first / second scatter
@@ -316,10 +310,6 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
   __shared__ u32 wsum[16];
   const int tid = threadIdx.x;
   int n_fresh = 0, n_oob = 0;
-#ifdef DOK_BULK_TIMING
-  u64 tacc[6] = {0, 0, 0, 0, 0, 0};
-  u64 tlast = wall_clock64();
-#endif
 
   // this workgroup's stretch of the input and its private write cursor of every bin
   i64 lo0, hi0;
@@ -409,7 +399,6 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
       if (tid * BPT + q < NB) cnt[tid * BPT + q] = 0;
     finish_tile(lo);
     __syncthreads();
-    BULK_TICK(0);
 
     // bins of the tile's rows and their ranks inside the bins
     int bn[RPT];
@@ -431,7 +420,6 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     for (int j = 0; j < RPT; j++)
       if (bn[j] >= 0) rk[j] = atomicAdd(&cnt[bn[j]], 1u);
     __syncthreads();
-    BULK_TICK(1);
 
     // bin offsets inside the tile, and where in global memory each bin's run goes
     u32 c[BPT], csum = 0;
@@ -452,7 +440,6 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
       ex += c[q];
     }
     __syncthreads();
-    BULK_TICK(2);
 
     #pragma unroll
     for (int j = 0; j < RPT; j++) {
@@ -465,7 +452,6 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     }
     if (lo + T < hi0) load_tile(lo + T);
     __syncthreads();
-    BULK_TICK(3);
 
     #pragma unroll
     for (int j = 0; j < RPT; j++) {
@@ -477,15 +463,8 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
         out_vals[dst] = svals[pos];
       }
     }
-    BULK_TICK(4);
     // the barriers at the top of the next tile order these reads before the next writes
   }
-#ifdef DOK_BULK_TIMING
-  if (threadIdx.x == 0 && LEVEL == DOK_BULK_TIMING) {
-    const int hslot[6] = {5, 6, 7, 12, 13, 14};
-    for (int q = 0; q < 6; q++) atomicAdd((u64 *)&t.header[hslot[q]], tacc[q]);
-  }
-#endif
   if (LEVEL == 1) {
     dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
     dok_wave_add_n(&t.header[DOK_H_NOOB], n_oob);
@@ -536,10 +515,6 @@ __device__ __forceinline__ int bulk_nth_bit(u32 m, u32 n) {
 // neither a clear of the table nor its read is paid for.
 template <int V, bool FRESH>
 __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, BulkWs ws) {
-#ifdef DOK_BULK_TIMING
-  u64 tacc[6] = {0, 0, 0, 0, 0, 0};
-  u64 tlast = wall_clock64();
-#endif
   typedef typename ValT<V>::type VT;
   constexpr int S = P8<V>::S;
   constexpr int R = DOK_BULK_R;
@@ -575,7 +550,6 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   __syncthreads();
 
   for (u32 p = p_lo; p < p_hi; p++) {
-    BULK_TICK(4);
     const u32 lo = ws.part_off[p], hi = ws.part_off[p + 1];
     const u32 carried = n_carry;                     // rows handed on by the range before (they sit
                                                      // at the head of the list already)
@@ -654,7 +628,6 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
       // zeroes of the empty copy)
       if (!fr || c0 == lo) __syncthreads();
       if (!FRESH && c0 == lo) fr = range_live == 0;
-      BULK_TICK(0);
 
       // look: act[j] = 0 nothing left to do, 1 write key and value into `slot`, 2 defer
       int act[RPT], slot[RPT];
@@ -742,7 +715,6 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
         }
       }
       if (!fr) __syncthreads();
-      BULK_TICK(1);
       // write
       #pragma unroll
       for (int j = 0; j < RPT; j++) {
@@ -765,7 +737,6 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           }
         }
       }
-      BULK_TICK(2);
 #undef BULK_VAL
     }
     __syncthreads();
@@ -813,7 +784,6 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
       if (tid == 0) n_carry = 0;                     // every thread has read it at the top of the range
     }
     __syncthreads();
-    BULK_TICK(3);
     const u32 total = n_list < (u32)DOK_BULK_LIST ? n_list : (u32)DOK_BULK_LIST;
     for (u32 e = tid; e < total; e += R) {
       const u64 key = lkey[e];
@@ -952,7 +922,6 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
         }
       }
     }
-    BULK_TICK(5);
     __syncthreads();
     {
       // the carried rows move to the head of the list, where the next range expects them
@@ -967,7 +936,6 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
       if (tid == 0) { n_carry = nc; range_live = 0; }
     }
     __syncthreads();
-    BULK_TICK(4);
 
     for (u32 u = tid; u < nbk * 8; u += R) {
       const u32 lb = u >> 3, w = (u & 7) * 2;
@@ -977,14 +945,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
       g[u] = y;
     }
     __syncthreads();
-    BULK_TICK(0);
   }
-#if defined(DOK_BULK_TIMING) && DOK_BULK_TIMING == 3
-  if (threadIdx.x == 0) {
-    const int hslot[6] = {5, 6, 7, 12, 13, 14};
-    for (int q = 0; q < 6; q++) atomicAdd((u64 *)&t.header[hslot[q]], tacc[q]);
-  }
-#endif
 
   // one header update per workgroup
   #pragma unroll

@@ -210,6 +210,16 @@ class SparseDOKTensor(object):
             return torch.empty(self.ndim, 0, device=self.device, dtype=torch.long)
         return idx[list(self._perm)] if self._is_permuted() else idx
 
+    def _items_coo_view(self):
+        """(indices [ndim, nnz] in this view's dimension order, values [nnz, 1]) from one pass."""
+        idx, values = self._hashmap.items_coo()
+        if idx is None:
+            return (torch.empty(self.ndim, 0, device=self.device, dtype=torch.long),
+                    torch.empty(0, 1, device=self.device, dtype=self.dtype))
+        if self._is_permuted():
+            idx = idx[list(self._perm)].contiguous()
+        return idx, values
+
     def values(self):
         values = self._hashmap.values()
         if values is None:
@@ -474,10 +484,12 @@ class SparseDOKTensor(object):
             return
         hm = self._hashmap
         if not hm._allocated:
-            # fixes the key/value widths; the entry itself is written again by the kernel below
+            # The reference stores the first element before anything else (sparse_dok_tensor_impl.py:
+            # 413-416), which its growth rule then counts; the kernel below writes it again.
             mats, _ = self._handle_selectors(expr)
             first_key = torch.stack([s.reshape(-1)[0] for s in self._to_storage_order(mats)], dim=0)[None]
             hm.set(first_key, src.reshape(-1)[:1, None].contiguous())
+            hm._header[_lib.DOK_H_NOOB] = 0       # an out-of-range first key is counted by the kernel below
         view = DokView()
         view.data = src.data_ptr()
         for j, st in enumerate(src.stride()):
@@ -531,12 +543,9 @@ class SparseDOKTensor(object):
         """Reference: set_items_sparse (sparse_dok_tensor_impl.py:235-340): clear every addressed
         element, grow, then store the source's nonzero entries through the selectors."""
         if isinstance(src, SparseDOKTensor):
-            keys, vals = src.storage().items()
-            if keys is None:
-                src_indices = torch.empty(src.ndim, 0, device=self.device, dtype=torch.long)
-                src_values = torch.empty(0, device=self.device, dtype=self.dtype)
-            else:
-                src_indices, src_values = keys.T.contiguous(), vals.flatten()
+            # coordinates in the order of the source's (possibly permuted) view
+            src_indices, vals = src._items_coo_view()
+            src_values = vals.flatten()
         else:
             if src.layout != torch.sparse_coo:
                 src = src.to_sparse_coo()
@@ -546,8 +555,10 @@ class SparseDOKTensor(object):
         src_values = src_values.to(device=self.device, dtype=self.dtype).contiguous()
         hm = self._hashmap
         if not hm._allocated:
+            # (reference: sparse_dok_tensor_impl.py:237-240)
             first_key = torch.stack([s.reshape(-1)[0] for s in self._to_storage_order(selectors)], dim=0)[None]
             hm.set(first_key, torch.zeros(1, 1, device=self.device, dtype=self.dtype))
+            hm._header[_lib.DOK_H_NOOB] = 0
         ix, _ = self._index_desc(selectors)
         lib = _lib.load()
         stream = _stream_ptr(self.device)

@@ -155,12 +155,12 @@ def test_bulk_reserved_patterns_and_full_table(cuda, bulk_always):
     hm = CudaClosedHashmap(n_buckets=100, device=cuda, rehash_threshold=1e9)
     keys = _unique_i64(np.random.default_rng(2), 400)[:, None]
     v = np.arange(400, dtype=np.float32)[:, None]
-    hm.set(*_to(cuda, keys, v))
-    with pytest.raises(RuntimeError):
-        hm.n_elements
-    slots = hm._n_phys * hm._slots_per_bucket
+    slots = 10 * 10                                  # 100 slots asked for = 10 buckets of 10
+    with pytest.raises(RuntimeError, match=f"full: {400 - slots} rows"):
+        hm.set(*_to(cuda, keys, v))
+    assert slots == hm._n_phys * hm._slots_per_bucket
     h = hm._header.cpu()
-    assert int(h[0]) == slots and int(h[1]) == 400 - slots
+    assert int(h[0]) == slots and int(h[1]) == 0     # reported once, then cleared
     out, found = hm.get(torch.from_numpy(keys).to(cuda))
     assert int(found.sum().item()) == slots
     assert torch.equal(out[found].cpu(), torch.from_numpy(v)[found.cpu()])

@@ -262,9 +262,11 @@ def test_tiny_and_full_tables(cuda):
     hm = CudaClosedHashmap(n_buckets=8, device=cuda, rehash_threshold=100.0)
     n_slots = 10   # one packed bucket of 8-byte keys / 4-byte values
     keys = torch.arange(n_slots + 6, device=cuda)[:, None]
-    hm.set(keys, torch.ones(n_slots + 6, 1, device=cuda))
-    with pytest.raises(RuntimeError, match="full"):
-        hm.n_elements
+    with pytest.raises(RuntimeError, match="full: 6 rows"):      # raised by the call that overflowed
+        hm.set(keys, torch.ones(n_slots + 6, 1, device=cuda))
+    assert hm.n_elements == n_slots                               # reported once; the map stays usable
+    _, f = hm.get(keys)
+    assert int(f.sum().item()) == n_slots
 
 
 def test_api_edges(cuda):
