@@ -15,6 +15,7 @@ DOK_OK = 0
 DOK_EINVAL = -1
 DOK_EUNSUPPORTED = -2
 DOK_ELAUNCH = -3
+DOK_ETOOLARGE = -4
 
 DOK_BUCKET_BYTES = 128
 DOK_MAX_DIMS = 8
@@ -78,6 +79,8 @@ SIGNATURES = {
     "dok_map_count_existing": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p]),
     "dok_compact_scratch_bytes": (c_int64, [POINTER(DokTable)]),
     "dok_map_compact": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
+    "dok_static_scratch_bytes": (c_int64, []),
+    "dok_map_compact_static": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "dok_coo_set": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p]),
     "dok_coo_compact": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "dok_map_rehash": (c_int32, [POINTER(DokTable), POINTER(DokTable), c_void_p]),
@@ -127,7 +130,11 @@ def check(rc, what):
     if rc == DOK_EINVAL:
         raise AssertionError(f"{what}: invalid argument")
     if rc == DOK_EUNSUPPORTED:
-        raise NotImplementedError(f"{what}: key/value width not supported by the table layouts")
+        raise NotImplementedError(f"{what}: not supported by the table layouts (a key/value row too wide for a "
+                                  "128-byte bucket, or a linearised coordinate space of 2^63 or more elements)")
+    if rc == DOK_ETOOLARGE:
+        raise ValueError(f"{what}: the table is larger than the library's own scratch memory serves; "
+                         "use the variant that takes a scratch buffer")
     if rc == DOK_ELAUNCH:
         msg = load().dok_last_hip_error().decode()
         raise DokError(f"{what}: HIP launch failed: {msg}")

@@ -4,14 +4,48 @@
 // device memory or synchronises.
 #include <hip/hip_runtime.h>
 #include <string.h>
+#include <atomic>
 #include "dok_device.h"
 #include "dok_packed8.h"
 #include "dok_tagged.h"
 #include "dok_bulk.h"
 
+// Scratch of dok_map_compact_static: device memory that belongs to the library, so that the call
+// needs no buffer from its caller.  Every GPU the library runs on holds its own copy of the array,
+// at its own address, from the moment the code object is loaded until the process ends.  In host
+// code this name is only a handle for hipGetSymbolAddress - never a pointer to hand to a kernel.
+static __device__ __align__(256) unsigned char dok_static_scratch[DOK_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char g_last_error[256] = "";
+
+// Device address of dok_static_scratch on each GPU, resolved at the first call on that GPU.
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_static_scratch[kMaxDevices];
+
+int static_scratch_of_current_device(void **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess && (dev < 0 || dev >= kMaxDevices)) e = hipErrorInvalidDevice;
+  void *p = nullptr;
+  if (e == hipSuccess) {
+    p = g_static_scratch[dev].load(std::memory_order_acquire);
+    if (!p) {
+      // (two threads may both get here: they obtain the same address)
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(dok_static_scratch));
+      if (e == hipSuccess && !p) e = hipErrorInvalidSymbol;
+      if (e == hipSuccess) g_static_scratch[dev].store(p, std::memory_order_release);
+    }
+  }
+  if (e != hipSuccess) {
+    strncpy(g_last_error, hipGetErrorString(e), sizeof(g_last_error) - 1);
+    g_last_error[sizeof(g_last_error) - 1] = 0;
+    return DOK_ELAUNCH;
+  }
+  *out = p;
+  return DOK_OK;
+}
 
 int note_launch() {
   hipError_t e = hipGetLastError();
@@ -392,6 +426,21 @@ int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out, int6
     if (rc) return rc;
   }
   return note_launch();
+}
+
+int64_t dok_static_scratch_bytes(void) { return DOK_STATIC_SCRATCH_BYTES; }
+
+int dok_map_compact_static(const dok_table_t *t, void *keys_out, void *values_out, int64_t capacity_rows,
+                           int64_t *count_out, void *stream) {
+  const int64_t need = dok_compact_scratch_bytes(t);
+  if (need < 0) return (int)need;
+  if (need > DOK_STATIC_SCRATCH_BYTES) return DOK_ETOOLARGE;     // before anything is launched
+  void *scratch = nullptr;
+  int rc = static_scratch_of_current_device(&scratch);
+  if (rc) return rc;
+  // every word of the scratch that is read is written first (chunk counts, then their prefix
+  // sums), so what an earlier call left behind does not matter
+  return dok_map_compact(t, keys_out, values_out, capacity_rows, count_out, scratch, stream);
 }
 
 int dok_coo_compact(const dok_table_t *t, int64_t *indices_out, void *values_out, int64_t capacity,

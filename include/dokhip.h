@@ -29,6 +29,7 @@ extern "C" {
 #define DOK_EINVAL       -1   /* bad argument (null pointer, negative count, misaligned buffer)   */
 #define DOK_EUNSUPPORTED -2   /* key/value width the table layouts cannot hold                   */
 #define DOK_ELAUNCH      -3   /* the HIP runtime refused a launch; see dok_last_hip_error()      */
+#define DOK_ETOOLARGE    -4   /* the table needs more scratch than dok_map_compact_static owns   */
 
 #define DOK_BUCKET_BYTES  128
 #define DOK_MAX_DIMS      8
@@ -177,6 +178,21 @@ int64_t dok_compact_scratch_bytes(const dok_table_t *t);
  * Reference: nonempty_mask / keys() / values() (cuda_closed_hashmap.py:157-172). */
 int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out,
                     int64_t capacity_rows, int64_t *count_out, void *scratch, void *stream);
+
+/* dok_map_compact for callers that cannot provide scratch memory because they cannot allocate:
+ * code under HIP graph capture, serving loops and harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  The scratch is a device array of DOK_STATIC_SCRATCH_BYTES that
+ * the library itself holds on every GPU it runs on (dok_static_scratch_bytes() returns that
+ * size); the call allocates and frees nothing.  Same outputs, in the same order, as
+ * dok_map_compact on the same table.
+ *   - A table whose dok_compact_scratch_bytes exceeds that size (more than about 2^28 buckets) is
+ *     refused with DOK_ETOOLARGE before anything is launched: use dok_map_compact.
+ *   - All calls on one GPU share the one array: calls that may overlap (different streams,
+ *     different host threads) race and must be ordered by the caller. */
+#define DOK_STATIC_SCRATCH_BYTES (8 << 20)
+int64_t dok_static_scratch_bytes(void);
+int dok_map_compact_static(const dok_table_t *t, void *keys_out, void *values_out,
+                           int64_t capacity_rows, int64_t *count_out, void *stream);
 
 /* Re-insert every live entry of src into dst (same key/value widths; dst cleared by the
  * caller; dst may have another size, seed or lin_dims of equal volume).

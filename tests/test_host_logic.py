@@ -84,6 +84,18 @@ def test_bad_descriptors_are_rejected_without_a_launch():
         _lib.check(_lib.DOK_EINVAL, "x")
 
 
+def test_static_compact_size_check_needs_no_gpu():
+    lib = _lib.load()
+    assert lib.dok_static_scratch_bytes() == 8 << 20
+    t = _lib.DokTable()
+    t.buckets, t.header, t.key_bytes, t.value_bytes = 4096, 8192, 8, 4
+    t.n_phys_buckets = (1 << 28) + 256              # one chunk counter more than the scratch holds
+    assert lib.dok_compact_scratch_bytes(ctypes.byref(t)) > lib.dok_static_scratch_bytes()
+    assert lib.dok_map_compact_static(ctypes.byref(t), None, None, 0, 8, None) == _lib.DOK_ETOOLARGE
+    with pytest.raises(ValueError):
+        _lib.check(_lib.DOK_ETOOLARGE, "x")
+
+
 def test_hashmap_before_any_set():
     hm = CudaClosedHashmap(n_buckets=64, device="cpu")
     assert hm.n_buckets == 64 and hm.n_elements == 0 and len(hm) == 0
