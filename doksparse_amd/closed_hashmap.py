@@ -785,15 +785,12 @@ class CudaClosedHashmap:
                 self._clear_table(desc)
                 _lib.check(lib.dok_map_rehash(ctypes.byref(old[2]), ctypes.byref(desc),
                                               _stream_ptr(self.device)), "rehash")
-            self._table, self._header, self._desc, self._n_phys = table, header, desc, n_phys
-            self._n_buckets = n_buckets
         else:
             self._clear_table(desc)
-            keys, values = self.items()
-            self._table, self._header, self._desc, self._n_phys = table, header, desc, n_phys
-            self._n_buckets = n_buckets
-            if keys.shape[0]:
-                self._launch_set(self._prep_rows(keys.reshape(-1, *self._key_shape), "keys"), values.contiguous())
+            _lib.check(lib.dok_map_rehash(ctypes.byref(old[2]), ctypes.byref(desc),
+                                          _stream_ptr(self.device)), "rehash")
+        self._table, self._header, self._desc, self._n_phys = table, header, desc, n_phys
+        self._n_buckets = n_buckets
         # the old table tensors stay referenced by `old` until the copies above are enqueued;
         # torch's allocator orders their reuse on the same stream
         del old

@@ -1,37 +1,42 @@
 // Tagged layout: keys and values of any width with 8*(1 + ceil(K/8) + ceil(V/8)) <= 128.
 //
 // A slot is W = 1 + KW + VW consecutive 8-byte words of a bucket:
-//     word 0            tag / lock word   (the only word ever CAS'd)
+//     word 0            low half:  tag / lock (the only 32 bits ever CAS'd)
+//                       high half: bucket metadata (slot 0 only, see below; zero elsewhere)
 //     words 1 .. KW     the key bytes, zero padded to 8*KW
 //     then VW words     the value bytes, zero padded to 8*VW
-// and a 128-byte bucket holds S = 16 / W slots.  Tag values:
+// and a 128-byte bucket holds S = 16 / W slots.  Tag values (32 bits):
 //     0                  EMPTY
 //     1                  TOMBSTONE
-//     (h & ~3) | 2       BUSY: claimed by a writer of a key whose 62-bit tag hash is h; key and
+//     (f & ~3) | 2       BUSY: claimed by a writer of a key whose 30-bit fingerprint is f; key and
 //                        value words are being written
-//     (h & ~3) | 3       FULL: key and value words are valid
+//     (f & ~3) | 3       FULL: key and value words are valid
 // Identity is always the full key: a tag match only selects the slots whose key words are then
 // compared, lane-parallel, against the query (each lane of the group holds one word of the
 // bucket and compares it with the word it should be).
 //
-// Query keys are staged in LDS as zero-padded words, one row per thread of the workgroup, so
-// that any lane of a group can fetch "word p of the row being served".
+// Metadata (high half of word 0 of the bucket) describes the keys whose HOME is this bucket, like
+// the metadata word of the packed layout:
+//     bits 1..23   displacement map: bit d set = some key was placed d buckets past this one
+//     bit 0        a key was placed 24 or more buckets past this one ...
+//     bits 24..31  ... and the largest such displacement, 255 standing for "255 or more"
+// Placement is linear probing over buckets (first free slot of the walk, a tombstone before an
+// EMPTY slot; a bucket never regains an EMPTY slot), so a lookup visits the home bucket and then
+// exactly the marked displacements - independent loads, no chain walk; with no mark set, the
+// home bucket alone decides a miss.  Only beyond 254 buckets does a lookup walk on until it
+// meets a bucket with an EMPTY slot.
+//
+// The rows a wave works on are staged in LDS as zero-padded words, one row per thread of the
+// workgroup, so that any lane of a group can fetch "word p of the row being served".
 #pragma once
 #include "dok_device.h"
 
-#define DOK_TG_EMPTY 0ULL
-#define DOK_TG_TOMB  1ULL
+#define DOK_TG_EMPTY 0u
+#define DOK_TG_TOMB  1u
 #define DOK_TG_MAXW  15
-// Ordering of "write the slot's key and value words" before "publish the FULL tag".  The data
-// words are written with agent-scope atomic stores, which gfx950 performs write-through to the
-// level every XCD shares; what remains to be ensured is that those stores have completed before
-// the tag store is issued, i.e. a wait for the wave's outstanding memory operations.  A
-// workgroup-scope release fence compiles to exactly that wait.  (An agent-scope release fence
-// adds a write-back of the whole L2, which exists for plain stores - there are none here - and
-// costs ten times the kernel's run time when issued once per inserted row.)
-#ifndef DOK_TG_RELEASE
-#define DOK_TG_RELEASE() __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup")
-#endif
+#define DOK_TG_NEAR  23                  // displacements with a bit of their own
+#define DOK_TG_NEARMASK 0x00fffffeu
+#define DOK_TG_FARCAP 255u               // stored largest far displacement saturates here
 
 struct TgGeom {
   int KW, VW, W, S;
@@ -75,135 +80,215 @@ __device__ __forceinline__ void tg_store_word(u8 *row, int k, int nbytes, int un
   }
 }
 
-// Per-thread preparation shared by all tagged batch kernels: stage the row's key words in LDS,
-// hash them, derive the home bucket and the FULL tag.
-__device__ __forceinline__ void tg_stage(const DevTable &t, const TgGeom &g, const u8 *keys, i64 i,
-                                         bool active, u64 *lds_keys, u32 &home, u64 &tag_full) {
+// LDS row of a staged batch row: word 0 = the row's FULL tag (low half), words 1 .. KW = the
+// zero-padded key words - exactly what the tag lane and the key lanes of a matching slot hold, so
+// lane p of a slot compares its bucket word with word p of the row.
+__device__ __forceinline__ int tg_rs(const TgGeom &g) { return g.KW + 1; }
+
+// Hash the key words already staged at krow[1 .. KW]; stores the FULL tag at krow[0].
+__device__ __forceinline__ void tg_hash_row(const DevTable &t, const TgGeom &g, u64 *krow,
+                                            u32 &home, u32 &tag_full) {
   u64 h = t.seed;
-  const u8 *row = keys + (size_t)i * g.K;
-  for (int k = 0; k < g.KW; k++) {
-    const u64 w = active ? tg_load_word(row, k, g.K, g.unit_k) : 0;
-    lds_keys[threadIdx.x * g.KW + k] = w;
-    h = dok_fmix64(h ^ w) + 0x9E3779B97F4A7C15ULL * (u64)(k + 1);
-  }
+  for (int k = 0; k < g.KW; k++) h = dok_fmix64(h ^ krow[1 + k]) + 0x9E3779B97F4A7C15ULL * (u64)(k + 1);
   const u64 h1 = dok_fmix64(h);
-  home = dok_reduce(h1, t.nb);
-  tag_full = (dok_fmix64(h1 ^ 0xD6E8FEB86659FD93ULL) & ~3ULL) | 3ULL;
+  home = dok_reduce(h1, t.nb);                       // upper half of the hash
+  tag_full = ((u32)h1 & ~3u) | 3u;                   // lower half
+  krow[0] = (u64)tag_full;
 }
 
 // Lane geometry inside a 16-lane group.
 struct TgLane {
-  int lane, gbase, l, slot, p;
+  int lane, gbase, l, slot, p, tag_lane;
   bool valid, is_tag, is_key, is_val;
-  u32 slotmask;
+  bool upper; int sh;        // where the group's 16 ballot bits sit (see P8Lane)
   __device__ __forceinline__ TgLane(const TgGeom &g) {
     lane = threadIdx.x & 63;
     gbase = lane & 48;
     l = lane & 15;
     slot = l / g.W;
     p = l - slot * g.W;
+    tag_lane = slot * g.W;
     valid = slot < g.S;
     is_tag = valid && p == 0;
     is_key = valid && p >= 1 && p <= g.KW;
     is_val = valid && p > g.KW;
-    slotmask = ((1u << g.W) - 1u) << (slot * g.W);
+    upper = lane >= 32;
+    sh = lane & 16;
+  }
+  __device__ __forceinline__ u32 grp(u64 m) const {
+    const u32 x = upper ? (u32)(m >> 32) : (u32)m;
+    return (x >> sh) & 0xffffu;
   }
 };
 
-// Group-wide view of one bucket for the row being served.
-struct TgView {
-  u32 hit;      // bit at the tag lane of every slot that is FULL with this row's key
-  u32 tagonly;  // bit at the tag lane of every slot whose tag equals the row's FULL tag
-  u32 busy;     // ... whose tag is the row's BUSY tag
-  u32 empty, tomb;
+// Wave-uniform lane masks of the geometry, made once per kernel.
+struct TgMasks {
+  u64 tagm;      // valid tag lanes
+  u64 notkey;    // every lane that is not a key lane
+  u32 kmask;     // KW + 1 ones: the tag lane and the key lanes of one slot
+  __device__ __forceinline__ TgMasks(const TgGeom &g, const TgLane &L) {
+    tagm = dok_ballot(L.is_tag);
+    notkey = ~dok_ballot(L.is_key);
+    kmask = (1u << (g.KW + 1)) - 1u;
+  }
 };
 
-__device__ __forceinline__ TgView tg_inspect(const TgGeom &g, const TgLane &L, bool has, u64 w,
-                                             u64 qfull, const u64 *lds_row) {
-  u64 expect = qfull;
-  if (L.is_key) expect = lds_row[L.p - 1];
-  const bool eq = L.valid && (L.is_val || w == expect);
-  const u32 geq = (u32)(dok_ballot(has && eq) >> L.gbase) & 0xffffu;
-  const bool slot_hit = L.valid && ((geq & L.slotmask) == L.slotmask);
-  TgView v;
-  v.hit = (u32)(dok_ballot(has && slot_hit && L.is_tag) >> L.gbase) & 0xffffu;
-  v.tagonly = (u32)(dok_ballot(has && L.is_tag && w == qfull) >> L.gbase) & 0xffffu;
-  v.busy = (u32)(dok_ballot(has && L.is_tag && w == (qfull & ~1ULL)) >> L.gbase) & 0xffffu;
-  v.empty = (u32)(dok_ballot(has && L.is_tag && w == DOK_TG_EMPTY) >> L.gbase) & 0xffffu;
-  v.tomb = (u32)(dok_ballot(has && L.is_tag && w == DOK_TG_TOMB) >> L.gbase) & 0xffffu;
-  return v;
+// Which slots of the buckets the wave just loaded (one per group, word `w` per lane) hold the key
+// of the row each group is serving: `expect` is the lane's word of that row (tag lanes: the FULL
+// tag, key lanes: the key word; other lanes: anything).  Returns a wave mask with a bit at the tag
+// lane of every matching slot.  Two compares, one shift and one compare per lane; the rest is
+// scalar mask arithmetic.
+__device__ __forceinline__ u64 tg_match64(const TgLane &L, const TgMasks &M, u64 w, u64 expect) {
+  const u64 mlo = __builtin_amdgcn_ballot_w64((u32)w == (u32)expect);
+  const u64 mhi = __builtin_amdgcn_ballot_w64((u32)(w >> 32) == (u32)(expect >> 32));
+  const u64 m = mlo & (mhi | M.notkey);              // tag lanes: low half only (the high half is metadata)
+  const u32 bits = (u32)(m >> L.lane) & M.kmask;
+  return __builtin_amdgcn_ballot_w64(bits == M.kmask) & M.tagm;
+}
+
+__device__ __forceinline__ u32 tg_wrap(u32 home, u32 d, u64 nb) {
+  const u64 b = (u64)home + d;
+  return (u32)(b >= nb ? b - nb : b);
 }
 
 // mode 0: get (write value or fallback + flag), 1: count, 2: remove.
 // Rows are taken in tiles of DOK_TPB (see DOK_TILE_LOOP); a wave only ever reads the LDS rows its
 // own lanes staged, so the tiles need no workgroup barrier between them.
+// Phase 1 serves the home bucket of each of a group's 16 rows as "issue 8 loads, resolve 8
+// rounds"; a round is a handful of instructions (tg_match64), and the value lanes of a matching
+// slot write the output row straight from the bucket words they hold.  Rows without a match are
+// finished by their owner lane: it reads the home bucket's metadata (the line has just been
+// fetched) and, with no displacement marked, writes the fallback row.  Phase 2 serves the rows
+// whose home bucket carries displacement marks and held no match, four rows per group and turn,
+// each at its next marked bucket.
 template <int MODE, bool STATS>
 __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g, const u8 *__restrict__ keys, i64 n,
                                                             u8 *__restrict__ values, u8 *__restrict__ flags,
                                                             i64 *count) {
   extern __shared__ u64 lds[];
-  u64 *lds_keys = lds;                          // [DOK_TPB][KW]
-  u64 *lds_fb = lds + DOK_TPB * g.KW;           // [VW]
+  const int RS = tg_rs(g);
+  u64 *lds_rows = lds;                          // [DOK_TPB][1 + KW]
+  u64 *lds_fb = lds + DOK_TPB * RS;             // [VW]
   if (MODE == 0 && threadIdx.x < g.VW) lds_fb[threadIdx.x] = g.fallback[threadIdx.x];
   __syncthreads();
   const TgLane L(g);
+  const TgMasks M(g, L);
   const int wave_row0 = threadIdx.x & ~63;      // first LDS row of this wave
+  // the word of the served row this lane compares its bucket word with: word p of the row for the
+  // tag and key lanes (any word for the others)
+  const int my_word = (L.is_tag || L.is_key) ? L.p : 0;
+  const u64 *exp0 = lds_rows + (wave_row0 + L.gbase) * RS + my_word;   // round r: exp0[r * RS]
+  const int tl = L.gbase + L.tag_lane;          // wave lane of this lane's slot's tag
   int n_found = 0, n_removed = 0, n_probe = 0, n_ops = 0;
 
   DOK_TILE_LOOP(n) {
     const i64 i = DOK_TILE_ROW();
     const bool active = i < n;
-    u32 b; u64 tag_full;
-    tg_stage(t, g, keys, i, active, lds_keys, b, tag_full);
-    const i64 wave_i0 = i - L.lane;             // batch row of lane 0
-    bool pend = active, found = false, removed = false;
-    u64 iters = 0;
-
-    u64 pm = dok_ballot(pend);
-    while (pm != 0) {
-      const u32 sub = (u32)(pm >> L.gbase) & 0xffffu;
-      const bool has = sub != 0;
-      const int r = has ? __builtin_ctz(sub) : 0;
-      const int j = L.gbase + r;
-      const u32 qb = dok_shfl32(b, j);
-      const u64 qfull = dok_shfl64(tag_full, j);
-      const u64 w = t.buckets[(u64)(has ? qb : 0u) * 16 + L.l];
-      const TgView v = tg_inspect(g, L, has, w, qfull, lds_keys + (wave_row0 + j) * g.KW);
-      const bool resolved = v.hit != 0 || v.empty != 0;
-      if (MODE == 0 && has && resolved) {
-        // the value lanes of the matching slot (or, on a miss, of slot 0 with the fallback)
-        // write the output row directly
-        const int hit_slot = v.hit ? (__builtin_ctz(v.hit) / g.W) : 0;
-        if (L.is_val && L.slot == hit_slot) {
-          const int k = L.p - 1 - g.KW;
-          const u64 word = v.hit ? w : lds_fb[k];
-          tg_store_word(values + (size_t)(wave_i0 + j) * g.V, k, g.V, g.unit_v, word);
-        }
-      }
-      if (has && L.l == r) {
-        n_probe++;
-        if (v.hit) {
-          found = true; pend = false;
-          if (MODE == 2) {
-            u64 *tagp = t.buckets + (u64)b * 16 + __builtin_ctz(v.hit);
-            removed = atomicCAS(tagp, qfull, DOK_TG_TOMB) == qfull;
-          }
-        } else if (v.empty) {
-          pend = false;
-        } else {
-          b = (b + 1 == t.nb) ? 0u : b + 1;
-          if (++iters >= t.nb) {
-            pend = false;
-            if (MODE == 0) {
-              // full ring without an empty slot: absent; the owner writes the fallback itself
-              for (int k = 0; k < g.VW; k++)
-                tg_store_word(values + (size_t)i * g.V, k, g.V, g.unit_v, lds_fb[k]);
-            }
-          }
-        }
-      }
-      pm = dok_ballot(pend);
+    u64 *krow = lds_rows + threadIdx.x * RS;
+    {
+      const u8 *row = keys + (size_t)i * g.K;
+      for (int k = 0; k < g.KW; k++) krow[1 + k] = active ? tg_load_word(row, k, g.K, g.unit_k) : 0;
     }
+    u32 home, qfull;
+    tg_hash_row(t, g, krow, home, qfull);
+    if (!active) home = 0;
+    const i64 wave_i0 = i - L.lane;             // batch row of lane 0
+    u8 *out_g = MODE == 0 ? values + (size_t)(wave_i0 + L.gbase) * g.V : nullptr;   // output row of the group's row 0
+    u64 my_hit64 = 0;
+
+    const u64 am = dok_ballot(active);
+    if (am != 0) {
+      #pragma unroll
+      for (int r0 = 0; r0 < 16; r0 += 8) {
+        u64 w[8];
+        #pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const u32 qb = dok_shfl32(home, L.gbase + r0 + u);
+          w[u] = t.buckets[(u64)qb * 16 + L.l];
+        }
+        #pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const int r = r0 + u;
+          // lanes of the groups whose row r is a real row
+          const u64 tr = (am >> r) & 0x0001000100010001ULL;
+          const u64 on64 = (tr << 16) - tr;
+          const u64 hit64 = tg_match64(L, M, w[u], exp0[r * RS]) & on64;
+          if (MODE == 0 && L.is_val && ((hit64 >> tl) & 1ULL))
+            tg_store_word(out_g + (size_t)r * g.V, L.p - 1 - g.KW, g.V, g.unit_v, w[u]);
+          my_hit64 = L.l == r ? hit64 : my_hit64;
+        }
+      }
+    }
+    const u32 my_hit = L.grp(my_hit64);
+    bool found = active && my_hit != 0;
+    u32 sb = home, sw = my_hit ? (u32)__builtin_ctz(my_hit) : 0u;
+    n_probe += active;
+    // rows without a match: the home bucket's metadata decides between "absent" and "look on"
+    u32 my_meta = 0;
+    if (active && !found) my_meta = (u32)(t.buckets[(u64)home * 16] >> 32);
+    bool open = active && !found && my_meta != 0;
+    if (MODE == 0 && active && !found && !open) {
+      for (int k = 0; k < g.VW; k++)
+        tg_store_word(values + (size_t)i * g.V, k, g.V, g.unit_v, lds_fb[k]);
+    }
+
+    // phase 2: the marked displacements, then (rare) the far ones
+    u32 cand = open ? (my_meta & DOK_TG_NEARMASK) : 0u;
+    bool far = open && (my_meta & 1u);
+    const u32 far_max = my_meta >> 24;
+    u32 far_d = DOK_TG_NEAR + 1;
+    u64 pm = dok_ballot(open);
+    while (pm != 0) {
+      const u32 d0 = cand ? (u32)__builtin_ctz(cand) : far_d;
+      const u32 b0 = tg_wrap(home, d0, t.nb);
+      u32 rest = L.grp(pm);
+      int rr[4];
+      bool hs[4];
+      u64 w[4];
+      #pragma unroll
+      for (int k = 0; k < 4; k++) {
+        hs[k] = rest != 0;
+        rr[k] = hs[k] ? __builtin_ctz(rest) : 0;
+        rest &= rest - 1;
+        const u32 qb = dok_shfl32(b0, L.gbase + rr[k]);
+        w[k] = t.buckets[(u64)(hs[k] ? qb : 0u) * 16 + L.l];
+      }
+      bool act = false;
+      u32 h = 0, e = 0;
+      #pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const u64 hit64 = tg_match64(L, M, w[k], exp0[rr[k] * RS]) & dok_ballot(hs[k]);
+        const u32 em = L.grp(dok_ballot(hs[k] && L.is_tag && (u32)w[k] == DOK_TG_EMPTY));
+        if (MODE == 0 && L.is_val && ((hit64 >> tl) & 1ULL))
+          tg_store_word(out_g + (size_t)rr[k] * g.V, L.p - 1 - g.KW, g.V, g.unit_v, w[k]);
+        const bool mine = hs[k] && L.l == rr[k];
+        act = act || mine;
+        h = mine ? L.grp(hit64) : h;
+        e = mine ? em : e;
+      }
+      if (act) {
+        n_probe++;
+        if (h) {
+          found = true; open = false;
+          sb = b0; sw = (u32)__builtin_ctz(h);
+        } else {
+          if (cand) cand &= cand - 1;
+          else {
+            if (far_max == DOK_TG_FARCAP && e) far = false;     // beyond the recorded range the chain ends at an EMPTY slot
+            far_d++;
+          }
+          open = cand != 0 || (far && (far_max == DOK_TG_FARCAP ? (u64)far_d < t.nb : far_d <= far_max));
+          if (!open && MODE == 0) {
+            for (int k = 0; k < g.VW; k++)
+              tg_store_word(values + (size_t)i * g.V, k, g.V, g.unit_v, lds_fb[k]);
+          }
+        }
+      }
+      pm = dok_ballot(open);
+    }
+    bool removed = false;
+    if (MODE == 2 && found)
+      removed = atomicCAS((u32 *)(t.buckets + (u64)sb * 16 + sw), qfull, DOK_TG_TOMB) == qfull;
     if (MODE == 0 && active) flags[i] = found ? 1 : 0;
     if (MODE == 2 && active && flags) flags[i] = removed ? 1 : 0;
     n_found += found;
@@ -218,119 +303,204 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
   }
 }
 
-// Upsert.  Protocol per row (owner lane acts, the group inspects):
-//   * slot FULL with the row's key  -> lock it (CAS FULL->BUSY), rewrite the value words,
+// Record in the home bucket's metadata that a key was placed d > 0 buckets further on.
+__device__ __forceinline__ void tg_mark(u64 *home_bucket, u32 d, u32 md_seen) {
+  u32 *meta = (u32 *)home_bucket + 1;
+  if (d <= DOK_TG_NEAR) {
+    if (!((md_seen >> d) & 1u)) atomicOr(meta, 1u << d);
+    return;
+  }
+  const u32 dm = d < DOK_TG_FARCAP ? d : DOK_TG_FARCAP;
+  u32 old = __hip_atomic_load(meta, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (;;) {
+    u32 mx = old >> 24;
+    if (dm > mx) mx = dm;
+    const u32 nw = (old & 0x00ffffffu) | (mx << 24) | 1u;
+    if (nw == old) break;
+    const u32 prev = atomicCAS(meta, old, nw);
+    if (prev == old) break;
+    old = prev;
+  }
+}
+
+#define DOK_TG_MAXS 5            // most slots a bucket can have (W >= 3)
+
+// Upsert of the (up to 64) rows a wave has staged in LDS: lane x owns LDS row threadIdx.x (tag and
+// key words in lds_rows, value words in lds_vals).  Every lane inspects the current bucket of its
+// own row by itself - it reads just the S tag words (slot 0's comes with the bucket metadata) and,
+// only where a tag equals its own, that slot's key words - so a turn costs a few loads per row and
+// no cross-lane work.  Protocol per row:
+//   * a slot FULL with the row's key -> lock it (CAS FULL->BUSY), rewrite the value words,
 //     publish FULL again.  Losing that CAS means an equal key of this batch holds the lock:
 //     its value stands and this row is done.
 //   * a slot BUSY with the row's tag -> its key is not readable yet: look again next turn.
 //   * a slot FULL with the row's tag but other key words -> look once more after an acquire
-//     fence (the key words may have been read before the writer's stores landed); a second
-//     mismatch is a genuine tag collision and the slot is skipped.
-//   * chain end (bucket with an EMPTY slot, or the ring walked) -> claim the first tombstone
-//     seen, else the first empty slot: CAS ->BUSY, write key and value words, release fence,
-//     publish FULL.  Losing the claim restarts the walk from the home bucket.
-// A BUSY holder finishes in straight-line code inside one loop turn, so waiting rows always
-// see it released.
+//     fence; a second mismatch is a genuine fingerprint collision and the slot is skipped.
+//   * otherwise the row's place is the first free slot of its walk (a tombstone of that bucket
+//     before an EMPTY slot).  That the key does not sit further on is established through the
+//     home bucket's displacement map, as in the packed layout: the marked buckets beyond the
+//     chosen slot are looked at, then the slot is claimed (CAS -> BUSY).  A lost claim makes the
+//     row look at that bucket again.
+// The slots won in a turn are then written by the groups, one row per round: lane p of the group
+// stores word p of the slot, so a slot costs one contiguous store instead of W scattered ones;
+// after a wait for those stores the owners publish FULL together.  The data words are written
+// with agent-scope atomic stores (write-through to the level all XCDs share); a BUSY holder
+// finishes in straight-line code inside one loop turn, so waiting rows always see it released.
+__device__ __forceinline__ void tg_insert_rows(const DevTable &t, const TgGeom &g, const TgLane &L,
+                                               const u64 *lds_rows, const u64 *lds_vals, u32 home, u32 qfull,
+                                               bool pend, int &st, int &fresh) {
+  const int RS = tg_rs(g);
+  const int wave_row0 = threadIdx.x & ~63;
+  const u64 *krow = lds_rows + threadIdx.x * RS;
+  if (!pend) home = 0;
+  const u32 qbusy = qfull & ~1u;
+  u32 cur = 0, md_home = 0;                       // displacement inspected this turn; home metadata
+  bool chosen = false, slot_tomb = false, confirm = false, far_unb = false;
+  u32 slot_d = 0, slot_w = 0, chk = 0, far_next = 0, far_to = 0;
+
+  u64 pm = dok_ballot(pend);
+  while (pm != 0) {
+    if (dok_ballot(confirm) != 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    const u32 b = pend ? tg_wrap(home, cur, t.nb) : 0u;
+    u64 *bucket = t.buckets + (u64)b * 16;
+
+    // ---- every owner looks at the tags of its bucket
+    u64 tw[DOK_TG_MAXS];
+    #pragma unroll
+    for (int s = 0; s < DOK_TG_MAXS; s++) {
+      tw[s] = 0;
+      if (s < g.S && pend) tw[s] = dok_load_coherent(bucket + s * g.W);
+    }
+    const u32 md = (u32)(tw[0] >> 32);
+    u32 candm = 0, emptym = 0, tombm = 0;          // one bit per slot
+    bool busy = false;
+    #pragma unroll
+    for (int s = 0; s < DOK_TG_MAXS; s++) {
+      if (s < g.S) {
+        const u32 t32 = (u32)tw[s];
+        candm |= (u32)(t32 == qfull) << s;
+        busy = busy || t32 == qbusy;
+        emptym |= (u32)(t32 == DOK_TG_EMPTY) << s;
+        tombm |= (u32)(t32 == DOK_TG_TOMB) << s;
+      }
+    }
+    // slots with the row's tag: compare the key words
+    int hit_s = -1;
+    bool tagonly = false;
+    if (pend) {
+      u32 c = candm;
+      while (c != 0 && hit_s < 0) {
+        const int s = __builtin_ctz(c);
+        c &= c - 1;
+        bool eq = true;
+        for (int k = 0; k < g.KW; k++) eq = eq && dok_load_coherent(bucket + s * g.W + 1 + k) == krow[1 + k];
+        if (eq) hit_s = s; else tagonly = true;
+      }
+    }
+
+    bool wr = false, wr_fresh = false;
+    u32 wr_b = 0, wr_w = 0;
+    if (pend) {
+      if (hit_s >= 0) {
+        const u32 sw = (u32)(hit_s * g.W);
+        if (atomicCAS((u32 *)(bucket + sw), qfull, qbusy) == qfull) { wr = true; wr_b = b; wr_w = sw; }
+        st = 1; pend = false;
+      } else if (busy) {
+        // wait for the holder to publish
+      } else if (tagonly && !confirm) {
+        confirm = true;
+      } else {
+        confirm = false;
+        if (!chosen) {
+          if (cur == 0) md_home = md;
+          if (tombm | emptym) {
+            chosen = true;
+            slot_tomb = tombm != 0;
+            slot_d = cur;
+            slot_w = (u32)(__builtin_ctz(tombm ? tombm : emptym) * g.W);
+            chk = cur < DOK_TG_NEAR ? (md_home & DOK_TG_NEARMASK & ~((2u << cur) - 1u)) : 0u;
+            far_unb = (md_home & 1u) && (md_home >> 24) == DOK_TG_FARCAP;
+            far_to = (md_home & 1u) ? (far_unb ? 0xffffffffu : (md_home >> 24)) : 0u;
+            far_next = cur + 1 > DOK_TG_NEAR + 1u ? cur + 1 : DOK_TG_NEAR + 1u;
+          } else if ((u64)cur + 1 >= t.nb) {
+            st = 0; pend = false;                          // no free slot anywhere
+          } else {
+            cur++;
+          }
+        } else if (far_unb && cur > DOK_TG_NEAR && emptym) {
+          far_to = 0;                                      // beyond the recorded range the chain ends at an EMPTY slot
+        }
+        if (pend && chosen) {
+          bool claim = false;
+          if (chk) { cur = (u32)__builtin_ctz(chk); chk &= chk - 1; }
+          else if (far_next <= far_to && (u64)far_next < t.nb) cur = far_next++;
+          else claim = true;
+          if (claim) {
+            const u32 tb = tg_wrap(home, slot_d, t.nb);
+            u32 *tagp = (u32 *)(t.buckets + (u64)tb * 16 + slot_w);
+            const u32 expect = slot_tomb ? DOK_TG_TOMB : DOK_TG_EMPTY;
+            if (atomicCAS(tagp, expect, qbusy) == expect) {
+              wr = true; wr_fresh = true; wr_b = tb; wr_w = slot_w;
+              st = 1; fresh = 1; pend = false;
+              if (slot_d > 0) tg_mark(t.buckets + (u64)home * 16, slot_d, md_home);
+            } else {
+              chosen = false; cur = slot_d;                // somebody took the slot: look at that bucket again
+            }
+          }
+        }
+      }
+    }
+
+    // ---- the slots won in this turn: payload by the groups, then the owners publish
+    const u64 wm = dok_ballot(wr);
+    if (wm != 0) {
+      const u32 wsub = L.grp(wm);
+      u32 wany = (u32)wm | (u32)(wm >> 32);
+      wany = (wany | (wany >> 16)) & 0xffffu;
+      #pragma unroll
+      for (int r = 0; r < 16; r++) {
+        if (!((wany >> r) & 1u)) continue;
+        const int j = L.gbase + r;
+        const u32 qb = dok_shfl32(wr_b, j), qw = dok_shfl32(wr_w, j);
+        const int first = dok_shfl32((u32)wr_fresh, j) ? 1 : 1 + g.KW;
+        if (((wsub >> r) & 1u) && L.l >= first && L.l < g.W) {
+          const u64 word = L.l <= g.KW ? lds_rows[(wave_row0 + j) * RS + L.l]
+                                       : lds_vals[(wave_row0 + j) * g.VW + L.l - 1 - g.KW];
+          dok_store_coherent(t.buckets + (u64)qb * 16 + qw + L.l, word);
+        }
+      }
+      // the payload stores have completed before any tag is published
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (wr) __hip_atomic_store((u32 *)(t.buckets + (u64)wr_b * 16 + wr_w), qfull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    pm = dok_ballot(pend);
+  }
+}
+
 __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, const u8 *__restrict__ keys,
                                                          const u8 *__restrict__ values, i64 n,
                                                          u8 *__restrict__ stored) {
   extern __shared__ u64 lds[];
-  u64 *lds_keys = lds;
+  const int RS = tg_rs(g);
+  u64 *lds_rows = lds;                          // [DOK_TPB][1 + KW]
+  u64 *lds_vals = lds + DOK_TPB * RS;           // [DOK_TPB][VW]
   const TgLane L(g);
-  const int wave_row0 = threadIdx.x & ~63;
-  const u64 *krow = lds_keys + threadIdx.x * g.KW;
   int n_fresh = 0, n_full = 0;
 
   DOK_TILE_LOOP(n) {
     const i64 i = DOK_TILE_ROW();
     const bool active = i < n;
-    u32 home; u64 tag_full;
-    tg_stage(t, g, keys, i, active, lds_keys, home, tag_full);
-    u32 b = home, tomb_b = DOK_NONE32;
-    int tomb_w = 0;
-    bool pend = active, confirm = false;
-    int st = 0, fresh = 0;
-    u64 iters = 0;
-    const u8 *vrow = values + (size_t)i * g.V;
-
-    // Turns: in every turn the current bucket of EVERY pending row of the wave is inspected (the
-    // loads of eight rows per group in flight together), then all owner lanes act at once - the
-    // claims, the slot writes and the publishing stores of a whole wave overlap instead of
-    // following one another row by row.  The first turn looks at the home buckets and settles
-    // most rows; rows that walk on (bucket full, a lost claim, a slot that is being written, a
-    // tag collision) stay pending for the next turn.
-    u64 pm = dok_ballot(pend);
-    while (pm != 0) {
-      if (dok_ballot(confirm) != 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-      const u32 sub = (u32)(pm >> L.gbase) & 0xffffu;          // this group's pending rows
-      u32 any = (u32)pm | (u32)(pm >> 32);
-      any = (any | (any >> 16)) & 0xffffu;                      // row numbers pending in some group
-      TgView v;
-      v.hit = v.tagonly = v.busy = v.empty = v.tomb = 0;
-      #pragma unroll
-      for (int r0 = 0; r0 < 16; r0 += 8) {
-        if (((any >> r0) & 0xffu) == 0) continue;
-        u64 w[8];
-        #pragma unroll
-        for (int u = 0; u < 8; u++) {
-          const u32 qb = dok_shfl32(b, L.gbase + r0 + u);
-          w[u] = 0;
-          if ((sub >> (r0 + u)) & 1u) w[u] = dok_load_coherent(t.buckets + (u64)qb * 16 + L.l);
-        }
-        #pragma unroll
-        for (int u = 0; u < 8; u++) {
-          if (!((any >> (r0 + u)) & 1u)) continue;
-          const int j = L.gbase + r0 + u;
-          const u64 qfull = dok_shfl64(tag_full, j);
-          const TgView x = tg_inspect(g, L, ((sub >> (r0 + u)) & 1u) != 0, w[u], qfull, lds_keys + (wave_row0 + j) * g.KW);
-          if (L.l == r0 + u) v = x;
-        }
-      }
-      if (pend) {
-        u64 *bucket = t.buckets + (u64)b * 16;
-        const u64 qfull = tag_full, qbusy = tag_full & ~1ULL;
-        if (v.hit) {
-          u64 *slot = bucket + __builtin_ctz(v.hit);
-          if (atomicCAS(slot, qfull, qbusy) == qfull) {
-            for (int k = 0; k < g.VW; k++)
-              dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
-            DOK_TG_RELEASE();
-            dok_store_coherent(slot, qfull);
-          }
-          st = 1; pend = false;
-        } else if (v.busy) {
-          // wait for the holder to publish
-        } else if ((v.tagonly & ~v.hit) != 0 && !confirm) {
-          confirm = true;
-        } else {
-          confirm = false;
-          if (tomb_b == DOK_NONE32 && v.tomb) { tomb_b = b; tomb_w = __builtin_ctz(v.tomb); }
-          const bool ring_done = (v.empty == 0) && (++iters >= t.nb);
-          if (v.empty || ring_done) {
-            if (tomb_b == DOK_NONE32 && v.empty == 0) {
-              st = 0; pend = false;                         // no free slot anywhere
-            } else {
-              u64 *slot; u64 expect;
-              if (tomb_b != DOK_NONE32) { slot = t.buckets + (u64)tomb_b * 16 + tomb_w; expect = DOK_TG_TOMB; }
-              else { slot = bucket + __builtin_ctz(v.empty); expect = DOK_TG_EMPTY; }
-              if (atomicCAS(slot, expect, qbusy) == expect) {
-                for (int k = 0; k < g.KW; k++) dok_store_coherent(slot + 1 + k, krow[k]);
-                for (int k = 0; k < g.VW; k++)
-                  dok_store_coherent(slot + 1 + g.KW + k, tg_load_word(vrow, k, g.V, g.unit_v));
-                DOK_TG_RELEASE();
-                dok_store_coherent(slot, qfull);
-                st = 1; fresh = 1; pend = false;
-              } else {
-                b = home; tomb_b = DOK_NONE32; iters = 0;   // lost the claim: walk again
-              }
-            }
-          } else {
-            b = (b + 1 == t.nb) ? 0u : b + 1;
-          }
-        }
-      }
-      pm = dok_ballot(pend);
+    u64 *krow = lds_rows + threadIdx.x * RS;
+    {
+      const u8 *kin = keys + (size_t)i * g.K, *vin = values + (size_t)i * g.V;
+      for (int k = 0; k < g.KW; k++) krow[1 + k] = active ? tg_load_word(kin, k, g.K, g.unit_k) : 0;
+      for (int k = 0; k < g.VW; k++)
+        lds_vals[threadIdx.x * g.VW + k] = active ? tg_load_word(vin, k, g.V, g.unit_v) : 0;
     }
+    u32 home, qfull;
+    tg_hash_row(t, g, krow, home, qfull);
+    int st = 0, fresh = 0;
+    tg_insert_rows(t, g, L, lds_rows, lds_vals, home, qfull, active, st, fresh);
     if (active && stored) stored[i] = (u8)st;
     n_fresh += fresh;
     n_full += (active && st == 0);
@@ -339,7 +509,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, c
   dok_wave_add_n(&t.header[DOK_H_NFULL], n_full);
 }
 
-// ---- read-out ---------------------------------------------------------------------------------
+// ---- table scans: read-out and rehash -----------------------------------------------------------
 #ifndef DOK_CHUNK
 #define DOK_CHUNK 256
 #endif
@@ -347,7 +517,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, c
 __device__ __forceinline__ bool tg_scan_load(const DevTable &t, const TgLane &L, i64 b, u64 &w) {
   const bool valid = b < (i64)t.nb;
   w = t.buckets[(u64)(valid ? b : (i64)t.nb - 1) * 16 + L.l];
-  return valid && L.is_tag && (w & 3ULL) == 3ULL;
+  return valid && L.is_tag && ((u32)w & 3u) == 3u;
 }
 
 __global__ __launch_bounds__(DOK_TPB) void tg_chunk_count_kernel(DevTable t, TgGeom g, i64 *chunk_counts, i64 n_chunks) {
@@ -376,7 +546,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_chunk_write_kernel(DevTable t, TgG
     const bool live_tag = tg_scan_load(t, L, wid * DOK_CHUNK + s * 4 + (L.lane >> 4), w);
     const u64 m = dok_ballot(live_tag);
     // every lane of a live slot learns the slot's output row from the tag lane's position
-    const int tag_lane = L.gbase + L.slot * g.W;
+    const int tag_lane = L.gbase + L.tag_lane;
     const bool slot_live = L.valid && ((m >> tag_lane) & 1ULL);
     const i64 row = base + __popcll(m & ((1ULL << tag_lane) - 1ULL));
     if (slot_live && row < cap) {
@@ -385,6 +555,47 @@ __global__ __launch_bounds__(DOK_TPB) void tg_chunk_write_kernel(DevTable t, TgG
     }
     base += __popcll(m);
   }
+}
+
+// Re-insert every live entry of `src` into `dst` (same widths, cleared by the caller).  A wave
+// scans a chunk of the source four buckets per step; the lanes that hold the words of a live slot
+// put them into the wave's LDS rows, packed, and whenever the rows of another step might not fit
+// any more the wave inserts what it has gathered.
+__global__ __launch_bounds__(DOK_TPB) void tg_rehash_kernel(DevTable src, DevTable dst, TgGeom g, i64 n_chunks) {
+  extern __shared__ u64 lds[];
+  const int RS = tg_rs(g);
+  u64 *lds_rows = lds;
+  u64 *lds_vals = lds + DOK_TPB * RS;
+  const i64 wid = (i64)blockIdx.x * (DOK_TPB / 64) + (threadIdx.x >> 6);
+  const TgLane L(g);
+  const int wave_row0 = threadIdx.x & ~63;
+  int n_fresh = 0, n_full = 0;
+  if (wid < n_chunks) {
+    int cnt = 0;
+    for (int s = 0; s < DOK_CHUNK / 4; s++) {
+      u64 w;
+      const bool live_tag = tg_scan_load(src, L, wid * DOK_CHUNK + s * 4 + (L.lane >> 4), w);
+      const u64 m = dok_ballot(live_tag);
+      const int tag_lane = L.gbase + L.tag_lane;
+      const bool slot_live = L.valid && ((m >> tag_lane) & 1ULL);
+      const int row = wave_row0 + cnt + __popcll(m & ((1ULL << tag_lane) - 1ULL));
+      if (slot_live && L.is_key) lds_rows[row * RS + L.p] = w;
+      if (slot_live && L.is_val) lds_vals[row * g.VW + L.p - 1 - g.KW] = w;
+      cnt += __popcll(m);
+      if (cnt + 4 * g.S > 64 || s == DOK_CHUNK / 4 - 1) {
+        const bool pend = L.lane < cnt;
+        u32 home, qfull;
+        tg_hash_row(dst, g, lds_rows + threadIdx.x * RS, home, qfull);
+        int st = 0, fresh = 0;
+        tg_insert_rows(dst, g, L, lds_rows, lds_vals, home, qfull, pend, st, fresh);
+        n_fresh += fresh;
+        n_full += (pend && st == 0);
+        cnt = 0;
+      }
+    }
+  }
+  dok_wave_add_n(&dst.header[DOK_H_NELEM], n_fresh);
+  dok_wave_add_n(&dst.header[DOK_H_NFULL], n_full);
 }
 
 // ---- host launchers -----------------------------------------------------------------------------
@@ -406,7 +617,21 @@ static int tg_geom(const DevTable &d, const void *fallback, TgGeom &g) {
 
 static bool tg_aligned(const void *p, int unit) { return ((uintptr_t)p & (uintptr_t)(unit - 1)) == 0; }
 
-static size_t tg_lds_bytes(const TgGeom &g) { return (size_t)(DOK_TPB * g.KW + g.VW) * 8; }
+static size_t tg_lds_lookup(const TgGeom &g) { return (size_t)(DOK_TPB * (g.KW + 1) + g.VW) * 8; }
+static size_t tg_lds_insert(const TgGeom &g) { return (size_t)DOK_TPB * (g.KW + 1 + g.VW) * 8; }
+
+// Most workgroups of the kernels that loop over tiles and end with one atomic per wave on a
+// counter: few workgroups keep those atomics cheap (same-address atomics serialise at ~12 ns
+// each), many even out the differing amounts of work of the tiles.
+#ifndef DOK_TG_COUNT_GRID
+#define DOK_TG_COUNT_GRID 8192u
+#endif
+#ifndef DOK_TG_REMOVE_GRID
+#define DOK_TG_REMOVE_GRID 4096u
+#endif
+#ifndef DOK_TG_SET_GRID
+#define DOK_TG_SET_GRID 8192u
+#endif
 
 static int tg_launch_get(const DevTable &d, const void *keys, i64 n, void *values, const void *fallback,
                          u8 *found, bool stats, hipStream_t s) {
@@ -417,34 +642,19 @@ static int tg_launch_get(const DevTable &d, const void *keys, i64 n, void *value
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
   const unsigned cgrid = grid < 2048u ? grid : 2048u;
   if (stats)
-    tg_lookup_kernel<0, true><<<cgrid, DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr);
+    tg_lookup_kernel<0, true><<<cgrid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr);
   else
-    tg_lookup_kernel<0, false><<<grid, DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr);
+    tg_lookup_kernel<0, false><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr);
   return DOK_OK;
 }
 
-// Most workgroups of the kernels that loop over tiles and end with one atomic per wave on a
-// counter.  Few workgroups keep those atomics cheap (same-address atomics serialise at ~12 ns
-// each), many even out the long probe chains of a loaded table; measured on 32M float32[3] ->
-// int64[5] rows at load factors 0.5 / 0.9: count 1.58 / 10.2 ms with 2048 workgroups,
-// 1.46 / 5.6 ms with 8192; set 9.6 / 22.7 ms with 2048, 9.0 / 15.4 ms with 32768; remove of 8M
-// 0.68 / 1.10 ms with 2048, 1.65 / 2.35 ms with 32768.
-#ifndef DOK_TG_COUNT_GRID
-#define DOK_TG_COUNT_GRID 8192u
-#endif
-#ifndef DOK_TG_REMOVE_GRID
-#define DOK_TG_REMOVE_GRID 2048u
-#endif
-#ifndef DOK_TG_SET_GRID
-#define DOK_TG_SET_GRID 32768u
-#endif
 static int tg_launch_count(const DevTable &d, const void *keys, i64 n, i64 *count, hipStream_t s) {
   TgGeom g;
   int rc = tg_geom(d, nullptr, g);
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_lookup_kernel<1, false><<<(grid < DOK_TG_COUNT_GRID ? grid : DOK_TG_COUNT_GRID), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, nullptr, nullptr, count);
+  tg_lookup_kernel<1, false><<<(grid < DOK_TG_COUNT_GRID ? grid : DOK_TG_COUNT_GRID), DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, nullptr, nullptr, count);
   return DOK_OK;
 }
 
@@ -454,7 +664,7 @@ static int tg_launch_remove(const DevTable &d, const void *keys, i64 n, u8 *remo
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_lookup_kernel<2, false><<<(grid < DOK_TG_REMOVE_GRID ? grid : DOK_TG_REMOVE_GRID), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, n, nullptr, removed, nullptr);
+  tg_lookup_kernel<2, false><<<(grid < DOK_TG_REMOVE_GRID ? grid : DOK_TG_REMOVE_GRID), DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, nullptr, removed, nullptr);
   return DOK_OK;
 }
 
@@ -464,7 +674,15 @@ static int tg_launch_set(const DevTable &d, const void *keys, const void *values
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k) || !tg_aligned(values, g.unit_v)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_set_kernel<<<(grid < DOK_TG_SET_GRID ? grid : DOK_TG_SET_GRID), DOK_TPB, tg_lds_bytes(g), s>>>(d, g, (const u8 *)keys, (const u8 *)values, n, stored);
+  tg_set_kernel<<<(grid < DOK_TG_SET_GRID ? grid : DOK_TG_SET_GRID), DOK_TPB, tg_lds_insert(g), s>>>(d, g, (const u8 *)keys, (const u8 *)values, n, stored);
+  return DOK_OK;
+}
+
+static int tg_launch_rehash(const DevTable &a, const DevTable &b, i64 n_chunks, hipStream_t s) {
+  TgGeom g;
+  int rc = tg_geom(a, nullptr, g);
+  if (rc) return rc;
+  tg_rehash_kernel<<<(unsigned)((n_chunks + 3) / 4), DOK_TPB, tg_lds_insert(g), s>>>(a, b, g, n_chunks);
   return DOK_OK;
 }
 

@@ -472,10 +472,14 @@ int dok_map_rehash(const dok_table_t *src, const dok_table_t *dst, void *stream)
   if (a.key_bytes != b.key_bytes || a.value_bytes != b.value_bytes || a.lin_ndim != b.lin_ndim) return DOK_EINVAL;
   if (a.buckets == b.buckets) return DOK_EINVAL;
   for (int k = 0; k < a.lin_ndim; k++) if (a.lin_dims[k] != b.lin_dims[k]) return DOK_EINVAL;
-  if (la != DOK_LAYOUT_PACKED8) return DOK_EUNSUPPORTED;   // tagged tables rehash through compact + set
   hipStream_t s = (hipStream_t)stream;
   const i64 n_chunks = chunks_of(a);
-  P8_DISPATCH(a.value_bytes, (p8_rehash_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(a, b, n_chunks)));
+  if (la == DOK_LAYOUT_PACKED8) {
+    P8_DISPATCH(a.value_bytes, (p8_rehash_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(a, b, n_chunks)));
+  } else {
+    rc = tg_launch_rehash(a, b, n_chunks, s);
+    if (rc) return rc;
+  }
   return note_launch();
 }
 
