@@ -276,6 +276,53 @@ def other_configs(device):
     return res
 
 
+def tagged_scale(device, n=32_000_000):
+    """The tagged layout (keys / values wider than 8 bytes) at scale: n float32[3] keys -> int64[5]
+    values, the row shape of the reference README's hashmap example, at load factors 0.5 and 0.75.
+    Kernel-level timings through the C ABI on preallocated buffers."""
+    from doksparse_amd import CudaClosedHashmap, _lib
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    lib = _lib.load()
+    res = {}
+    gen = torch.Generator(device=device)
+    gen.manual_seed(1002)
+    k = torch.rand(n, 3, generator=gen, device=device)
+    v = torch.randint(0, 2**63 - 1, (n, 5), generator=gen, device=device)
+    q = torch.cat([k[: n // 2], torch.rand(n - n // 2, 3, generator=gen, device=device) + 1.0])
+    q = q[torch.randperm(n, generator=gen, device=device)].contiguous()
+    out_v = torch.empty(n, 5, device=device, dtype=torch.long)
+    out_f = torch.empty(n, device=device, dtype=torch.bool)
+    quarter = k[: n // 4].contiguous()
+    stream = _stream_ptr(device)
+    for lf, tag in ((0.5, "lf05"), (0.75, "lf075")):
+        hm = CudaClosedHashmap(n_buckets=int(n / lf), device=device, rehash_threshold=1.0, seed=4242)
+        hm.set(k[:8], v[:8])
+        desc = ctypes.byref(hm._desc)
+        clear = lambda: _lib.check(lib.dok_table_clear(desc, stream), "clear")
+        set_ = lambda: _lib.check(lib.dok_map_set(desc, k.data_ptr(), v.data_ptr(), n, None, stream), "set")
+        get = lambda: _lib.check(lib.dok_map_get(desc, q.data_ptr(), n, out_v.data_ptr(), None,
+                                                 out_f.data_ptr(), stream), "get")
+        rem = lambda: _lib.check(lib.dok_map_remove(desc, quarter.data_ptr(), n // 4, out_f.data_ptr(), stream), "remove")
+        s_avg, _ = time_kernel(set_, 3, prep=clear)
+        assert hm.n_elements == n
+        o_avg, _ = time_kernel(set_, 3)
+        get()
+        assert int(out_f.sum().item()) == n // 2
+        g_avg, _ = time_kernel(get, 5)
+        probe = hm.probe_stats(q)
+        r_avg, _ = time_kernel(rem, 1)
+        assert hm.n_elements == n - n // 4
+        res[f"tagged_set_mops_{tag}"] = round(n / s_avg / 1e3, 1)
+        res[f"tagged_overwrite_mops_{tag}"] = round(n / o_avg / 1e3, 1)
+        res[f"tagged_get_mops_{tag}"] = round(n / g_avg / 1e3, 1)
+        res[f"tagged_remove_mops_{tag}"] = round((n // 4) / r_avg / 1e3, 1)
+        res[f"tagged_probe_len_{tag}"] = round(probe, 4)
+        res[f"tagged_table_bytes_{tag}"] = hm._n_phys * 128
+        del hm
+    res["tagged_keys"] = n
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -287,6 +334,10 @@ def main():
     ap.add_argument("--quick", action="store_true", help="skip the set and load-factor-0.9 legs")
     ap.add_argument("--configs", action="store_true",
                     help="also time the four non-headline configurations (reported under extra)")
+    ap.add_argument("--tagged", action="store_true",
+                    help="also time the tagged layout at 32M float32[3] -> int64[5] keys (reported under extra)")
+    ap.add_argument("--only-tagged", action="store_true",
+                    help="run nothing but the --tagged leg and print its figures (for profiling that leg)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one read-only pass over the whole table (the live-entry count of "
                          "the read-out path); with the table clear that every run does, this gives "
@@ -302,6 +353,9 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.only_tagged:
+        print(json.dumps({"extra": tagged_scale(device)}), flush=True)
+        return
     n = args.keys
     gen = torch.Generator(device=device)
     gen.manual_seed(1003)
@@ -454,10 +508,13 @@ def main():
         results["load_factor_09_physical"] = round(n / (hm9._n_phys * hm9._slots_per_bucket), 4)
         del hm9
 
-    if args.configs:
+    if args.configs or args.tagged:
         del keys, values, queries, out_v, out_f
         torch.cuda.empty_cache()
+    if args.configs:
         results.update(other_configs(device))
+    if args.tagged:
+        results.update(tagged_scale(device))
 
     achieved = n * B_GET / (k_avg * 1e-3) / 1e9
     line = {

@@ -157,8 +157,8 @@ __device__ __forceinline__ u32 tg_wrap(u32 home, u32 d, u64 nb) {
 // Phase 1 serves the home bucket of each of a group's 16 rows as "issue 8 loads, resolve 8
 // rounds"; a round is a handful of instructions (tg_match64), and the value lanes of a matching
 // slot write the output row straight from the bucket words they hold.  Rows without a match are
-// finished by their owner lane: it reads the home bucket's metadata (the line has just been
-// fetched) and, with no displacement marked, writes the fallback row.  Phase 2 serves the rows
+// finished by their owner lane: with no displacement marked in the home bucket's metadata (passed
+// on through LDS by the lane that held it) it writes the fallback row.  Phase 2 serves the rows
 // whose home bucket carries displacement marks and held no match, four rows per group and turn,
 // each at its next marked bucket.
 template <int MODE, bool STATS>
@@ -215,6 +215,9 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
           const u64 hit64 = tg_match64(L, M, w[u], exp0[r * RS]) & on64;
           if (MODE == 0 && L.is_val && ((hit64 >> tl) & 1ULL))
             tg_store_word(out_g + (size_t)r * g.V, L.p - 1 - g.KW, g.V, g.unit_v, w[u]);
+          // the bucket's metadata (lane 0 holds it) is left for the row's owner in the unused
+          // upper half of the row's tag word
+          if (L.l == 0) ((u32 *)(lds_rows + (wave_row0 + L.gbase + r) * RS))[1] = (u32)(w[u] >> 32);
           my_hit64 = L.l == r ? hit64 : my_hit64;
         }
       }
@@ -225,7 +228,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
     n_probe += active;
     // rows without a match: the home bucket's metadata decides between "absent" and "look on"
     u32 my_meta = 0;
-    if (active && !found) my_meta = (u32)(t.buckets[(u64)home * 16] >> 32);
+    if (active && !found) my_meta = ((const u32 *)krow)[1];
     bool open = active && !found && my_meta != 0;
     if (MODE == 0 && active && !found && !open) {
       for (int k = 0; k < g.VW; k++)
@@ -630,7 +633,7 @@ static size_t tg_lds_insert(const TgGeom &g) { return (size_t)DOK_TPB * (g.KW + 
 #define DOK_TG_REMOVE_GRID 4096u
 #endif
 #ifndef DOK_TG_SET_GRID
-#define DOK_TG_SET_GRID 8192u
+#define DOK_TG_SET_GRID 32768u
 #endif
 
 static int tg_launch_get(const DevTable &d, const void *keys, i64 n, void *values, const void *fallback,

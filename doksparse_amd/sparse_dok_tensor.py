@@ -33,6 +33,31 @@ from .util import str2dtype, next_power_of_2, shape_to_stride
 
 _INT_DTYPES = {torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8}
 
+# A tensor whose index space a single 8-byte linear key cannot hold (2^63 elements or more), or
+# with more dimensions than the fused indexing kernels take, keeps its coordinates as they are:
+# the map's key rows are the int64[ndim] coordinate vectors themselves (the reference's own key
+# format, sparse_dok_tensor.py:45-69) on the multi-word table layout, and indexing goes through
+# materialised coordinate rows and the batched get / set / remove kernels.  One tag word, ndim key
+# words and the value word have to fit a 128-byte bucket.
+_WIDE_MAX_DIMS = 14
+
+
+def _is_wide(size):
+    volume = 1
+    for s in size:
+        volume *= max(int(s), 1)
+    return len(size) > DOK_MAX_DIMS or volume >= 2**63
+
+
+def _make_storage(size, n_buckets, device, rehash_factor=2.0, rehash_threshold=0.75):
+    """An empty map keyed the way a tensor of this size needs it."""
+    if len(size) > _WIDE_MAX_DIMS:
+        raise NotImplementedError(f"tensors of more than {_WIDE_MAX_DIMS} dimensions: a coordinate row "
+                                  "no longer fits a 128-byte bucket")
+    coord_dims = None if _is_wide(size) else tuple(int(s) for s in size)
+    return CudaClosedHashmap(n_buckets=n_buckets, device=device, coord_dims=coord_dims,
+                             rehash_factor=rehash_factor, rehash_threshold=rehash_threshold)
+
 
 # `nonzero` of a boolean mask needs a device-to-host synchronisation (its result's shape). Code
 # that indexes with the same mask tensor again and again pays that every time, so the index
@@ -76,38 +101,75 @@ class SparseDOKTensor(object):
         else:
             self._dtype = str2dtype(dtype)
 
+        self._wide = _is_wide(self._size)
         if storage is not None:
             self._hashmap = self._adopt_storage(storage)
         else:
             n_buckets = 32 if indices is None else next_power_of_2(values.shape[0])
-            self._hashmap = CudaClosedHashmap(n_buckets=n_buckets, device=self.device,
-                                              coord_dims=tuple(self._size))
+            self._hashmap = _make_storage(self._size, n_buckets, self.device)
         if indices is not None:
             assert values is not None
             assert len(indices.shape) == 2
             assert len(values.shape) == 1
             assert indices.shape[1] == values.shape[0]
             assert indices.shape[0] == self.ndim
-            vals = values.to(device=self.device, dtype=self.dtype)[:, None]
-            if self._hashmap._coord_dims == tuple(self._size):
-                self._hashmap.set_coo(indices.to(self.device), vals)
-            else:
-                self._hashmap.set(indices.T.to(self.device), vals)
+            self._store_coo(indices.to(self.device), values.to(device=self.device, dtype=self.dtype)[:, None])
+
+    def _store_coo(self, indices, vals):
+        """Upsert entries given as [ndim, n] coordinates (this view's dimension order must be the
+        storage's) and [n, 1] values; coordinates outside the size are skipped."""
+        hm = self._hashmap
+        if self._wide:
+            rows = indices.T.contiguous()
+            ok = self._rows_in_range(rows)
+            if not bool(ok.all()):
+                rows, vals = rows[ok], vals[ok]
+            hm.set(rows, vals)
+        elif hm._coord_dims == tuple(self._size):
+            hm.set_coo(indices, vals)
+        else:
+            hm.set(indices.T, vals)
 
     def _adopt_storage(self, storage):
-        """Use `storage` directly if it is keyed by coordinates of this size; otherwise move its
-        entries into a coordinate-keyed map (the fused kernels need the linearised key)."""
-        if storage._coord_dims == tuple(self._size):
+        """Use `storage` directly if it is keyed the way this tensor needs (linearised coordinates
+        of this size, or plain coordinate rows for a wide tensor); otherwise move its entries
+        into such a map."""
+        if self._wide:
+            if storage._coord_dims is None and (not storage._allocated or (
+                    storage._key_dtype == torch.long and storage._key_shape == (self.ndim,))):
+                return storage
+        elif storage._coord_dims == tuple(self._size):
             return storage
-        new = CudaClosedHashmap(n_buckets=storage.n_buckets, device=storage.device,
-                                coord_dims=tuple(self._size),
-                                rehash_factor=storage._rehash_factor,
-                                rehash_threshold=storage._rehash_threshold)
+        new = _make_storage(self._size, storage.n_buckets, storage.device,
+                            storage._rehash_factor, storage._rehash_threshold)
         if storage._allocated:
             keys, values = storage.items()
             if keys.shape[0]:
-                new.set(keys.reshape(-1, self.ndim).long(), values)
+                rows = keys.reshape(-1, self.ndim).long()
+                if self._wide:
+                    ok = self._rows_in_range(rows)
+                    rows, values = rows[ok], values[ok]
+                new.set(rows, values)
         return new
+
+    # ------------------------------------------------------------------ wide tensors
+    def _storage_sizes(self):
+        """Sizes in the storage's dimension order, as a device tensor."""
+        return torch.tensor(self._to_storage_order(list(self._size)), device=self.device, dtype=torch.long)
+
+    def _rows_in_range(self, rows):
+        return ((rows >= 0) & (rows < self._storage_sizes())).all(dim=1)
+
+    def _wide_rows(self, mats):
+        """[n, ndim] int64 coordinate rows, in the storage's dimension order, of materialised
+        selectors (the reference's stack + transpose, sparse_dok_tensor.py:304-311, in one copy)."""
+        return torch.stack(self._to_storage_order(list(mats)), dim=-1).reshape(-1, self.ndim)
+
+    def _ensure_widths(self):
+        """Fix the key / value widths of an unallocated map without storing anything."""
+        if not self._hashmap._allocated:
+            self._hashmap.set(torch.empty(0, self.ndim, device=self.device, dtype=torch.long),
+                              torch.empty(0, 1, device=self.device, dtype=self.dtype))
 
     def _is_permuted(self):
         return self._perm != tuple(range(self.ndim))
@@ -195,7 +257,10 @@ class SparseDOKTensor(object):
 
     @property
     def sparsity(self):
-        return 1 - self._nnz() / float(np.prod(self.shape))
+        volume = 1
+        for n in self.shape:
+            volume *= int(n)                      # (Python integers: the volume may exceed 64 bits)
+        return 1 - self._nnz() / float(volume) if volume else 0.0
 
     def clone(self, deepclone=True):
         new = SparseDOKTensor(size=tuple(self._size), device=self.device, dtype=self.dtype)
@@ -205,14 +270,15 @@ class SparseDOKTensor(object):
 
     # ------------------------------------------------------------------ read-out
     def indices(self):
-        idx, _ = self._hashmap.items_coo()
-        if idx is None:
-            return torch.empty(self.ndim, 0, device=self.device, dtype=torch.long)
-        return idx[list(self._perm)] if self._is_permuted() else idx
+        return self._items_coo_view()[0]
 
     def _items_coo_view(self):
         """(indices [ndim, nnz] in this view's dimension order, values [nnz, 1]) from one pass."""
-        idx, values = self._hashmap.items_coo()
+        if self._wide:
+            keys, values = self._hashmap.items()
+            idx = None if keys is None else keys.T.contiguous()
+        else:
+            idx, values = self._hashmap.items_coo()
         if idx is None:
             return (torch.empty(self.ndim, 0, device=self.device, dtype=torch.long),
                     torch.empty(0, 1, device=self.device, dtype=self.dtype))
@@ -236,12 +302,7 @@ class SparseDOKTensor(object):
         self._hashmap.set_values(selectors=selectors, new_values=new_values[:, None])
 
     def to_sparse_coo(self):
-        idx, values = self._hashmap.items_coo()
-        if idx is None:
-            idx = torch.empty(self.ndim, 0, device=self.device, dtype=torch.long)
-            values = torch.empty(0, 1, device=self.device, dtype=self.dtype)
-        if self._is_permuted():
-            idx = idx[list(self._perm)]
+        idx, values = self._items_coo_view()
         return torch.sparse_coo_tensor(indices=idx, values=values.flatten(), size=tuple(self.shape),
                                        device=self.device)
 
@@ -256,7 +317,11 @@ class SparseDOKTensor(object):
         hm = self._hashmap
         storage_shape = self._to_storage_order(list(self.shape))
         dense = torch.zeros(tuple(storage_shape), device=self.device, dtype=self.dtype)
-        if hm._allocated and dense.numel():
+        if self._wide:
+            keys, values = hm.items()
+            if keys is not None and keys.shape[0]:
+                dense[tuple(keys.T)] = values.flatten()
+        elif hm._allocated and dense.numel():
             lib = _lib.load()
             _lib.check(lib.dok_to_dense(ctypes.byref(hm._desc), dense.data_ptr(), _stream_ptr(self.device)),
                        "to_dense")
@@ -273,17 +338,20 @@ class SparseDOKTensor(object):
     def _rekey(self, new_size, fn):
         """Rebuild the storage for `new_size`, mapping the [ndim, nnz] indices through fn."""
         old = self._hashmap
-        new = CudaClosedHashmap(n_buckets=old.n_buckets, device=self.device, coord_dims=tuple(new_size),
-                                rehash_factor=old._rehash_factor, rehash_threshold=old._rehash_threshold)
+        new = _make_storage(new_size, old.n_buckets, self.device, old._rehash_factor, old._rehash_threshold)
+        idx = values = None
         if old._allocated:
             keys, values = old.items()
             if keys.shape[0]:
-                idx = keys.T[list(self._perm)] if self._is_permuted() else keys.T
-                new.set(fn(idx).T.contiguous(), values)
-                new._header[_lib.DOK_H_NOOB] = 0      # entries outside the new size are dropped
+                idx = fn(keys.T[list(self._perm)] if self._is_permuted() else keys.T)
         self._hashmap = new
         self._size = torch.Size(new_size)
         self._perm = tuple(range(len(new_size)))
+        self._wide = _is_wide(self._size)
+        if idx is not None:
+            self._store_coo(idx.contiguous(), values)
+            if not self._wide:
+                new._header[_lib.DOK_H_NOOB] = 0      # entries outside the new size are dropped
 
     # ------------------------------------------------------------------ selectors
     def _normalise_slice(self, sl, dim):
@@ -446,6 +514,8 @@ class SparseDOKTensor(object):
 
     # ------------------------------------------------------------------ indexing
     def __getitem__(self, selectors):
+        if self._wide:
+            return self._wide_getitem(selectors)
         ix, out_shape, scalar_positions, keep = self._plan(selectors)
         hm = self._hashmap
         if not hm._allocated:
@@ -462,6 +532,45 @@ class SparseDOKTensor(object):
                 values = values.squeeze(i)
         return values
 
+    def _wide_getitem(self, selectors):
+        mats, scalar_positions = self._handle_selectors(selectors)
+        out_shape = tuple(mats[0].shape)
+        hm = self._hashmap
+        if not hm._allocated or mats[0].numel() == 0:
+            values = torch.zeros(out_shape, device=self.device, dtype=self.dtype)
+        else:
+            values, _ = hm.get(self._wide_rows(mats))          # absent (and out-of-range) coordinates read 0
+            values = values.reshape(out_shape)
+        for i in reversed(scalar_positions):
+            if i < values.ndim:
+                values = values.squeeze(i)
+        return values
+
+    def _wide_set_items_dense(self, src, mats):
+        """`_set_items_dense` for a wide tensor: same growth rule, coordinate rows through the
+        batched upsert."""
+        rows = self._wide_rows(mats)
+        src = src.reshape(-1, 1)
+        n_sel = rows.shape[0]
+        if n_sel == 0:
+            return
+        ok = self._rows_in_range(rows)
+        n_oob = n_sel - int(ok.sum().item())
+        if n_oob:
+            rows, src = rows[ok], src[ok]
+        hm = self._hashmap
+        if rows.shape[0]:
+            if not hm._allocated:
+                hm.set(rows[:1], src[:1].contiguous())            # (sparse_dok_tensor_impl.py:413-416)
+            limit = hm.n_buckets * hm._rehash_threshold
+            if hm._n_upper + n_sel > limit:
+                n_now = hm.n_elements
+                if n_now + n_sel > limit:
+                    hm.rehash(int(np.ceil((n_now + n_sel) * hm._rehash_factor)))
+            hm.set(rows, src.contiguous())
+        if n_oob:
+            raise IndexError(f"{n_oob} coordinates fall outside the tensor of size {tuple(self.shape)}")
+
     def __setitem__(self, selectors, values):
         if isinstance(values, SparseDOKTensor) or (isinstance(values, Tensor) and values.is_sparse):
             mats, _ = self._handle_selectors(selectors)
@@ -469,6 +578,13 @@ class SparseDOKTensor(object):
             assert tuple(values.shape) == out_shape, \
                 f"expecting the value shape to be {out_shape}, got {tuple(values.shape)} instead"
             return self._set_items_sparse(values, mats)
+        if self._wide:
+            mats, _ = self._handle_selectors(selectors)
+            out_shape = tuple(mats[0].shape)
+            if not isinstance(values, Tensor):
+                values = torch.tensor(values, device=self.device, dtype=self.dtype)
+            values = torch.broadcast_to(values.to(device=self.device, dtype=self.dtype), out_shape)
+            return self._wide_set_items_dense(values, mats)
         ix, out_shape, _, keep = self._plan(selectors)
         if not isinstance(values, Tensor):
             values = torch.tensor(values, device=self.device, dtype=self.dtype)
@@ -514,13 +630,26 @@ class SparseDOKTensor(object):
         """Sparse-valued gather: a SparseDOKTensor over the index space holding the addressed
         entries (reference: :342-350 and get_items, sparse_dok_tensor_impl.py:148-233)."""
         selectors, _ = self._handle_selectors(selectors)
-        ix, out_shape = self._index_desc(selectors)
+        out_shape = tuple(selectors[0].shape)
         if len(out_shape) == 0:
             raise NotImplementedError("sparse-valued indexing needs at least one result axis")
         out = SparseDOKTensor(size=out_shape, device=self.device, dtype=self.dtype)
         hm = self._hashmap
         if not hm._allocated:
             return out
+        if self._wide or out._wide:
+            # through coordinate rows: look up, keep the hits, key them by their index vector
+            n = 0
+            if selectors[0].numel():
+                values, found = hm.get(self._wide_rows(selectors))
+                at = found.nonzero().flatten()
+                n = int(at.shape[0])
+            out._hashmap = _make_storage(out_shape, int(n * 2.0), self.device)
+            out._ensure_widths()
+            if n:
+                out._store_coo(torch.stack(torch.unravel_index(at, out_shape)), values[at])
+            return out
+        ix, out_shape = self._index_desc(selectors)
         lib = _lib.load()
         stream = _stream_ptr(self.device)
         n = 0
@@ -554,6 +683,8 @@ class SparseDOKTensor(object):
         src_indices = src_indices.to(self.device)
         src_values = src_values.to(device=self.device, dtype=self.dtype).contiguous()
         hm = self._hashmap
+        if self._wide:
+            return self._wide_set_items_sparse(src_indices, src_values, selectors)
         if not hm._allocated:
             # (reference: sparse_dok_tensor_impl.py:237-240)
             first_key = torch.stack([s.reshape(-1)[0] for s in self._to_storage_order(selectors)], dim=0)[None]
@@ -576,12 +707,41 @@ class SparseDOKTensor(object):
                                               src_values.data_ptr(), n_src, mask, stream), "__setitem__")
         hm._n_upper = n_now + n_src
 
+    def _wide_set_items_sparse(self, src_indices, src_values, mats):
+        hm = self._hashmap
+        rows_all = self._wide_rows(mats)
+        if not hm._allocated:
+            first = rows_all[:1]
+            if first.shape[0] and bool(self._rows_in_range(first).all()):
+                hm.set(first, torch.zeros(1, 1, device=self.device, dtype=self.dtype))   # (sparse_dok_tensor_impl.py:237-240)
+            else:
+                self._ensure_widths()
+        if rows_all.shape[0]:
+            hm._remove_rows(rows_all)
+        n_src = int(src_values.shape[0])
+        n_now = hm.n_elements
+        hm.rehash(int(np.ceil((n_now + n_src) * hm._rehash_factor * 2)))
+        if n_src:
+            shape = torch.tensor(tuple(mats[0].shape), device=self.device, dtype=torch.long)[:, None]
+            keep = (src_values != 0) & ((src_indices >= 0) & (src_indices < shape)).all(dim=0)
+            at = tuple(src_indices[:, keep])
+            rows = torch.stack([m[at] for m in self._to_storage_order(list(mats))], dim=-1).reshape(-1, self.ndim)
+            vals = src_values[keep][:, None]
+            ok = self._rows_in_range(rows)
+            if rows.shape[0]:
+                hm.set(rows[ok], vals[ok].contiguous())
+        hm._n_upper = n_now + n_src
+
     def count_items(self, selectors):
         """Number of addressed elements that are stored (reference: count_items,
         sparse_dok_tensor_impl.py:56-108)."""
         selectors, _ = self._handle_selectors(selectors)
         count = torch.zeros(1, device=self.device, dtype=torch.long)
         hm = self._hashmap
+        if self._wide:
+            if hm._allocated and selectors[0].numel():
+                count += hm.count_existing(self._wide_rows(selectors))
+            return count
         if hm._allocated and selectors[0].numel():
             ix, _ = self._index_desc(selectors)
             lib = _lib.load()
@@ -593,6 +753,10 @@ class SparseDOKTensor(object):
         """Remove every addressed element (reference: zero_items, sparse_dok_tensor_impl.py:110-146)."""
         selectors, _ = self._handle_selectors(selectors)
         hm = self._hashmap
+        if self._wide:
+            if hm._allocated and selectors[0].numel():
+                hm._remove_rows(self._wide_rows(selectors))
+            return
         if hm._allocated and selectors[0].numel():
             ix, _ = self._index_desc(selectors)
             lib = _lib.load()
@@ -710,10 +874,8 @@ class SparseDOKTensor(object):
     def _map_values(self, fn):
         keys, values = self._hashmap.items()
         new = SparseDOKTensor(size=tuple(self._size), device=self.device, dtype=self.dtype)
-        new._hashmap = CudaClosedHashmap(n_buckets=self._hashmap.n_buckets, device=self.device,
-                                         coord_dims=tuple(self._size),
-                                         rehash_factor=self._hashmap._rehash_factor,
-                                         rehash_threshold=self._hashmap._rehash_threshold)
+        new._hashmap = _make_storage(self._size, self._hashmap.n_buckets, self.device,
+                                     self._hashmap._rehash_factor, self._hashmap._rehash_threshold)
         if keys is not None and keys.shape[0]:
             if self._is_permuted():
                 keys = keys[:, list(self._perm)].contiguous()

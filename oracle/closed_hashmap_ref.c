@@ -265,7 +265,7 @@ void ref_batch_hash(const ref_table_t *t, const uint8_t *keys, ll_t n, ll_t *h1,
 
 /* ---- DOK kernels --------------------------------------------------------------------------*/
 
-#define REF_MAX_DIMS 8
+#define REF_MAX_DIMS 16
 
 /* One strided view: tensor_accessor.cu:1-121.  Strides are in elements; 0 = broadcast. */
 typedef struct {

@@ -27,7 +27,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libref_hashmap.so")
 _lib = None
 
-MAX_DIMS = 8
+MAX_DIMS = 16
 
 
 class RefTable(ctypes.Structure):

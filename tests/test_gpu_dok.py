@@ -642,3 +642,153 @@ def test_random_sparse_valued_indexing_against_the_oracle(cuda):
             assert torch.equal(dok.to_dense().cpu(), ref.to_dense()), (shape, sel)
             n_set += 1
     assert n_get > 150 and n_set > 100
+
+
+# ---- wide tensors: index spaces of 2^63 elements or more, or more than 8 dimensions ---------------
+
+def _wide_pair(size, nnz, seed, dev, dtype=torch.float32):
+    from doksparse_amd import SparseDOKTensor
+    rng = np.random.default_rng(seed)
+    idx = np.stack([rng.integers(0, s, size=nnz, dtype=np.int64) for s in size])
+    idx = np.unique(idx, axis=1)
+    idx = torch.from_numpy(idx[:, rng.permutation(idx.shape[1])])
+    vals = torch.from_numpy(rng.integers(1, 1000, size=idx.shape[1])).to(dtype)
+    dok = SparseDOKTensor(size, idx.to(dev), vals.to(dev), device=dev)
+    ref = RefSparseDOKTensor(size, idx, vals, rng=np.random.default_rng(seed))
+    return dok, ref, idx, vals
+
+
+@pytest.mark.parametrize("size", [(2**40, 2**40), (2**31, 2**31, 2**31), (2**62, 5), (2**21,) * 4])
+def test_wide_index_space_construct_getitem_setitem_roundtrip(cuda, size):
+    """Tensors whose volume is 2^63 or more keep their coordinates as multi-word keys: construct,
+    gather (hits, misses, broadcast and slice selectors), scatter (new and present coordinates,
+    with growth), read-out - all against the oracle."""
+    dok, ref, idx, vals = _wide_pair(size, 5000, 11, cuda)
+    assert dok._wide and dok._nnz() == ref._nnz() == idx.shape[1]
+    assert dok.storage().n_buckets == ref._hashmap.n_buckets
+    assert same_entries(dok, ref)
+    rng = np.random.default_rng(12)
+    nd = len(size)
+    # gather: stored coordinates mixed with random ones
+    pick = torch.from_numpy(rng.integers(0, idx.shape[1], size=3000))
+    rand = torch.from_numpy(np.stack([rng.integers(0, s, size=3000, dtype=np.int64) for s in size]))
+    q = torch.cat([idx[:, pick], rand], dim=1)[:, torch.from_numpy(rng.permutation(6000))]
+    sel = tuple(q[d] for d in range(nd))
+    exp = ref[sel]
+    got = dok[tuple(x.to(cuda) for x in sel)]
+    assert got.shape == exp.shape and torch.equal(got.cpu(), exp) and int((exp != 0).sum()) >= 3000
+    # a broadcast block with a slice at the end: rows of stored first coordinates x a window
+    first = idx[0, :7]
+    last0 = int(idx[-1, 0])
+    lo = max(0, min(last0 - 3, size[-1] - 8))
+    sel = (first[:, None],) + tuple(idx[d, :5][None, :] for d in range(1, nd - 1)) + (slice(lo, lo + 8),)
+    exp = ref[sel]
+    got = dok[tuple(x.to(cuda) if isinstance(x, torch.Tensor) else x for x in sel)]
+    assert got.shape == exp.shape and torch.equal(got.cpu(), exp)
+    # scalar selectors
+    one = tuple(int(idx[d, 0]) for d in range(nd))
+    assert dok[one].item() == vals[0].item()       # (the reference, and so the oracle, raises here by accident)
+    # scatter: half present, half new coordinates; enough to grow the table
+    new = torch.from_numpy(np.stack([rng.integers(0, s, size=4000, dtype=np.int64) for s in size]))
+    w = torch.cat([idx[:, :4000], new], dim=1)
+    wv = torch.from_numpy(rng.integers(-500, 500, size=8000)).float()
+    wsel = tuple(w[d] for d in range(nd))
+    ref[wsel] = wv
+    dok[tuple(x.to(cuda) for x in wsel)] = wv.to(cuda)
+    assert dok.storage().n_buckets == ref._hashmap.n_buckets
+    a = sorted_coo(dok.indices(), dok.values())
+    b = sorted_coo(ref.indices(), ref.values())
+    ub, first_of = np.unique(b[0], axis=1, return_index=True)       # (the oracle may hold a repeated coordinate twice)
+    assert np.array_equal(a[0], ub) and dok._nnz() == ub.shape[1]
+    assert torch.equal(dok[tuple(x.to(cuda) for x in wsel)].cpu(), ref[wsel])
+    # out-of-range coordinates: reads give 0, writes raise
+    far = tuple(torch.tensor([s + 5]) for s in size)
+    assert dok[tuple(x.to(cuda) for x in far)].item() == 0
+    with pytest.raises(IndexError):
+        dok[tuple(x.to(cuda) for x in far)] = torch.ones(1, device=cuda)
+    # count / remove
+    csel = tuple(q[d].to(cuda) for d in range(nd))
+    n_before = dok._nnz()
+    cnt = int(dok.count_items(csel).item())
+    dok.zero_items(csel)
+    assert int(dok.count_items(csel).item()) == 0
+    def rows(a):                                       # [nd, n] coordinates -> n comparable records
+        return np.ascontiguousarray(a.T).view([("", np.int64)] * nd).ravel()
+    stored_q = np.isin(rows(q.numpy()), rows(ub))
+    assert cnt == int(stored_q.sum()) >= 3000
+    assert n_before - dok._nnz() == np.unique(rows(q.numpy())[stored_q]).shape[0]
+    assert "nnz=" in repr(dok)
+
+
+def test_wide_many_dimensions_against_the_oracle(cuda):
+    """A 10-dimensional tensor (more dimensions than the fused kernels take): random expressions,
+    assignments, views, dense read-out and sparse-valued indexing against the oracle."""
+    from doksparse_amd import SparseDOKTensor
+    size = (3, 2, 4, 3, 2, 3, 2, 2, 3, 2)
+    dok, ref, idx, vals = _wide_pair(size, 3000, 21, cuda)
+    assert dok._wide and dok.ndim == 10 and same_entries(dok, ref)
+    assert torch.equal(dok.to_dense().cpu(), ref.to_dense())
+    rng = np.random.default_rng(22)
+    compared = 0
+    for _ in range(40):
+        sel = _random_selectors(rng, size)
+        dsel = tuple(s.to(cuda) if isinstance(s, torch.Tensor) else s for s in sel)
+        try:
+            exp = ref[sel]
+        except Exception:
+            continue
+        got = dok[dsel]
+        assert got.shape == exp.shape and torch.equal(got.cpu(), exp), sel
+        val = float(rng.integers(-50, 50))
+        try:
+            ref[sel] = torch.full(exp.shape, val)
+        except Exception:
+            continue
+        dok[dsel] = torch.full(exp.shape, val, device=cuda)
+        assert torch.equal(dok.to_dense().cpu(), ref.to_dense()), sel
+        compared += 1
+    assert compared >= 15
+    # a permuted view shares the storage
+    order = (9, 0, 5, 2, 7, 1, 8, 3, 6, 4)
+    v = dok.permute(*order)
+    dense = ref.to_dense()
+    assert torch.equal(v.to_dense().cpu(), dense.permute(*order))
+    pos = tuple(int(x) for x in idx[:, 0])
+    vpos = tuple(pos[o] for o in order)
+    v[vpos] = 777.0
+    assert dok[pos].item() == 777.0
+    dense[pos] = 777.0
+    # sparse-valued gather and scatter
+    sel = (torch.tensor([0, 2, 1])[:, None], slice(None), torch.tensor([3, 0])[None, :], 1, 0, 2, 1, 0, 2, 1)
+    dsel = tuple(s.to(cuda) if isinstance(s, torch.Tensor) else s for s in sel)
+    sp = dok.__spgetitem__(dsel)
+    want = dok[dsel]
+    assert torch.equal(sp.to_dense().cpu().reshape(want.shape), want.cpu())
+    # (result axes: the 3 x 2 broadcast block at the first tensor selector's position, then the slice)
+    assert tuple(want.shape) == (3, 2, 2)
+    src = torch.zeros(3, 2, 2)
+    src[0, 1, 0], src[2, 0, 1] = 5.0, -6.0
+    dok[dsel] = src.to_sparse().to(cuda)
+    for bi, c0 in enumerate((0, 2, 1)):
+        for bj, c2 in enumerate((3, 0)):
+            for sl in range(2):
+                dense[c0, sl, c2, 1, 0, 2, 1, 0, 2, 1] = src[bi, bj, sl]
+    assert torch.equal(dok.to_dense().cpu(), dense)
+
+
+def test_permuted_dok_tensor_as_sparse_source(cuda):
+    """`a[sel] = b.t()` with a DOK source that is a permuted view: the source's coordinates are
+    taken in the view's dimension order."""
+    from doksparse_amd import SparseDOKTensor
+    g = torch.Generator().manual_seed(5)
+    b_dense = torch.zeros(6, 4)
+    b_dense[torch.randint(0, 6, (9,), generator=g), torch.randint(0, 4, (9,), generator=g)] = torch.randn(9, generator=g)
+    b = SparseDOKTensor.from_dense(b_dense.to(cuda))
+    a = SparseDOKTensor((10, 12), device=cuda)
+    a_dense = torch.zeros(10, 12)
+    a[2:6, 3:9] = b.t()
+    a_dense[2:6, 3:9] = b_dense.t()
+    assert torch.equal(a.to_dense().cpu(), a_dense)
+    a[torch.tensor([7, 1, 0, 9])[:, None].to(cuda), torch.tensor([0, 11, 5, 2, 3, 8])[None, :].to(cuda)] = b.permute(1, 0)
+    a_dense[torch.tensor([7, 1, 0, 9])[:, None], torch.tensor([0, 11, 5, 2, 3, 8])[None, :]] = b_dense.t()
+    assert torch.equal(a.to_dense().cpu(), a_dense)

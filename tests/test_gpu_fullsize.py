@@ -173,6 +173,13 @@ def test_cfg3_full_size_int64_to_float32(cuda, load_factor):
     assert check(mixed) == n // 2
     del mixed
 
+    # the batch of the configuration itself: 2^26 queries, half of them hits whose rank among the
+    # stored keys is drawn Zipf(1.1), half uniform misses, shuffled; every row is compared
+    from bench import make_queries
+    zipf, n_hit = make_queries(keys, n, gen, cuda)
+    assert abs(check(zipf) - n_hit) <= 64          # (a uniform "miss" can hit a stored key by chance)
+    del zipf
+
     # bulk upsert into the populated table: a quarter overwritten, nothing new
     values[: n // 4] += 1.0
     hm.set(keys[: n // 4, None], values[: n // 4, None])

@@ -89,12 +89,13 @@ def _check_get(hm, ref, q, dev, fallback=None):
     assert np.array_equal(np.ascontiguousarray(v.cpu().numpy()).view(np.uint8), np.ascontiguousarray(rv).view(np.uint8))
 
 
-def test_cfg2_float_triple_keys_wide_values(cuda):
-    """README-shaped map at 1/8 scale: float32[3] keys hashed over raw bytes, int64[5] values
-    (tagged layout): set, get hits+misses, remove 25 %, get again."""
+@pytest.mark.parametrize("n,capacity", [(131072, 2**18), (1_000_000, 2**21)])
+def test_cfg2_float_triple_keys_wide_values(cuda, n, capacity):
+    """README-shaped map, at 1/8 scale and at its full size (1,000,000 keys, capacity 2^21):
+    float32[3] keys hashed over raw bytes, int64[5] values (tagged layout): set, get of as many
+    hits as misses, remove 25 %, get again, overwrite + re-insert."""
     from doksparse_amd import CudaClosedHashmap
     rng = np.random.default_rng(1002)
-    n = 131072
     keys = rng.random((n, 3), dtype=np.float32)
     keys = np.unique(keys, axis=0)
     rng.shuffle(keys)
@@ -102,8 +103,8 @@ def test_cfg2_float_triple_keys_wide_values(cuda):
     vals = rng.integers(0, 2**63 - 1, size=(n, 5), dtype=np.int64)
     misses = rng.random((n, 3), dtype=np.float32) + 1.0            # disjoint from [0, 1)
 
-    hm = CudaClosedHashmap(n_buckets=2**18, device=cuda)
-    ref = RefClosedHashmap(n_buckets=2**18, rng=np.random.default_rng(8))
+    hm = CudaClosedHashmap(n_buckets=capacity, device=cuda)
+    ref = RefClosedHashmap(n_buckets=capacity, rng=np.random.default_rng(8))
     k, v = _to(cuda, keys, vals)
     hm.set(k, v)
     ref.set(keys, vals)
@@ -552,3 +553,45 @@ def test_keys_beyond_freed_slots_are_overwritten_not_duplicated(cuda, capacity):
         ks, _ = hm.items()
         assert np.unique(ks.cpu().numpy()).shape[0] == n       # no key in two slots
         _check_get(hm, ref, keys, cuda, fallback=0)
+
+
+def test_tagged_map_grows_on_the_device_like_the_reference(cuda):
+    """A multi-word map that starts small: every growth re-inserts the entries with the
+    device-side rehash; sizes, contents and lookups follow the oracle through the growths,
+    through removals and through an explicit rehash."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(77)
+    hm = CudaClosedHashmap(n_buckets=64, device=cuda)
+    ref = RefClosedHashmap(n_buckets=64, rng=np.random.default_rng(9))
+    pool = np.unique(rng.integers(-2**40, 2**40, size=(60000, 3), dtype=np.int64), axis=0)
+    rng.shuffle(pool)
+    done = 0
+    for step, n in enumerate((10, 100, 1000, 7000, 30000)):
+        keys = pool[done: done + n]
+        done += n
+        vals = rng.standard_normal((n, 2)).astype(np.float32)
+        hm.set(*_to(cuda, keys, vals)); ref.set(keys, vals)
+        assert hm.n_buckets == ref.n_buckets and hm.n_elements == ref.n_elements == done
+        if step == 3:
+            gone = pool[:done][rng.permutation(done)[: done // 3]]
+            m = hm.remove(torch.from_numpy(gone).to(cuda))
+            assert np.array_equal(m.cpu().numpy(), ref.remove(gone))
+            done_live = hm.n_elements
+            assert done_live == ref.n_elements
+            # the removed keys go back in with the next batch
+            pool = np.concatenate([pool[:done][~_isin_rows(pool[:done], gone)], pool[done:], gone])
+            done = done_live
+    _assert_same_map(hm, ref)
+    q = np.concatenate([pool[:done], rng.integers(2**41, 2**42, size=(5000, 3), dtype=np.int64)])
+    _check_get(hm, ref, q, cuda)
+    hm.rehash(3 * hm.n_buckets); ref.rehash(3 * ref.n_buckets)
+    assert hm.n_buckets == ref.n_buckets and hm.n_elements == ref.n_elements
+    _check_get(hm, ref, q, cuda)
+    _assert_same_map(hm, ref)
+
+
+def _isin_rows(a, b):
+    """Mask over the rows of `a` that occur among the rows of `b`."""
+    va = np.ascontiguousarray(a).view([("", a.dtype)] * a.shape[1]).ravel()
+    vb = np.ascontiguousarray(b).view([("", b.dtype)] * b.shape[1]).ravel()
+    return np.isin(va, vb)
