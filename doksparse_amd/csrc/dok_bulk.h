@@ -798,8 +798,11 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
         const u64 mw = ((volatile u64 *)tb)[DOK_P8_META * LD + lhome];
         // bit 0 stands for the home bucket here: the look has checked it, but a row that met a
         // fingerprint mark may find the key there by now
-        u32 mk = ((u32)mw & ~1u) | (u32)lflag[e];
-        const u32 far_hi = ((u32)mw & 1u) ? (u32)(mw >> 32) : 0u;
+        // (a key that was ever placed away from this bucket has its filter bit set here; without
+        // the bit there is nothing to look for beyond the home bucket)
+        const bool maybe_away = ((u32)(mw >> 32) & p8_fbit(h)) != 0;
+        u32 mk = (maybe_away ? ((u32)mw & ~1u) : 0u) | (u32)lflag[e];
+        const u32 far_hi = (maybe_away && ((u32)mw & 1u)) ? ((u32)(mw >> 32) & 0xffu) : 0u;
         u32 d = 0;
         while (true) {
           if (mk) { d = (u32)__builtin_ctz(mk); mk &= mk - 1; }
@@ -824,6 +827,8 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
             break;
           }
         }
+        // a saturated record of the largest displacement: the key may sit further on still
+        if (!done && far_hi == DOK_P8_FARCAP) beyond = true;
         if (!done && !beyond) {
           // one row per key goes on
           u32 i = (u32)(h >> 8) & (HSET - 1);
@@ -886,16 +891,14 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
           *(VT *)((char *)(tb + (S + ((ts * V) >> 3)) * LD + T) + ((ts * V) & 7)) = val;
           const u32 td = (u32)((int)T - lhome);
           if (td > 0 && lhome >= 0) {
-            u32 *meta = (u32 *)(tb + DOK_P8_META * LD + lhome);
-            if (td >= 32) { atomicMax(meta + 1, td); atomicOr(meta, 1u); }
-            else atomicOr(meta, 1u << td);
+            p8_mark(tb + DOK_P8_META * LD + lhome, td, p8_fbit(h), 0);
           } else if (td > 0) {
             // A carried row: its home bucket went back to HBM with plain stores a moment ago,
             // and an atomic on that line from inside this kernel is not ordered against
-            // them.  The mark is noted down (in the part of keysB this workgroup has consumed)
-            // and applied by the kernel that runs after the merge.
+            // them.  The mark (with the key's filter bit) is noted down (in the part of keysB this
+            // workgroup has consumed) and applied by the kernel that runs after the merge.
             const u32 mi = atomicAdd(&n_meta, 1u);
-            ws.keysB[def_base + mi] = ((u64)home << 32) | (u64)td;
+            ws.keysB[def_base + mi] = ((u64)home << 32) | ((u64)p8_fidx(h) << 24) | (u64)(td & 0xffffffu);
           }
           n_fresh++;
           done = true;
@@ -988,13 +991,15 @@ __global__ __launch_bounds__(DOK_BULK_R) void bulk_edge_kernel(DevTable t, BulkW
   const u32 def_base = ws.part_off[p_lo], top = ws.part_off[p_hi];
   const u32 note_base = def_base + ws.meta_cnt[blockIdx.x], a_base = def_base + ws.def_cnt[blockIdx.x];
   bool have = (u32)tid < n_rows;
-  u64 key = 0, sk = 0, home = 0;
+  u64 key = 0, sk = 0, home = 0, fidx = 0;
   VT val = 0;
   if (have) {
     key = ws.keysA[top - 1 - tid];
     val = (VT)dok_load_val<V>(ws.valsA, (i64)(top - 1 - tid));
     sk = key ^ DOK_P8_XOR;
-    home = p8_home(sk, t);
+    const u64 h = p8_hash(sk, t);
+    home = dok_reduce(h, t.nb);
+    fidx = p8_fidx(h);
   }
   if (tid == 0) { n_note = 0; n_a = 0; }
   int n_fresh = 0;
@@ -1050,7 +1055,7 @@ __global__ __launch_bounds__(DOK_BULK_R) void bulk_edge_kernel(DevTable t, BulkW
         *(VT *)((char *)(tb + (S + ((ts * V) >> 3)) * LD + T) + ((ts * V) & 7)) = val;
         // the displacement mark belongs to a bucket of another range: noted for the kernel that follows
         const u64 td = b0 + T - home;
-        ws.keysB[note_base + atomicAdd(&n_note, 1u)] = (home << 32) | td;
+        ws.keysB[note_base + atomicAdd(&n_note, 1u)] = (home << 32) | (fidx << 24) | (td & 0xffffffULL);
         n_fresh++;
         have = false;
         break;
@@ -1095,11 +1100,9 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
   // displacement marks the merge could not set itself (see there)
   const u32 n_marks = ws.meta_cnt[blockIdx.x];
   for (u32 i = threadIdx.x; i < n_marks; i += DOK_TPB) {
+    // home bucket (32 bits) | the key's filter bit number (8) | displacement (24)
     const u64 note = ws.keysB[base + i];
-    const u32 td = (u32)note;
-    u32 *meta = (u32 *)(t.buckets + (note >> 32) * 16 + DOK_P8_META);
-    if (td >= 32) { atomicMax(meta + 1, td); atomicOr(meta, 1u); }
-    else atomicOr(meta, 1u << td);
+    p8_mark(t.buckets + (note >> 32) * 16 + DOK_P8_META, (u32)note & 0xffffffu, 256u << ((u32)(note >> 24) & 0xffu), 0);
   }
   // the rows from the bottom of the stretch, and - if bulk_edge_kernel has not taken them - the
   // rows listed from its top downwards

@@ -7,7 +7,12 @@
 //                              bits 1..31  displacement map: bit d set = some key was placed d
 //                                          buckets past this one
 //                              bit 0       a key was placed 32 or more buckets past this one
-//                              bits 32..63 the largest such far displacement
+//                              bits 32..39 the largest such far displacement, 255 standing for
+//                                          "255 or more" (the walk then ends at the first bucket
+//                                          with an EMPTY slot)
+//                              bits 40..63 filter: every key placed away from this bucket sets the
+//                                          bit its hash selects; a lookup whose bit is clear
+//                                          cannot be a displaced key and ends at the home bucket
 // (V=4: 10 slots, V=8: 7, V=2: 12, V=1: 13).  The stored key word is  key XOR DOK_P8_XOR,
 // and the two words 0 and 1 mean EMPTY and TOMBSTONE, so a cleared table is all zero bytes and
 // the slot word itself is the target of the claiming 64-bit compare-and-swap: an insert is one
@@ -43,8 +48,32 @@ template <int V> struct P8 {
   }
 };
 
-__device__ __forceinline__ u32 p8_home(u64 sk, const DevTable &t) {
-  return dok_reduce(dok_fmix64(sk ^ t.seed), t.nb);
+// Hash of a stored key word.  Its upper half picks the home bucket, its lower half the filter bit.
+__device__ __forceinline__ u64 p8_hash(u64 sk, const DevTable &t) { return dok_fmix64(sk ^ t.seed); }
+__device__ __forceinline__ u32 p8_home(u64 sk, const DevTable &t) { return dok_reduce(p8_hash(sk, t), t.nb); }
+
+#define DOK_P8_FARCAP 255u
+#define DOK_P8_FBITS 24
+// The key's bit among bits 8..31 of the metadata word's upper half.
+__device__ __forceinline__ u32 p8_fidx(u64 h) { return (((u32)h & 0xffffu) * DOK_P8_FBITS) >> 16; }
+__device__ __forceinline__ u32 p8_fbit(u64 h) { return 256u << p8_fidx(h); }
+
+// Record in the home bucket's metadata word (global memory or an LDS copy) that a key with filter
+// bit `fbit` was placed d > 0 buckets further on.  `seen`: a view of the word taken earlier (0 if
+// none) - what it already shows need not be written again.
+__device__ __forceinline__ void p8_mark(u64 *meta, u32 d, u32 fbit, u64 seen) {
+  const u64 want = ((u64)fbit << 32) | (d < 32 ? 1ULL << d : 1ULL);
+  if ((seen & want) != want) atomicOr(meta, want);
+  if (d >= 32) {
+    u32 *hi = (u32 *)meta + 1;
+    const u32 dm = d < DOK_P8_FARCAP ? d : DOK_P8_FARCAP;
+    u32 old = *(volatile u32 *)hi;
+    while ((old & 0xffu) < dm) {
+      const u32 prev = atomicCAS(hi, old, (old & ~0xffu) | dm);
+      if (prev == old) break;
+      old = prev;
+    }
+  }
 }
 
 // Keeps the compiler from hoisting the 16 per-round "is this my row" masks out of the tile loop
@@ -128,7 +157,7 @@ __device__ __forceinline__ int p8_pick(u32 free_mask, int start) {   // free_mas
 #define DOK_P8_WI 4  // rows per group per phase-2 turn of the insert
 #endif
 template <int V>
-__device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 nb, u64 sk, u32 b,
+__device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 nb, u64 sk, u32 b, u32 fbit,
                                           bool pend, bool &found, u64 &val, u32 &slot_b,
                                           int &slot_s, int &nprobe) {
   const P8Lane L;
@@ -136,7 +165,7 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
   int l = L.l;
   DOK_OPAQUE(l);
   const u32 home = b;
-  u32 meta = 0;                 // low word of the home bucket's metadata
+  u32 meta = 0, mhi = 0;        // the home bucket's metadata word
   bool open = false;            // row still unresolved after its home bucket
   slot_b = home;
 
@@ -159,11 +188,12 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
         const u64 q = dok_shfl64(sk, gbase + r);
         P8Probe<V> pr;
         pr.match(L, w[u], q);
-        const u32 md = dok_shfl32((u32)w[u], gbase + DOK_P8_META);
+        const u64 mw = dok_shfl64(w[u], gbase + DOK_P8_META);
         const bool mine = l == r;
         my_gm = mine ? pr.gm : my_gm;
         my_ge = mine ? pr.ge : my_ge;
-        meta = mine ? md : meta;
+        meta = mine ? (u32)mw : meta;
+        mhi = mine ? (u32)(mw >> 32) : mhi;
         DOK_SCHED_FENCE();
       }
     }
@@ -176,7 +206,9 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
       my_v = *(const T *)((const char *)(buckets + (u64)home * 16) + 8 * P8<V>::S + V * s1);
     }
     if (pend) { found = hit1; slot_s = s1; if (hit1) val = my_v; }
-    open = pend && my_gm == 0 && meta != 0;
+    // a key placed away from its home has set its filter bit there: with the bit clear the
+    // home bucket alone decides, whatever other keys it has sent on
+    open = pend && my_gm == 0 && meta != 0 && (mhi & fbit) != 0;
     nprobe += pend;
   }
 
@@ -184,8 +216,10 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
   // to be visited; the far walk (displacements >= 32, rare even in a 97 % full table) follows.
   u32 cand = open ? (meta & ~1u) : 0u;
   bool far = open && (meta & 1u);
-  u32 far_d = 32, far_max = 0;
-  if (far) far_max = (u32)(buckets[(u64)home * 16 + DOK_P8_META] >> 32);
+  u32 far_d = 32, far_max = mhi & 0xffu;
+  // a saturated record: the far walk goes on to the first bucket with an EMPTY slot (or once round)
+  const bool far_unb = far_max == DOK_P8_FARCAP;
+  if (far_unb) far_max = nb > 0xffffffffULL ? 0xffffffffu : (u32)nb - 1u;
   bool hit2 = false;
   u64 pm = dok_ballot(open);
   while (pm != 0) {
@@ -220,7 +254,7 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
       w1[k] = buckets[(u64)(h1[k] ? qb1 : 0u) * 16 + l];
     }
     bool act = false;
-    u32 gm0 = 0, gm1 = 0;
+    u32 gm0 = 0, gm1 = 0, gee = 0;
     #pragma unroll
     for (int k = 0; k < DOK_P8_WL; k++) {
       const u64 q = dok_shfl64(sk, gbase + rr[k]);
@@ -231,6 +265,7 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
       act = act || mine;
       gm0 = mine ? p0.gm : gm0;
       gm1 = mine ? (h1[k] ? p1.gm : 0u) : gm1;
+      gee = mine ? (p0.ge | (h1[k] ? p1.ge : 0u)) : gee;
     }
     if (act) {
       nprobe += 1 + (d1 != 0);
@@ -239,6 +274,7 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
         slot_b = gm0 ? b0 : b1;
         slot_s = __builtin_ctz(gm0 ? gm0 : gm1);
       } else {
+        if (far_unb && cand == 0 && gee != 0) far = false;   // an EMPTY slot ends the unrecorded part of the chain
         // drop the visited displacements
         if (cand) {
           cand &= cand - 1;
@@ -284,7 +320,7 @@ __device__ __forceinline__ bool p8_side_get(const DevTable &t, u64 sk, u64 &val)
 // acting together.  A key placed d > 0 buckets past its home raises the home bucket's recorded largest
 // displacement to d.
 template <int V>
-__device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val, u32 home,
+__device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val, u32 home, u32 fbit,
                                           bool pend, int &st, int &fresh) {
   const P8Lane L;
   const int gbase = L.gbase;
@@ -398,14 +434,8 @@ __device__ __forceinline__ void p8_insert(u64 *buckets, u64 nb, u64 sk, u64 val,
             const u64 old = atomicCAS(tp + ts, expect, sk);
             if (old == expect) {
               P8<V>::store(tp, ts, val);
-              // mark the displacement in the home bucket's metadata (skipped when the view
-              // of it taken in phase 1 already shows the mark)
-              if (td >= 32) {
-                atomicMax((u32 *)(hb + DOK_P8_META) + 1, td);
-                if (!(md_home & 1u)) atomicOr((u32 *)(hb + DOK_P8_META), 1u);
-              } else if (td > 0 && !((md_home >> td) & 1u)) {
-                atomicOr((u32 *)(hb + DOK_P8_META), 1u << td);
-              }
+              // mark the displacement and the key's filter bit in the home bucket's metadata
+              if (td > 0) p8_mark(hb + DOK_P8_META, td, fbit, 0);
               st = 1; fresh = 1; pend = false;
             } else if (old == sk) {
               st = 1; pend = false;                     // an equal key of this batch won the slot
@@ -447,7 +477,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
     bool pend = ok;
     if (ok && sk < 2) { found = p8_side_get(t, sk, val); pend = false; }
     u32 sb = 0; int ss = 0, nprobe = 0;
-    p8_lookup<V>(t.buckets, t.nb, sk, pend ? p8_home(sk, t) : 0u, pend, found, val, sb, ss, nprobe);
+    const u64 h = p8_hash(sk, t);
+    p8_lookup<V>(t.buckets, t.nb, sk, pend ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), pend, found, val, sb, ss, nprobe);
     if (active) {
       dok_store_val<V>(values, i, val);
       found_out[i] = found ? 1 : 0;
@@ -498,9 +529,9 @@ __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 nex
   bool act = false;
   u64 sk = 0, val = 0;
   i64 idx = 0;
-  u32 home = 0, d = 0, md_home = 0, far_home = 0;
+  u32 home = 0, fbit = 0, d = 0, md_home = 0, far_home = 0;
   // once the walk has met a free slot: the slot, and what is left to look at before the claim
-  bool chosen = false, slot_tomb = false;
+  bool chosen = false, slot_tomb = false, far_unb = false;
   u32 slot_d = 0, cd = 0, chk = 0, far_next = 0, far_to = 0;
   int slot_s = 0;
 
@@ -522,7 +553,8 @@ __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 nex
             n_fresh += p8_side_set(t, sk, val);
             if (stored) stored[i] = 1;
           } else {
-            act = true; idx = i; home = p8_home(sk, t); d = 0; chosen = false;
+            const u64 h = p8_hash(sk, t);
+            act = true; idx = i; home = dok_reduce(h, nb); fbit = p8_fbit(h); d = 0; chosen = false;
           }
         }
       }
@@ -597,12 +629,19 @@ __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 nex
           slot_s = p8_pick(gt ? gt : ge, start);
           chk = d < 31 ? (md_home & ~((2u << d) - 1u)) : 0u;
           far_next = d + 1 > 32u ? d + 1 : 32u;
-          far_to = (md_home & 1u) ? far_home : 0u;
+          far_to = (md_home & 1u) ? (far_home & 0xffu) : 0u;
+          far_unb = far_to == DOK_P8_FARCAP;
+          if (far_unb) far_to = nb > 0xffffffffULL ? 0xffffffffu : (u32)nb - 1u;
+          // without the key's filter bit in its home bucket the key was never placed elsewhere
+          if (!(far_home & fbit)) { chk = 0; far_to = 0; }
         } else if ((u64)d + 1 >= nb) {
           st = 0;                                    // no free slot anywhere
         } else {
           d++;
         }
+      }
+      else if (far_unb && cd >= 32u && ge) {
+        far_to = 0;                                    // an EMPTY slot ends the unrecorded part of the chain
       }
       if (st < 0 && chosen) {
         if (chk) { cd = (u32)__builtin_ctz(chk); chk &= chk - 1; }
@@ -617,13 +656,7 @@ __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 nex
         const u64 old = atomicCAS(tp + slot_s, expect, sk);
         if (old == expect) {
           P8<V>::store(tp, slot_s, val);
-          u64 *hb = buckets + (u64)home * 16;
-          if (td >= 32) {
-            atomicMax((u32 *)(hb + DOK_P8_META) + 1, td);
-            if (!(md_home & 1u)) atomicOr((u32 *)(hb + DOK_P8_META), 1u);
-          } else if (td > 0 && !((md_home >> td) & 1u)) {
-            atomicOr((u32 *)(hb + DOK_P8_META), 1u << td);
-          }
+          if (td > 0) p8_mark(buckets + (u64)home * 16 + DOK_P8_META, td, fbit, ((u64)far_home << 32) | md_home);
           st = 1; n_fresh++;
         } else if (old == sk) {
           st = 1;                                    // an equal key of this batch won the slot
@@ -689,7 +722,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const vo
       pend = false;
     }
     u32 sb = 0; int ss = 0, nprobe = 0;
-    p8_lookup<V>(t.buckets, t.nb, sk, pend ? p8_home(sk, t) : 0u, pend, found, val, sb, ss, nprobe);
+    const u64 h = p8_hash(sk, t);
+    p8_lookup<V>(t.buckets, t.nb, sk, pend ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), pend, found, val, sb, ss, nprobe);
     if (found) removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
     if (active && removed_out) removed_out[i] = removed ? 1 : 0;
     n_removed += removed;
@@ -712,7 +746,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_count_kernel(DevTable t, const voi
     bool pend = ok;
     if (ok && sk < 2) { found = p8_side_get(t, sk, val); pend = false; }
     u32 sb = 0; int ss = 0, nprobe = 0;
-    p8_lookup<V>(t.buckets, t.nb, sk, pend ? p8_home(sk, t) : 0u, pend, found, val, sb, ss, nprobe);
+    const u64 h = p8_hash(sk, t);
+    p8_lookup<V>(t.buckets, t.nb, sk, pend ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), pend, found, val, sb, ss, nprobe);
     n_found += found;
   }
   dok_wave_add_n(count, n_found);
@@ -844,7 +879,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_rehash_kernel(DevTable src, DevTab
     const int vw = l < P8<V>::S ? P8<V>::value_word(l) : 15;
     const u64 val = P8<V>::extract(dok_shfl64(w, gbase + vw), l);
     int st = 0, fresh = 0;
-    p8_insert<V>(dst.buckets, dst.nb, w, val, live ? p8_home(w, dst) : 0u, live, st, fresh);
+    const u64 h = p8_hash(w, dst);
+    p8_insert<V>(dst.buckets, dst.nb, w, val, live ? dok_reduce(h, dst.nb) : 0u, p8_fbit(h), live, st, fresh);
     n_fresh += fresh;
     n_full += (live && st == 0);
   }
@@ -892,7 +928,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_getitem_kernel(DevTable t, DevInde
     bool found = false;
     u64 val = 0;
     u32 sb = 0; int ss = 0, nprobe = 0;
-    p8_lookup<V>(t.buckets, t.nb, sk, ok ? p8_home(sk, t) : 0u, ok, found, val, sb, ss, nprobe);
+    const u64 h = p8_hash(sk, t);
+    p8_lookup<V>(t.buckets, t.nb, sk, ok ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), ok, found, val, sb, ss, nprobe);
     if (active) dok_store_val<V>(out, e, val);
   }
 }
@@ -919,7 +956,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_countitems_kernel(DevTable t, DevI
     bool found = false;
     u64 val = 0;
     u32 sb = 0; int ss = 0, nprobe = 0;
-    p8_lookup<V>(t.buckets, t.nb, sk, ok ? p8_home(sk, t) : 0u, ok, found, val, sb, ss, nprobe);
+    const u64 h = p8_hash(sk, t);
+    p8_lookup<V>(t.buckets, t.nb, sk, ok ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), ok, found, val, sb, ss, nprobe);
     n_found += found;
   }
   dok_wave_add_n(count, n_found);
@@ -937,7 +975,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_zeroitems_kernel(DevTable t, DevIn
     bool found = false, removed = false;
     u64 val = 0;
     u32 sb = 0; int ss = 0, nprobe = 0;
-    p8_lookup<V>(t.buckets, t.nb, sk, ok ? p8_home(sk, t) : 0u, ok, found, val, sb, ss, nprobe);
+    const u64 h = p8_hash(sk, t);
+    p8_lookup<V>(t.buckets, t.nb, sk, ok ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), ok, found, val, sb, ss, nprobe);
     if (found) removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
     n_removed += removed;
   }
@@ -958,10 +997,12 @@ __global__ __launch_bounds__(DOK_TPB) void p8_getitem_sparse_kernel(DevTable t, 
     bool found = false;
     u64 val = 0;
     u32 sb = 0; int ss = 0, nprobe = 0;
-    p8_lookup<V>(t.buckets, t.nb, sk, ok ? p8_home(sk, t) : 0u, ok, found, val, sb, ss, nprobe);
+    const u64 h = p8_hash(sk, t);
+    p8_lookup<V>(t.buckets, t.nb, sk, ok ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), ok, found, val, sb, ss, nprobe);
     const u64 ok2 = (u64)e ^ DOK_P8_XOR;
     int st = 0, fresh = 0;
-    p8_insert<V>(out.buckets, out.nb, ok2, val, found ? p8_home(ok2, out) : 0u, found, st, fresh);
+    const u64 h2 = p8_hash(ok2, out);
+    p8_insert<V>(out.buckets, out.nb, ok2, val, found ? dok_reduce(h2, out.nb) : 0u, p8_fbit(h2), found, st, fresh);
     n_fresh += fresh;
     n_full += (found && st == 0);
   }
