@@ -20,11 +20,13 @@
 //     bits 1..23   displacement map: bit d set = some key was placed d buckets past this one
 //     bit 0        a key was placed 24 or more buckets past this one ...
 //     bits 24..31  ... and the largest such displacement, 255 standing for "255 or more"
+// Buckets of two or more slots also keep a filter in the (otherwise unused) high half of slot 1's
+// tag word: every key placed away from this bucket sets the one of 32 bits its hash selects.
 // Placement is linear probing over buckets (first free slot of the walk, a tombstone before an
 // EMPTY slot; a bucket never regains an EMPTY slot), so a lookup visits the home bucket and then
-// exactly the marked displacements - independent loads, no chain walk; with no mark set, the
-// home bucket alone decides a miss.  Only beyond 254 buckets does a lookup walk on until it
-// meets a bucket with an EMPTY slot.
+// exactly the marked displacements - independent loads, no chain walk; with no mark set, or with
+// the key's filter bit clear, the home bucket alone decides a miss.  Only beyond 254 buckets does
+// a lookup walk on until it meets a bucket with an EMPTY slot.
 //
 // The rows a wave works on are staged in LDS as zero-padded words, one row per thread of the
 // workgroup, so that any lane of a group can fetch "word p of the row being served".
@@ -95,6 +97,8 @@ __device__ __forceinline__ void tg_hash_row(const DevTable &t, const TgGeom &g, 
   tag_full = ((u32)h1 & ~3u) | 3u;                   // lower half
   krow[0] = (u64)tag_full;
 }
+// The key's bit in its home bucket's filter (from the fingerprint bits of its tag).
+__device__ __forceinline__ u32 tg_fbit(u32 tag_full) { return 1u << ((tag_full >> 2) & 31u); }
 
 // Lane geometry inside a 16-lane group.
 struct TgLane {
@@ -169,6 +173,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
   const int RS = tg_rs(g);
   u64 *lds_rows = lds;                          // [DOK_TPB][1 + KW]
   u64 *lds_fb = lds + DOK_TPB * RS;             // [VW]
+  u32 *lds_meta = (u32 *)(lds_fb + g.VW);       // [DOK_TPB][2]: metadata and filter of each row's home bucket
   if (MODE == 0 && threadIdx.x < g.VW) lds_fb[threadIdx.x] = g.fallback[threadIdx.x];
   __syncthreads();
   const TgLane L(g);
@@ -179,6 +184,10 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
   const int my_word = (L.is_tag || L.is_key) ? L.p : 0;
   const u64 *exp0 = lds_rows + (wave_row0 + L.gbase) * RS + my_word;   // round r: exp0[r * RS]
   const int tl = L.gbase + L.tag_lane;          // wave lane of this lane's slot's tag
+  // lane 0 of a group holds the bucket's metadata, lane W (slot 1's tag lane) its filter
+  const bool has_filter = g.S >= 2;
+  const bool meta_lane = L.l == 0 || (has_filter && L.l == g.W);
+  u32 *meta_out = lds_meta + (wave_row0 + L.gbase) * 2 + (L.l != 0);   // round r: meta_out[2 * r]
   int n_found = 0, n_removed = 0, n_probe = 0, n_ops = 0;
 
   DOK_TILE_LOOP(n) {
@@ -215,9 +224,8 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
           const u64 hit64 = tg_match64(L, M, w[u], exp0[r * RS]) & on64;
           if (MODE == 0 && L.is_val && ((hit64 >> tl) & 1ULL))
             tg_store_word(out_g + (size_t)r * g.V, L.p - 1 - g.KW, g.V, g.unit_v, w[u]);
-          // the bucket's metadata (lane 0 holds it) is left for the row's owner in the unused
-          // upper half of the row's tag word
-          if (L.l == 0) ((u32 *)(lds_rows + (wave_row0 + L.gbase + r) * RS))[1] = (u32)(w[u] >> 32);
+          // the bucket's metadata and filter are left in LDS for the row's owner
+          if (meta_lane) meta_out[2 * r] = (u32)(w[u] >> 32);
           my_hit64 = L.l == r ? hit64 : my_hit64;
         }
       }
@@ -228,7 +236,11 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
     n_probe += active;
     // rows without a match: the home bucket's metadata decides between "absent" and "look on"
     u32 my_meta = 0;
-    if (active && !found) my_meta = ((const u32 *)krow)[1];
+    if (active && !found) {
+      my_meta = lds_meta[threadIdx.x * 2];
+      // a key placed away from its home has set its filter bit there
+      if (has_filter && !(lds_meta[threadIdx.x * 2 + 1] & tg_fbit(qfull))) my_meta = 0;
+    }
     bool open = active && !found && my_meta != 0;
     if (MODE == 0 && active && !found && !open) {
       for (int k = 0; k < g.VW; k++)
@@ -306,9 +318,11 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
   }
 }
 
-// Record in the home bucket's metadata that a key was placed d > 0 buckets further on.
-__device__ __forceinline__ void tg_mark(u64 *home_bucket, u32 d, u32 md_seen) {
+// Record in the home bucket's metadata that a key was placed d > 0 buckets further on, and (W > 0:
+// the bucket has a filter, in slot 1's tag word) the key's filter bit.
+__device__ __forceinline__ void tg_mark(u64 *home_bucket, u32 d, u32 md_seen, int W, u32 fbit, u32 filt_seen) {
   u32 *meta = (u32 *)home_bucket + 1;
+  if (W > 0 && !(filt_seen & fbit)) atomicOr((u32 *)(home_bucket + W) + 1, fbit);
   if (d <= DOK_TG_NEAR) {
     if (!((md_seen >> d) & 1u)) atomicOr(meta, 1u << d);
     return;
@@ -357,7 +371,9 @@ __device__ __forceinline__ void tg_insert_rows(const DevTable &t, const TgGeom &
   const u64 *krow = lds_rows + threadIdx.x * RS;
   if (!pend) home = 0;
   const u32 qbusy = qfull & ~1u;
-  u32 cur = 0, md_home = 0;                       // displacement inspected this turn; home metadata
+  const u32 fbit = tg_fbit(qfull);
+  const bool has_filter = g.S >= 2;
+  u32 cur = 0, md_home = 0, filt_home = 0;        // displacement inspected this turn; home metadata and filter
   bool chosen = false, slot_tomb = false, confirm = false, far_unb = false;
   u32 slot_d = 0, slot_w = 0, chk = 0, far_next = 0, far_to = 0;
 
@@ -415,7 +431,7 @@ __device__ __forceinline__ void tg_insert_rows(const DevTable &t, const TgGeom &
       } else {
         confirm = false;
         if (!chosen) {
-          if (cur == 0) md_home = md;
+          if (cur == 0) { md_home = md; filt_home = (u32)(tw[1] >> 32); }
           if (tombm | emptym) {
             chosen = true;
             slot_tomb = tombm != 0;
@@ -425,6 +441,8 @@ __device__ __forceinline__ void tg_insert_rows(const DevTable &t, const TgGeom &
             far_unb = (md_home & 1u) && (md_home >> 24) == DOK_TG_FARCAP;
             far_to = (md_home & 1u) ? (far_unb ? 0xffffffffu : (md_home >> 24)) : 0u;
             far_next = cur + 1 > DOK_TG_NEAR + 1u ? cur + 1 : DOK_TG_NEAR + 1u;
+            // without the key's filter bit in its home bucket the key was never placed elsewhere
+            if (has_filter && !(filt_home & fbit)) { chk = 0; far_to = 0; }
           } else if ((u64)cur + 1 >= t.nb) {
             st = 0; pend = false;                          // no free slot anywhere
           } else {
@@ -445,7 +463,7 @@ __device__ __forceinline__ void tg_insert_rows(const DevTable &t, const TgGeom &
             if (atomicCAS(tagp, expect, qbusy) == expect) {
               wr = true; wr_fresh = true; wr_b = tb; wr_w = slot_w;
               st = 1; fresh = 1; pend = false;
-              if (slot_d > 0) tg_mark(t.buckets + (u64)home * 16, slot_d, md_home);
+              if (slot_d > 0) tg_mark(t.buckets + (u64)home * 16, slot_d, md_home, has_filter ? g.W : 0, fbit, filt_home);
             } else {
               chosen = false; cur = slot_d;                // somebody took the slot: look at that bucket again
             }
@@ -620,7 +638,7 @@ static int tg_geom(const DevTable &d, const void *fallback, TgGeom &g) {
 
 static bool tg_aligned(const void *p, int unit) { return ((uintptr_t)p & (uintptr_t)(unit - 1)) == 0; }
 
-static size_t tg_lds_lookup(const TgGeom &g) { return (size_t)(DOK_TPB * (g.KW + 1) + g.VW) * 8; }
+static size_t tg_lds_lookup(const TgGeom &g) { return (size_t)(DOK_TPB * (g.KW + 1) + g.VW + DOK_TPB) * 8; }
 static size_t tg_lds_insert(const TgGeom &g) { return (size_t)DOK_TPB * (g.KW + 1 + g.VW) * 8; }
 
 // Most workgroups of the kernels that loop over tiles and end with one atomic per wave on a
