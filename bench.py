@@ -225,7 +225,7 @@ def other_configs(device):
     res["cfg1_set_ms"] = round(timed(lambda: hm.set(k[:65536, None], v))[0], 4)
     hm.get(k[:, None])                  # (the first call of a size pays for the allocation of its outputs)
     res["cfg1_get_ms"] = round(timed(lambda: hm.get(k[:, None]))[0], 4)
-    res["cfg1_remove_ms"] = round(timed(lambda: hm._remove_rows(k[:32768, None].contiguous()))[0], 4)
+    res["cfg1_remove_ms"] = round(timed(lambda: hm._remove_rows(k[:32768, None].contiguous(), unique=True))[0], 4)
 
     # cfg2: 1M float32[3] keys -> int64[5], capacity 2^21 (tagged layout)
     gen.manual_seed(1002)
@@ -237,7 +237,7 @@ def other_configs(device):
     res["cfg2_set_ms"] = round(timed(lambda: hm2.set(k2, v2))[0], 4)
     hm2.get(q2)
     res["cfg2_get_ms"] = round(timed(lambda: hm2.get(q2))[0], 4)
-    res["cfg2_remove_ms"] = round(timed(lambda: hm2._remove_rows(k2[:250_000].contiguous()))[0], 4)
+    res["cfg2_remove_ms"] = round(timed(lambda: hm2._remove_rows(k2[:250_000].contiguous(), unique=True))[0], 4)
     del hm, hm2, k2, v2, q2
 
     # cfg4: 2-D 1e6 x 1e6 float32, 50M entries
@@ -288,7 +288,7 @@ def other_configs(device):
     res["cfg5_64_getitems_ms"] = round(timed(gets)[0], 3)
     n_gone = lin.numel() // 5
     gone = coords[:, :n_gone].T.contiguous()
-    res["cfg5_remove_20M_ms"] = round(timed(lambda: dok.storage()._remove_rows(gone))[0], 3)
+    res["cfg5_remove_20M_ms"] = round(timed(lambda: dok.storage()._remove_rows(gone, unique=True))[0], 3)
     fresh = torch.stack([torch.randint(0, s, (n_gone,), generator=gen, device=device) for s in size], dim=1)
     fv = torch.randn(n_gone, 1, generator=gen, device=device).half()
     res["cfg5_reinsert_20M_ms"] = round(timed(lambda: dok.storage().set(fresh, fv))[0], 3)
@@ -322,7 +322,7 @@ def tagged_scale(device, n=32_000_000):
         set_ = lambda: _lib.check(lib.dok_map_set(desc, k.data_ptr(), v.data_ptr(), n, None, stream), "set")
         get = lambda: _lib.check(lib.dok_map_get(desc, q.data_ptr(), n, out_v.data_ptr(), None,
                                                  out_f.data_ptr(), stream), "get")
-        rem = lambda: _lib.check(lib.dok_map_remove(desc, quarter.data_ptr(), n // 4, out_f.data_ptr(), stream), "remove")
+        rem = lambda: _lib.check(lib.dok_map_remove_unique(desc, quarter.data_ptr(), n // 4, out_f.data_ptr(), stream), "remove")
         s_avg, _ = time_kernel(set_, 3, prep=clear)
         assert hm.n_elements == n
         o_avg, _ = time_kernel(set_, 3)
@@ -504,13 +504,19 @@ def main():
         half = keys[: n // 2]
         rem_f = torch.empty(n // 2, device=device, dtype=torch.uint8)
         def raw_remove():
-            _dl.check(_dl.load().dok_map_remove(ctypes.byref(hm._desc), half.data_ptr(), n // 2, rem_f.data_ptr(),
-                                                _stream_ptr(device)), "remove")
+            # (the keys are distinct: the variant CudaClosedHashmap.remove runs after its unique)
+            _dl.check(_dl.load().dok_map_remove_unique(ctypes.byref(hm._desc), half.data_ptr(), n // 2,
+                                                       rem_f.data_ptr(), _stream_ptr(device)), "remove")
         raw_remove()
         assert bool(rem_f.all()) and hm.n_elements == n - n // 2
         r_avg, _ = time_kernel(raw_remove, 5, prep=lambda: raw_set(half, values[: n // 2]))
         results["remove_ms_lf05"] = round(r_avg, 4)
         results["remove_mops_lf05"] = round((n // 2) / r_avg / 1e3, 1)
+        def raw_remove_cas():                  # any batch, equal keys allowed: one compare-and-swap per row
+            _dl.check(_dl.load().dok_map_remove(ctypes.byref(hm._desc), half.data_ptr(), n // 2, rem_f.data_ptr(),
+                                                _stream_ptr(device)), "remove")
+        rc_avg, _ = time_kernel(raw_remove_cas, 3, prep=lambda: raw_set(half, values[: n // 2]))
+        results["remove_cas_mops_lf05"] = round((n // 2) / rc_avg / 1e3, 1)
         del half, rem_f
         del hm
         torch.cuda.empty_cache()

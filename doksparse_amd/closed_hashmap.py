@@ -683,15 +683,17 @@ class CudaClosedHashmap:
             unique_keys = keys.reshape(-1).unique().reshape(-1, *self._key_shape)
         else:
             unique_keys = keys.unique(dim=0)
-        return self._remove_rows(self._prep_rows(unique_keys, "keys"))
+        return self._remove_rows(self._prep_rows(unique_keys, "keys"), unique=True)
 
-    def _remove_rows(self, keys):
-        """Remove without the sort: mask aligned with ``keys`` (equal rows: one reports True)."""
+    def _remove_rows(self, keys, unique=False):
+        """Remove without the sort: mask aligned with ``keys`` (equal rows: one reports True).
+        unique=True: the caller vouches that no row occurs twice (no atomic per row is needed then)."""
         n = keys.shape[0]
         is_removed = torch.empty(n, device=self.device, dtype=torch.bool)
         lib = _lib.load()
-        _lib.check(lib.dok_map_remove(ctypes.byref(self._desc), keys.data_ptr(), n,
-                                      is_removed.data_ptr(), _stream_ptr(self.device)), "remove")
+        fn = lib.dok_map_remove_unique if unique else lib.dok_map_remove
+        _lib.check(fn(ctypes.byref(self._desc), keys.data_ptr(), n,
+                      is_removed.data_ptr(), _stream_ptr(self.device)), "remove")
         return is_removed
 
     def count_existing(self, keys):

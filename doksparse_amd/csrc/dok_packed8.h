@@ -703,8 +703,10 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void p8_set_kernel(DevTa
   });
 }
 
-// Tombstone the matching slot with a CAS so that equal keys in one batch remove it once.
-template <int V, int KF>
+// Tombstone the matching slot: with a CAS, so that equal keys in one batch remove it once, or -
+// UNIQUE: the caller vouches that the batch holds no key twice - with a plain store, as the
+// reference does after its host-side unique (one returning atomic in HBM less per row).
+template <int V, int KF, bool UNIQUE>
 __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                             u8 *__restrict__ removed_out) {
   int n_removed = 0;
@@ -724,7 +726,10 @@ __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const vo
     u32 sb = 0; int ss = 0, nprobe = 0;
     const u64 h = p8_hash(sk, t);
     p8_lookup<V>(t.buckets, t.nb, sk, pend ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), pend, found, val, sb, ss, nprobe);
-    if (found) removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
+    if (found) {
+      if (UNIQUE) { t.buckets[(u64)sb * 16 + ss] = DOK_P8_TOMB; removed = true; }
+      else removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
+    }
     if (active && removed_out) removed_out[i] = removed ? 1 : 0;
     n_removed += removed;
   }

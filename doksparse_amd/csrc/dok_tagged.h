@@ -155,7 +155,8 @@ __device__ __forceinline__ u32 tg_wrap(u32 home, u32 d, u64 nb) {
   return (u32)(b >= nb ? b - nb : b);
 }
 
-// mode 0: get (write value or fallback + flag), 1: count, 2: remove.
+// mode 0: get (write value or fallback + flag), 1: count, 2: remove, 3: remove of a batch that
+// holds no key twice (the tombstone is a plain store instead of a compare-and-swap).
 // Rows are taken in tiles of DOK_TPB (see DOK_TILE_LOOP); a wave only ever reads the LDS rows its
 // own lanes staged, so the tiles need no workgroup barrier between them.
 // Phase 1 serves the home bucket of each of a group's 16 rows as "issue 8 loads, resolve 8
@@ -304,14 +305,15 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
     bool removed = false;
     if (MODE == 2 && found)
       removed = atomicCAS((u32 *)(t.buckets + (u64)sb * 16 + sw), qfull, DOK_TG_TOMB) == qfull;
+    if (MODE == 3 && found) { *(u32 *)(t.buckets + (u64)sb * 16 + sw) = DOK_TG_TOMB; removed = true; }
     if (MODE == 0 && active) flags[i] = found ? 1 : 0;
-    if (MODE == 2 && active && flags) flags[i] = removed ? 1 : 0;
+    if (MODE >= 2 && active && flags) flags[i] = removed ? 1 : 0;
     n_found += found;
     n_removed += removed;
     n_ops += active;
   }
   if (MODE == 1) dok_wave_add_n(count, n_found);
-  if (MODE == 2) dok_wave_add_n(&t.header[DOK_H_NELEM], -n_removed);
+  if (MODE >= 2) dok_wave_add_n(&t.header[DOK_H_NELEM], -n_removed);
   if (STATS) {
     dok_wave_add_n(&t.header[DOK_H_NPROBE], n_probe);
     dok_wave_add_n(&t.header[DOK_H_NOPS], n_ops);
@@ -679,13 +681,17 @@ static int tg_launch_count(const DevTable &d, const void *keys, i64 n, i64 *coun
   return DOK_OK;
 }
 
-static int tg_launch_remove(const DevTable &d, const void *keys, i64 n, u8 *removed, hipStream_t s) {
+static int tg_launch_remove(const DevTable &d, const void *keys, i64 n, u8 *removed, bool unique, hipStream_t s) {
   TgGeom g;
   int rc = tg_geom(d, nullptr, g);
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k)) return DOK_EINVAL;
-  const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_lookup_kernel<2, false><<<(grid < DOK_TG_REMOVE_GRID ? grid : DOK_TG_REMOVE_GRID), DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, nullptr, removed, nullptr);
+  const unsigned tiles = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
+  const unsigned grid = tiles < DOK_TG_REMOVE_GRID ? tiles : DOK_TG_REMOVE_GRID;
+  if (unique)
+    tg_lookup_kernel<3, false><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, nullptr, removed, nullptr);
+  else
+    tg_lookup_kernel<2, false><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, nullptr, removed, nullptr);
   return DOK_OK;
 }
 

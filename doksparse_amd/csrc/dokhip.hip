@@ -365,7 +365,7 @@ int dok_coo_build_bulk(const dok_table_t *t, const int64_t *indices, const void 
   return set_bulk(t, indices, values, n, true, true, workspace, workspace_bytes, stream);
 }
 
-int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t *removed, void *stream) {
+static int map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t *removed, bool unique, void *stream) {
   DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
@@ -374,12 +374,24 @@ int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t *r
   if (!keys) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   if (layout == DOK_LAYOUT_PACKED8) {
-    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_remove_kernel<V, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
+    if (unique) {
+      P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_remove_kernel<V, KF, true><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
+    } else {
+      P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_remove_kernel<V, KF, false><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
+    }
   } else {
-    rc = tg_launch_remove(d, keys, n, removed, s);
+    rc = tg_launch_remove(d, keys, n, removed, unique, s);
     if (rc) return rc;
   }
   return note_launch();
+}
+
+int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t *removed, void *stream) {
+  return map_remove(t, keys, n, removed, false, stream);
+}
+
+int dok_map_remove_unique(const dok_table_t *t, const void *keys, int64_t n, uint8_t *removed, void *stream) {
+  return map_remove(t, keys, n, removed, true, stream);
 }
 
 int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n, int64_t *count, void *stream) {

@@ -161,6 +161,15 @@ int dok_map_build_bulk(const dok_table_t *t, const void *keys, const void *value
 int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n,
                    uint8_t *removed, void *stream);
 
+/* dok_map_remove for a batch in which no key occurs twice - what the reference's kernel is given,
+ * because CudaClosedHashmap.remove passes its keys through unique(dim=0) first
+ * (cuda_closed_hashmap.py:438) and the kernel then stores the REMOVED marker without any atomic
+ * (closed_hashmap_impl_class.cu:459-484).  The tombstone is a plain store here as well, which
+ * saves one returning atomic in HBM per row.  With a key twice in the batch both rows would
+ * report 1 and header[DOK_H_NELEM] would shrink twice: use dok_map_remove for such batches. */
+int dok_map_remove_unique(const dok_table_t *t, const void *keys, int64_t n,
+                          uint8_t *removed, void *stream);
+
 /* count[0] += number of rows whose key is present.  count is a device int64.
  * Reference: ClosedHashmap::exists (closed_hashmap_impl_class.cu:253-278). */
 int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n,
