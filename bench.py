@@ -30,13 +30,15 @@ HBM_PEAK_GBS = 8000.0
 # hold the runs.  The figures belong to one state of the kernel sources, named by `csrc_sha16`
 # (see csrc_sha16()): when the sources have changed since, nothing measured is reported.
 PROFILED = {
-    "csrc_sha16": "unset",
-    "get_lf05": None,         # p8_get_kernel, load factor 0.5
-    "get_lf09": None,         # p8_get_kernel, load factor 0.9
-    "set_bulk_lf05": None,    # the bulk upsert's kernels together, into a cleared table
-    "build_lf05": None,       # the bulk build's kernels together, into uninitialised memory
-    "set_cas_lf05": None,     # p8_set_kernel (one compare-and-swap per row)
-    "remove_lf05": None,      # p8_remove_kernel, half of the keys
+    "csrc_sha16": "8bbba435b5185ec5",
+    "get_lf05": 6.658e9,         # p8_get_kernel, load factor 0.5
+    "get_lf09": 6.946e9,         # p8_get_kernel, load factor 0.9
+    "set_bulk_lf05": 8.868e9,    # the bulk upsert's kernels together, into a cleared table
+    "build_lf05": 7.143e9,       # the bulk build's kernels together, into uninitialised memory
+    "set_bulk_lf09": 7.388e9,
+    "build_lf09": 6.429e9,
+    "set_cas_lf05": 1.615e10,    # p8_set_kernel (one compare-and-swap per row)
+    "remove_lf05": 5.669e9,      # p8_remove_kernel, half of the keys, plain-store tombstones
 }
 # algorithmic bytes per op for 8-byte keys and 4-byte values: one 128-byte bucket line per op,
 # plus the batch row and the outputs
@@ -343,6 +345,61 @@ def tagged_scale(device, n=32_000_000):
     return res
 
 
+def dok_scale(device):
+    """The DOK indexing kernels at scale, kernel-level through the C ABI on preallocated buffers:
+    a 2-D 1e6 x 1e6 float32 tensor of 50M entries (BASELINE configuration 4); gather of 2^26
+    stored coordinates through `__getitem__`'s kernel, scatter of 10M coordinates (half present,
+    half new) through `__setitem__`'s, and the read-out of all entries."""
+    from doksparse_amd import SparseDOKTensor, _lib
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    lib = _lib.load()
+    res = {}
+    gen = torch.Generator(device=device)
+    gen.manual_seed(1004)
+    lin = torch.unique(torch.randint(0, 10**12, (50_000_000,), generator=gen, device=device))
+    lin = lin[torch.randperm(lin.numel(), generator=gen, device=device)]
+    coords = torch.stack([lin // 10**6, lin % 10**6])
+    vals = torch.randn(lin.numel(), generator=gen, device=device)
+    dok = SparseDOKTensor((10**6, 10**6), coords, vals, device=device)
+    hm = dok.storage()
+    hm.rehash(120_000_000)                       # room for the scatter below without a growth
+    nnz = hm.n_elements
+    stream = _stream_ptr(device)
+    # gather: 2^26 stored coordinates, in random order
+    n_g = 1 << 26
+    pick = torch.randint(0, lin.numel(), (n_g,), generator=gen, device=device)
+    r, c = coords[0][pick].contiguous(), coords[1][pick].contiguous()
+    ix, out_shape, _, keep = dok._plan((r, c))
+    out = torch.empty(n_g, device=device, dtype=torch.float32)
+    gather = lambda: _lib.check(lib.dok_getitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), out.data_ptr(), stream), "getitem")
+    gather()
+    assert torch.equal(out, vals[pick])
+    g_avg, _ = time_kernel(gather, 5)
+    res["dok_getitem_2p26_ms"] = round(g_avg, 4)
+    res["dok_getitem_2p26_mops"] = round(n_g / g_avg / 1e3, 1)
+    del pick, r, c, out, ix, keep
+    # scatter: 5M present + 5M new coordinates
+    sc = torch.cat([coords[:, :5_000_000], torch.randint(0, 10**6, (2, 5_000_000), generator=gen, device=device)], dim=1)
+    sc = sc[:, torch.randperm(sc.shape[1], generator=gen, device=device)].contiguous()
+    sv = torch.randn(sc.shape[1], generator=gen, device=device)
+    ix, _, _, keep = dok._plan((sc[0], sc[1]))
+    view = _lib.DokView()
+    view.data = sv.data_ptr()
+    view.strides[0] = 1
+    scatter = lambda: _lib.check(lib.dok_setitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), ctypes.byref(view), stream), "setitem")
+    s_first, _ = timed(scatter)                   # half of the rows are new
+    s_avg, _ = time_kernel(scatter, 3)            # every row present
+    res["dok_setitem_10M_ms"] = round(s_first, 4)
+    res["dok_setitem_10M_overwrite_ms"] = round(s_avg, 4)
+    assert hm.n_elements > nnz
+    # read-out of every entry as [ndim, nnz] coordinates + values
+    ro, _ = timed(lambda: hm.items_coo())
+    ro, _ = timed(lambda: hm.items_coo())
+    res["dok_readout_ms"] = round(ro, 4)
+    res["dok_entries"] = hm.n_elements
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -359,6 +416,8 @@ def main():
                     help="also time the tagged layout at 32M float32[3] -> int64[5] keys (reported under extra)")
     ap.add_argument("--only-tagged", action="store_true",
                     help="run nothing but the --tagged leg and print its figures (for profiling that leg)")
+    ap.add_argument("--only-dok", action="store_true",
+                    help="run nothing but the DOK indexing kernels at scale and print their figures (for profiling)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one read-only pass over the whole table (the live-entry count of "
                          "the read-out path); with the table clear that every run does, this gives "
@@ -376,6 +435,9 @@ def main():
     torch.cuda.set_device(device)
     if args.only_tagged:
         print(json.dumps({"extra": tagged_scale(device)}), flush=True)
+        return
+    if args.only_dok:
+        print(json.dumps({"extra": dok_scale(device)}), flush=True)
         return
     n = args.keys
     gen = torch.Generator(device=device)
@@ -567,6 +629,8 @@ def main():
         for name, entry, ms_key, ops in (("get_lf09", "get_lf09", "get_kernel_ms_lf09", n),
                                          ("set_lf05", "set_bulk_lf05", "set_bulk_ms_lf05", n),
                                          ("build_lf05", "build_lf05", "build_ms_lf05", n),
+                                         ("set_lf09", "set_bulk_lf09", "set_bulk_ms_lf09", n),
+                                         ("build_lf09", "build_lf09", "build_ms_lf09", n),
                                          ("set_per_row_lf05", "set_cas_lf05", "set_cas_kernel_ms_lf05", n),
                                          ("remove_lf05", "remove_lf05", "remove_ms_lf05", n // 2)):
             ms = results.get(ms_key)
