@@ -584,13 +584,26 @@ def main():
         torch.cuda.empty_cache()
 
         # ---------------- load factor 0.9 ---------------------------------------------------
-        hm9 = build_map(keys, values, cap09, device)
-        assert hm9.n_elements == n
-        raw_get9, raw_set9, raw_clear9 = raw_calls(hm9)
-        v, f = hm9.get(queries[:, None])
-        assert int(f.sum().item()) == n_hit
-        del v, f
-        g9, _ = time_kernel(lambda: raw_get9(queries, out_v, out_f), 10)
+        # Which keys end up away from their home bucket depends on the order in which the rows of a
+        # build arrive (atomic reservations), and the hottest key of the Zipf batch alone is 5 % of
+        # the queries: the table is therefore built four times and the get figures are means over
+        # the builds (the spread is reported beside them).
+        g9s, p9s = [], []
+        for rep in range(4):
+            hm9 = build_map(keys, values, cap09, device)
+            assert hm9.n_elements == n
+            raw_get9, raw_set9, raw_clear9 = raw_calls(hm9)
+            if rep == 0:
+                v, f = hm9.get(queries[:, None])
+                assert int(f.sum().item()) == n_hit
+                del v, f
+            g9s.append(time_kernel(lambda: raw_get9(queries, out_v, out_f), 5)[0])
+            p9s.append(hm9.probe_stats(queries[:, None]))
+            if rep < 3:
+                del hm9, raw_get9, raw_set9, raw_clear9
+        g9 = float(np.mean(g9s))
+        results["get_kernel_ms_lf09_builds"] = [round(x, 4) for x in g9s]
+        results["probe_len_lf09_builds"] = [round(x, 4) for x in p9s]
         s9, _ = time_kernel(lambda: raw_set9(keys, values), 3, prep=raw_clear9)
         results["set_cas_mops_lf09"] = round(n / s9 / 1e3, 1)
         bulk9 = raw_bulk_set(hm9, n)
@@ -608,7 +621,7 @@ def main():
         results["get_kernel_ms_lf09"] = round(g9, 4)
         results["get_mops_lf09"] = round(n / g9 / 1e3, 1)
         results["set_mops_lf09"] = round(n / s9 / 1e3, 1)
-        results["probe_len_lf09"] = round(hm9.probe_stats(queries[:, None]), 4)
+        results["probe_len_lf09"] = round(float(np.mean(p9s)), 4)
         results["load_factor_09_physical"] = round(n / (hm9._n_phys * hm9._slots_per_bucket), 4)
         del hm9
 

@@ -35,14 +35,16 @@ def _stream_ptr(device):
 
 # A batch goes through the bulk insert (partition by table range, merge each range in LDS)
 # instead of the per-row compare-and-swap kernel when it is large in absolute terms and holds at
-# least this many rows per physical bucket.  The bulk path costs about 35 us per million rows
-# plus 59 us per million buckets (it streams the whole table once) plus ~0.13 ms of launches;
-# the per-row kernel about 66 us per million rows (MI355X, 8-byte keys, 4-byte values).
+# least this many rows per physical bucket.  The bulk path costs about 22 us per million rows
+# plus 45 us per million buckets (it streams the whole table once) plus ~0.05 ms of launches;
+# the per-row kernel about 66 us per million rows (MI355X, 8-byte keys, 4-byte values; measured
+# 1M .. 33M rows: at 2 rows per bucket the bulk path is 1.1x to 1.4x faster, at 5 rows 1.5x to
+# 1.9x, at 1.25 rows 0.8x to 0.97x).
 # In a table that ends up nearly full the per-row kernel walks longer chains (about 100 us per
 # million rows into a table at 85 % with tombstones), so there the bulk path pays from fewer
 # rows per bucket on.
-BULK_MIN_ROWS = 1 << 23
-BULK_MIN_ROWS_PER_BUCKET = 2.5
+BULK_MIN_ROWS = 1 << 20
+BULK_MIN_ROWS_PER_BUCKET = 2.0
 BULK_MIN_ROWS_PER_BUCKET_LOADED = 1.5
 BULK_LOADED_FILL = 0.7
 
@@ -774,7 +776,7 @@ class CudaClosedHashmap:
         table, header, desc, n_phys, slots, layout = self._alloc_table(n_buckets, clear=False)
         if layout == _lib.DOK_LAYOUT_PACKED8:
             ws = None
-            if self._n_upper >= BULK_MIN_ROWS and self._n_upper >= BULK_MIN_ROWS_PER_BUCKET * n_phys:
+            if self._n_upper >= (1 << 23) and self._n_upper >= 2.5 * n_phys:
                 # (the upper bound is only a hint for picking the path; both give the same table)
                 nbytes = int(lib.dok_rehash_bulk_workspace_bytes(ctypes.byref(old[2]), ctypes.byref(desc)))
                 if nbytes > 0:

@@ -8,13 +8,15 @@
 //
 //   1. the table is cut into ranges of DOK_BULK_R consecutive buckets; the range of a row is
 //      (home bucket) / DOK_BULK_R;
-//   2. two count + scan + scatter passes (first by range / 256 (range / 1024 for very large tables), then by range inside
-//      each first-level bin) move every (key, value) row next to the other rows of its range.
-//      Every workgroup of a scatter owns a fixed stretch of the input; the count pass records how
-//      many of that stretch's rows go to each bin, a prefix sum over the workgroups turns the
-//      counts into the workgroup's private write cursors, and the scatter therefore needs no
-//      atomic on global memory.  A scatter tile is staged in LDS ordered by bin, so the global
-//      writes are runs of consecutive addresses;
+//   2. two scatter passes (first by range / 256 (range / 1024 for very large tables), then by
+//      range inside each first-level bin) move every (key, value) row next to the other rows of
+//      its range.  Nothing is counted beforehand: every bin owns a region of fixed capacity in the
+//      pass's output - the rows a uniform hash sends there on average plus seven standard
+//      deviations - and a workgroup that has staged a tile of rows in LDS, ordered by bin,
+//      reserves the run of each bin with ONE atomic add on that bin's fill counter (a few hundred
+//      atomics per tile of thousands of rows, issued while the tile is being staged, so their
+//      latency is hidden).  Rows that find their bin's region full (batches with very many
+//      equal keys) go to a spill list that the ordinary insert works through at the end;
 //   3. one workgroup per range copies the range's buckets into LDS, places the range's rows
 //      there and streams the buckets back (a table that holds nothing yet is not read: the
 //      copy starts empty, and the clear of the table is saved as well);
@@ -23,8 +25,9 @@
 //   5. the handful of rows left (overflow of the per-range lists, keys that may sit at far
 //      displacements) are handed, packed, to the ordinary insert, which runs last.
 //
-// Every step is exact for any input: bin sizes are counted, not estimated, and a batch whose
-// rows all fall into one range merely degrades to step 5's ordinary insert.
+// Every step is exact for any input: a bin that receives more rows than its region holds spills
+// the surplus, and a batch whose rows all fall into one range merely degrades to step 5's
+// ordinary insert.
 #pragma once
 #include "dok_packed8.h"
 
@@ -69,11 +72,12 @@
 struct BulkWs {
   u64 *keysA, *keysB;       // [n] each: rows after the first / second scatter
   void *valsA, *valsB;      // [n] values of value_bytes each
-  u32 *wg_hist;             // [n_big][GRID]: rows of workgroup w's stretch that go to first-level bin b;
-                            //                after the scan, the exclusive prefix sum over w
-  u32 *big_off;             // [n_big + 1]    start of every first-level bin in keysA
-  u32 *sub_hist;            // [n_big << sublog][ch]: the same for the ch stretches of a first-level bin
-  u32 *part_off;            // [(n_big << sublog) + 1]  start of every range in keysB
+  u32 *big_cnt;             // [n_big]             rows reserved so far in first-level bin b, whose region is
+                            //                     keysA[b * big_cap, (b + 1) * big_cap)
+  u32 *part_cnt;            // [n_big << sublog]   the same for range p: keysB[p * part_cap, (p + 1) * part_cap)
+  u64 *spill_keys;          // [spill_cap] rows that found their bin's region full
+  void *spill_vals;
+  u32 *spill_cnt;           // [1]
   u32 *def_cnt;             // [GRID] rows each merge workgroup handed to the ordinary insert
   u32 *meta_cnt;            // [GRID] displacement marks each merge workgroup left to be applied
   u32 *edge_cnt;            // [GRID] rows each merge workgroup could not place in the last range of its block
@@ -81,8 +85,20 @@ struct BulkWs {
   u32 sublog;               // log2 of the ranges per first-level bin
   u32 g1;                   // workgroups of the first pass (a multiple of 64, at most DOK_BULK_GRID)
   u32 ch;                   // stretches (workgroups) per first-level bin in the second pass
+  u32 big_cap, part_cap;    // rows a first-level bin's / a range's region holds
+  u32 spill_cap;
   i64 share;                // rows per workgroup in the first pass
 };
+
+// The rows of first-level bin b / of range p that the passes have delivered.
+__device__ __forceinline__ u32 bulk_big_n(const BulkWs &ws, u32 b) {
+  const u32 c = ws.big_cnt[b];
+  return c < ws.big_cap ? c : ws.big_cap;
+}
+__device__ __forceinline__ u32 bulk_part_n(const BulkWs &ws, u32 p) {
+  const u32 c = ws.part_cnt[p];
+  return c < ws.part_cap ? c : ws.part_cap;
+}
 
 // Exclusive prefix sum of one value per thread over the workgroup (blockDim.x a multiple of 64,
 // at most 1024).  `wsum` is LDS scratch of 16 words.  Ends with a barrier.
@@ -171,7 +187,7 @@ __device__ __forceinline__ void bulk_stretch1(const BulkWs &ws, i64 n, u32 w, i6
   if (lo > hi) lo = hi;
 }
 __device__ __forceinline__ void bulk_stretch2(const BulkWs &ws, u32 b, u32 c, i64 &lo, i64 &hi) {
-  const i64 lo0 = ws.big_off[b], hi0 = ws.big_off[b + 1];
+  const i64 lo0 = (i64)b * ws.big_cap, hi0 = lo0 + bulk_big_n(ws, b);
   const i64 len = (hi0 - lo0 + ws.ch - 1) / ws.ch;
   lo = lo0 + (i64)c * len;
   hi = lo + len;
@@ -179,21 +195,24 @@ __device__ __forceinline__ void bulk_stretch2(const BulkWs &ws, u32 b, u32 c, i6
   if (lo > hi) lo = hi;
 }
 
-// ---- pass 1, count: rows of every workgroup's stretch per first-level bin ------------------------
-// EMIT: the keys are coordinate rows of several words each; their linearised form is written to
-// keysB (free until the second scatter) so that the first scatter reads 8 bytes per row instead
-// of the coordinates a second time.
-template <int KF, bool EMIT, int ND>
-__global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count1_kernel(DevTable t, const void *__restrict__ keys, i64 n,
-                                                                   BulkWs ws) {
-  // Few bins and 64 lanes per atomic instruction mean many lanes on one address, which the LDS
-  // serialises; four copies of the histogram, picked by the lane, thin that out.
-  __shared__ u32 cnt[4 * DOK_BULK_MAXBIG];
-  for (int b = threadIdx.x; b < 4 * DOK_BULK_MAXBIG; b += DOK_BULK_CTPB) cnt[b] = 0;
-  __syncthreads();
-  const u32 copy = (threadIdx.x & 3) * DOK_BULK_MAXBIG;
-  // rows a thread has in flight: 8 to 16 eight-byte loads
-  constexpr int U = ND <= 2 ? 8 : ND <= 4 ? 4 : 2;
+// ---- set-up: every fill counter to zero (and, for a build, the table header) ------------------------
+__global__ __launch_bounds__(DOK_TPB) void bulk_init_kernel(BulkWs ws, i64 *header) {
+  const u32 n_parts = ws.n_big << ws.sublog;
+  for (u32 i = blockIdx.x * DOK_TPB + threadIdx.x; i < n_parts; i += gridDim.x * DOK_TPB) ws.part_cnt[i] = 0;
+  if (blockIdx.x == 0) {
+    for (u32 i = threadIdx.x; i < ws.n_big; i += DOK_TPB) ws.big_cnt[i] = 0;
+    if (threadIdx.x == 0) ws.spill_cnt[0] = 0;
+    if (header && threadIdx.x < DOK_HEADER_WORDS) header[threadIdx.x] = 0;
+  }
+}
+
+// ---- coordinate rows of three and more dimensions are linearised once, into keysB (free until the
+// second scatter), so that the first scatter reads 8 bytes per row and holds one word per row in
+// registers instead of the coordinates; all ones marks a row outside the table's coordinate space.
+template <int KF, int ND>
+__global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_linearise_kernel(DevTable t, const void *__restrict__ keys, i64 n,
+                                                                      BulkWs ws) {
+  constexpr int U = ND <= 4 ? 4 : 2;
   i64 lo, hi;
   bulk_stretch1(ws, n, blockIdx.x, lo, hi);
   for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += U * DOK_BULK_CTPB) {
@@ -203,92 +222,13 @@ __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count1_kernel(DevTable t, 
       const i64 i = i0 + u * DOK_BULK_CTPB;
       if (i < hi) bulk_fetch<KF, ND>(t, keys, i, n, raw[u]);
     }
-    u64 key[U];
-    bool ok[U];
     #pragma unroll
     for (int u = 0; u < U; u++) {
       const i64 i = i0 + u * DOK_BULK_CTPB;
-      key[u] = 0;
-      ok[u] = i < hi && bulk_finish<KF, ND>(t, raw[u], key[u]) == 1;
-      if (EMIT && i < hi) ws.keysB[i] = ok[u] ? key[u] : ~0ULL;
+      u64 key = 0;
+      if (i < hi) ws.keysB[i] = bulk_finish<KF, ND>(t, raw[u], key) == 1 ? key : ~0ULL;
     }
-    #pragma unroll
-    for (int u = 0; u < U; u++)
-      if (ok[u] && (key[u] ^ DOK_P8_XOR) >= 2)
-        atomicAdd(&cnt[copy + (bulk_range_of(key[u], t) >> ws.sublog)], 1u);
   }
-  __syncthreads();
-  for (int b = threadIdx.x; b < (int)ws.n_big; b += DOK_BULK_CTPB)
-    ws.wg_hist[(size_t)b * ws.g1 + blockIdx.x] =
-        cnt[b] + cnt[DOK_BULK_MAXBIG + b] + cnt[2 * DOK_BULK_MAXBIG + b] + cnt[3 * DOK_BULK_MAXBIG + b];
-}
-
-// ---- pass 1, scan: per bin over the workgroups, then over the bins ---------------------------------
-__global__ __launch_bounds__(DOK_BULK_GRID) void bulk_scan1a_kernel(BulkWs ws) {
-  __shared__ u32 wsum[16];
-  u32 *row = ws.wg_hist + (size_t)blockIdx.x * ws.g1;
-  const u32 c = row[threadIdx.x];
-  u32 total;
-  row[threadIdx.x] = bulk_block_scan(c, wsum, total);
-  if (threadIdx.x == 0) ws.big_off[blockIdx.x] = total;      // the bin's size; scan1b turns it into a start
-}
-__global__ __launch_bounds__(DOK_BULK_MAXBIG) void bulk_scan1b_kernel(BulkWs ws) {
-  __shared__ u32 wsum[16];
-  const u32 b = threadIdx.x;
-  const u32 c = b < ws.n_big ? ws.big_off[b] : 0u;
-  u32 total;
-  const u32 off = bulk_block_scan(c, wsum, total);
-  if (b < ws.n_big) ws.big_off[b] = off;
-  if (b == 0) ws.big_off[ws.n_big] = total;
-}
-
-// ---- pass 2, count: rows of every stretch of a first-level bin per range -----------------------------
-template <int SL>
-__global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_count2_kernel(DevTable t, BulkWs ws) {
-  constexpr int SUB = 1 << SL;
-  __shared__ u32 cnt[4 * SUB];                       // four copies, as in the first count
-  const u32 b = blockIdx.x / ws.ch, c = blockIdx.x % ws.ch;
-  for (int s = threadIdx.x; s < 4 * SUB; s += DOK_BULK_CTPB) cnt[s] = 0;
-  __syncthreads();
-  const u32 copy = (threadIdx.x & 3) * SUB;
-  i64 lo, hi;
-  bulk_stretch2(ws, b, c, lo, hi);
-  for (i64 i0 = lo + threadIdx.x; i0 < hi; i0 += 8 * DOK_BULK_CTPB) {
-    u64 key[8];
-    #pragma unroll
-    for (int u = 0; u < 8; u++) {
-      const i64 i = i0 + u * DOK_BULK_CTPB;
-      key[u] = i < hi ? ws.keysA[i] : 0;
-    }
-    #pragma unroll
-    for (int u = 0; u < 8; u++)
-      if (i0 + u * DOK_BULK_CTPB < hi) atomicAdd(&cnt[copy + (bulk_range_of(key[u], t) & (SUB - 1))], 1u);
-  }
-  __syncthreads();
-  for (int s = threadIdx.x; s < SUB; s += DOK_BULK_CTPB)
-    ws.sub_hist[((size_t)b * SUB + s) * ws.ch + c] =
-        cnt[s] + cnt[SUB + s] + cnt[2 * SUB + s] + cnt[3 * SUB + s];
-}
-
-// ---- pass 2, scan: per range over the stretches, then over the ranges of the bin ---------------------
-template <int SL>
-__global__ __launch_bounds__(1 << SL) void bulk_scan2_kernel(BulkWs ws) {
-  constexpr int SUB = 1 << SL;
-  __shared__ u32 wsum[16];
-  const u32 b = blockIdx.x;
-  const size_t idx = (size_t)b * SUB + threadIdx.x;
-  u32 *row = ws.sub_hist + idx * ws.ch;
-  u32 run = 0;
-  for (u32 c = 0; c < ws.ch; c++) {
-    const u32 x = row[c];
-    row[c] = run;
-    run += x;
-  }
-  u32 total;
-  const u32 ex = bulk_block_scan(run, wsum, total);
-  const u32 base = ws.big_off[b];
-  ws.part_off[idx] = base + ex;
-  if (b == ws.n_big - 1 && threadIdx.x == SUB - 1) ws.part_off[idx + 1] = base + ex + run;
 }
 
 // ---- scatter: LEVEL 1 moves the caller's rows into first-level bins (keysA/valsA), LEVEL 2 moves
@@ -304,6 +244,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
   constexpr int NB = LEVEL == 1 ? DOK_BULK_MAXBIG : (1 << SL);
   constexpr int BPT = NB >= DOK_BULK_TPB ? NB / DOK_BULK_TPB : 1;   // consecutive bins per thread
   __shared__ u32 cnt[NB], off[NB], gbase[NB];
+  __shared__ u16 room[NB];                  // rows of a bin's run that its region still holds (a tile has < 65535 rows)
   __shared__ u64 skeys[T];
   __shared__ VT svals[T];
   __shared__ u16 sbins[T];                  // bin of every staged row (saves a second hash)
@@ -311,21 +252,18 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
   const int tid = threadIdx.x;
   int n_fresh = 0, n_oob = 0;
 
-  // this workgroup's stretch of the input and its private write cursor of every bin
+  // this workgroup's stretch of the input; the fill counters and the region size of its output bins
   i64 lo0, hi0;
   const void *kin = keys_in, *vin = vals_in;
   u64 *out_keys;
   VT *out_vals;
-  u32 cursor[BPT];
+  u32 *fill;                                // fill[bin]: rows reserved so far in the bin's region
+  u32 first_bin, n_bins, cap;               // (global number of this workgroup's bin 0; bins in use; region size)
   if (LEVEL == 1) {
     bulk_stretch1(ws, n, blockIdx.x, lo0, hi0);
     out_keys = ws.keysA;
     out_vals = (VT *)ws.valsA;
-    #pragma unroll
-    for (int q = 0; q < BPT; q++) {
-      const u32 b = tid * BPT + q;
-      cursor[q] = b < ws.n_big ? ws.big_off[b] + ws.wg_hist[(size_t)b * ws.g1 + blockIdx.x] : 0u;
-    }
+    fill = ws.big_cnt; first_bin = 0; n_bins = ws.n_big; cap = ws.big_cap;
   } else {
     const u32 b = blockIdx.x / ws.ch, c = blockIdx.x % ws.ch;
     bulk_stretch2(ws, b, c, lo0, hi0);
@@ -333,11 +271,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     vin = ws.valsA;
     out_keys = ws.keysB;
     out_vals = (VT *)ws.valsB;
-    #pragma unroll
-    for (int q = 0; q < BPT; q++) {
-      const size_t idx = (size_t)b * NB + tid * BPT + q;
-      cursor[q] = tid * BPT + q < NB ? ws.part_off[idx] + ws.sub_hist[idx * ws.ch + c] : 0u;
-    }
+    first_bin = b * NB; fill = ws.part_cnt + first_bin; n_bins = NB; cap = ws.part_cap;
   }
 
   // The rows of a tile sit in registers from their load to their place in the LDS staging area;
@@ -421,22 +355,22 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
       if (bn[j] >= 0) rk[j] = atomicAdd(&cnt[bn[j]], 1u);
     __syncthreads();
 
-    // bin offsets inside the tile, and where in global memory each bin's run goes
-    u32 c[BPT], csum = 0;
+    // bin offsets inside the tile; the run of every bin is reserved in the bin's region with one
+    // atomic add on its fill counter, whose result is only needed for the write-out below
+    u32 c[BPT], got[BPT], csum = 0;
     #pragma unroll
     for (int q = 0; q < BPT; q++) {
-      c[q] = tid * BPT + q < NB ? cnt[tid * BPT + q] : 0u;
+      const u32 bin = tid * BPT + q;
+      c[q] = bin < NB ? cnt[bin] : 0u;
       csum += c[q];
+      got[q] = 0;
+      if (c[q] != 0 && bin < n_bins) got[q] = atomicAdd(&fill[bin], c[q]);
     }
     u32 total;
     u32 ex = bulk_block_scan(csum, wsum, total);
     #pragma unroll
     for (int q = 0; q < BPT; q++) {
-      if (tid * BPT + q < NB) {
-        off[tid * BPT + q] = ex;
-        gbase[tid * BPT + q] = cursor[q];
-      }
-      cursor[q] += c[q];
+      if (tid * BPT + q < NB) off[tid * BPT + q] = ex;
       ex += c[q];
     }
     __syncthreads();
@@ -451,6 +385,15 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
       }
     }
     if (lo + T < hi0) load_tile(lo + T);
+    #pragma unroll
+    for (int q = 0; q < BPT; q++) {
+      const u32 bin = tid * BPT + q;
+      if (bin < NB) {
+        gbase[bin] = (first_bin + bin) * cap + got[q];       // (fits 32 bits: checked with the plan)
+        const u32 left = got[q] < cap ? cap - got[q] : 0u;
+        room[bin] = (u16)(left < 0xffffu ? left : 0xffffu);
+      }
+    }
     __syncthreads();
 
     #pragma unroll
@@ -458,9 +401,15 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
       const u32 pos = tid + j * DOK_BULK_TPB;
       if (pos < total) {
         const u32 b = sbins[pos];
-        const u32 dst = gbase[b] + (pos - off[b]);
-        out_keys[dst] = skeys[pos];
-        out_vals[dst] = svals[pos];
+        const u32 r = pos - off[b];
+        if (r < room[b]) {
+          out_keys[gbase[b] + r] = skeys[pos];
+          out_vals[gbase[b] + r] = svals[pos];
+        } else {
+          // the bin's region is full: the row goes to the ordinary insert
+          const u32 at = atomicAdd(ws.spill_cnt, 1u);
+          if (at < ws.spill_cap) { ws.spill_keys[at] = skeys[pos]; ((VT *)ws.spill_vals)[at] = svals[pos]; }
+        }
       }
     }
     // the barriers at the top of the next tile order these reads before the next writes
@@ -545,12 +494,12 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
   const u32 per = (ws.n_part + gridDim.x - 1) / gridDim.x;
   const u32 p_lo = blockIdx.x * per < ws.n_part ? blockIdx.x * per : ws.n_part;
   const u32 p_hi = p_lo + per < ws.n_part ? p_lo + per : ws.n_part;
-  const u32 def_base = ws.part_off[p_lo], blk_end = ws.part_off[p_hi];
+  const u32 def_base = p_lo * ws.part_cap, blk_end = p_hi * ws.part_cap;
   if (tid == 0) { n_def = 0; n_carry = 0; n_meta = 0; range_live = 0; n_edge = 0; }
   __syncthreads();
 
   for (u32 p = p_lo; p < p_hi; p++) {
-    const u32 lo = ws.part_off[p], hi = ws.part_off[p + 1];
+    const u32 lo = p * ws.part_cap, hi = lo + bulk_part_n(ws, p);
     const u32 carried = n_carry;                     // rows handed on by the range before (they sit
                                                      // at the head of the list already)
     if (!FRESH && lo == hi && carried == 0) continue;   // nothing to do in this range
@@ -988,7 +937,7 @@ __global__ __launch_bounds__(DOK_BULK_R) void bulk_edge_kernel(DevTable t, BulkW
   const u32 n_rows = ws.edge_cnt[blockIdx.x];
   // (more rows than threads: left to the ordinary insert, which reads the list as it is)
   if (n_rows == 0 || n_rows > (u32)R || p_hi >= ws.n_part) return;
-  const u32 def_base = ws.part_off[p_lo], top = ws.part_off[p_hi];
+  const u32 def_base = p_lo * ws.part_cap, top = p_hi * ws.part_cap;
   const u32 note_base = def_base + ws.meta_cnt[blockIdx.x], a_base = def_base + ws.def_cnt[blockIdx.x];
   bool have = (u32)tid < n_rows;
   u64 key = 0, sk = 0, home = 0, fidx = 0;
@@ -1096,7 +1045,7 @@ template <int V>
 __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kernel(DevTable t, BulkWs ws) {
   const u32 per = (ws.n_part + gridDim.x - 1) / gridDim.x;
   const u32 p_lo = blockIdx.x * per < ws.n_part ? blockIdx.x * per : ws.n_part;
-  const i64 base = ws.part_off[p_lo];
+  const i64 base = (i64)p_lo * ws.part_cap;
   // displacement marks the merge could not set itself (see there)
   const u32 n_marks = ws.meta_cnt[blockIdx.x];
   for (u32 i = threadIdx.x; i < n_marks; i += DOK_TPB) {
@@ -1107,8 +1056,14 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
   // the rows from the bottom of the stretch, and - if bulk_edge_kernel has not taken them - the
   // rows listed from its top downwards
   const u32 p_hi = p_lo + per < ws.n_part ? p_lo + per : ws.n_part;
-  const i64 top = ws.part_off[p_hi];
-  const i64 n_a = ws.def_cnt[blockIdx.x], n = n_a + ws.edge_cnt[blockIdx.x];
+  const i64 top = (i64)p_hi * ws.part_cap;
+  // ... and this workgroup's share of the rows that found their bin's region full
+  const i64 n_sp_all = ws.spill_cnt[0] < ws.spill_cap ? ws.spill_cnt[0] : ws.spill_cap;
+  const i64 sp_per = (n_sp_all + gridDim.x - 1) / gridDim.x;
+  const i64 sp_lo = sp_per * blockIdx.x < n_sp_all ? sp_per * blockIdx.x : n_sp_all;
+  const i64 n_sp = sp_lo + sp_per < n_sp_all ? sp_per : n_sp_all - sp_lo;
+  const i64 n_a = ws.def_cnt[blockIdx.x], n_e = n_a + ws.edge_cnt[blockIdx.x], n = n_e + n_sp;
+  if (blockIdx.x == 0 && threadIdx.x == 0) t.header[DOK_H_NSPILL] = n_sp_all;
   const i64 waves = DOK_TPB / 64, wave = threadIdx.x >> 6;
   const i64 share = (n + waves - 1) / waves;
   i64 lo = wave * share, hi = lo + share;
@@ -1117,6 +1072,11 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
   const u64 *keys = ws.keysA;
   const void *vals = ws.valsA;
   p8_stream_insert_rows<V>(t, lo, hi, nullptr, [&](i64 i, u64 &key, u64 &val) -> int {
+    if (i >= n_e) {
+      key = ws.spill_keys[sp_lo + (i - n_e)];
+      val = dok_load_val<V>(ws.spill_vals, sp_lo + (i - n_e));
+      return 0;
+    }
     const i64 at = i < n_a ? base + i : top - 1 - (i - n_a);
     key = keys[at];
     val = dok_load_val<V>(vals, at);
@@ -1127,9 +1087,20 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
 // ---- host side -----------------------------------------------------------------------------------
 struct BulkPlan {
   u32 n_part, n_big, sublog, ch, g1, gm;
+  u32 big_cap, part_cap, spill_cap;
   i64 share;
-  size_t o_keysA, o_keysB, o_valsA, o_valsB, o_wg_hist, o_big_off, o_sub_hist, o_part_off, o_def_cnt, o_meta_cnt, o_edge_cnt, bytes;
+  size_t o_keysA, o_keysB, o_valsA, o_valsB, o_big_cnt, o_part_cnt, o_spill_keys, o_spill_vals, o_spill_cnt,
+         o_def_cnt, o_meta_cnt, o_edge_cnt, bytes;
 };
+
+// Rows the region of a bin holds that receives `mean` rows on average (the hash spreads the rows
+// uniformly over the buckets, so a bin's share is binomial): the mean plus `sigmas` standard
+// deviations and a little, a multiple of `unit`, and never more than all the rows.
+static inline u64 bulk_region_rows(double mean, double sigmas, u64 unit, u64 all_rows) {
+  u64 cap = (u64)(mean + sigmas * __builtin_sqrt(mean) + 2.0 * (double)unit) + 1;
+  if (cap > all_rows) cap = all_rows;
+  return (cap + unit - 1) / unit * unit;
+}
 
 static inline size_t bulk_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -1157,15 +1128,31 @@ static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p, u32 g1 = DOK_BULK_G
   p.share = ((tiles + g1 - 1) / g1) * DOK_BULK_T;
   p.gm = p.n_part < gm ? p.n_part : gm;
   const size_t parts = (size_t)n_big << p.sublog;
+  // Regions: a first-level bin covers (256 << sublog) of the nb buckets, a range 256 of them.  Six
+  // resp. five standard deviations of slack: a region that still overflows (one range in a million
+  // at five) spills a few rows to the ordinary insert.
+  const double buckets = (double)d.nb;
+  const double f_big = (double)((u64)DOK_BULK_R << p.sublog) / buckets, f_part = (double)DOK_BULK_R / buckets;
+  const u64 big_cap = bulk_region_rows((double)n_cap * (f_big < 1.0 ? f_big : 1.0), 6.0, 64, (u64)n_cap);
+  const u64 part_cap = bulk_region_rows((double)n_cap * (f_part < 1.0 ? f_part : 1.0), 5.0, 16, (u64)n_cap);
+  const u64 rowsA_1 = (u64)n_big * big_cap, rowsB = (u64)parts * part_cap;
+  if (rowsA_1 >= 0xffff0000ULL || rowsB >= 0xffff0000ULL) return false;      // positions are 32 bits
+  // keysA also serves the merge as scratch, addressed like keysB; keysB first holds the linearised
+  // keys of a coordinate source (n rows)
+  const u64 rowsA = rowsA_1 > rowsB ? rowsA_1 : rowsB;
+  const u64 rowsB2 = (d.lin_ndim >= 3 && rowsB < (u64)n) ? (u64)n : rowsB;
+  p.big_cap = (u32)big_cap; p.part_cap = (u32)part_cap;
+  p.spill_cap = (u32)n_cap;                                                   // (every row may spill: n_cap < 2^31)
   size_t o = 0;
-  p.o_keysA = o; o = bulk_align(o + 8 * (size_t)n_cap);
-  p.o_keysB = o; o = bulk_align(o + 8 * (size_t)n_cap);
-  p.o_valsA = o; o = bulk_align(o + (size_t)d.value_bytes * (size_t)n_cap);
-  p.o_valsB = o; o = bulk_align(o + (size_t)d.value_bytes * (size_t)n_cap);
-  p.o_wg_hist = o; o = bulk_align(o + 4 * (size_t)n_big * DOK_BULK_GRID);
-  p.o_big_off = o; o = bulk_align(o + 4 * (DOK_BULK_MAXBIG + 1));
-  p.o_sub_hist = o; o = bulk_align(o + 4 * parts * ch);
-  p.o_part_off = o; o = bulk_align(o + 4 * (parts + 1));
+  p.o_keysA = o; o = bulk_align(o + 8 * (size_t)rowsA);
+  p.o_keysB = o; o = bulk_align(o + 8 * (size_t)rowsB2);
+  p.o_valsA = o; o = bulk_align(o + (size_t)d.value_bytes * (size_t)rowsA);
+  p.o_valsB = o; o = bulk_align(o + (size_t)d.value_bytes * (size_t)rowsB);
+  p.o_spill_keys = o; o = bulk_align(o + 8 * (size_t)p.spill_cap);
+  p.o_spill_vals = o; o = bulk_align(o + (size_t)d.value_bytes * (size_t)p.spill_cap);
+  p.o_big_cnt = o; o = bulk_align(o + 4 * (size_t)DOK_BULK_MAXBIG);
+  p.o_part_cnt = o; o = bulk_align(o + 4 * parts);
+  p.o_spill_cnt = o; o = bulk_align(o + 4);
   p.o_def_cnt = o; o = bulk_align(o + 4 * DOK_BULK_GRID);
   p.o_meta_cnt = o; o = bulk_align(o + 4 * DOK_BULK_GRID);
   p.o_edge_cnt = o; o = bulk_align(o + 4 * DOK_BULK_GRID);
@@ -1179,10 +1166,14 @@ static void bulk_bind(const BulkPlan &p, void *workspace, BulkWs &ws) {
   ws.keysB = (u64 *)(w + p.o_keysB);
   ws.valsA = w + p.o_valsA;
   ws.valsB = w + p.o_valsB;
-  ws.wg_hist = (u32 *)(w + p.o_wg_hist);
-  ws.big_off = (u32 *)(w + p.o_big_off);
-  ws.sub_hist = (u32 *)(w + p.o_sub_hist);
-  ws.part_off = (u32 *)(w + p.o_part_off);
+  ws.big_cnt = (u32 *)(w + p.o_big_cnt);
+  ws.part_cnt = (u32 *)(w + p.o_part_cnt);
+  ws.spill_keys = (u64 *)(w + p.o_spill_keys);
+  ws.spill_vals = w + p.o_spill_vals;
+  ws.spill_cnt = (u32 *)(w + p.o_spill_cnt);
+  ws.big_cap = p.big_cap;
+  ws.part_cap = p.part_cap;
+  ws.spill_cap = p.spill_cap;
   ws.def_cnt = (u32 *)(w + p.o_def_cnt);
   ws.meta_cnt = (u32 *)(w + p.o_meta_cnt);
   ws.edge_cnt = (u32 *)(w + p.o_edge_cnt);
@@ -1243,26 +1234,21 @@ static void bulk_launch_nd(const DevTable &d, const void *keys, const void *valu
                            void *workspace, hipStream_t s) {
   BulkWs ws;
   bulk_bind(p, workspace, ws);
-  if (FRESH) dok_fill_kernel<<<1, DOK_TPB, 0, s>>>(d.buckets, 0, d.header);
-  // coordinate rows of three and more dimensions are linearised once, by the count
-  constexpr bool EMIT = ND >= 3;
-  bulk_count1_kernel<KF, EMIT, ND><<<p.g1, DOK_BULK_CTPB, 0, s>>>(d, keys, n, ws);
-  bulk_scan1a_kernel<<<p.n_big, p.g1, 0, s>>>(ws);
-  bulk_scan1b_kernel<<<1, DOK_BULK_MAXBIG, 0, s>>>(ws);
-  if constexpr (EMIT)
+  bulk_init_kernel<<<64, DOK_TPB, 0, s>>>(ws, FRESH ? d.header : nullptr);
+  // coordinate rows of three and more dimensions are linearised first (see bulk_linearise_kernel)
+  constexpr bool LIN = ND >= 3;
+  if constexpr (LIN) {
+    bulk_linearise_kernel<KF, ND><<<p.g1, DOK_BULK_CTPB, 0, s>>>(d, keys, n, ws);
     bulk_scatter_kernel<V, DOK_KF_LIN, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, ws.keysB, values, n, ws);
-  else
+  } else {
     bulk_scatter_kernel<V, KF, 1, DOK_BULK_SUBLOG, ND><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, keys, values, n, ws);
+  }
   // narrow values: small second-pass tiles when the workgroups' stretches are short
   const bool smallt = V <= 2 && n / ((i64)p.n_big * p.ch) < DOK_BULK_T2S_BELOW;
   if (p.sublog == DOK_BULK_SUBLOG) {
-    bulk_count2_kernel<DOK_BULK_SUBLOG><<<p.n_big * p.ch, DOK_BULK_CTPB, 0, s>>>(d, ws);
-    bulk_scan2_kernel<DOK_BULK_SUBLOG><<<p.n_big, 1 << DOK_BULK_SUBLOG, 0, s>>>(ws);
     if (smallt) bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG, 0, V <= 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
     else bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
   } else {
-    bulk_count2_kernel<DOK_BULK_SUBLOG_WIDE><<<p.n_big * p.ch, DOK_BULK_CTPB, 0, s>>>(d, ws);
-    bulk_scan2_kernel<DOK_BULK_SUBLOG_WIDE><<<p.n_big, 1 << DOK_BULK_SUBLOG_WIDE, 0, s>>>(ws);
     bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG_WIDE><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
   }
   bulk_merge_kernel<V, FRESH><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);

@@ -41,6 +41,8 @@ extern "C" {
 #define DOK_H_NPROBE      2   /* buckets visited, accumulated by the *_stats entry points         */
 #define DOK_H_NOOB        3   /* rows whose coordinates fell outside lin_dims (skipped)           */
 #define DOK_H_NOPS        4   /* rows processed by the *_stats entry points                       */
+#define DOK_H_NSPILL      5   /* rows the last bulk insert handed to the per-row insert because
+                                 their range's region of the partition was full (statistics)       */
 /* words 8..11: side slots for the two 8-byte key patterns the packed layout reserves            */
 
 /* Physical layouts (chosen from the key/value widths by dok_layout_of). */

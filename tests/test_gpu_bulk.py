@@ -534,6 +534,13 @@ def test_build_with_many_equal_keys(cuda, bulk_always, distinct):
     assert bool((keys[v[:, 0].long()] == keys).all())      # the value is the index of a row with this key
     ks, _ = hm.items()
     assert torch.equal(torch.sort(ks[:, 0]).values, torch.unique(keys))
+    # the same rows again, now as an upsert into the populated table (every row of a key beyond
+    # what its range's region of the partition holds takes the spill list)
+    hm.set(keys[:, None], (vals + n)[:, None])
+    assert hm.n_elements == int(torch.unique(keys).numel())
+    v, f = hm.get(keys[:, None])
+    assert bool(f.all()) and bool((v[:, 0] >= n).all())
+    assert bool((keys[(v[:, 0] - n).long()] == keys).all())
 
 
 @pytest.mark.parametrize("size", [(900_000,), (5000, 3000), (300, 77, 50), (40, 30, 20, 16), (12, 9, 8, 7, 11),

@@ -262,8 +262,9 @@ def test_bulk_path_decision():
     S = 10                                        # slots per bucket of int64 -> float32
     # the headline build: 64M rows into 2^27 slots
     assert bulk_pays(64 * M, 128 * M // S, S, 0)
-    # small batches never
-    assert not bulk_pays(4 * M, 4 * M // S, S, 0)
+    # small batches never; from a million rows on with at least 2 rows per bucket
+    assert not bulk_pays(M // 2, M // 2 // S, S, 0)
+    assert bulk_pays(4 * M, 4 * M // S, S, 0) and bulk_pays(M, M // 2, S, 0) and not bulk_pays(M, M, S, 0)
     # a large batch that is thin against the table (1.25 rows per bucket, table stays empty)
     assert not bulk_pays(16 * M, int(16 * M / 1.25), S, 0)
     # the same density pays once the table ends up more than 70 % full ...
