@@ -408,7 +408,9 @@ def test_completely_full_tables_exercise_far_displacements(cuda, vdtype):
     # (buckets, rows per set call).  One call for all rows: the waves race, and where the last keys
     # end up differs from run to run.  One row per call: a fixed order, the same table every
     # time - that case must show a far displacement.
-    for n_phys, step in ((40, None), (64, None), (200, None), (120, 1)):
+    # (700 buckets: displacements beyond the 254 the metadata records, where the walk runs to the
+    # ring's end)
+    for n_phys, step in ((40, None), (64, None), (200, None), (700, None), (120, 1)):
         cap = n_phys * slots                                   # every physical slot
         keys = np.unique(rng.integers(0, 2**62, size=cap + 64, dtype=np.int64))[:cap, None]
         vals = rng.integers(-100, 100, size=(cap, 1)).astype(vdtype)
@@ -595,3 +597,70 @@ def _isin_rows(a, b):
     va = np.ascontiguousarray(a).view([("", a.dtype)] * a.shape[1]).ravel()
     vb = np.ascontiguousarray(b).view([("", b.dtype)] * b.shape[1]).ravel()
     return np.isin(va, vb)
+
+
+@pytest.mark.parametrize("kshape,kdt,vshape,vdt", [
+    ((3,), np.float32, (5,), np.int64),        # 2 slots of 8 words per bucket
+    ((2,), np.int64, (1,), np.float32),        # 4 slots of 4 words
+    ((13,), np.int64, (1,), np.float16),       # 1 slot of 15 words (no filter word)
+])
+def test_full_multiword_tables_take_the_far_walk(cuda, kshape, kdt, vshape, vdt):
+    """Multi-word tables filled to the last physical slot: the last keys land dozens to hundreds of
+    buckets past their home - beyond the 23 displacements with a bit of their own, and (in the
+    larger tables) beyond the 254 the metadata can record, where a lookup walks on to the ring's
+    end.  Then tombstone churn at 100 % load.  Everything against the oracle."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(41)
+    probe = CudaClosedHashmap(n_buckets=1, device=cuda)
+    probe.set(torch.zeros((1, *kshape), dtype=torch.from_numpy(np.zeros(1, kdt)).dtype, device=cuda),
+              torch.zeros((1, *vshape), dtype=torch.from_numpy(np.zeros(1, vdt)).dtype, device=cuda))
+    slots = probe._slots_per_bucket
+    for n_phys, step in ((40, None), (200, None), (700, None), (90, 1)):
+        cap = n_phys * slots
+        if kdt == np.float32:
+            keys = rng.random((cap + 64, *kshape), dtype=np.float32)
+        else:
+            keys = rng.integers(-2**40, 2**40, size=(cap + 64, *kshape)).astype(kdt)
+        keys = np.unique(keys, axis=0)
+        rng.shuffle(keys)
+        keys = keys[:cap]
+        assert keys.shape[0] == cap
+        vals = rng.integers(-100, 100, size=(cap, *vshape)).astype(vdt)
+        hm = CudaClosedHashmap(n_buckets=cap, device=cuda, rehash_threshold=1.0, seed=77)
+        ref = RefClosedHashmap(n_buckets=cap, rehash_threshold=1.0, rng=np.random.default_rng(1))
+        k, v = _to(cuda, keys, vals)
+        for lo in range(0, cap, step or cap):
+            hm.set(k[lo: lo + (step or cap)], v[lo: lo + (step or cap)])
+        ref.set(keys, vals)
+        assert hm.n_elements == ref.n_elements == cap and hm._n_phys == n_phys
+        words = hm._table.view(torch.int64).reshape(n_phys, 16).cpu().numpy()
+        meta = (words[:, 0] >> 32) & 0xffffffff
+        if step:
+            assert (meta & 1).any(), "no far displacement was produced; the test lost its point"
+        if kdt == np.float32:
+            absent = rng.random((cap, *kshape), dtype=np.float32) + 1.0
+        else:
+            absent = rng.integers(2**41, 2**42, size=(cap, *kshape)).astype(kdt)
+        q = np.concatenate([keys, absent])
+        _check_get(hm, ref, q, cuda, fallback=-3)
+        assert hm.probe_stats(torch.from_numpy(q).to(cuda)) >= 1.0
+        for _ in range(3):                                      # churn at full load
+            gone = keys[rng.permutation(cap)[: cap // 3]]
+            m = hm.remove(torch.from_numpy(gone).to(cuda))
+            assert np.array_equal(m.cpu().numpy(), ref.remove(gone))
+            if kdt == np.float32:
+                fresh = rng.random((gone.shape[0], *kshape), dtype=np.float32) + 2.0 + _
+            else:
+                fresh = np.unique(rng.integers(2**43 + _ * 2**41, 2**43 + (_ + 1) * 2**41, size=(cap, *kshape)).astype(kdt),
+                                  axis=0)[: gone.shape[0]]
+            fresh = np.unique(fresh, axis=0)
+            assert fresh.shape[0] == gone.shape[0]
+            fv = rng.integers(-100, 100, size=(fresh.shape[0], *vshape)).astype(vdt)
+            a, b = _to(cuda, fresh, fv)
+            hm.set(a, b)
+            ref.set(fresh, fv)
+            keys = np.concatenate([keys[~_isin_rows(keys, gone)], fresh])
+            assert hm.n_elements == ref.n_elements == cap
+            _check_get(hm, ref, q, cuda)
+            _check_get(hm, ref, keys, cuda)
+        _assert_same_map(hm, ref)
