@@ -30,15 +30,15 @@ HBM_PEAK_GBS = 8000.0
 # hold the runs.  The figures belong to one state of the kernel sources, named by `csrc_sha16`
 # (see csrc_sha16()): when the sources have changed since, nothing measured is reported.
 PROFILED = {
-    "csrc_sha16": "8bbba435b5185ec5",
+    "csrc_sha16": "8f9152004384ec4f",
     "get_lf05": 6.658e9,         # p8_get_kernel, load factor 0.5
-    "get_lf09": 6.946e9,         # p8_get_kernel, load factor 0.9
-    "set_bulk_lf05": 8.868e9,    # the bulk upsert's kernels together, into a cleared table
-    "build_lf05": 7.143e9,       # the bulk build's kernels together, into uninitialised memory
-    "set_bulk_lf09": 7.388e9,
-    "build_lf09": 6.429e9,
+    "get_lf09": 7.190e9,         # p8_get_kernel, load factor 0.9 (mean over four builds)
+    "set_bulk_lf05": 7.611e9,    # the bulk upsert's kernels together, into a cleared table
+    "build_lf05": 5.890e9,       # the bulk build's kernels together, into uninitialised memory
+    "set_bulk_lf09": 6.080e9,
+    "build_lf09": 5.125e9,
     "set_cas_lf05": 1.615e10,    # p8_set_kernel (one compare-and-swap per row)
-    "remove_lf05": 5.669e9,      # p8_remove_kernel, half of the keys, plain-store tombstones
+    "remove_lf05": 5.688e9,      # p8_remove_kernel, half of the keys, plain-store tombstones
 }
 # algorithmic bytes per op for 8-byte keys and 4-byte values: one 128-byte bucket line per op,
 # plus the batch row and the outputs
