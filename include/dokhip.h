@@ -130,12 +130,16 @@ int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int6
 
 /* Bulk upsert: the same result as dok_map_set (stored == NULL) for a batch that is large
  * against the table - rule of thumb: more than one row per physical bucket.  Instead of one
- * compare-and-swap in HBM per row, the batch is partitioned by table range (two counting
- * scatter passes through `workspace`) and every range of buckets is merged in LDS, so the
- * table is streamed through the GPU once.  Packed layout only.
+ * compare-and-swap in HBM per row, the batch is partitioned by table range (two scatter passes
+ * through `workspace`, each bin of a pass owning a region of fixed capacity there) and every
+ * range of buckets is merged in LDS, so the table is streamed through the GPU once.  Rows whose
+ * bin's region is full (batches with very many equal keys) take the per-row insert at the end;
+ * header[DOK_H_NSPILL] says how many.  Packed layout only.
  *   dok_bulk_workspace_bytes: device bytes dok_map_set_bulk / dok_coo_set_bulk need for n rows;
  *     0 if the bulk path cannot take this table or n (tagged layout, n >= 2^31, more than
  *     2^28 buckets: use dok_map_set), negative on a bad table.
+ *     (about 3.4 times the bytes of the batch: two partition buffers with slack and the spill
+ *     list, plus 4 bytes per 256 buckets of the table).
  *   workspace: device, 256-byte aligned, at least that many bytes; contents need no
  *     initialisation and are garbage afterwards.  Calls sharing one workspace must be ordered.
  * Reference: the same closed_hashmap_set launch as dok_map_set, at the batch sizes of
