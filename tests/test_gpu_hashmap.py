@@ -664,3 +664,57 @@ def test_full_multiword_tables_take_the_far_walk(cuda, kshape, kdt, vshape, vdt)
             _check_get(hm, ref, q, cuda)
             _check_get(hm, ref, keys, cuda)
         _assert_same_map(hm, ref)
+
+
+def test_multiword_layout_random_geometries_against_a_dict(cuda):
+    """Differential test of the multi-word layout against a Python dict: random key / value widths
+    (one to five slots per bucket), loads up to 99 % or growth from 64 slots, batches with equal
+    keys, removals with repeats, several rounds.  After every round the whole key pool is looked
+    up and compared."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(2024)
+    geoms = [((3,), np.float32, (5,), np.int64), ((2,), np.int64, (1,), np.float32), ((13,), np.int64, (1,), np.float16),
+             ((3,), np.int32, (1,), np.int8), ((4,), np.int64, (2,), np.int64), ((1,), np.int64, (3,), np.float32),
+             ((5,), np.int16, (3,), np.int16)]
+    for case in range(14):
+        ks, kdt, vs, vdt = geoms[case % len(geoms)]
+        universe = int(10 ** rng.uniform(2, 4.3))
+        grow = case % 3 == 2
+        cap = 64 if grow else int(universe / float(rng.uniform(0.3, 0.99))) + 4
+        lim = 2**14 if kdt == np.int16 else 2**30
+        pool = np.unique(rng.integers(-lim, lim, size=(universe, *ks)).astype(kdt), axis=0)
+        universe = pool.shape[0]
+        hm = CudaClosedHashmap(n_buckets=cap, device=cuda, rehash_threshold=0.75 if grow else 1e9,
+                               seed=int(rng.integers(1, 1 << 40)))
+        model = {}
+        for rnd in range(int(rng.integers(2, 5))):
+            n = int(universe * rng.uniform(0.1, 0.9)) + 1
+            idx = rng.integers(0, universe, size=n)
+            v = rng.integers(-100, 100, size=(n, *vs)).astype(vdt)
+            hm.set(*_to(cuda, pool[idx], v))
+            rows_of = {}
+            for i, key in enumerate(idx.tolist()):
+                rows_of.setdefault(key, []).append(i)
+            uk = np.array(sorted(rows_of))
+            got, f = hm.get(torch.from_numpy(pool[uk]).to(cuda))
+            got = got.cpu().numpy()
+            assert bool(f.all())
+            for j, key in enumerate(uk.tolist()):       # each key holds the value of ONE of its rows, untorn
+                assert any(np.array_equal(v[r].view(np.uint8), got[j].view(np.uint8)) for r in rows_of[key]), (case, rnd, key)
+                model[key] = got[j].copy()
+            assert hm.n_elements == len(model)
+            gidx = rng.integers(0, universe, size=int(universe * rng.uniform(0.05, 0.6)) + 1)
+            mask = hm._remove_rows(torch.from_numpy(pool[gidx]).to(cuda).contiguous()).cpu().numpy()
+            gone = set(gidx.tolist())
+            assert int(mask.sum()) == len(gone & set(model))       # repeated keys are removed once
+            for key in gone:
+                model.pop(key, None)
+            assert hm.n_elements == len(model)
+            allv, allf = hm.get(torch.from_numpy(pool).to(cuda))
+            allv, allf = allv.cpu().numpy(), allf.cpu().numpy()
+            present = np.zeros(universe, dtype=bool)
+            present[list(model)] = True
+            assert np.array_equal(allf, present), (case, rnd)
+            for key, val in model.items():
+                assert np.array_equal(allv[key].view(np.uint8), val.view(np.uint8)), (case, rnd, key)
+        assert hm.items()[0].shape[0] == len(model)
