@@ -845,4 +845,10 @@ class CudaClosedHashmap:
         return self.set(keys, values)
 
     def __delitem__(self, keys):
-        return self.remove(keys)
+        # `del hm[keys]` discards the mask, so the sort that only orders the mask is skipped
+        if not self._allocated:
+            raise RuntimeError("store something first")
+        if keys.shape[0] == 0:
+            return
+        self._check_keys(keys)
+        self._remove_rows(self._prep_rows(keys, "keys"))

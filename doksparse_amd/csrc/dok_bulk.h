@@ -38,9 +38,19 @@
 #define DOK_BULK_SUBLOG 8                   // log2 of the ranges per first-level bin ...
 #define DOK_BULK_SUBLOG_WIDE 10             // ... and for tables of more than 1024 << 8 ranges
 #define DOK_BULK_MAXBIG 1024                // first-level bins at most
-#ifndef DOK_BULK_TPB
-#define DOK_BULK_TPB 512
+// Threads per scatter workgroup.  One workgroup per CU with the large tiles either way (a tile
+// fills the LDS); 16 waves instead of 8 make the second pass, whose workgroups take one or two
+// tiles each, 12 % faster and the first pass over plain keys 3 %; the first pass over coordinate
+// rows or over a table's buckets (more registers per row, more loads per row) loses with them.
+#ifndef DOK_BULK_TPB_FEW
+#define DOK_BULK_TPB_FEW 512
 #endif
+#ifndef DOK_BULK_TPB_MANY
+#define DOK_BULK_TPB_MANY 1024
+#endif
+constexpr int bulk_tpb(int level, int key_format, int coord_dims) {
+  return level == 1 && (coord_dims > 0 || key_format == DOK_KF_TABLE) ? DOK_BULK_TPB_FEW : DOK_BULK_TPB_MANY;
+}
 // Rows per scatter tile.  A tile is staged in LDS whole (8 + V + 2 bytes per row), and the larger
 // it is, the longer the runs of rows that leave for one bin: for 8-byte keys with 4-byte values
 // one workgroup per CU with a tile that nearly fills the LDS beats two with half the tile
@@ -234,15 +244,16 @@ __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_linearise_kernel(DevTable 
 // ---- scatter: LEVEL 1 moves the caller's rows into first-level bins (keysA/valsA), LEVEL 2 moves
 // the rows of each first-level bin into their ranges (keysB/valsB) ---------------------------------
 template <int V, int KF, int LEVEL, int SL = DOK_BULK_SUBLOG, int ND = 0, bool SMALLT = false>
-__global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, const void *__restrict__ keys_in,
+__global__ __launch_bounds__(bulk_tpb(LEVEL, KF, ND)) void bulk_scatter_kernel(DevTable t, const void *__restrict__ keys_in,
                                                                     const void *__restrict__ vals_in, i64 n, BulkWs ws) {
   typedef typename ValT<V>::type VT;
   constexpr int T = LEVEL == 1 ? (V == 8 ? DOK_BULK_T1V8 : DOK_BULK_T)
                                : (V == 8 ? DOK_BULK_T2V8 : SMALLT ? DOK_BULK_T2S : DOK_BULK_T2);
-  static_assert(T % DOK_BULK_TPB == 0, "every thread stages the same number of rows");
-  constexpr int RPT = T / DOK_BULK_TPB;
+  constexpr int TPB = bulk_tpb(LEVEL, KF, ND);
+  static_assert(T % TPB == 0, "every thread stages the same number of rows");
+  constexpr int RPT = T / TPB;
   constexpr int NB = LEVEL == 1 ? DOK_BULK_MAXBIG : (1 << SL);
-  constexpr int BPT = NB >= DOK_BULK_TPB ? NB / DOK_BULK_TPB : 1;   // consecutive bins per thread
+  constexpr int BPT = NB >= TPB ? NB / TPB : 1;   // consecutive bins per thread
   __shared__ u32 cnt[NB], off[NB], gbase[NB];
   __shared__ u16 room[NB];                  // rows of a bin's run that its region still holds (a tile has < 65535 rows)
   __shared__ u64 skeys[T];
@@ -289,7 +300,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     const i64 hi = lo + T < hi0 ? lo + T : hi0;
     #pragma unroll
     for (int j = 0; j < RPT; j++) {
-      const i64 i = lo + j * DOK_BULK_TPB + tid;
+      const i64 i = lo + j * TPB + tid;
       k[j] = 0; v[j] = 0;
       if (COORDS) raw[COORDS ? j : 0] = BulkRaw<KF, ND>{};
       if (i < hi) {
@@ -314,7 +325,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
     #pragma unroll
     for (int j = 0; j < RPT; j++) {
       st[j] = 0;
-      if (lo + j * DOK_BULK_TPB + tid < hi) {
+      if (lo + j * TPB + tid < hi) {
         if constexpr (COORDS) {
           st[j] = bulk_finish<KF, ND>(t, raw[j], k[j]);
         } else {
@@ -398,7 +409,7 @@ __global__ __launch_bounds__(DOK_BULK_TPB) void bulk_scatter_kernel(DevTable t, 
 
     #pragma unroll
     for (int j = 0; j < RPT; j++) {
-      const u32 pos = tid + j * DOK_BULK_TPB;
+      const u32 pos = tid + j * TPB;
       if (pos < total) {
         const u32 b = sbins[pos];
         const u32 r = pos - off[b];
@@ -1212,7 +1223,7 @@ static bool bulk_plan_for(const DevTable &d, i64 n, BulkPlan &p, i64 n_cap = -1)
   static u32 g1 = 0, gm = 0;
   if (g1 == 0) {
     constexpr int ND = (KF == DOK_KF_COLS || KF == DOK_KF_ROWS) ? 2 : 0;   // (the dimensions do not change the LDS use)
-    g1 = bulk_resident(bulk_scatter_kernel<V, KF, 1, DOK_BULK_SUBLOG, ND>, DOK_BULK_TPB, DOK_BULK_GRID, 64);
+    g1 = bulk_resident(bulk_scatter_kernel<V, KF, 1, DOK_BULK_SUBLOG, ND>, bulk_tpb(1, KF, ND), DOK_BULK_GRID, 64);
     gm = bulk_resident(bulk_merge_kernel<V, false>, DOK_BULK_R, DOK_BULK_GRID, 1);
   }
   return bulk_plan(d, n, p, g1, gm, n_cap);
@@ -1239,17 +1250,17 @@ static void bulk_launch_nd(const DevTable &d, const void *keys, const void *valu
   constexpr bool LIN = ND >= 3;
   if constexpr (LIN) {
     bulk_linearise_kernel<KF, ND><<<p.g1, DOK_BULK_CTPB, 0, s>>>(d, keys, n, ws);
-    bulk_scatter_kernel<V, DOK_KF_LIN, 1><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, ws.keysB, values, n, ws);
+    bulk_scatter_kernel<V, DOK_KF_LIN, 1><<<p.g1, bulk_tpb(1, DOK_KF_LIN, 0), 0, s>>>(d, ws.keysB, values, n, ws);
   } else {
-    bulk_scatter_kernel<V, KF, 1, DOK_BULK_SUBLOG, ND><<<p.g1, DOK_BULK_TPB, 0, s>>>(d, keys, values, n, ws);
+    bulk_scatter_kernel<V, KF, 1, DOK_BULK_SUBLOG, ND><<<p.g1, bulk_tpb(1, KF, ND), 0, s>>>(d, keys, values, n, ws);
   }
   // narrow values: small second-pass tiles when the workgroups' stretches are short
   const bool smallt = V <= 2 && n / ((i64)p.n_big * p.ch) < DOK_BULK_T2S_BELOW;
   if (p.sublog == DOK_BULK_SUBLOG) {
-    if (smallt) bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG, 0, V <= 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
-    else bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
+    if (smallt) bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG, 0, V <= 2><<<p.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
+    else bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
   } else {
-    bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG_WIDE><<<p.n_big * p.ch, DOK_BULK_TPB, 0, s>>>(d, nullptr, nullptr, n, ws);
+    bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG_WIDE><<<p.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
   }
   bulk_merge_kernel<V, FRESH><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
   if (p.gm > 1) bulk_edge_kernel<V><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);

@@ -299,6 +299,14 @@ def test_api_edges(cuda):
     assert bool(hm.get(kk)[1].all())
     assert hm.count_existing(torch.arange(0, 25, device=cuda)[:, None]).item() == sum(
         1 for x in range(25) if x in {1, 2} | set(range(0, 20, 2)))
+    # del hm[keys]: rows may repeat and may be absent
+    before = hm.n_elements
+    del hm[torch.tensor([[2], [2], [18], [99]], device=cuda)]
+    assert hm.n_elements == before - 2
+    assert hm.get(torch.tensor([[2], [18], [1]], device=cuda))[1].tolist() == [False, False, True]
+    del hm[torch.zeros(0, 1, dtype=torch.long, device=cuda)]
+    with pytest.raises(AssertionError):
+        del hm[torch.zeros(2, 2, dtype=torch.long, device=cuda)]
 
 
 def test_probe_stats_are_in_the_expected_band(cuda):
