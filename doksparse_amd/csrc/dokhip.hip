@@ -47,6 +47,36 @@ int static_scratch_of_current_device(void **out) {
   return DOK_OK;
 }
 
+// Makes the device of the caller's stream current for the duration of a call (kernels launch on
+// the current device; a process that drives several GPUs may call with another one current).
+// The null stream belongs to whatever device is current, so there is nothing to switch then.
+// A process that sees one GPU (the usual one-process-per-GPU set-up) skips the query, which costs
+// 2 to 3 microseconds per call.
+int visible_devices() {
+  static std::atomic<int> count{0};
+  int c = count.load(std::memory_order_relaxed);
+  if (c == 0) {
+    if (hipGetDeviceCount(&c) != hipSuccess || c < 1) c = 1;
+    count.store(c, std::memory_order_relaxed);
+  }
+  return c;
+}
+struct DeviceScope {
+  int prev = -1;
+  bool switched = false;
+  explicit DeviceScope(hipStream_t s) {
+    hipDevice_t dev = -1;
+    if (s != nullptr && visible_devices() > 1 && hipStreamGetDevice(s, &dev) == hipSuccess &&
+        hipGetDevice(&prev) == hipSuccess && prev != (int)dev)
+      switched = hipSetDevice((int)dev) == hipSuccess;
+  }
+  ~DeviceScope() {
+    if (switched) (void)hipSetDevice(prev);
+  }
+  DeviceScope(const DeviceScope &) = delete;
+  DeviceScope &operator=(const DeviceScope &) = delete;
+};
+
 int note_launch() {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
@@ -224,6 +254,7 @@ int dok_table_clear(const dok_table_t *t, void *stream) {
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   // a fill kernel rather than a memset node, so that the call can be captured into a graph
   const i64 words = (i64)d.nb * 16;
   dok_fill_kernel<<<(unsigned)((words / 4 + DOK_TPB - 1) / DOK_TPB), DOK_TPB, 0, s>>>(d.buckets, words, d.header);
@@ -239,6 +270,7 @@ int dok_map_get(const dok_table_t *t, const void *keys, int64_t n, void *values_
   if (n == 0) return DOK_OK;
   if (!keys || !values_out || !found) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   if (layout == DOK_LAYOUT_PACKED8) {
     const u64 fb = fallback_word(fallback, d.value_bytes);
     P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, false, KF><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
@@ -258,6 +290,7 @@ int dok_map_get_stats(const dok_table_t *t, const void *keys, int64_t n, void *v
   if (n == 0) return DOK_OK;
   if (!keys || !values_out || !found) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   if (layout == DOK_LAYOUT_PACKED8) {
     const u64 fb = fallback_word(fallback, d.value_bytes);
     P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, true, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
@@ -277,6 +310,7 @@ int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int6
   if (n == 0) return DOK_OK;
   if (!keys || !values) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   if (layout == DOK_LAYOUT_PACKED8) {
     const unsigned grid = grid_counting(n);
     P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_set_kernel<V, KF><<<grid, DOK_TPB, 0, s>>>(d, keys, values, n, stored, rows_per_wave(n, grid))));
@@ -296,6 +330,7 @@ int dok_coo_set(const dok_table_t *t, const int64_t *indices, const void *values
   if (n == 0) return DOK_OK;
   if (!indices || !values) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   { constexpr int KF = DOK_KF_COLS;
     const unsigned grid = grid_counting(n);
     P8_DISPATCH(d.value_bytes, (p8_set_kernel<V, KF><<<grid, DOK_TPB, 0, s>>>(d, indices, values, n, nullptr, rows_per_wave(n, grid)))); }
@@ -326,6 +361,7 @@ static int set_bulk(const dok_table_t *t, const void *keys, const void *values, 
   if (layout != DOK_LAYOUT_PACKED8 || !bulk_plan(d, n, p)) return DOK_EUNSUPPORTED;
   if (((uintptr_t)workspace & 255) != 0 || workspace_bytes < (int64_t)p.bytes) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   // the launch plan shares the workspace layout of the sizing plan above and only narrows the grids
 #define BULK_GO (bulk_plan_for<V, KF>(d, n, p),                                                    \
                  fresh ? bulk_launch<V, KF, true>(d, keys, values, n, p, workspace, s)             \
@@ -373,6 +409,7 @@ static int map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t
   if (n == 0) return DOK_OK;
   if (!keys) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   if (layout == DOK_LAYOUT_PACKED8) {
     if (unique) {
       P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_remove_kernel<V, KF, true><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
@@ -402,6 +439,7 @@ int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n, in
   if (n == 0) return DOK_OK;
   if (!keys || !count) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   if (layout == DOK_LAYOUT_PACKED8) {
     P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_count_kernel<V, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, (i64 *)count)));
   } else {
@@ -425,6 +463,7 @@ int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out, int6
   if (!count_out || !scratch || capacity_rows < 0) return DOK_EINVAL;
   if (((uintptr_t)scratch & 7) != 0) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   const i64 n_chunks = chunks_of(d);
   i64 *offs = (i64 *)scratch;
   if (layout == DOK_LAYOUT_PACKED8) {
@@ -447,6 +486,7 @@ int dok_map_compact_static(const dok_table_t *t, void *keys_out, void *values_ou
   const int64_t need = dok_compact_scratch_bytes(t);
   if (need < 0) return (int)need;
   if (need > DOK_STATIC_SCRATCH_BYTES) return DOK_ETOOLARGE;     // before anything is launched
+  const DeviceScope on_stream_device((hipStream_t)stream);      // (the scratch of the GPU the stream runs on)
   void *scratch = nullptr;
   int rc = static_scratch_of_current_device(&scratch);
   if (rc) return rc;
@@ -464,6 +504,7 @@ int dok_coo_compact(const dok_table_t *t, int64_t *indices_out, void *values_out
   if (!count_out || !scratch || capacity < 0) return DOK_EINVAL;
   if (((uintptr_t)scratch & 7) != 0) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   const i64 n_chunks = chunks_of(d);
   i64 *offs = (i64 *)scratch;
   P8_DISPATCH(d.value_bytes, (p8_chunk_count_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks)));
@@ -485,6 +526,7 @@ int dok_map_rehash(const dok_table_t *src, const dok_table_t *dst, void *stream)
   if (a.buckets == b.buckets) return DOK_EINVAL;
   for (int k = 0; k < a.lin_ndim; k++) if (a.lin_dims[k] != b.lin_dims[k]) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   const i64 n_chunks = chunks_of(a);
   if (la == DOK_LAYOUT_PACKED8) {
     P8_DISPATCH(a.value_bytes, (p8_rehash_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(a, b, n_chunks)));
@@ -533,6 +575,7 @@ int dok_map_rehash_bulk(const dok_table_t *src, const dok_table_t *dst, void *wo
   if (!bulk_plan(b, n_in, p, DOK_BULK_GRID, DOK_BULK_GRID, n_cap)) return DOK_EUNSUPPORTED;
   if (((uintptr_t)workspace & 255) != 0 || workspace_bytes < (int64_t)p.bytes) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   constexpr int KF = DOK_KF_TABLE;
   P8_DISPATCH(b.value_bytes, (bulk_plan_for<V, KF>(b, n_in, p, n_cap),
                               bulk_launch<V, KF, true>(b, a.buckets, nullptr, n_in, p, workspace, s)));
@@ -549,6 +592,7 @@ int dok_getitem_dense(const dok_table_t *t, const dok_index_t *ix, void *out, vo
   if (di.n_elems == 0) return DOK_OK;
   if (!out || di.n_elems > kMaxRows) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   P8_DISPATCH(d.value_bytes, (p8_getitem_kernel<V><<<grid_for(di.n_elems), DOK_TPB, 0, s>>>(d, di, out)));
   return note_launch();
 }
@@ -563,6 +607,7 @@ int dok_setitem_dense(const dok_table_t *t, const dok_index_t *ix, const dok_vie
   if (di.n_elems == 0) return DOK_OK;
   if (di.n_elems > kMaxRows) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   const unsigned grid = grid_counting(di.n_elems);
   P8_DISPATCH(d.value_bytes, (p8_setitem_kernel<V><<<grid, DOK_TPB, 0, s>>>(d, di, rows_per_wave(di.n_elems, grid))));
   return note_launch();
@@ -577,6 +622,7 @@ int dok_count_items(const dok_table_t *t, const dok_index_t *ix, int64_t *count,
   if (di.n_elems == 0) return DOK_OK;
   if (!count || di.n_elems > kMaxRows) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   P8_DISPATCH(d.value_bytes, (p8_countitems_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di, (i64 *)count)));
   return note_launch();
 }
@@ -590,6 +636,7 @@ int dok_zero_items(const dok_table_t *t, const dok_index_t *ix, void *stream) {
   if (di.n_elems == 0) return DOK_OK;
   if (di.n_elems > kMaxRows) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   P8_DISPATCH(d.value_bytes, (p8_zeroitems_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di)));
   return note_launch();
 }
@@ -609,6 +656,7 @@ int dok_getitem_sparse(const dok_table_t *t, const dok_index_t *ix, const dok_ta
   if (di.n_elems == 0) return DOK_OK;
   if (di.n_elems > kMaxRows) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   P8_DISPATCH(d.value_bytes, (p8_getitem_sparse_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di, o)));
   return note_launch();
 }
@@ -624,6 +672,7 @@ int dok_setitem_sparse(const dok_table_t *t, const dok_index_t *ix, const int64_
   if (n_src == 0) return DOK_OK;
   if (!src_values || (!src_indices && di.sel_ndim > 0)) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   const unsigned grid = grid_counting(n_src);
   P8_DISPATCH(d.value_bytes, (p8_setitem_sparse_kernel<V><<<grid, DOK_TPB, 0, s>>>(
       d, di, (const i64 *)src_indices, src_values, n_src, nonzero_mask, rows_per_wave(n_src, grid))));
@@ -639,6 +688,7 @@ int dok_to_dense(const dok_table_t *t, void *dense, void *stream) {
   for (int k = 0; k < d.lin_ndim; k++) volume *= d.lin_dims[k];
   if (volume == 0) return DOK_OK;
   hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
   const i64 n_chunks = chunks_of(d);
   P8_DISPATCH(d.value_bytes, (p8_to_dense_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, dense, n_chunks, volume)));
   return note_launch();
@@ -653,6 +703,7 @@ int dok_line_gather(const dok_table_t *t, int64_t n, uint64_t seed, uint32_t *ou
   const i64 groups = (n + 7) / 8;
   i64 blocks = (groups * 16 + DOK_TPB - 1) / DOK_TPB;
   if (blocks > 16384) blocks = 16384;
+  const DeviceScope on_stream_device((hipStream_t)stream);
   dok_line_gather_kernel<<<(unsigned)blocks, DOK_TPB, 0, (hipStream_t)stream>>>(
       (const u64 *)d.buckets, d.nb, n, seed, out);
   return note_launch();

@@ -10,6 +10,9 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Calls
  *     enqueue work and return; they do not synchronise.  Operations on one table
  *     must be ordered on one stream (or by events); distinct tables are independent.
+ *     Kernels run on the GPU the stream belongs to, whichever GPU is current in the
+ *     calling thread (the null stream: on the current one); every buffer of a call must
+ *     live on that GPU.
  *   - Return value: DOK_OK or a negative DOK_E* code.  No call throws or aborts.
  *   - Flags (`found`, `stored`, `removed`) are one byte per row, 0 or 1.
  *
