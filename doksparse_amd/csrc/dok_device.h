@@ -107,6 +107,42 @@ __device__ __forceinline__ void dok_wave_add_n(i64 *counter, int v) {
   if (v != 0 && (threadIdx.x & 63) == 0) atomicAdd((u64 *)counter, (u64)(i64)v);
 }
 
+// The same over a whole workgroup: one atomic per workgroup and counter instead of one per wave.
+// The adds of a kernel all go to the same few header words and are served one after the other
+// (about 10 ns each), which a small batch would otherwise wait for longer than for its rows.
+// Every thread of the workgroup must get here (the function holds a barrier), and a kernel calls
+// it once.
+template <int N>
+__device__ __forceinline__ void dok_block_add(i64 *const (&counter)[N], const int (&value)[N]) {
+  __shared__ int part[16][N];
+  const int wave = threadIdx.x >> 6, n_waves = (blockDim.x + 63) >> 6;
+  #pragma unroll
+  for (int k = 0; k < N; k++) {
+    int v = value[k];
+    #pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    if ((threadIdx.x & 63) == 0) part[wave][k] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x < N) {
+    int sum = 0;
+    for (int w = 0; w < n_waves; w++) sum += part[w][threadIdx.x];
+    if (sum != 0) atomicAdd((u64 *)counter[threadIdx.x], (u64)(i64)sum);
+  }
+}
+__device__ __forceinline__ void dok_block_add1(i64 *c0, int v0) {
+  i64 *const c[1] = {c0}; const int v[1] = {v0};
+  dok_block_add<1>(c, v);
+}
+__device__ __forceinline__ void dok_block_add2(i64 *c0, int v0, i64 *c1, int v1) {
+  i64 *const c[2] = {c0, c1}; const int v[2] = {v0, v1};
+  dok_block_add<2>(c, v);
+}
+__device__ __forceinline__ void dok_block_add3(i64 *c0, int v0, i64 *c1, int v1, i64 *c2, int v2) {
+  i64 *const c[3] = {c0, c1, c2}; const int v[3] = {v0, v1, v2};
+  dok_block_add<3>(c, v);
+}
+
 // Zero `words` 8-byte words (a multiple of 4) and the table header.
 __global__ __launch_bounds__(DOK_TPB) void dok_fill_kernel(u64 *p, i64 words, i64 *header) {
   const i64 i = ((i64)blockIdx.x * DOK_TPB + threadIdx.x) * 4;

@@ -487,8 +487,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
     n_ops += active;
   }
   if (STATS) {
-    dok_wave_add_n(&t.header[DOK_H_NPROBE], n_probe);
-    dok_wave_add_n(&t.header[DOK_H_NOPS], n_ops);
+    dok_block_add2(&t.header[DOK_H_NPROBE], n_probe, &t.header[DOK_H_NOPS], n_ops);
   }
 }
 
@@ -675,9 +674,7 @@ __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 nex
       }
     }
   }
-  dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
-  dok_wave_add_n(&t.header[DOK_H_NFULL], n_full);
-  dok_wave_add_n(&t.header[DOK_H_NOOB], n_oob);
+  dok_block_add3(&t.header[DOK_H_NELEM], n_fresh, &t.header[DOK_H_NFULL], n_full, &t.header[DOK_H_NOOB], n_oob);
 }
 
 // Rows [0, n) split into one contiguous share per wave of the grid.
@@ -733,7 +730,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const vo
     if (active && removed_out) removed_out[i] = removed ? 1 : 0;
     n_removed += removed;
   }
-  dok_wave_add_n(&t.header[DOK_H_NELEM], -n_removed);
+  dok_block_add1(&t.header[DOK_H_NELEM], -n_removed);
 }
 
 template <int V, int KF>
@@ -755,7 +752,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_count_kernel(DevTable t, const voi
     p8_lookup<V>(t.buckets, t.nb, sk, pend ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), pend, found, val, sb, ss, nprobe);
     n_found += found;
   }
-  dok_wave_add_n(count, n_found);
+  dok_block_add1(count, n_found);
 }
 
 // ---- table scans: read-out, rehash, densify ------------------------------------------------
@@ -965,7 +962,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_countitems_kernel(DevTable t, DevI
     p8_lookup<V>(t.buckets, t.nb, sk, ok ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), ok, found, val, sb, ss, nprobe);
     n_found += found;
   }
-  dok_wave_add_n(count, n_found);
+  dok_block_add1(count, n_found);
 }
 
 template <int V>
@@ -985,7 +982,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_zeroitems_kernel(DevTable t, DevIn
     if (found) removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
     n_removed += removed;
   }
-  dok_wave_add_n(&t.header[DOK_H_NELEM], -n_removed);
+  dok_block_add1(&t.header[DOK_H_NELEM], -n_removed);
 }
 
 // Sparse-valued getitem: every element of the index space whose coordinate is stored in `t` is
@@ -1011,8 +1008,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_getitem_sparse_kernel(DevTable t, 
     n_fresh += fresh;
     n_full += (found && st == 0);
   }
-  dok_wave_add_n(&out.header[DOK_H_NELEM], n_fresh);
-  dok_wave_add_n(&out.header[DOK_H_NFULL], n_full);
+  dok_block_add2(&out.header[DOK_H_NELEM], n_fresh, &out.header[DOK_H_NFULL], n_full);
 }
 
 // Sparse-valued setitem: source entry k has index vector src_indices[j*n_src + k] (j over the

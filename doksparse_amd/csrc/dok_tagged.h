@@ -312,12 +312,9 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
     n_removed += removed;
     n_ops += active;
   }
-  if (MODE == 1) dok_wave_add_n(count, n_found);
-  if (MODE >= 2) dok_wave_add_n(&t.header[DOK_H_NELEM], -n_removed);
-  if (STATS) {
-    dok_wave_add_n(&t.header[DOK_H_NPROBE], n_probe);
-    dok_wave_add_n(&t.header[DOK_H_NOPS], n_ops);
-  }
+  if (MODE == 1 || MODE >= 2 || STATS)
+    dok_block_add3(MODE == 1 ? count : &t.header[DOK_H_NELEM], MODE == 1 ? n_found : -n_removed,
+                   &t.header[DOK_H_NPROBE], STATS ? n_probe : 0, &t.header[DOK_H_NOPS], STATS ? n_ops : 0);
 }
 
 // Record in the home bucket's metadata that a key was placed d > 0 buckets further on, and (W > 0:
@@ -528,8 +525,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, c
     n_fresh += fresh;
     n_full += (active && st == 0);
   }
-  dok_wave_add_n(&t.header[DOK_H_NELEM], n_fresh);
-  dok_wave_add_n(&t.header[DOK_H_NFULL], n_full);
+  dok_block_add2(&t.header[DOK_H_NELEM], n_fresh, &t.header[DOK_H_NFULL], n_full);
 }
 
 // ---- table scans: read-out and rehash -----------------------------------------------------------
