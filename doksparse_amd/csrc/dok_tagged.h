@@ -178,6 +178,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
   u64 *lds_rows = lds;                          // [DOK_TPB][1 + KW]
   u64 *lds_fb = lds + DOK_TPB * RS;             // [VW]
   u32 *lds_meta = (u32 *)(lds_fb + g.VW);       // [DOK_TPB][2]: metadata and filter of each row's home bucket
+  u8 *lds_out = (u8 *)(lds_meta + DOK_TPB * 2); // [DOK_TPB][V]: the tile's output rows (get)
   if (MODE == 0 && threadIdx.x < g.VW) lds_fb[threadIdx.x] = g.fallback[threadIdx.x];
   __syncthreads();
   const TgLane L(g);
@@ -207,7 +208,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
     tg_hash_row(t, g, krow, home, qfull);
     if (!active) home = 0;
     const i64 wave_i0 = i - L.lane;             // batch row of lane 0
-    u8 *out_g = MODE == 0 ? values + (size_t)(wave_i0 + L.gbase) * g.V : nullptr;   // output row of the group's row 0
+    u8 *out_g = lds_out + (size_t)(wave_row0 + L.gbase) * g.V;   // (staged) output row of the group's row 0
     u64 my_hit64 = 0;
 
     const u64 am = dok_ballot(active);
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
     bool open = active && !found && my_meta != 0;
     if (MODE == 0 && active && !found && !open) {
       for (int k = 0; k < g.VW; k++)
-        tg_store_word(values + (size_t)i * g.V, k, g.V, unit_v, lds_fb[k]);
+        tg_store_word(lds_out + (size_t)threadIdx.x * g.V, k, g.V, unit_v, lds_fb[k]);
     }
 
     // phase 2: the marked displacements, then (rare) the far ones
@@ -300,7 +301,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
           open = cand != 0 || (far && (far_max == DOK_TG_FARCAP ? (u64)far_d < t.nb : far_d <= far_max));
           if (!open && MODE == 0) {
             for (int k = 0; k < g.VW; k++)
-              tg_store_word(values + (size_t)i * g.V, k, g.V, unit_v, lds_fb[k]);
+              tg_store_word(lds_out + (size_t)threadIdx.x * g.V, k, g.V, unit_v, lds_fb[k]);
           }
         }
       }
@@ -310,6 +311,18 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
     if (MODE == 2 && found)
       removed = atomicCAS((u32 *)(t.buckets + (u64)sb * 16 + sw), qfull, DOK_TG_TOMB) == qfull;
     if (MODE == 3 && found) { *(u32 *)(t.buckets + (u64)sb * 16 + sw) = DOK_TG_TOMB; removed = true; }
+    if (MODE == 0 && am != 0) {
+      // the wave's output rows leave LDS as one contiguous stretch
+      const int ne = __popcll(am) * (g.V / unit_v);
+      const u8 *src = lds_out + (size_t)wave_row0 * g.V;
+      u8 *dst = values + (size_t)wave_i0 * g.V;
+      for (int e = L.lane; e < ne; e += 64) {
+        if (unit_v == 8) ((u64 *)dst)[e] = ((const u64 *)src)[e];
+        else if (unit_v == 4) ((u32 *)dst)[e] = ((const u32 *)src)[e];
+        else if (unit_v == 2) ((u16 *)dst)[e] = ((const u16 *)src)[e];
+        else dst[e] = src[e];
+      }
+    }
     if (MODE == 0 && active) flags[i] = found ? 1 : 0;
     if (MODE >= 2 && active && flags) flags[i] = removed ? 1 : 0;
     n_found += found;
@@ -640,7 +653,7 @@ static int tg_geom(const DevTable &d, const void *fallback, TgGeom &g) {
 
 static bool tg_aligned(const void *p, int unit) { return ((uintptr_t)p & (uintptr_t)(unit - 1)) == 0; }
 
-static size_t tg_lds_lookup(const TgGeom &g) { return (size_t)(DOK_TPB * (g.KW + 1) + g.VW + DOK_TPB) * 8; }
+static size_t tg_lds_lookup(const TgGeom &g) { return (size_t)(DOK_TPB * (g.KW + 1) + g.VW + DOK_TPB + (DOK_TPB * g.V + 7) / 8) * 8; }
 static size_t tg_lds_insert(const TgGeom &g) { return (size_t)DOK_TPB * (g.KW + 1 + g.VW) * 8; }
 
 // Most workgroups of the kernels that loop over tiles and end with one atomic per wave on a
