@@ -514,6 +514,76 @@ __device__ __forceinline__ void tg_insert_rows(const DevTable &t, const TgGeom &
   }
 }
 
+// Placement of rows whose keys are all different and absent from the table, into a table without
+// tombstones that nothing else touches while the kernel runs: the destination of a rehash.
+// Slots then only ever go from EMPTY to FULL, so no key is compared and no slot is locked: a row
+// claims the first EMPTY slot of its walk (CAS EMPTY -> FULL; a stale view of a taken slot only
+// costs a failed claim) and the group writes the payload with plain stores - one compare-and-swap
+// and one store per row where the upsert protocol takes three write-through transactions.
+__device__ __forceinline__ void tg_place_rows(const DevTable &t, const TgGeom &g, const TgLane &L,
+                                              const u64 *lds_rows, const u64 *lds_vals, u32 home, u32 qfull,
+                                              bool pend, int &st) {
+  const int RS = tg_rs(g);
+  const int wave_row0 = threadIdx.x & ~63;
+  if (!pend) home = 0;
+  const u32 fbit = tg_fbit(qfull);
+  const bool has_filter = g.S >= 2;
+  u32 cur = 0, md_home = 0, filt_home = 0;
+  u64 pm = dok_ballot(pend);
+  while (pm != 0) {
+    bool wr = false;
+    u32 wr_b = 0, wr_w = 0;
+    if (pend) {
+      const u32 b = tg_wrap(home, cur, t.nb);
+      u64 *bucket = t.buckets + (u64)b * 16;
+      u32 emptym = 0;
+      #pragma unroll
+      for (int s = 0; s < DOK_TG_MAXS; s++) {
+        if (s < g.S) {
+          const u64 tw = bucket[s * g.W];
+          emptym |= (u32)((u32)tw == DOK_TG_EMPTY) << s;
+          if (cur == 0 && s == 0) md_home = (u32)(tw >> 32);
+          if (cur == 0 && s == 1) filt_home = (u32)(tw >> 32);
+        }
+      }
+      while (emptym != 0 && !wr) {
+        const int s = __builtin_ctz(emptym);
+        emptym &= emptym - 1;
+        if (atomicCAS((u32 *)(bucket + s * g.W), DOK_TG_EMPTY, qfull) == DOK_TG_EMPTY) {
+          wr = true; wr_b = b; wr_w = (u32)(s * g.W);
+        }
+      }
+      if (wr) {
+        st = 1; pend = false;
+        if (cur > 0) tg_mark(t.buckets + (u64)home * 16, cur, md_home, has_filter ? g.W : 0, fbit, filt_home);
+      } else if ((u64)cur + 1 >= t.nb) {
+        st = 0; pend = false;                              // no free slot anywhere
+      } else {
+        cur++;
+      }
+    }
+    // the slots won in this turn: lane p of the row's group stores word p
+    const u64 wm = dok_ballot(wr);
+    if (wm != 0) {
+      const u32 wsub = L.grp(wm);
+      u32 wany = (u32)wm | (u32)(wm >> 32);
+      wany = (wany | (wany >> 16)) & 0xffffu;
+      #pragma unroll
+      for (int r = 0; r < 16; r++) {
+        if (!((wany >> r) & 1u)) continue;
+        const int j = L.gbase + r;
+        const u32 qb = dok_shfl32(wr_b, j), qw = dok_shfl32(wr_w, j);
+        if (((wsub >> r) & 1u) && L.l >= 1 && L.l < g.W) {
+          const u64 word = L.l <= g.KW ? lds_rows[(wave_row0 + j) * RS + L.l]
+                                       : lds_vals[(wave_row0 + j) * g.VW + L.l - 1 - g.KW];
+          t.buckets[(u64)qb * 16 + qw + L.l] = word;
+        }
+      }
+    }
+    pm = dok_ballot(pend);
+  }
+}
+
 __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, const u8 *__restrict__ keys,
                                                          const u8 *__restrict__ values, i64 n,
                                                          u8 *__restrict__ stored) {
@@ -622,9 +692,9 @@ __global__ __launch_bounds__(DOK_TPB) void tg_rehash_kernel(DevTable src, DevTab
         const bool pend = L.lane < cnt;
         u32 home, qfull;
         tg_hash_row(dst, g, lds_rows + threadIdx.x * RS, home, qfull);
-        int st = 0, fresh = 0;
-        tg_insert_rows(dst, g, L, lds_rows, lds_vals, home, qfull, pend, st, fresh);
-        n_fresh += fresh;
+        int st = 0;
+        tg_place_rows(dst, g, L, lds_rows, lds_vals, home, qfull, pend, st);
+        n_fresh += (pend && st == 1);
         n_full += (pend && st == 0);
         cnt = 0;
       }
