@@ -726,3 +726,39 @@ def test_multiword_layout_random_geometries_against_a_dict(cuda):
             for key, val in model.items():
                 assert np.array_equal(allv[key].view(np.uint8), val.view(np.uint8)), (case, rnd, key)
         assert hm.items()[0].shape[0] == len(model)
+
+
+@pytest.mark.parametrize("kshape,kdt,vshape,vdt", [((3,), np.float32, (5,), np.int64), ((2,), np.int64, (1,), np.float32),
+                                                   ((9,), np.int64, (3,), np.int16)])
+def test_multiword_rehash_into_a_table_without_a_free_slot_to_spare(cuda, kshape, kdt, vshape, vdt):
+    """rehash(n_elements): the device-side rehash fills the new table to (nearly) its last slot, so
+    rows walk far from their home buckets and leave far displacement records; every key must still
+    be found, absent keys must not, and the map must keep working afterwards."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(31)
+    n = 5000
+    keys = np.unique(rng.integers(-2**20, 2**20, size=(n, *kshape)).astype(kdt), axis=0)
+    n = keys.shape[0]
+    vals = rng.integers(-1000, 1000, size=(n, *vshape)).astype(vdt)
+    absent = (rng.integers(2**21, 2**22, size=(2000, *kshape))).astype(kdt)
+    hm = CudaClosedHashmap(n_buckets=4 * n, device=cuda, rehash_threshold=1e9)
+    hm.set(*_to(cuda, keys, vals))
+    gone = rng.permutation(n)[: n // 5]
+    hm._remove_rows(torch.from_numpy(keys[gone]).to(cuda).contiguous())       # tombstones do not travel
+    live = np.ones(n, dtype=bool); live[gone] = False
+    hm.rehash(int(live.sum()))
+    assert hm.n_elements == int(live.sum()) and hm.n_buckets == int(live.sum())
+    got, found = hm.get(torch.from_numpy(keys).to(cuda))
+    assert np.array_equal(found.cpu().numpy(), live)
+    assert np.array_equal(got.cpu().numpy()[live], vals[live])
+    assert not bool(hm.get(torch.from_numpy(absent).to(cuda))[1].any())
+    # the removed keys fit again only after a growth; overwrites work in the full table
+    hm.set(*_to(cuda, keys[live][:100], vals[live][:100] + 1))
+    assert np.array_equal(hm.get(torch.from_numpy(keys[live][:100]).to(cuda))[0].cpu().numpy(), vals[live][:100] + 1)
+    hm.rehash(2 * n)
+    hm.set(*_to(cuda, keys[gone], vals[gone]))
+    assert hm.n_elements == n
+    got, found = hm.get(torch.from_numpy(keys).to(cuda))
+    assert bool(found.all())
+    expect = vals.copy(); idx = np.flatnonzero(live)[:100]; expect[idx] += 1
+    assert np.array_equal(got.cpu().numpy(), expect)
