@@ -477,6 +477,44 @@ def test_reductions_and_elementwise_glue(cuda):
     assert torch.equal(dok.reshape(20, 60).to_dense().cpu(), dense.reshape(20, 60))
 
 
+def test_constructors_clone_resize_and_conversions(cuda):
+    """from_sparse_coo / from_storage / clone / resize / to_sparse_csr / __torch_function__ / repr
+    (reference: sparse_dok_tensor.py:71-118, 195-215), against the dense tensor."""
+    from doksparse_amd import SparseDOKTensor, sparse_dok_tensor
+    gen = torch.Generator(device="cpu"); gen.manual_seed(21)
+    dense = torch.zeros(24, 18)
+    mask = torch.rand(24, 18, generator=gen) < 0.25
+    dense[mask] = torch.randn(int(mask.sum()), generator=gen)
+    coo = dense.to_sparse().to(cuda)
+    dok = SparseDOKTensor.from_sparse_coo(coo)
+    assert torch.equal(dok.to_dense().cpu(), dense) and dok._nnz() == int(mask.sum())
+    assert torch.equal(sparse_dok_tensor((24, 18), coo.indices(), coo.values(), device=cuda).to_dense().cpu(), dense)
+    # the storage of one tensor makes another: same table, same entries
+    twin = SparseDOKTensor.from_storage(dok.storage())
+    assert tuple(twin.shape) == (24, 18) and torch.equal(twin.to_dense().cpu(), dense)
+    # deep clone is independent, shallow clone shares the table
+    deep, shallow = dok.clone(), dok.clone(deepclone=False)
+    dok[torch.tensor([0], device=cuda), torch.tensor([0], device=cuda)] = torch.tensor([7.0], device=cuda)
+    changed = dense.clone(); changed[0, 0] = 7.0
+    assert torch.equal(deep.to_dense().cpu(), dense)
+    assert torch.equal(shallow.to_dense().cpu(), changed) and torch.equal(dok.to_dense().cpu(), changed)
+    # conversions
+    csr = dok.to_sparse_csr()
+    assert csr.layout == torch.sparse_csr and torch.equal(csr.to_dense().cpu(), changed)
+    assert torch.equal(dok.to_sparse_coo().to_dense().cpu(), changed)
+    assert torch.allclose(torch.sparse.sum(dok).cpu(), changed.sum(), atol=1e-5)      # via __torch_function__
+    text = repr(dok)
+    assert "SparseDOKTensor" in text and f"nnz={dok._nnz()}" in text
+    # resize: growing keeps every entry, shrinking keeps the entries inside the new size
+    grown = deep.clone().resize(30, 40)
+    assert tuple(grown.shape) == (30, 40)
+    big = torch.zeros(30, 40); big[:24, :18] = dense
+    assert torch.equal(grown.to_dense().cpu(), big)
+    shrunk = deep.clone().resize(10)                       # second dimension unchanged
+    assert tuple(shrunk.shape) == (10, 18) and torch.equal(shrunk.to_dense().cpu(), dense[:10])
+    assert shrunk._nnz() == int(mask[:10].sum())
+
+
 def _random_selectors(rng, shape):
     """A random indexing expression over the leading dimensions of `shape`: integers, slices,
     index tensors that broadcast to one shape, lists, and at most one 1-D mask (kept apart
