@@ -762,3 +762,39 @@ def test_multiword_rehash_into_a_table_without_a_free_slot_to_spare(cuda, kshape
     assert bool(found.all())
     expect = vals.copy(); idx = np.flatnonzero(live)[:100]; expect[idx] += 1
     assert np.array_equal(got.cpu().numpy(), expect)
+
+
+def test_raw_table_attributes_and_set_values(cuda):
+    """The reference's raw-table surface (cuda_closed_hashmap.py:157-177, 233-273): keys() /
+    values() / uuid() / nonempty_mask / _keys / _values / _uuid / _n_elements and set_values, whose
+    selectors address the live entries in values() order."""
+    from doksparse_amd import CudaClosedHashmap
+    hm = CudaClosedHashmap(n_buckets=64, device=cuda)
+    assert hm._keys is None and hm._values is None
+    assert hm._uuid.shape == (64,) and bool((hm._uuid == hm._empty_marker).all())
+    assert hm.nonempty_mask.shape == (0,)
+    k = torch.arange(10, 40, device=cuda)[:, None]
+    v = torch.arange(30, device=cuda, dtype=torch.float32)[:, None] * 2
+    hm.set(k, v)
+    hm.remove(k[:5])
+    assert hm.key_type == torch.int64 and hm.value_type == torch.float32
+    assert hm.key_shape == (1,) and hm.value_shape == (1,)
+    assert int(hm._n_elements) == len(hm) == 25 and hm._n_elements.device.type == "cuda"
+    keys, values = hm.keys(), hm.values()
+    assert keys.shape == (25, 1) and values.shape == (25, 1)
+    assert torch.equal(values, (keys - 10).float() * 2)                   # the two read-outs agree row by row
+    assert torch.equal(hm._keys, keys) and torch.equal(hm._values, values)
+    assert hm.nonempty_mask.shape == (25,) and bool(hm.nonempty_mask.all())
+    assert hm.uuid().shape == (25,) and torch.equal(hm.uuid(), hm.get_uuid(keys))
+    assert torch.unique(hm.uuid()).numel() == 25
+    # set_values: by position in values() order, boolean or integer selectors
+    sel = torch.zeros(25, dtype=torch.bool, device=cuda); sel[::3] = True
+    hm.set_values(sel, torch.full((int(sel.sum()), 1), -1.0, device=cuda))
+    got, found = hm.get(keys)
+    assert bool(found.all())
+    expect = values.clone(); expect[sel] = -1.0
+    assert torch.equal(got, expect) and len(hm) == 25
+    hm.set_values(torch.tensor([0, 24], device=cuda), torch.tensor([[5.0], [6.0]], device=cuda))
+    keys2, values2 = hm.items()
+    look = dict(zip(keys2.flatten().tolist(), values2.flatten().tolist()))
+    assert look[int(keys[0])] == 5.0 and look[int(keys[24])] == 6.0
