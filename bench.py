@@ -360,7 +360,7 @@ def tagged_scale(device, n=32_000_000):
 
 def dok_scale(device):
     """The DOK indexing kernels at scale, kernel-level through the C ABI on preallocated buffers:
-    a 2-D 1e6 x 1e6 float32 tensor of 50M entries (BASELINE configuration 4); gather of 2^26
+    a 2-D 1e6 x 1e6 float32 tensor of 50M entries (the fourth benchmark configuration); gather of 2^26
     stored coordinates through `__getitem__`'s kernel, scatter of 10M coordinates (half present,
     half new) through `__setitem__`'s, and the read-out of all entries."""
     from doksparse_amd import SparseDOKTensor, _lib
