@@ -439,9 +439,10 @@ class CudaClosedHashmap:
         return t
 
     def _check_keys(self, keys):
-        assert keys.dtype == self._key_dtype
-        assert keys.device == self.device
-        assert tuple(keys.shape[1:]) == self._key_shape
+        assert keys.dtype == self._key_dtype, f"keys are {keys.dtype}, the map holds {self._key_dtype}"
+        assert keys.device == self.device, f"keys are on {keys.device}, the map is on {self.device}"
+        assert tuple(keys.shape[1:]) == self._key_shape, \
+            f"key rows have shape {tuple(keys.shape[1:])}, the map holds {self._key_shape}"
 
     # ------------------------------------------------------------------ set / get / remove
     def _bulk_workspace(self, n):
@@ -501,15 +502,19 @@ class CudaClosedHashmap:
 
     def set(self, new_keys, new_values):
         """Upsert a batch (reference: cuda_closed_hashmap.py:321-384).  Returns None."""
-        assert new_keys.shape[0] == new_values.shape[0]
+        assert new_keys.shape[0] == new_values.shape[0], \
+            f"{new_keys.shape[0]} key rows but {new_values.shape[0]} value rows"
         if not self._allocated:
-            assert new_keys.device == new_values.device == self.device
+            assert new_keys.device == new_values.device == self.device, \
+                f"keys on {new_keys.device}, values on {new_values.device}, the map is on {self.device}"
             self._init_storage(new_keys, new_values)
         else:
             self._check_keys(new_keys)
-            assert new_values.dtype == self._value_dtype
-            assert new_values.device == self.device
-            assert tuple(new_values.shape[1:]) == self._value_shape
+            assert new_values.dtype == self._value_dtype, \
+                f"values are {new_values.dtype}, the map holds {self._value_dtype}"
+            assert new_values.device == self.device, f"values are on {new_values.device}, the map is on {self.device}"
+            assert tuple(new_values.shape[1:]) == self._value_shape, \
+                f"value rows have shape {tuple(new_values.shape[1:])}, the map holds {self._value_shape}"
         n = new_keys.shape[0]
         try:
             if n:
