@@ -68,6 +68,7 @@ SIGNATURES = {
     "dok_last_hip_error": (c_char_p, []),
     "dok_table_clear": (c_int32, [POINTER(DokTable), c_void_p]),
     "dok_map_get": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "dok_map_get_dev_fallback": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "dok_map_get_stats": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "dok_map_set": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "dok_bulk_workspace_bytes": (c_int64, [POINTER(DokTable), c_int64]),

@@ -90,6 +90,38 @@ def _next_prime(n):
     return m
 
 
+_SAME_SIZE_INT = {1: torch.int8, 2: torch.int16, 4: torch.int32, 8: torch.int64}
+
+
+def _ordered_bits(t):
+    """Floating-point rows as integers of the same width whose order is the order of the values
+    and whose equality is equality of the BIT PATTERNS - the identity the table goes by: two NaNs
+    of one bit pattern are one key, -0.0 and +0.0 are two (`torch.unique` on the float values has
+    it the other way round).  A float's bits, read as a signed integer, already sort like the
+    float when the sign is clear; with the sign set the order is reversed, which flipping the
+    other bits undoes.  The map is its own inverse.  Integer and bool rows come back unchanged."""
+    if not t.dtype.is_floating_point:
+        return t
+    bits = t.view(_SAME_SIZE_INT[t.element_size()])
+    width = 8 * t.element_size()
+    return bits ^ ((bits >> (width - 1)) & ((1 << (width - 1)) - 1))
+
+
+def unique_rows(keys):
+    """Distinct rows of `keys` by bit pattern, sorted (row-wise lexicographically) by value: what
+    `keys.unique(dim=0)` gives (reference: cuda_closed_hashmap.py:438) wherever the two notions of
+    equality agree, i.e. for every batch without NaNs and without both zeros in one column."""
+    ordered = _ordered_bits(keys)
+    if keys[0].numel() == 1:
+        # one element per key: the 1-D sort gives the order of unique(dim=0) far faster
+        uniq = ordered.reshape(-1).unique().reshape(-1, *keys.shape[1:])
+    else:
+        uniq = ordered.unique(dim=0)
+    if keys.dtype.is_floating_point:
+        uniq = _ordered_bits(uniq.view(keys.dtype)).view(keys.dtype)
+    return uniq
+
+
 class _TableState:
     """Physical state of one table.  Shallow clones of a map share one instance, so a rehash or
     an insert through any of them is seen by all."""
@@ -635,7 +667,7 @@ class CudaClosedHashmap:
         if n == 0:
             return 0
         if self._layout != _lib.DOK_LAYOUT_PACKED8:
-            return int(keys.unique(dim=0).shape[0])
+            return int(unique_rows(keys).shape[0])        # distinct by bit pattern, as the table sees them
         lib = _lib.load()
         kb = 8 if self._coord_dims is not None else self._key_bytes
         n_phys = int(lib.dok_phys_buckets_for(2 * n, kb, 1))
@@ -660,10 +692,17 @@ class CudaClosedHashmap:
             return (torch.empty(0, *self._value_shape, device=self.device, dtype=self._value_dtype),
                     torch.empty(0, device=self.device, dtype=torch.bool))
         self._check_keys(keys)
-        fb = None
-        if fallback_value is not None:
+        # The fallback row.  A tensor on the map's device stays there and is read by the kernel: no
+        # copy to the host, no synchronisation, and the call can be captured into a HIP graph and
+        # see the row's contents at replay time (the reference passes a device array too,
+        # closed_hashmap_impl.py:103-109).  Anything else becomes a few bytes passed by value.
+        fb = fb_dev = None
+        if isinstance(fallback_value, Tensor) and fallback_value.device == self.device:
+            assert fallback_value.dtype == self._value_dtype
+            fb_dev = torch.broadcast_to(fallback_value, self._value_shape).contiguous()
+        elif fallback_value is not None:
             if not isinstance(fallback_value, Tensor):
-                fallback_value = torch.tensor(fallback_value, device=self.device, dtype=self._value_dtype)
+                fallback_value = torch.tensor(fallback_value, dtype=self._value_dtype)
             assert fallback_value.dtype == self._value_dtype
             row = torch.empty(self._value_shape, dtype=self._value_dtype)
             row.copy_(torch.broadcast_to(fallback_value.cpu(), self._value_shape))
@@ -673,24 +712,25 @@ class CudaClosedHashmap:
         values = torch.empty(n, *self._value_shape, device=self.device, dtype=self._value_dtype)
         is_found = torch.empty(n, device=self.device, dtype=torch.bool)
         lib = _lib.load()
-        _lib.check(lib.dok_map_get(ctypes.byref(self._desc), keys.data_ptr(), n, values.data_ptr(),
-                                   fb, is_found.data_ptr(), _stream_ptr(self.device)), "get")
+        if fb_dev is not None:
+            _lib.check(lib.dok_map_get_dev_fallback(ctypes.byref(self._desc), keys.data_ptr(), n, values.data_ptr(),
+                                                    fb_dev.data_ptr(), is_found.data_ptr(),
+                                                    _stream_ptr(self.device)), "get")
+        else:
+            _lib.check(lib.dok_map_get(ctypes.byref(self._desc), keys.data_ptr(), n, values.data_ptr(),
+                                       fb, is_found.data_ptr(), _stream_ptr(self.device)), "get")
         return values, is_found
 
     def remove(self, keys):
-        """Remove a batch of keys; returns the mask over ``keys.unique(dim=0)``
-        (reference: cuda_closed_hashmap.py:423-454)."""
+        """Remove a batch of keys; returns the mask over the distinct rows of ``keys`` in sorted
+        order - ``keys.unique(dim=0)``, except that rows are told apart by bit pattern like the
+        table does (see `unique_rows`; reference: cuda_closed_hashmap.py:423-454)."""
         if not self._allocated:
             raise RuntimeError("store something first")
         if keys.shape[0] == 0:
             return torch.zeros(0, device=keys.device, dtype=torch.bool)
         self._check_keys(keys)
-        if keys[0].numel() == 1:
-            # one element per key: the 1-D sort gives the order of unique(dim=0) far faster
-            unique_keys = keys.reshape(-1).unique().reshape(-1, *self._key_shape)
-        else:
-            unique_keys = keys.unique(dim=0)
-        return self._remove_rows(self._prep_rows(unique_keys, "keys"), unique=True)
+        return self._remove_rows(self._prep_rows(unique_rows(keys), "keys"), unique=True)
 
     def _remove_rows(self, keys, unique=False):
         """Remove without the sort: mask aligned with ``keys`` (equal rows: one reports True).

@@ -11,8 +11,8 @@
 //   2. two scatter passes (first by range / 256 (range / 1024 for very large tables), then by
 //      range inside each first-level bin) move every (key, value) row next to the other rows of
 //      its range.  Nothing is counted beforehand: every bin owns a region of fixed capacity in the
-//      pass's output - the rows a uniform hash sends there on average plus seven standard
-//      deviations - and a workgroup that has staged a tile of rows in LDS, ordered by bin,
+//      pass's output - the rows a uniform hash sends there on average plus six (first level) resp.
+//      five (ranges) standard deviations - and a workgroup that has staged a tile of rows in LDS, ordered by bin,
 //      reserves the run of each bin with ONE atomic add on that bin's fill counter (a few hundred
 //      atomics per tile of thousands of rows, issued while the tile is being staged, so their
 //      latency is hidden).  Rows that find their bin's region full (batches with very many
@@ -31,9 +31,7 @@
 #pragma once
 #include "dok_packed8.h"
 
-#ifndef DOK_BULK_RLOG
 #define DOK_BULK_RLOG 8                     // log2 of the buckets per range: 256 buckets = 32 KiB
-#endif
 #define DOK_BULK_R (1 << DOK_BULK_RLOG)
 #define DOK_BULK_SUBLOG 8                   // log2 of the ranges per first-level bin ...
 #define DOK_BULK_SUBLOG_WIDE 10             // ... and for tables of more than 1024 << 8 ranges
@@ -42,12 +40,8 @@
 // fills the LDS); 16 waves instead of 8 make the second pass, whose workgroups take one or two
 // tiles each, 12 % faster and the first pass over plain keys 3 %; the first pass over coordinate
 // rows or over a table's buckets (more registers per row, more loads per row) loses with them.
-#ifndef DOK_BULK_TPB_FEW
 #define DOK_BULK_TPB_FEW 512
-#endif
-#ifndef DOK_BULK_TPB_MANY
 #define DOK_BULK_TPB_MANY 1024
-#endif
 constexpr int bulk_tpb(int level, int key_format, int coord_dims) {
   return level == 1 && (coord_dims > 0 || key_format == DOK_KF_TABLE) ? DOK_BULK_TPB_FEW : DOK_BULK_TPB_MANY;
 }
@@ -55,28 +49,16 @@ constexpr int bulk_tpb(int level, int key_format, int coord_dims) {
 // it is, the longer the runs of rows that leave for one bin: for 8-byte keys with 4-byte values
 // one workgroup per CU with a tile that nearly fills the LDS beats two with half the tile
 // (scatter of 64M rows: 0.57 -> 0.47 ms).  All sizes are measured choices.
-#ifndef DOK_BULK_T
 #define DOK_BULK_T 8192                     // first pass (up to 1024 bins: 12 KiB of bin arrays)
-#endif
-#ifndef DOK_BULK_T1V8
 #define DOK_BULK_T1V8 6144                  //   ... with 8-byte values
-#endif
-#ifndef DOK_BULK_T2
 #define DOK_BULK_T2 10240                   // second pass
-#endif
-#ifndef DOK_BULK_T2S
 #define DOK_BULK_T2S 4096                   //   ... with 1- and 2-byte values when a workgroup's stretch is short
-#endif                                      //   (three workgroups per CU with small tiles are faster then)
+                                            //   (three workgroups per CU with small tiles are faster then)
 #define DOK_BULK_T2S_BELOW 16384            //   ... which is: fewer rows than this per workgroup
-#ifndef DOK_BULK_T2V8
 #define DOK_BULK_T2V8 8192                  //   ... with 8-byte values
-#endif
-#ifndef DOK_BULK_CTPB
 #define DOK_BULK_CTPB 1024                  // threads per workgroup of the count kernels: they only stream
-#endif                                      // keys, and the bytes in flight per CU bound their rate
-#ifndef DOK_BULK_GRID
+                                            // keys, and the bytes in flight per CU bound their rate
 #define DOK_BULK_GRID 1024                  // most workgroups the first pass and the merge are given
-#endif
 
 // Device view of the caller's workspace.
 struct BulkWs {
@@ -454,9 +436,7 @@ __global__ __launch_bounds__(bulk_tpb(LEVEL, KF, ND)) void bulk_scatter_kernel(D
 // there).  Rows that find no room up to the range's last bucket move on to the next range of the
 // same workgroup, or - out of the block's last range - to bulk_edge_kernel; rows that found no
 // room on the list, and a few awkward cases, are handed to the ordinary insert.
-#ifndef DOK_BULK_C
 #define DOK_BULK_C (6 * DOK_BULK_R)
-#endif
 #define DOK_BULK_FPW 8                          // 32-bit fingerprint words per bucket
 #define DOK_BULK_LIST (2 * DOK_BULK_R)          // capacity of a range's list
 

@@ -110,8 +110,8 @@ __device__ __forceinline__ void dok_wave_add_n(i64 *counter, int v) {
 // The same over a whole workgroup: one atomic per workgroup and counter instead of one per wave.
 // The adds of a kernel all go to the same few header words and are served one after the other
 // (about 10 ns each), which a small batch would otherwise wait for longer than for its rows.
-// Every thread of the workgroup must get here (the function holds a barrier), and a kernel calls
-// it once.
+// Every thread of the workgroup must get here (the function holds barriers: no call after a
+// per-wave early return).
 template <int N>
 __device__ __forceinline__ void dok_block_add(i64 *const (&counter)[N], const int (&value)[N]) {
   __shared__ int part[16][N];
@@ -129,6 +129,7 @@ __device__ __forceinline__ void dok_block_add(i64 *const (&counter)[N], const in
     for (int w = 0; w < n_waves; w++) sum += part[w][threadIdx.x];
     if (sum != 0) atomicAdd((u64 *)counter[threadIdx.x], (u64)(i64)sum);
   }
+  __syncthreads();           // `part` may be written again by a later call
 }
 __device__ __forceinline__ void dok_block_add1(i64 *c0, int v0) {
   i64 *const c[1] = {c0}; const int v[1] = {v0};

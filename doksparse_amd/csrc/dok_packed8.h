@@ -147,15 +147,9 @@ __device__ __forceinline__ int p8_pick(u32 free_mask, int start) {   // free_mas
 // up to DOK_P8_WL of its open rows and loads the next two marked buckets of each (independent
 // loads), folds the outcomes into the owners, which then act together.  Two rows per turn
 // measured best: most turns have few open rows and wider turns only add instructions.
-#ifndef DOK_P8_U
 #define DOK_P8_U 8
-#endif
-#ifndef DOK_P8_WL
 #define DOK_P8_WL 2  // rows per group per phase-2 turn of the lookup
-#endif
-#ifndef DOK_P8_WI
 #define DOK_P8_WI 4  // rows per group per phase-2 turn of the insert
-#endif
 template <int V>
 __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 nb, u64 sk, u32 b, u32 fbit,
                                           bool pend, bool &found, u64 &val, u32 &slot_b,
@@ -464,7 +458,10 @@ __device__ __forceinline__ int p8_side_set(const DevTable &t, u64 sk, u64 val) {
 template <int V, bool STATS, int KF>
 __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void *__restrict__ keys, i64 n,
                                                          void *__restrict__ values, u8 *__restrict__ found_out,
-                                                         u64 fallback) {
+                                                         u64 fallback, const void *__restrict__ fallback_dev) {
+  // the fallback value: an immediate, or - fallback_dev set - read from device memory by the kernel
+  // itself, as the reference's kernel reads its fallback array
+  if (fallback_dev) fallback = dok_load_val<V>(fallback_dev, 0);
   int n_probe = 0, n_ops = 0;
   DOK_TILE_LOOP(n) {
     const i64 i = DOK_TILE_ROW();
@@ -491,9 +488,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
   }
 }
 
-#ifndef DOK_STREAM_WAVES
 #define DOK_STREAM_WAVES 8   // waves per SIMD the streaming kernels are compiled for
-#endif
 // Streaming insert.  Every lane carries one row at some point of its walk (bucket home + d); a
 // pass loads the current bucket of all 64 rows (batched as in phase 1 of p8_insert), the owners
 // decide and claim together, and lanes whose row is finished take the next rows of the wave's
@@ -512,7 +507,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
 //
 // `src(i, key, val)` produces row i: 0 = insert key -> val, 1 = the row addresses nothing inside
 // the table's coordinate space (counted, reported as not stored), 2 = skip the row silently.
-// The header counters are updated once per wave at the end.
+// The header counters are updated once per workgroup at the end (dok_block_add3: every thread of
+// the workgroup has to reach the end of this function, exactly once per kernel).
 // The core works through the rows [next, end) that the caller assigns to this wave.
 template <int V, class Src>
 __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 next, i64 end,

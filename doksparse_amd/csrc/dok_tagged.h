@@ -172,14 +172,17 @@ __device__ __forceinline__ u32 tg_wrap(u32 home, u32 d, u64 nb) {
 template <int MODE, bool STATS, int UV = 0>
 __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g, const u8 *__restrict__ keys, i64 n,
                                                             u8 *__restrict__ values, u8 *__restrict__ flags,
-                                                            i64 *count) {
+                                                            i64 *count, const u8 *__restrict__ fallback_dev = nullptr) {
   extern __shared__ u64 lds[];
   const int RS = tg_rs(g);
   u64 *lds_rows = lds;                          // [DOK_TPB][1 + KW]
   u64 *lds_fb = lds + DOK_TPB * RS;             // [VW]
   u32 *lds_meta = (u32 *)(lds_fb + g.VW);       // [DOK_TPB][2]: metadata and filter of each row's home bucket
   u8 *lds_out = (u8 *)(lds_meta + DOK_TPB * 2); // [DOK_TPB][V]: the tile's output rows (get)
-  if (MODE == 0 && threadIdx.x < g.VW) lds_fb[threadIdx.x] = g.fallback[threadIdx.x];
+  // the fallback row: part of the geometry argument, or - fallback_dev set - read from device memory
+  if (MODE == 0 && threadIdx.x < g.VW)
+    lds_fb[threadIdx.x] = fallback_dev ? tg_load_word(fallback_dev, threadIdx.x, g.V, UV ? UV : g.unit_v)
+                                       : g.fallback[threadIdx.x];
   __syncthreads();
   const TgLane L(g);
   const TgMasks M(g, L);
@@ -616,9 +619,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, c
 }
 
 // ---- table scans: read-out and rehash -----------------------------------------------------------
-#ifndef DOK_CHUNK
 #define DOK_CHUNK 256
-#endif
 
 __device__ __forceinline__ bool tg_scan_load(const DevTable &t, const TgLane &L, i64 b, u64 &w) {
   const bool valid = b < (i64)t.nb;
@@ -729,32 +730,29 @@ static size_t tg_lds_insert(const TgGeom &g) { return (size_t)DOK_TPB * (g.KW + 
 // Most workgroups of the kernels that loop over tiles and end with one atomic per wave on a
 // counter: few workgroups keep those atomics cheap (same-address atomics serialise at ~12 ns
 // each), many even out the differing amounts of work of the tiles.
-#ifndef DOK_TG_COUNT_GRID
 #define DOK_TG_COUNT_GRID 8192u
-#endif
-#ifndef DOK_TG_REMOVE_GRID
 #define DOK_TG_REMOVE_GRID 4096u
-#endif
-#ifndef DOK_TG_SET_GRID
 #define DOK_TG_SET_GRID 32768u
-#endif
 
+// fallback: host pointer to the fallback row (NULL = zeros); fb_dev: device pointer to it instead
 static int tg_launch_get(const DevTable &d, const void *keys, i64 n, void *values, const void *fallback,
-                         u8 *found, bool stats, hipStream_t s) {
+                         const void *fb_dev, u8 *found, bool stats, hipStream_t s) {
   TgGeom g;
   int rc = tg_geom(d, fallback, g);
   if (rc) return rc;
   if (!tg_aligned(keys, g.unit_k) || !tg_aligned(values, g.unit_v)) return DOK_EINVAL;
+  if (fb_dev && !tg_aligned(fb_dev, g.unit_v)) return DOK_EINVAL;
+  const u8 *fbd = (const u8 *)fb_dev;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
   const unsigned cgrid = grid < 2048u ? grid : 2048u;
   if (stats)
-    tg_lookup_kernel<0, true><<<cgrid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr);
+    tg_lookup_kernel<0, true><<<cgrid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr, fbd);
   else if (g.unit_v == 8)
-    tg_lookup_kernel<0, false, 8><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr);
+    tg_lookup_kernel<0, false, 8><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr, fbd);
   else if (g.unit_v == 4)
-    tg_lookup_kernel<0, false, 4><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr);
+    tg_lookup_kernel<0, false, 4><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr, fbd);
   else
-    tg_lookup_kernel<0, false><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr);
+    tg_lookup_kernel<0, false><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr, fbd);
   return DOK_OK;
 }
 

@@ -15,6 +15,7 @@
 // at its own address, from the moment the code object is loaded until the process ends.  In host
 // code this name is only a handle for hipGetSymbolAddress - never a pointer to hand to a kernel.
 static __device__ __align__(256) unsigned char dok_static_scratch[DOK_STATIC_SCRATCH_BYTES];
+static_assert(DOK_STATIC_SCRATCH_BYTES >= (((1LL << 28) / DOK_CHUNK) + 1) * 8, "serves tables of up to 2^28 buckets");
 
 namespace {
 
@@ -185,19 +186,10 @@ int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *s
 }
 
 // One workgroup per tile of DOK_TPB rows (kernels without counters) ...
-#ifndef DOK_GET_GRID_CAP
-#define DOK_GET_GRID_CAP 0
-#endif
-inline unsigned grid_for(i64 n) {
-  const i64 tiles = (n + DOK_TPB - 1) / DOK_TPB;
-  if (DOK_GET_GRID_CAP > 0 && tiles > DOK_GET_GRID_CAP) return DOK_GET_GRID_CAP;
-  return (unsigned)tiles;
-}
+inline unsigned grid_for(i64 n) { return (unsigned)((n + DOK_TPB - 1) / DOK_TPB); }
 // ... or a fixed grid that fills the machine (8 workgroups on each of 256 CUs) and loops over the
 // tiles, for kernels that end with per-wave atomics on the table header.
-#ifndef DOK_COUNT_GRID
 #define DOK_COUNT_GRID 2048
-#endif
 inline unsigned grid_counting(i64 n) {
   const i64 tiles = (n + DOK_TPB - 1) / DOK_TPB;
   return (unsigned)(tiles < DOK_COUNT_GRID ? tiles : DOK_COUNT_GRID);
@@ -261,8 +253,10 @@ int dok_table_clear(const dok_table_t *t, void *stream) {
   return note_launch();
 }
 
-int dok_map_get(const dok_table_t *t, const void *keys, int64_t n, void *values_out,
-                const void *fallback, uint8_t *found, void *stream) {
+// Shared body of the get entry points.  fallback: host pointer (NULL = zeros); fb_dev: device
+// pointer that the kernel reads instead.
+static int map_get(const dok_table_t *t, const void *keys, int64_t n, void *values_out, const void *fallback,
+                   const void *fb_dev, uint8_t *found, bool stats, void *stream) {
   DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
@@ -272,33 +266,34 @@ int dok_map_get(const dok_table_t *t, const void *keys, int64_t n, void *values_
   hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
   if (layout == DOK_LAYOUT_PACKED8) {
+    if (fb_dev && ((uintptr_t)fb_dev & (uintptr_t)(d.value_bytes - 1)) != 0) return DOK_EINVAL;
     const u64 fb = fallback_word(fallback, d.value_bytes);
-    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, false, KF><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
+    if (stats) {
+      P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, true, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb, fb_dev)));
+    } else {
+      P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, false, KF><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb, fb_dev)));
+    }
   } else {
-    rc = tg_launch_get(d, keys, n, values_out, fallback, found, false, s);
+    rc = tg_launch_get(d, keys, n, values_out, fallback, fb_dev, found, stats, s);
     if (rc) return rc;
   }
   return note_launch();
 }
 
+int dok_map_get(const dok_table_t *t, const void *keys, int64_t n, void *values_out,
+                const void *fallback, uint8_t *found, void *stream) {
+  return map_get(t, keys, n, values_out, fallback, nullptr, found, false, stream);
+}
+
+int dok_map_get_dev_fallback(const dok_table_t *t, const void *keys, int64_t n, void *values_out,
+                             const void *fallback_dev, uint8_t *found, void *stream) {
+  if (!fallback_dev) return DOK_EINVAL;
+  return map_get(t, keys, n, values_out, nullptr, fallback_dev, found, false, stream);
+}
+
 int dok_map_get_stats(const dok_table_t *t, const void *keys, int64_t n, void *values_out,
                       const void *fallback, uint8_t *found, void *stream) {
-  DevTable d; int layout;
-  int rc = make_dev_table(t, d, layout);
-  if (rc) return rc;
-  if (n < 0 || n > kMaxRows) return DOK_EINVAL;
-  if (n == 0) return DOK_OK;
-  if (!keys || !values_out || !found) return DOK_EINVAL;
-  hipStream_t s = (hipStream_t)stream;
-  const DeviceScope on_stream_device(s);
-  if (layout == DOK_LAYOUT_PACKED8) {
-    const u64 fb = fallback_word(fallback, d.value_bytes);
-    P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, true, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb)));
-  } else {
-    rc = tg_launch_get(d, keys, n, values_out, fallback, found, true, s);
-    if (rc) return rc;
-  }
-  return note_launch();
+  return map_get(t, keys, n, values_out, fallback, nullptr, found, true, stream);
 }
 
 int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int64_t n,

@@ -117,7 +117,16 @@ int dok_table_clear(const dok_table_t *t, void *stream);
 int dok_map_get(const dok_table_t *t, const void *keys, int64_t n,
                 void *values_out, const void *fallback, uint8_t *found, void *stream);
 
-/* Same, and adds the buckets visited / rows processed to header[DOK_H_NPROBE/NOPS]. */
+/* dok_map_get with the fallback row in DEVICE memory (value_bytes bytes, aligned like a value
+ * row; never NULL): the kernel reads it, so the host neither copies nor synchronises, and a call
+ * captured into a HIP graph sees the row's current contents at every replay.
+ * Reference: the `fallback` array argument of closed_hashmap_get (closed_hashmap_impl.cu:7-23),
+ * a device tensor made by ClosedHashmapImplCuda.get (closed_hashmap_impl.py:103-109). */
+int dok_map_get_dev_fallback(const dok_table_t *t, const void *keys, int64_t n,
+                             void *values_out, const void *fallback_dev, uint8_t *found,
+                             void *stream);
+
+/* Same as dok_map_get, and adds the buckets visited / rows processed to header[DOK_H_NPROBE/NOPS]. */
 int dok_map_get_stats(const dok_table_t *t, const void *keys, int64_t n,
                       void *values_out, const void *fallback, uint8_t *found, void *stream);
 
@@ -203,17 +212,21 @@ int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out,
  * the library itself holds on every GPU it runs on (dok_static_scratch_bytes() returns that
  * size); the call allocates and frees nothing.  Same outputs, in the same order, as
  * dok_map_compact on the same table.
- *   - A table whose dok_compact_scratch_bytes exceeds that size (more than about 2^28 buckets) is
+ *   - A table whose dok_compact_scratch_bytes exceeds that size (more than 2^28 buckets) is
  *     refused with DOK_ETOOLARGE before anything is launched: use dok_map_compact.
  *   - All calls on one GPU share the one array: calls that may overlap (different streams,
  *     different host threads) race and must be ordered by the caller. */
-#define DOK_STATIC_SCRATCH_BYTES (8 << 20)
+#define DOK_STATIC_SCRATCH_BYTES ((8 << 20) + 256)
 int64_t dok_static_scratch_bytes(void);
 int dok_map_compact_static(const dok_table_t *t, void *keys_out, void *values_out,
                            int64_t capacity_rows, int64_t *count_out, void *stream);
 
-/* Re-insert every live entry of src into dst (same key/value widths; dst cleared by the
- * caller; dst may have another size, seed or lin_dims of equal volume).
+/* Re-insert every live entry of src into dst (same key/value widths; dst may have another size
+ * or seed).  dst must be EMPTY: cleared by the caller (dok_table_clear) and not written by anything
+ * else while the call runs.  On the multi-word layout the entries are placed without comparing
+ * keys (src holds no key twice, an empty dst none at all), so a dst that already holds entries
+ * would end up with keys stored twice and a wrong entry count; the packed layout happens to
+ * upsert, which callers must not rely on.
  * Reference: CudaClosedHashmap.rehash (cuda_closed_hashmap.py:456-468). */
 int dok_map_rehash(const dok_table_t *src, const dok_table_t *dst, void *stream);
 

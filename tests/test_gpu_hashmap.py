@@ -798,3 +798,107 @@ def test_raw_table_attributes_and_set_values(cuda):
     keys2, values2 = hm.items()
     look = dict(zip(keys2.flatten().tolist(), values2.flatten().tolist()))
     assert look[int(keys[0])] == 5.0 and look[int(keys[24])] == 6.0
+
+
+def _bytes_dict(keys, vals):
+    return {k.tobytes(): v.tobytes() for k, v in zip(np.ascontiguousarray(keys), np.ascontiguousarray(vals))}
+
+
+@pytest.mark.parametrize("kshape,vshape", [((1,), (1,)), ((3,), (5,))])
+def test_remove_tells_float_keys_apart_by_bit_pattern(cuda, kshape, vshape):
+    """The table's key identity is the key row's bytes.  `remove` must agree with it: a NaN key
+    given twice in one batch is ONE key (removed once, counted once), and -0.0 / +0.0 are TWO keys
+    (both removed) - `torch.unique` on the float values has both the other way round.  Checked
+    against a dict keyed by the rows' bytes, on the packed layout (one float32 per key) and on the
+    multi-word layout (float32[3] keys)."""
+    from doksparse_amd import CudaClosedHashmap
+    from doksparse_amd.closed_hashmap import unique_rows
+    nan = np.float32("nan")
+    width = kshape[0]
+    base = np.array([nan, 0.0, -0.0, 1.5, -2.0, np.inf, -np.inf], dtype=np.float32)
+    keys = np.stack([np.roll(base, s) for s in range(width)], axis=1)            # [7, width], distinct by bytes
+    rng = np.random.default_rng(3)
+    vals = rng.integers(1, 2**31, size=(keys.shape[0],) + vshape).astype(np.int64 if vshape[0] > 1 else np.int32)
+    hm = CudaClosedHashmap(n_buckets=64, device=cuda)
+    k, v = _to(cuda, keys, vals)
+    hm.set(k, v)
+    model = _bytes_dict(keys, vals)
+    assert hm.n_elements == len(model) == 7
+    got_v, got_f = hm.get(k)
+    assert bool(got_f.all()) and np.array_equal(got_v.cpu().numpy(), vals)
+
+    # the batch: the NaN row twice, both zeros, one absent key, one ordinary key twice
+    absent = np.full((1, width), 7.25, dtype=np.float32)
+    batch = np.concatenate([keys[0:1], keys[0:1], keys[1:2], keys[2:3], absent, keys[3:4], keys[3:4]])
+    uniq = unique_rows(torch.from_numpy(batch)).numpy()
+    assert uniq.shape[0] == 5                                                  # NaN once, -0.0 and +0.0 apart
+    assert len({r.tobytes() for r in uniq}) == 5
+    expect = np.array([r.tobytes() in model for r in uniq])
+    m = hm.remove(torch.from_numpy(batch).to(cuda))
+    assert np.array_equal(m.cpu().numpy(), expect)
+    for r in uniq:
+        model.pop(r.tobytes(), None)
+    assert hm.n_elements == len(model) == 3
+    rk, rv = hm.items()
+    assert _bytes_dict(rk.cpu().numpy().reshape(-1, width), rv.cpu().numpy()) == model
+    _, f = hm.get(k)
+    assert f.cpu().numpy().tolist() == [False, False, False, False, True, True, True]
+    # a batch holding a key twice that would cross the growth threshold: the exact count of distinct
+    # new keys (multi-word layout: a sort of the rows) goes by bit pattern as well
+    small = CudaClosedHashmap(n_buckets=8, device=cuda)
+    rep = np.concatenate([keys[0:1]] * 4 + [keys[1:3]] + [keys[0:1]] * 4)       # 3 distinct keys in 10 rows
+    small.set(torch.from_numpy(rep).to(cuda), torch.from_numpy(np.concatenate([vals[0:1]] * 4 + [vals[1:3]] + [vals[0:1]] * 4)).to(cuda))
+    assert small.n_elements == 3 and small.n_buckets == 8                       # 3 <= int(0.75 * 8): no growth
+
+
+@pytest.mark.parametrize("vshape,vdt", [((1,), np.float32), ((5,), np.int64), ((1,), np.int64), ((3,), np.int16)])
+def test_device_resident_fallback_row(cuda, vshape, vdt):
+    """A fallback row given as a device tensor is read by the kernel (dok_map_get_dev_fallback): same
+    results as the host-side fallback, and a captured get sees the row's contents at replay time."""
+    import ctypes
+    from doksparse_amd import CudaClosedHashmap, _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(17)
+    n = 5000
+    keys = _unique_i64(rng, 2 * n)
+    vals = rng.integers(-1000, 1000, size=(n,) + vshape).astype(vdt)
+    hm = CudaClosedHashmap(n_buckets=4 * n, device=cuda)
+    k, v = _to(cuda, keys[:n, None], vals)
+    hm.set(k, v)
+    q = torch.from_numpy(keys[rng.permutation(2 * n)][:, None]).to(cuda)
+    fb_host = (np.arange(vshape[0]) - 7).astype(vdt)
+    want_v, want_f = hm.get(q, fallback_value=torch.from_numpy(fb_host))        # a CPU tensor: passed by value
+    fb = torch.from_numpy(fb_host).to(cuda)
+    got_v, got_f = hm.get(q, fallback_value=fb)
+    assert torch.equal(got_f, want_f) and torch.equal(got_v, want_v)
+    assert bool((got_v[~got_f] == fb).all()) and int((~got_f).sum()) == n
+    # broadcast of a one-element device tensor over the value row
+    one = torch.tensor([-9], device=cuda, dtype=fb.dtype)
+    b_v, _ = hm.get(q, fallback_value=one)
+    assert bool((b_v[~got_f] == -9).all()) and torch.equal(b_v[got_f], want_v[got_f])
+    # captured: the row changes between replays
+    out_v = torch.zeros_like(want_v)
+    out_f = torch.zeros_like(want_f)
+    desc = ctypes.byref(hm._desc)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            assert lib.dok_map_get_dev_fallback(desc, q.data_ptr(), q.shape[0], out_v.data_ptr(), fb.data_ptr(),
+                                                out_f.data_ptr(), st) == 0
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(4):
+        out_v.zero_()
+        out_f.zero_()
+        if rep % 2 == 1:
+            fb.add_(100)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_f, want_f) and torch.equal(out_v[want_f], want_v[want_f])
+        assert bool((out_v[~want_f] == fb).all())
+        (torch.randn(1000, device=cuda) @ torch.randn(1000, device=cuda)).item()   # unrelated eager work
+    # a NULL device row is refused
+    assert lib.dok_map_get_dev_fallback(desc, q.data_ptr(), q.shape[0], out_v.data_ptr(), None, out_f.data_ptr(),
+                                        None) == _lib.DOK_EINVAL

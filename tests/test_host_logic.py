@@ -86,10 +86,12 @@ def test_bad_descriptors_are_rejected_without_a_launch():
 
 def test_static_compact_size_check_needs_no_gpu():
     lib = _lib.load()
-    assert lib.dok_static_scratch_bytes() == 8 << 20
+    assert lib.dok_static_scratch_bytes() == (8 << 20) + 256
     t = _lib.DokTable()
     t.buckets, t.header, t.key_bytes, t.value_bytes = 4096, 8192, 8, 4
-    t.n_phys_buckets = (1 << 28) + 256              # one chunk counter more than the scratch holds
+    t.n_phys_buckets = 1 << 28                      # the documented limit itself is served
+    assert lib.dok_compact_scratch_bytes(ctypes.byref(t)) <= lib.dok_static_scratch_bytes()
+    t.n_phys_buckets = (1 << 28) + 256 * 32         # more chunk counters than the scratch holds
     assert lib.dok_compact_scratch_bytes(ctypes.byref(t)) > lib.dok_static_scratch_bytes()
     assert lib.dok_map_compact_static(ctypes.byref(t), None, None, 0, 8, None) == _lib.DOK_ETOOLARGE
     with pytest.raises(ValueError):

@@ -41,7 +41,7 @@ def _compact_both(lib, hm, dev):
 def test_static_compact_matches_compact_on_two_calls(cuda, kshape, kdtype, vshape, vdtype):
     from doksparse_amd import CudaClosedHashmap, _lib
     lib = _lib.load()
-    assert lib.dok_static_scratch_bytes() == 8 << 20
+    assert lib.dok_static_scratch_bytes() == (8 << 20) + 256
     g = torch.Generator().manual_seed(77)
     # the second table is smaller: fewer chunks of the shared scratch are used than the first
     # call left written
@@ -77,7 +77,7 @@ def test_static_compact_refuses_a_table_beyond_its_scratch(cuda):
     # must return before it launches anything on the (much smaller) real table
     big = _lib.DokTable()
     ctypes.memmove(ctypes.byref(big), ctypes.byref(hm._desc), ctypes.sizeof(big))
-    big.n_phys_buckets = (1 << 28) + 256
+    big.n_phys_buckets = (1 << 28) + 256 * 32
     count = torch.zeros(1, device=cuda, dtype=torch.long)
     rc = lib.dok_map_compact_static(ctypes.byref(big), None, None, 0, count.data_ptr(), None)
     assert rc == _lib.DOK_ETOOLARGE
@@ -85,3 +85,36 @@ def test_static_compact_refuses_a_table_beyond_its_scratch(cuda):
         _lib.check(rc, "compact")
     torch.cuda.synchronize()
     assert hm.n_elements == 10
+
+
+def test_static_compact_allocates_no_device_memory(cuda):
+    """What the entry point is for: with the outputs allocated beforehand, calls of
+    dok_map_compact_static leave the device's free memory as it was (no hipMalloc, no hipFree, no
+    growth of torch's pool), while giving the right rows."""
+    from doksparse_amd import CudaClosedHashmap, _lib
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    lib = _lib.load()
+    n = 200_000
+    g = torch.Generator().manual_seed(78)
+    keys = torch.unique(torch.randint(0, 2**62, (n,), generator=g))[:, None].to(cuda)
+    n = keys.shape[0]
+    hm = CudaClosedHashmap(n_buckets=1 << 19, device=cuda)
+    hm.set(keys, torch.arange(n, device=cuda, dtype=torch.float32)[:, None])
+    assert hm.n_elements == n
+    desc, stream = ctypes.byref(hm._desc), _stream_ptr(cuda)
+    out_k = torch.zeros(n, 1, device=cuda, dtype=torch.long)
+    out_v = torch.zeros(n, 1, device=cuda, dtype=torch.float32)
+    count = torch.zeros(1, device=cuda, dtype=torch.long)
+    # warm-up: resolves the scratch symbol on this device and loads the kernels
+    assert lib.dok_map_compact_static(desc, out_k.data_ptr(), out_v.data_ptr(), n, count.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info(cuda)
+    reserved_before = torch.cuda.memory_reserved(cuda)
+    for _ in range(3):
+        out_k.zero_(); out_v.zero_(); count.zero_()          # (in place: no allocation)
+        assert lib.dok_map_compact_static(desc, out_k.data_ptr(), out_v.data_ptr(), n, count.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(cuda)
+    assert free_after == free_before and torch.cuda.memory_reserved(cuda) == reserved_before
+    assert int(count.item()) == n
+    assert torch.equal(torch.sort(out_k[:, 0]).values, torch.sort(keys[:, 0]).values)
