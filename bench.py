@@ -5,10 +5,12 @@ MI355X, load factors 0.5 and 0.9 (synthetic data).
 One "step" is one `get` of a 64M-query batch (50% hits drawn Zipf(1.1) over the stored keys,
 50% uniform misses) against the load-factor-0.5 table.  The JSON line also carries set
 throughput, the load-factor-0.9 figures, mean probe lengths, the HBM roofline of the get kernel
-and a CPU baseline (the reference algorithm restated in C, timed on this machine's cores over a
-bounded sample of the same workload).
+(`roofline.achieved` / `frac`: the bytes that crossed the HBM interface, from profiler counters,
+over the kernel's live duration), the other four benchmark configurations, the multi-word layout
+and the DOK indexing kernels at scale (`roofline.other_legs`), and a CPU baseline (the reference
+algorithm restated in C, timed on this machine's cores on the benchmark's own keys and queries).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--keys N] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--keys N] [--no-cpu] [--headline-only]
 """
 import argparse
 import ctypes
@@ -39,6 +41,15 @@ PROFILED = {
     "build_lf09": 5.124e9,
     "set_cas_lf05": 1.615e10,    # p8_set_kernel (one compare-and-swap per row)
     "remove_lf05": 5.688e9,      # p8_remove_kernel, half of the keys, plain-store tombstones
+    # bench.py --only-tagged (profiles/tagged_32M_f32x3_i64x5.txt), load factor 0.5
+    "tagged_set_lf05": 11.84e9,        # tg_set_kernel, 32M fresh float32[3] -> int64[5] rows
+    "tagged_overwrite_lf05": None,
+    "tagged_get_lf05": 6.07e9,         # tg_lookup_kernel<0, false, 8>, 32M queries
+    "tagged_remove_lf05": None,
+    # bench.py --only-dok (profiles/dok_indexing_50M_2d_f32.txt)
+    "dok_getitem_2p26": 10.69e9,       # p8_getitem_kernel<4>, 2^26 stored coordinates of a 2-D tensor
+    "dok_setitem_10M": 2.24e9,         # p8_setitem_kernel<4>, 10M coordinates, half of them new
+    "dok_readout": None,
 }
 # algorithmic bytes per op for 8-byte keys and 4-byte values: one 128-byte bucket line per op,
 # plus the batch row and the outputs
@@ -259,6 +270,7 @@ def other_configs(device):
     del del_me
     ms, dok = timed(lambda: SparseDOKTensor((10**6, 10**6), coords, vals, device=device))
     res["cfg4_construct_50M_ms"] = round(ms, 3)
+    res["cfg4_entries"] = int(lin.numel())
     rows = torch.randint(0, 10**6, (4096, 1), generator=gen, device=device)
     cols = torch.randint(0, 10**6, (1, 256), generator=gen, device=device)
     dok[rows, cols]
@@ -286,6 +298,7 @@ def other_configs(device):
     store = new_store()
     ms, dok = timed(lambda: SparseDOKTensor(size, coords, vals, device=device, storage=store))
     res["cfg5_construct_100M_ms"] = round(ms, 3)
+    res["cfg5_entries"] = int(lin.numel())
     i_list = torch.randint(0, 4096, (64,), generator=gen, device=device).tolist()
     idx = torch.randint(0, 64, (128, 1), generator=gen, device=device)
     mask = torch.tensor([True, False, True, True, False, False, True, False], device=device)
@@ -293,6 +306,7 @@ def other_configs(device):
         for i in i_list:
             dok[i, :512, idx, mask]
     gets()
+    res["cfg5_lookups_per_64_getitems"] = 64 * 512 * 128 * int(mask.sum().item())
     res["cfg5_64_getitems_ms"] = round(timed(gets)[0], 3)
     # the host's share: time to enqueue the 64 calls (selector normalisation, descriptor, launch),
     # without waiting for the GPU
@@ -347,6 +361,8 @@ def tagged_scale(device, n=32_000_000):
         probe = hm.probe_stats(q)
         r_avg, _ = time_kernel(rem, 1)
         assert hm.n_elements == n - n // 4
+        for nm, ms in (("set", s_avg), ("overwrite", o_avg), ("get", g_avg), ("remove", r_avg)):
+            res[f"tagged_{nm}_ms_{tag}"] = round(ms, 4)
         res[f"tagged_set_mops_{tag}"] = round(n / s_avg / 1e3, 1)
         res[f"tagged_overwrite_mops_{tag}"] = round(n / o_avg / 1e3, 1)
         res[f"tagged_get_mops_{tag}"] = round(n / g_avg / 1e3, 1)
@@ -410,6 +426,47 @@ def dok_scale(device):
     ro, _ = timed(lambda: hm.items_coo())
     res["dok_readout_ms"] = round(ro, 4)
     res["dok_entries"] = hm.n_elements
+    del dok, hm, coords, vals, lin, sc, sv, ix, keep
+    torch.cuda.empty_cache()
+    res.update(dok_wide_scale(device))
+    return res
+
+
+def dok_wide_scale(device, nnz=10_000_000, n_q=1 << 22):
+    """A tensor whose coordinates do not fit one 8-byte key, (2^40, 2^40), beside one of the same
+    content whose do, (2^20, 2^20): the same 10M entries (the small tensor's coordinates, spread
+    over 2^40 by a shift), construction, gather of 4M elements (half stored) and scatter of 4M
+    (half present, half new; no growth), through the Python API, best of 3."""
+    from doksparse_amd import SparseDOKTensor
+    res = {}
+    gen = torch.Generator(device=device)
+    gen.manual_seed(4040)
+    lin = torch.unique(torch.randint(0, 2**40, (nnz,), generator=gen, device=device))
+    lin = lin[torch.randperm(lin.numel(), generator=gen, device=device)]
+    small = torch.stack([lin >> 20, lin & 0xFFFFF])
+    vals = torch.randn(lin.numel(), generator=gen, device=device)
+    qs = torch.cat([small[:, : n_q // 2], torch.randint(0, 2**20, (2, n_q // 2), generator=gen, device=device)], dim=1)
+    qs = qs[:, torch.randperm(n_q, generator=gen, device=device)].contiguous()
+    sv = torch.randn(n_q, generator=gen, device=device)
+    for tag, size, shift in (("dok_lin", (2**20, 2**20), 0), ("dok_wide", (2**40, 2**40), 20)):
+        coords, q = (small << shift).contiguous(), (qs << shift).contiguous()
+        best = {"construct": 1e9, "getitem": 1e9, "setitem": 1e9}
+        for _ in range(3):
+            ms, dok = timed(lambda: SparseDOKTensor(size, coords, vals, device=device))
+            best["construct"] = min(best["construct"], ms)
+            dok.storage().rehash(4 * lin.numel())          # room for the scatter: no growth inside the timed call
+            got = dok[q[0], q[1]]
+            best["getitem"] = min(best["getitem"], timed(lambda: dok[q[0], q[1]])[0])
+            def scatter():
+                dok[q[0], q[1]] = sv
+            best["setitem"] = min(best["setitem"], timed(scatter)[0])
+            # (a coordinate the random half happens to hold twice keeps either of its two values)
+            assert int((dok[q[0], q[1]] != sv).sum().item()) <= 16
+            del dok
+        assert int((got != 0).sum().item()) >= n_q // 2
+        res[f"{tag}_construct_10M_ms"] = round(best["construct"], 4)
+        res[f"{tag}_getitem_4M_ms"] = round(best["getitem"], 4)
+        res[f"{tag}_setitem_4M_ms"] = round(best["setitem"], 4)
     return res
 
 
@@ -423,12 +480,15 @@ def main():
                     help="keys of the CPU baseline (default: the full configuration, a 2.7 GB host table)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--quick", action="store_true", help="skip the set and load-factor-0.9 legs")
-    ap.add_argument("--configs", action="store_true",
-                    help="also time the four non-headline configurations (reported under extra)")
-    ap.add_argument("--tagged", action="store_true",
-                    help="also time the tagged layout at 32M float32[3] -> int64[5] keys (reported under extra)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="skip the four non-headline configurations, the multi-word layout at 32M keys and "
+                         "the DOK indexing kernels at scale (all reported under roofline.other_legs / extra)")
+    ap.add_argument("--configs", action="store_true", help="(kept for old command lines: these legs now always run)")
+    ap.add_argument("--tagged", action="store_true", help="(kept for old command lines: this leg now always runs)")
     ap.add_argument("--only-tagged", action="store_true",
                     help="run nothing but the --tagged leg and print its figures (for profiling that leg)")
+    ap.add_argument("--only-wide", action="store_true",
+                    help="run nothing but the wide-tensor legs of --only-dok")
     ap.add_argument("--only-dok", action="store_true",
                     help="run nothing but the DOK indexing kernels at scale and print their figures (for profiling)")
     ap.add_argument("--calibrate", action="store_true",
@@ -448,6 +508,9 @@ def main():
     torch.cuda.set_device(device)
     if args.only_tagged:
         print(json.dumps({"extra": tagged_scale(device)}), flush=True)
+        return
+    if args.only_wide:
+        print(json.dumps({"extra": dok_wide_scale(device)}), flush=True)
         return
     if args.only_dok:
         print(json.dumps({"extra": dok_scale(device)}), flush=True)
@@ -638,19 +701,61 @@ def main():
         results["load_factor_09_physical"] = round(n / (hm9._n_phys * hm9._slots_per_bucket), 4)
         del hm9
 
-    if args.configs or args.tagged:
+    default_workload = n == (1 << 26)
+    legs = {}
+    if not args.headline_only and not args.quick:
         del keys, values, queries, out_v, out_f
         torch.cuda.empty_cache()
-    if args.configs:
-        results.update(other_configs(device))
-    if args.tagged:
-        results.update(tagged_scale(device))
+        # the other four configurations at API level (host time included): durations only
+        cfg = other_configs(device)
+        results.update(cfg)
+        for name, ms_key, ops in (("cfg1_set_65536", "cfg1_set_ms", 65536), ("cfg1_get_131072", "cfg1_get_ms", 131072),
+                                  ("cfg1_remove_32768", "cfg1_remove_ms", 32768),
+                                  ("cfg2_set_1M_f32x3_i64x5", "cfg2_set_ms", 1_000_000),
+                                  ("cfg2_get_2M", "cfg2_get_ms", 2_000_000), ("cfg2_remove_250K", "cfg2_remove_ms", 250_000),
+                                  ("cfg4_construct_50M", "cfg4_construct_50M_ms", cfg["cfg4_entries"]),
+                                  ("cfg4_getitem_4096x256", "cfg4_getitem_4096x256_ms", 4096 * 256),
+                                  ("cfg4_setitem_10M_with_growth", "cfg4_setitem_10M_ms", 10_000_000),
+                                  ("cfg4_setitem_10M_overwrite", "cfg4_setitem_10M_again_ms", 10_000_000),
+                                  ("cfg5_construct_100M", "cfg5_construct_100M_ms", cfg["cfg5_entries"]),
+                                  ("cfg5_64_getitems", "cfg5_64_getitems_ms", cfg["cfg5_lookups_per_64_getitems"]),
+                                  ("cfg5_remove_20M", "cfg5_remove_20M_ms", cfg["cfg5_entries"] // 5),
+                                  ("cfg5_reinsert_20M", "cfg5_reinsert_20M_ms", cfg["cfg5_entries"] // 5)):
+            legs[name] = {"ms": cfg[ms_key], "mops": round(ops / cfg[ms_key] / 1e3, 1), "level": "api"}
+        torch.cuda.empty_cache()
+        # the multi-word layout and the DOK indexing kernels at scale: kernel level, with profiled bytes
+        tg = tagged_scale(device)
+        results.update(tg)
+        nt = tg["tagged_keys"]
+        torch.cuda.empty_cache()
+        dk = dok_scale(device)
+        results.update(dk)
+        for name, entry, ms, ops in (
+                ("tagged_set_32M_lf05", "tagged_set_lf05", tg["tagged_set_ms_lf05"], nt),
+                ("tagged_overwrite_32M_lf05", "tagged_overwrite_lf05", tg["tagged_overwrite_ms_lf05"], nt),
+                ("tagged_get_32M_lf05", "tagged_get_lf05", tg["tagged_get_ms_lf05"], nt),
+                ("tagged_remove_8M_lf05", "tagged_remove_lf05", tg["tagged_remove_ms_lf05"], nt // 4),
+                ("tagged_set_32M_lf075", None, tg["tagged_set_ms_lf075"], nt),
+                ("tagged_get_32M_lf075", None, tg["tagged_get_ms_lf075"], nt),
+                ("dok_getitem_2p26", "dok_getitem_2p26", dk["dok_getitem_2p26_ms"], 1 << 26),
+                ("dok_setitem_10M", "dok_setitem_10M", dk["dok_setitem_10M_ms"], 10_000_000),
+                ("dok_readout_55M", "dok_readout", dk["dok_readout_ms"], dk["dok_entries"]),
+                ("dok_lin_2p20x2p20_getitem_4M", None, dk.get("dok_lin_getitem_4M_ms"), 1 << 22),
+                ("dok_lin_2p20x2p20_setitem_4M", None, dk.get("dok_lin_setitem_4M_ms"), 1 << 22),
+                ("dok_lin_2p20x2p20_construct_10M", None, dk.get("dok_lin_construct_10M_ms"), 10_000_000),
+                ("dok_wide_2p40x2p40_getitem_4M", None, dk.get("dok_wide_getitem_4M_ms"), 1 << 22),
+                ("dok_wide_2p40x2p40_setitem_4M", None, dk.get("dok_wide_setitem_4M_ms"), 1 << 22),
+                ("dok_wide_2p40x2p40_construct_10M", None, dk.get("dok_wide_construct_10M_ms"), 10_000_000)):
+            if ms is None:
+                continue
+            m = measured(entry, ms) if entry else None
+            legs[name] = {"ms": ms, "mops": round(ops / ms / 1e3, 1), "level": "kernel",
+                          "traffic": m and m["traffic"], "bytes_per_op": m and round(m["traffic"] / ops, 1),
+                          "measured_gbs": m and m["gbs"], "frac_measured": m and m["frac"]}
 
-    achieved = n * B_GET / (k_avg * 1e-3) / 1e9
-    default_workload = n == (1 << 26)
+    line_model_gbs = n * B_GET / (k_avg * 1e-3) / 1e9
     m_get = measured("get_lf05", k_avg) if default_workload else None
     # the other legs the metric names, with measured HBM bytes (never a per-op model)
-    legs = {}
     if default_workload:
         for name, entry, ms_key, ops in (("get_lf09", "get_lf09", "get_kernel_ms_lf09", n),
                                          ("set_lf05", "set_bulk_lf05", "set_bulk_ms_lf05", n),
@@ -685,19 +790,22 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "achieved": round(achieved, 1),
+            # achieved / frac: the bytes that crossed the HBM interface per launch (rocprofv3
+            # FETCH_SIZE + WRITE_SIZE, `traffic`) over the kernel's live duration; null when no
+            # profile of the current kernel sources exists
+            "achieved": m_get and m_get["gbs"],
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "frac": m_get and m_get["frac"],
             "traffic": m_get and m_get["traffic"],
             "kernel": "p8_get_kernel<4, false, 0>",
-            "bytes_per_op": B_GET,
             "kernel_ms": round(k_avg, 4),
-            # `achieved` / `frac` count one 128-byte bucket line per query whether or not it came
-            # from HBM (the Zipf half of the batch is largely cache-resident); the two below are
-            # the bytes that did cross the HBM interface, from the counters
-            "measured_gbs": m_get and m_get["gbs"],
-            "frac_measured": m_get and m_get["frac"],
+            # the line-granular model: one 128-byte bucket line per query plus the batch row and the
+            # outputs, whether or not the line came from HBM (the Zipf half of the batch is largely
+            # cache-resident, so this exceeds what the memory interface carried)
+            "model_bytes_per_op": B_GET,
+            "line_model_gbs": round(line_model_gbs, 1),
+            "frac_line_model": round(line_model_gbs / HBM_PEAK_GBS, 4),
             # what this GPU reaches on uniformly random 128-byte lines of the same table
             "random_line_ceiling_gbs": results.get("line_gather_gbs_lf05"),
             "profiled_csrc_sha16": PROFILED["csrc_sha16"],

@@ -18,7 +18,8 @@ DOK_ELAUNCH = -3
 DOK_ETOOLARGE = -4
 
 DOK_BUCKET_BYTES = 128
-DOK_MAX_DIMS = 8
+DOK_MAX_DIMS = 14          # most dimensions of a coordinate table / an index space
+DOK_LIN_DIMS = 8           # ... of a table of linearised coordinates and of its index spaces
 DOK_HEADER_WORDS = 16
 DOK_H_NELEM = 0
 DOK_H_NFULL = 1

@@ -15,8 +15,10 @@ What differs underneath (and why callers do not see it):
 * The hash-constant keyword arguments are accepted and kept for ``get_hash`` / ``get_uuid`` /
   ``test_uniformity``; slot placement uses the library's own hash.
 * ``coord_dims`` (not in the reference) makes the map coordinate-keyed: key rows are int64
-  coordinates inside ``coord_dims`` and are stored as one linearised 8-byte key.  This is how
-  ``SparseDOKTensor`` uses the map.
+  coordinates inside ``coord_dims``.  They are stored as one linearised 8-byte key where that is
+  possible (at most 8 dimensions, fewer than 2^63 elements) and as the coordinate rows themselves,
+  on the multi-word layout, otherwise (`coord_rows_needed`).  This is how ``SparseDOKTensor``
+  uses the map.
 """
 import ctypes
 import math
@@ -26,7 +28,7 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from ._lib import DokTable, DOK_BUCKET_BYTES, DOK_HEADER_WORDS, DOK_MAX_DIMS
+from ._lib import DokTable, DOK_BUCKET_BYTES, DOK_HEADER_WORDS, DOK_MAX_DIMS, DOK_LIN_DIMS
 
 
 def _stream_ptr(device):
@@ -47,6 +49,15 @@ BULK_MIN_ROWS = 1 << 20
 BULK_MIN_ROWS_PER_BUCKET = 2.0
 BULK_MIN_ROWS_PER_BUCKET_LOADED = 1.5
 BULK_LOADED_FILL = 0.7
+
+
+def coord_rows_needed(dims):
+    """Whether coordinates inside `dims` have to be kept as int64 rows (multi-word keys) because one
+    8-byte linear key cannot hold them, or the table has more dimensions than linearised tables take."""
+    volume = 1
+    for s in dims:
+        volume *= max(int(s), 1)
+    return len(dims) > DOK_LIN_DIMS or volume >= 2**63
 
 
 def bulk_pays(n, n_phys, slots_per_bucket, n_upper):
@@ -159,6 +170,7 @@ class CudaClosedHashmap:
         rehash_threshold=0.75,
         coord_dims=None,
         seed=None,
+        coord_rows=None,
     ):
         self._st = _TableState()
         self._empty_marker = -1
@@ -177,6 +189,16 @@ class CudaClosedHashmap:
                 key_perm = torch.tensor(key_perm, dtype=torch.long, device=self.device)
             self._key_perm = key_perm.to(device=self.device, dtype=torch.long)
         self._coord_dims = None if coord_dims is None else tuple(int(d) for d in coord_dims)
+        if self._coord_dims is not None and len(self._coord_dims) > DOK_MAX_DIMS:
+            raise NotImplementedError(f"coordinate tables of more than {DOK_MAX_DIMS} dimensions: a coordinate "
+                                      "row no longer fits a 128-byte bucket")
+        # key format of a coordinate table: linearised (False) or int64 rows (True); None = rows only
+        # where a linear key cannot hold the coordinates
+        self._coord_rows = False
+        if self._coord_dims is not None:
+            need = coord_rows_needed(self._coord_dims)
+            assert coord_rows is None or coord_rows or not need, "these coordinates do not fit a linear key"
+            self._coord_rows = need or (bool(coord_rows) and len(self._coord_dims) >= 2)
         self._seed = int(seed) if seed is not None else int(np.random.randint(1, 2**62, dtype=np.int64))
 
         # physical state; the table itself is allocated at the first set(), when the key and
@@ -214,7 +236,7 @@ class CudaClosedHashmap:
         d.header = header.data_ptr()
         d.n_phys_buckets = n_phys
         d.seed = self._seed
-        d.key_bytes = 8 if self._coord_dims is not None else self._key_bytes
+        d.key_bytes = self._stored_key_bytes()
         d.value_bytes = self._value_bytes
         if self._coord_dims is not None:
             d.lin_ndim = len(self._coord_dims)
@@ -224,11 +246,18 @@ class CudaClosedHashmap:
             d.lin_ndim = 0
         return d
 
+    def _stored_key_bytes(self):
+        """Bytes of a key as the table stores it: a coordinate table linearises its rows into 8
+        bytes unless the coordinate space is too large for that."""
+        if self._coord_dims is not None and not self._coord_rows:
+            return 8
+        return self._key_bytes
+
     def _alloc_table(self, n_buckets, clear=True):
         """New table tensors and their descriptor.  clear=False leaves the memory uninitialised:
         only for a caller that clears it (_clear_table) or builds it in bulk right away."""
         lib = _lib.load()
-        kb = 8 if self._coord_dims is not None else self._key_bytes
+        kb = self._stored_key_bytes()
         slots = ctypes.c_int32(0)
         layout = lib.dok_layout_of(kb, self._value_bytes, ctypes.byref(slots))
         _lib.check(min(layout, 0), "CudaClosedHashmap")
@@ -611,9 +640,6 @@ class CudaClosedHashmap:
 
     def _set_coo_rows(self, indices, values):
         n = indices.shape[1]
-        if self._layout != _lib.DOK_LAYOUT_PACKED8:
-            self._ensure_cleared()
-            return self.set(indices.T, values)
         indices = self._prep_rows(indices, "indices")
         values = self._prep_rows(values, "values")
 
@@ -642,9 +668,6 @@ class CudaClosedHashmap:
         assert self._coord_dims is not None
         if not self._allocated:
             return None, None
-        if self._layout != _lib.DOK_LAYOUT_PACKED8:
-            keys, values = self.items()
-            return keys.T.contiguous(), values
         lib = _lib.load()
         scratch = torch.empty(int(lib.dok_compact_scratch_bytes(ctypes.byref(self._desc))) // 8,
                               device=self.device, dtype=torch.long)
@@ -667,9 +690,15 @@ class CudaClosedHashmap:
         if n == 0:
             return 0
         if self._layout != _lib.DOK_LAYOUT_PACKED8:
+            if self._coord_dims is not None:
+                # rows outside the coordinate space are skipped by the insert
+                dims = torch.tensor(self._coord_dims, device=keys.device, dtype=torch.long)
+                keys = keys[((keys >= 0) & (keys < dims)).all(dim=1)]
+                if keys.shape[0] == 0:
+                    return 0
             return int(unique_rows(keys).shape[0])        # distinct by bit pattern, as the table sees them
         lib = _lib.load()
-        kb = 8 if self._coord_dims is not None else self._key_bytes
+        kb = self._stored_key_bytes()
         n_phys = int(lib.dok_phys_buckets_for(2 * n, kb, 1))
         table = torch.empty(n_phys * DOK_BUCKET_BYTES, device=self.device, dtype=torch.uint8)
         header = torch.empty(DOK_HEADER_WORDS, device=self.device, dtype=torch.long)
@@ -851,7 +880,7 @@ class CudaClosedHashmap:
             prime1=self._prime1, prime2=self._prime2, alpha1=self._alpha1, alpha2=self._alpha2,
             beta1=self._beta1, beta2=self._beta2, key_perm=self._key_perm,
             rehash_factor=self._rehash_factor, rehash_threshold=self._rehash_threshold,
-            coord_dims=self._coord_dims, seed=self._seed,
+            coord_dims=self._coord_dims, seed=self._seed, coord_rows=self._coord_rows or None,
         )
         if not deepclone:
             new._st = self._st

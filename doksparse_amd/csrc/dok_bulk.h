@@ -1251,7 +1251,7 @@ template <int V, int KF, bool FRESH = false>
 static void bulk_launch(const DevTable &d, const void *keys, const void *values, i64 n, const BulkPlan &p,
                         void *workspace, hipStream_t s) {
   if constexpr (KF == DOK_KF_COLS || KF == DOK_KF_ROWS) {
-    switch (d.lin_ndim) {                              // 1 .. DOK_MAX_DIMS, checked with the descriptor
+    switch (d.lin_ndim) {                              // 1 .. DOK_LIN_DIMS, checked with the descriptor
       case 1: return bulk_launch_nd<V, KF, 1, FRESH>(d, keys, values, n, p, workspace, s);
       case 2: return bulk_launch_nd<V, KF, 2, FRESH>(d, keys, values, n, p, workspace, s);
       case 3: return bulk_launch_nd<V, KF, 3, FRESH>(d, keys, values, n, p, workspace, s);

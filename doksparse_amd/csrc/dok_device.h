@@ -20,6 +20,11 @@ typedef unsigned char u8;
 
 #define DOK_TPB 256          // threads per workgroup
 #define DOK_NONE32 0xffffffffu
+// Most dimensions of a coordinate table whose keys are LINEARISED coordinates (one 8-byte key on
+// the packed layout), and of the index spaces its fused indexing kernels take: their descriptor
+// arrays have this many entries and their loops unroll to it.  Tables of more dimensions (up to
+// DOK_MAX_DIMS), or of 2^63 elements and more, keep their coordinates as multi-word keys.
+#define DOK_LIN_DIMS 8
 
 // Batch kernels walk the rows in tiles of DOK_TPB; a workgroup takes tiles blockIdx.x,
 // blockIdx.x + gridDim.x, ...  The host launches one workgroup per tile for kernels without
@@ -41,10 +46,10 @@ struct DevTable {
   int value_bytes;
   int lin_ndim;
   int pad_;
-  i64 lin_dims[DOK_MAX_DIMS];
-  i64 lin_strides[DOK_MAX_DIMS];   // row-major strides of lin_dims
-  u64 lin_magic[DOK_MAX_DIMS];     // division by lin_strides[d] as multiply + shift (dok_div_stride);
-  int lin_shift[DOK_MAX_DIMS];     // set by the host for strides above 1
+  i64 lin_dims[DOK_MAX_DIMS];        // (a multi-word coordinate table uses all of them)
+  i64 lin_strides[DOK_LIN_DIMS];   // row-major strides of lin_dims
+  u64 lin_magic[DOK_LIN_DIMS];     // division by lin_strides[d] as multiply + shift (dok_div_stride);
+  int lin_shift[DOK_LIN_DIMS];     // set by the host for strides above 1
 };
 
 // n / d for the stride d that (magic, shift) were made for (host: div_magic in dokhip.hip).  The
@@ -61,13 +66,13 @@ struct DevIndex {
   int ndim;
   int sel_ndim;
   i64 n_elems;
-  i64 shape[DOK_MAX_DIMS];
-  i64 estride[DOK_MAX_DIMS];       // C-contiguous strides of `shape`
-  const i64 *sel[DOK_MAX_DIMS];              // NULL: the coordinate is sbase + offset itself
-  i64 sbase[DOK_MAX_DIMS];
-  i64 sstride[DOK_MAX_DIMS][DOK_MAX_DIMS];
+  i64 shape[DOK_LIN_DIMS];
+  i64 estride[DOK_LIN_DIMS];       // C-contiguous strides of `shape`
+  const i64 *sel[DOK_LIN_DIMS];              // NULL: the coordinate is sbase + offset itself
+  i64 sbase[DOK_LIN_DIMS];
+  i64 sstride[DOK_LIN_DIMS][DOK_LIN_DIMS];
   const void *src;
-  i64 vstride[DOK_MAX_DIMS];
+  i64 vstride[DOK_LIN_DIMS];
 };
 
 __device__ __forceinline__ u64 dok_fmix64(u64 x) {
@@ -188,16 +193,16 @@ __global__ __launch_bounds__(DOK_TPB) void dok_line_gather_kernel(const u64 *__r
 // streaming kernels of the bulk path, where the loads of many rows must overlap, have a loader
 // of their own.)
 __device__ __forceinline__ bool dok_linearise(const DevTable &t, const i64 *row, u64 &key) {
-  i64 c[DOK_MAX_DIMS];
+  i64 c[DOK_LIN_DIMS];
   #pragma unroll
-  for (int d = 0; d < DOK_MAX_DIMS; d++) {
+  for (int d = 0; d < DOK_LIN_DIMS; d++) {
     c[d] = 0;
     if (d < t.lin_ndim) c[d] = row[d];               // loads only: they overlap
   }
   bool ok = true;
   u64 k = 0;
   #pragma unroll
-  for (int d = 0; d < DOK_MAX_DIMS; d++) {
+  for (int d = 0; d < DOK_LIN_DIMS; d++) {
     if (d < t.lin_ndim) {
       ok = ok && ((u64)c[d] < (u64)t.lin_dims[d]);
       k += (u64)c[d] * (u64)t.lin_strides[d];
@@ -225,16 +230,16 @@ __device__ __forceinline__ bool dok_load_key8(const DevTable &t, const void *key
   if (KF == DOK_KF_ROWS) return dok_linearise(t, (const i64 *)keys + i * t.lin_ndim, key);
   if (KF == DOK_KF_U64) { key = ((const u64 *)keys)[i]; return true; }
   if (KF == DOK_KF_COLS) {
-    i64 c[DOK_MAX_DIMS];
+    i64 c[DOK_LIN_DIMS];
     #pragma unroll
-    for (int d = 0; d < DOK_MAX_DIMS; d++) {
+    for (int d = 0; d < DOK_LIN_DIMS; d++) {
       c[d] = 0;
       if (d < t.lin_ndim) c[d] = ((const i64 *)keys)[(i64)d * n + i];
     }
     bool ok = true;
     u64 k = 0;
     #pragma unroll
-    for (int d = 0; d < DOK_MAX_DIMS; d++) {
+    for (int d = 0; d < DOK_LIN_DIMS; d++) {
       if (d < t.lin_ndim) {
         ok = ok && ((u64)c[d] < (u64)t.lin_dims[d]);
         k += (u64)c[d] * (u64)t.lin_strides[d];
@@ -293,17 +298,17 @@ template <int V> __device__ __forceinline__ void dok_store_val(void *values, i64
 // maximum with uniform guards so that idx[] stays in registers; the host zeroes the strides of
 // unused axes.
 __device__ __forceinline__ bool dok_gather_at(const DevTable &t, const DevIndex &ix,
-                                              const i64 (&idx)[DOK_MAX_DIMS], u64 &key, i64 &voff) {
+                                              const i64 (&idx)[DOK_LIN_DIMS], u64 &key, i64 &voff) {
   // first every dimension's selector is read, then the values are used: a use next to its load
   // would make the loads of the dimensions wait for one another
-  i64 g[DOK_MAX_DIMS];
+  i64 g[DOK_LIN_DIMS];
   #pragma unroll
-  for (int d = 0; d < DOK_MAX_DIMS; d++) {
+  for (int d = 0; d < DOK_LIN_DIMS; d++) {
     g[d] = 0;
     if (d < ix.ndim) {
       i64 off = 0;
       #pragma unroll
-      for (int j = 0; j < DOK_MAX_DIMS; j++)
+      for (int j = 0; j < DOK_LIN_DIMS; j++)
         if (j < ix.sel_ndim) off += idx[j] * ix.sstride[d][j];
       const i64 *sp = ix.sel[d];
       g[d] = off;
@@ -313,7 +318,7 @@ __device__ __forceinline__ bool dok_gather_at(const DevTable &t, const DevIndex 
   bool ok = true;
   u64 k = 0;
   #pragma unroll
-  for (int d = 0; d < DOK_MAX_DIMS; d++) {
+  for (int d = 0; d < DOK_LIN_DIMS; d++) {
     if (d < ix.ndim) {
       const i64 c = ix.sbase[d] + g[d];
       ok = ok && ((u64)c < (u64)t.lin_dims[d]);
@@ -322,7 +327,7 @@ __device__ __forceinline__ bool dok_gather_at(const DevTable &t, const DevIndex 
   }
   i64 vo = 0;
   #pragma unroll
-  for (int j = 0; j < DOK_MAX_DIMS; j++)
+  for (int j = 0; j < DOK_LIN_DIMS; j++)
     if (j < ix.sel_ndim) vo += idx[j] * ix.vstride[j];
   voff = vo;
   key = k;
@@ -332,11 +337,11 @@ __device__ __forceinline__ bool dok_gather_at(const DevTable &t, const DevIndex 
 // The same for element e (row-major offset) of the index space: unravel e over `shape` first.
 __device__ __forceinline__ bool dok_gather_key(const DevTable &t, const DevIndex &ix, i64 e,
                                                u64 &key, i64 &voff) {
-  i64 idx[DOK_MAX_DIMS];
+  i64 idx[DOK_LIN_DIMS];
   if (ix.n_elems <= 0x7fffffffLL) {
     u32 rem = (u32)e;
     #pragma unroll
-    for (int j = 0; j < DOK_MAX_DIMS; j++) {
+    for (int j = 0; j < DOK_LIN_DIMS; j++) {
       idx[j] = 0;
       if (j < ix.sel_ndim) {
         u32 s = (u32)ix.estride[j];
@@ -348,7 +353,7 @@ __device__ __forceinline__ bool dok_gather_key(const DevTable &t, const DevIndex
   } else {
     u64 rem = (u64)e;
     #pragma unroll
-    for (int j = 0; j < DOK_MAX_DIMS; j++) {
+    for (int j = 0; j < DOK_LIN_DIMS; j++) {
       idx[j] = 0;
       if (j < ix.sel_ndim) {
         u64 s = (u64)ix.estride[j];

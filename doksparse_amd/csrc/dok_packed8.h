@@ -1017,10 +1017,10 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void p8_setitem_sparse_k
                                                                     i64 n_src, u64 nonzero_mask,
                                                                     i64 rows_per_wave) {
   p8_stream_insert<V>(t, n_src, rows_per_wave, nullptr, [&](i64 k, u64 &key, u64 &val) -> int {
-    i64 idx[DOK_MAX_DIMS];
+    i64 idx[DOK_LIN_DIMS];
     bool inside = true;
     #pragma unroll
-    for (int j = 0; j < DOK_MAX_DIMS; j++) {
+    for (int j = 0; j < DOK_LIN_DIMS; j++) {
       idx[j] = 0;
       if (j < ix.sel_ndim) {
         idx[j] = src_indices[(i64)j * n_src + k];

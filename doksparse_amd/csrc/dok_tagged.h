@@ -32,6 +32,7 @@
 // workgroup, so that any lane of a group can fetch "word p of the row being served".
 #pragma once
 #include "dok_device.h"
+#include "dok_packed8.h"
 
 #define DOK_TG_EMPTY 0u
 #define DOK_TG_TOMB  1u
@@ -81,6 +82,149 @@ __device__ __forceinline__ void tg_store_word(u8 *row, int k, int nbytes, int un
       if (base + q < nbytes) row[base + q] = (u8)(w >> (8 * q));
   }
 }
+
+// ---- where the rows of a batch come from ---------------------------------------------------------
+// Every kernel of this layout stages the rows it works on in LDS (key words at krow[1 .. KW], value
+// words at vrow[0 .. VW)); a *row source* says how row i gets there.  stage() returns 0 = a row,
+// 1 = the row addresses nothing inside the table's coordinate space (set kernels count it in
+// header[DOK_H_NOOB]; lookups treat it as absent), 2 = skip the row silently.  vrow may be NULL
+// (lookups).  A table with lin_ndim > 0 holds int64 coordinate rows - the key format of the
+// reference's SparseDOKTensor (sparse_dok_tensor.py:45-69) - and its sources check every
+// coordinate against lin_dims.
+
+// Key rows and value rows as contiguous byte rows: the batched map entry points.
+struct TgRows {
+  const u8 *keys, *values;
+  __device__ __forceinline__ int stage(const DevTable &t, const TgGeom &g, i64 i, u64 *krow, u64 *vrow) const {
+    const u8 *kin = keys + (size_t)i * g.K;
+    for (int k = 0; k < g.KW; k++) krow[1 + k] = tg_load_word(kin, k, g.K, g.unit_k);
+    if (vrow) {
+      const u8 *vin = values + (size_t)i * g.V;
+      for (int k = 0; k < g.VW; k++) vrow[k] = tg_load_word(vin, k, g.V, g.unit_v);
+    }
+    bool ok = true;
+    for (int d = 0; d < t.lin_ndim; d++) ok = ok && krow[1 + d] < (u64)t.lin_dims[d];
+    return ok ? 0 : 1;
+  }
+};
+
+// Coordinates the way a COO tensor holds them: indices[d * n + i]; values[i] (coordinate tables).
+struct TgCols {
+  const i64 *indices;
+  i64 n;
+  const u8 *values;
+  __device__ __forceinline__ int stage(const DevTable &t, const TgGeom &g, i64 i, u64 *krow, u64 *vrow) const {
+    bool ok = true;
+    for (int d0 = 0; d0 < g.KW; d0 += 4) {
+      u64 c[4];
+      #pragma unroll
+      for (int u = 0; u < 4; u++) { c[u] = 0; if (d0 + u < g.KW) c[u] = (u64)indices[(i64)(d0 + u) * n + i]; }   // loads first
+      #pragma unroll
+      for (int u = 0; u < 4; u++)
+        if (d0 + u < g.KW) { krow[1 + d0 + u] = c[u]; ok = ok && c[u] < (u64)t.lin_dims[d0 + u]; }
+    }
+    if (vrow)
+      for (int k = 0; k < g.VW; k++) vrow[k] = tg_load_word(values + (size_t)i * g.V, k, g.V, g.unit_v);
+    return ok ? 0 : 1;
+  }
+};
+
+// Kernel-argument form of dok_index_t for tables of up to DOK_MAX_DIMS dimensions (+ optional
+// source-value view, + the source entries of a sparse-valued scatter).
+struct DevIndexW {
+  int ndim, sel_ndim;
+  i64 n_elems;
+  i64 shape[DOK_MAX_DIMS];
+  i64 estride[DOK_MAX_DIMS];       // C-contiguous strides of `shape`
+  const i64 *sel[DOK_MAX_DIMS];    // NULL: the coordinate is sbase + offset itself
+  i64 sbase[DOK_MAX_DIMS];
+  i64 sstride[DOK_MAX_DIMS][DOK_MAX_DIMS];
+  const void *src;
+  i64 vstride[DOK_MAX_DIMS];
+};
+
+// The selectors applied: on entry krow[1 + d] holds the element offset into dimension d's selector,
+// on exit the coordinate.  Four dimensions at a time, their loads issued before the first is used.
+__device__ __forceinline__ bool tg_apply_selectors(const DevTable &t, const DevIndexW &ix, u64 *krow) {
+  bool ok = true;
+  for (int d0 = 0; d0 < ix.ndim; d0 += 4) {
+    i64 c[4];
+    #pragma unroll
+    for (int u = 0; u < 4; u++) {
+      c[u] = 0;
+      if (d0 + u < ix.ndim) {
+        const i64 off = (i64)krow[1 + d0 + u];
+        const i64 *sp = ix.sel[d0 + u];
+        c[u] = sp ? sp[off] : off;
+      }
+    }
+    #pragma unroll
+    for (int u = 0; u < 4; u++) {
+      if (d0 + u < ix.ndim) {
+        const i64 x = c[u] + ix.sbase[d0 + u];
+        ok = ok && (u64)x < (u64)t.lin_dims[d0 + u];
+        krow[1 + d0 + u] = (u64)x;
+      }
+    }
+  }
+  return ok;
+}
+
+// Element e of the broadcast index space of an indexing expression: the fused form of the
+// reference's stack + transpose of the broadcast selectors (sparse_dok_tensor.py:302-311) and of the
+// accessor arithmetic of its DOK kernels (tensor_accessor.cu:50-87).  e is unravelled over the index
+// space; the offsets into the selectors accumulate in the row's own LDS words (the number of
+// dimensions is a run-time value here, and registers cannot be indexed by one).
+struct TgIndexSrc {
+  DevIndexW ix;
+  __device__ __forceinline__ int stage(const DevTable &t, const TgGeom &g, i64 e, u64 *krow, u64 *vrow) const {
+    for (int d = 0; d < ix.ndim; d++) krow[1 + d] = 0;
+    i64 vo = 0;
+    u64 rem = (u64)e;
+    const bool small = ix.n_elems <= 0x7fffffffLL;
+    for (int j = 0; j < ix.sel_ndim; j++) {
+      u64 q;
+      if (small) { const u32 st = (u32)ix.estride[j]; const u32 q32 = (u32)rem / st; rem = (u32)rem - q32 * st; q = q32; }
+      else { const u64 st = (u64)ix.estride[j]; q = rem / st; rem -= q * st; }
+      vo += (i64)q * ix.vstride[j];
+      for (int d = 0; d < ix.ndim; d++) {
+        const i64 st = ix.sstride[d][j];
+        if (st) krow[1 + d] += q * (u64)st;          // (most strides are 0: a selector varies along few axes)
+      }
+    }
+    const bool ok = tg_apply_selectors(t, ix, krow);
+    if (vrow) vrow[0] = tg_load_word((const u8 *)ix.src + (size_t)vo * g.V, 0, g.V, g.V);
+    return ok ? 0 : 1;
+  }
+};
+
+// Source entry k of a sparse-valued scatter: index vector src_indices[j * n_src + k] over the axes of
+// the index space, value src_values[k]; entries that are zero under nonzero_mask are skipped
+// (reference: sparse_dok_set_items_sparse_v1, sparse_dok_tensor_impl.cu:163-211).
+struct TgSparseSrc {
+  DevIndexW ix;
+  const i64 *src_indices;
+  const u8 *src_values;
+  i64 n_src;
+  u64 nonzero_mask;
+  __device__ __forceinline__ int stage(const DevTable &t, const TgGeom &g, i64 k, u64 *krow, u64 *vrow) const {
+    const u64 val = tg_load_word(src_values + (size_t)k * g.V, 0, g.V, g.V);
+    if ((val & nonzero_mask) == 0) return 2;
+    for (int d = 0; d < ix.ndim; d++) krow[1 + d] = 0;
+    bool inside = true;
+    for (int j = 0; j < ix.sel_ndim; j++) {
+      const u64 q = (u64)src_indices[(i64)j * n_src + k];
+      inside = inside && q < (u64)ix.shape[j];
+      for (int d = 0; d < ix.ndim; d++) {
+        const i64 st = ix.sstride[d][j];
+        if (st) krow[1 + d] += q * (u64)st;
+      }
+    }
+    if (!inside) return 1;                            // (before any selector is read at such an offset)
+    if (vrow) vrow[0] = val;
+    return tg_apply_selectors(t, ix, krow) ? 0 : 1;
+  }
+};
 
 // LDS row of a staged batch row: word 0 = the row's FULL tag (low half), words 1 .. KW = the
 // zero-padded key words - exactly what the tag lane and the key lanes of a matching slot hold, so
@@ -169,10 +313,14 @@ __device__ __forceinline__ u32 tg_wrap(u32 home, u32 d, u64 nb) {
 // UV: the access granule of the value rows (8 or 4) as a compile-time constant, or 0 = g.unit_v:
 // with it each of the 16 unrolled rounds carries one store instead of a switch over the four
 // granules (4 % at 16M lookups of 40-byte values).
-template <int MODE, bool STATS, int UV = 0>
-__global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g, const u8 *__restrict__ keys, i64 n,
-                                                            u8 *__restrict__ values, u8 *__restrict__ flags,
-                                                            i64 *count, const u8 *__restrict__ fallback_dev = nullptr) {
+// MODE 4 (sparse-valued gather): as get, but the value of every row found goes, under the key i,
+// into `out`, a packed table of VP-byte values (i = the element's offset in the index space).
+// Src: where the rows come from (see the row sources above).
+template <int MODE, bool STATS, int UV, class Src, int VP = 0>
+__device__ __forceinline__ void tg_lookup_body(const DevTable &t, const TgGeom &g, const Src &src, i64 n,
+                                               u8 *__restrict__ values, u8 *__restrict__ flags,
+                                               i64 *count, const u8 *__restrict__ fallback_dev,
+                                               const DevTable *out) {
   extern __shared__ u64 lds[];
   const int RS = tg_rs(g);
   u64 *lds_rows = lds;                          // [DOK_TPB][1 + KW]
@@ -180,7 +328,8 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
   u32 *lds_meta = (u32 *)(lds_fb + g.VW);       // [DOK_TPB][2]: metadata and filter of each row's home bucket
   u8 *lds_out = (u8 *)(lds_meta + DOK_TPB * 2); // [DOK_TPB][V]: the tile's output rows (get)
   // the fallback row: part of the geometry argument, or - fallback_dev set - read from device memory
-  if (MODE == 0 && threadIdx.x < g.VW)
+  constexpr bool VALUES = MODE == 0 || MODE == 4;   // the value rows of the hits are staged in lds_out
+  if (VALUES && threadIdx.x < g.VW)
     lds_fb[threadIdx.x] = fallback_dev ? tg_load_word(fallback_dev, threadIdx.x, g.V, UV ? UV : g.unit_v)
                                        : g.fallback[threadIdx.x];
   __syncthreads();
@@ -197,16 +346,14 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
   const bool has_filter = g.S >= 2;
   const bool meta_lane = L.l == 0 || (has_filter && L.l == g.W);
   u32 *meta_out = lds_meta + (wave_row0 + L.gbase) * 2 + (L.l != 0);   // round r: meta_out[2 * r]
-  int n_found = 0, n_removed = 0, n_probe = 0, n_ops = 0;
+  int n_found = 0, n_removed = 0, n_probe = 0, n_ops = 0, n_fresh = 0, n_full = 0;
 
   DOK_TILE_LOOP(n) {
     const i64 i = DOK_TILE_ROW();
-    const bool active = i < n;
+    const bool inside = i < n;                  // the tile's rows inside the batch
     u64 *krow = lds_rows + threadIdx.x * RS;
-    {
-      const u8 *row = keys + (size_t)i * g.K;
-      for (int k = 0; k < g.KW; k++) krow[1 + k] = active ? tg_load_word(row, k, g.K, g.unit_k) : 0;
-    }
+    // `active`: a row that is looked up (rows addressing nothing inside the coordinate space are absent)
+    const bool active = inside && src.stage(t, g, i, krow, nullptr) == 0;
     u32 home, qfull;
     tg_hash_row(t, g, krow, home, qfull);
     if (!active) home = 0;
@@ -215,6 +362,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
     u64 my_hit64 = 0;
 
     const u64 am = dok_ballot(active);
+    const u64 im = dok_ballot(inside);
     if (am != 0) {
       #pragma unroll
       for (int r0 = 0; r0 < 16; r0 += 8) {
@@ -231,7 +379,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
           const u64 tr = (am >> r) & 0x0001000100010001ULL;
           const u64 on64 = (tr << 16) - tr;
           const u64 hit64 = tg_match64(L, M, w[u], exp0[r * RS]) & on64;
-          if (MODE == 0 && L.is_val && ((hit64 >> tl) & 1ULL))
+          if (VALUES && L.is_val && ((hit64 >> tl) & 1ULL))
             tg_store_word(out_g + (size_t)r * g.V, L.p - 1 - g.KW, g.V, unit_v, w[u]);
           // the bucket's metadata and filter are left in LDS for the row's owner
           if (meta_lane) meta_out[2 * r] = (u32)(w[u] >> 32);
@@ -251,7 +399,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
       if (has_filter && !(lds_meta[threadIdx.x * 2 + 1] & tg_fbit(qfull))) my_meta = 0;
     }
     bool open = active && !found && my_meta != 0;
-    if (MODE == 0 && active && !found && !open) {
+    if (VALUES && inside && !found && !open) {
       for (int k = 0; k < g.VW; k++)
         tg_store_word(lds_out + (size_t)threadIdx.x * g.V, k, g.V, unit_v, lds_fb[k]);
     }
@@ -283,7 +431,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
       for (int k = 0; k < 4; k++) {
         const u64 hit64 = tg_match64(L, M, w[k], exp0[rr[k] * RS]) & dok_ballot(hs[k]);
         const u32 em = L.grp(dok_ballot(hs[k] && L.is_tag && (u32)w[k] == DOK_TG_EMPTY));
-        if (MODE == 0 && L.is_val && ((hit64 >> tl) & 1ULL))
+        if (VALUES && L.is_val && ((hit64 >> tl) & 1ULL))
           tg_store_word(out_g + (size_t)rr[k] * g.V, L.p - 1 - g.KW, g.V, unit_v, w[k]);
         const bool mine = hs[k] && L.l == rr[k];
         act = act || mine;
@@ -302,7 +450,7 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
             far_d++;
           }
           open = cand != 0 || (far && (far_max == DOK_TG_FARCAP ? (u64)far_d < t.nb : far_d <= far_max));
-          if (!open && MODE == 0) {
+          if (!open && VALUES) {
             for (int k = 0; k < g.VW; k++)
               tg_store_word(lds_out + (size_t)threadIdx.x * g.V, k, g.V, unit_v, lds_fb[k]);
           }
@@ -314,9 +462,9 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
     if (MODE == 2 && found)
       removed = atomicCAS((u32 *)(t.buckets + (u64)sb * 16 + sw), qfull, DOK_TG_TOMB) == qfull;
     if (MODE == 3 && found) { *(u32 *)(t.buckets + (u64)sb * 16 + sw) = DOK_TG_TOMB; removed = true; }
-    if (MODE == 0 && am != 0) {
+    if (MODE == 0 && im != 0) {
       // the wave's output rows leave LDS as one contiguous stretch
-      const int ne = __popcll(am) * (g.V / unit_v);
+      const int ne = __popcll(im) * (g.V / unit_v);
       const u8 *src = lds_out + (size_t)wave_row0 * g.V;
       u8 *dst = values + (size_t)wave_i0 * g.V;
       for (int e = L.lane; e < ne; e += 64) {
@@ -326,15 +474,41 @@ __global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g
         else dst[e] = src[e];
       }
     }
-    if (MODE == 0 && active) flags[i] = found ? 1 : 0;
-    if (MODE >= 2 && active && flags) flags[i] = removed ? 1 : 0;
+    if (MODE == 0 && inside && flags) flags[i] = found ? 1 : 0;
+    if ((MODE == 2 || MODE == 3) && inside && flags) flags[i] = removed ? 1 : 0;
+    if constexpr (MODE == 4) {
+      // every row found goes into `out` under the key i, by the packed layout's cooperative insert
+      // (the whole wave takes part; its rows' values sit in the wave's own lds_out rows)
+      const u64 ok2 = (u64)i ^ DOK_P8_XOR;
+      const u64 val = found ? tg_load_word(lds_out + (size_t)threadIdx.x * g.V, 0, g.V, unit_v) : 0;
+      const u64 h2 = p8_hash(ok2, *out);
+      int st = 0, fresh = 0;
+      p8_insert<VP>(out->buckets, out->nb, ok2, val, found ? dok_reduce(h2, out->nb) : 0u, p8_fbit(h2), found, st, fresh);
+      n_fresh += fresh;
+      n_full += (found && st == 0);
+    }
     n_found += found;
     n_removed += removed;
-    n_ops += active;
+    n_ops += inside;
   }
-  if (MODE == 1 || MODE >= 2 || STATS)
+  if constexpr (MODE == 4)
+    dok_block_add2(&out->header[DOK_H_NELEM], n_fresh, &out->header[DOK_H_NFULL], n_full);
+  else if (MODE == 1 || MODE == 2 || MODE == 3 || STATS)
     dok_block_add3(MODE == 1 ? count : &t.header[DOK_H_NELEM], MODE == 1 ? n_found : -n_removed,
                    &t.header[DOK_H_NPROBE], STATS ? n_probe : 0, &t.header[DOK_H_NOPS], STATS ? n_ops : 0);
+}
+
+template <int MODE, bool STATS, int UV, class Src>
+__global__ __launch_bounds__(DOK_TPB) void tg_lookup_kernel(DevTable t, TgGeom g, Src src, i64 n,
+                                                            u8 *__restrict__ values, u8 *__restrict__ flags,
+                                                            i64 *count, const u8 *__restrict__ fallback_dev) {
+  tg_lookup_body<MODE, STATS, UV, Src>(t, g, src, n, values, flags, count, fallback_dev, nullptr);
+}
+
+// Sparse-valued gather from a multi-word coordinate table into a packed one keyed by the index space.
+template <int VP>
+__global__ __launch_bounds__(DOK_TPB) void tg_getitem_sparse_kernel(DevTable t, TgGeom g, TgIndexSrc src, DevTable out) {
+  tg_lookup_body<4, false, 0, TgIndexSrc, VP>(t, g, src, src.ix.n_elems, nullptr, nullptr, nullptr, nullptr, &out);
 }
 
 // Record in the home bucket's metadata that a key was placed d > 0 buckets further on, and (W > 0:
@@ -587,39 +761,35 @@ __device__ __forceinline__ void tg_place_rows(const DevTable &t, const TgGeom &g
   }
 }
 
-__global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, const u8 *__restrict__ keys,
-                                                         const u8 *__restrict__ values, i64 n,
-                                                         u8 *__restrict__ stored) {
+// Upsert of the rows a source delivers (see the row sources above).
+template <class Src>
+__global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, Src src, i64 n, u8 *__restrict__ stored) {
   extern __shared__ u64 lds[];
   const int RS = tg_rs(g);
   u64 *lds_rows = lds;                          // [DOK_TPB][1 + KW]
   u64 *lds_vals = lds + DOK_TPB * RS;           // [DOK_TPB][VW]
   const TgLane L(g);
-  int n_fresh = 0, n_full = 0;
+  int n_fresh = 0, n_full = 0, n_oob = 0;
 
   DOK_TILE_LOOP(n) {
     const i64 i = DOK_TILE_ROW();
-    const bool active = i < n;
+    const bool inside = i < n;
     u64 *krow = lds_rows + threadIdx.x * RS;
-    {
-      const u8 *kin = keys + (size_t)i * g.K, *vin = values + (size_t)i * g.V;
-      for (int k = 0; k < g.KW; k++) krow[1 + k] = active ? tg_load_word(kin, k, g.K, g.unit_k) : 0;
-      for (int k = 0; k < g.VW; k++)
-        lds_vals[threadIdx.x * g.VW + k] = active ? tg_load_word(vin, k, g.V, g.unit_v) : 0;
-    }
+    const int code = inside ? src.stage(t, g, i, krow, lds_vals + threadIdx.x * g.VW) : 2;
+    const bool active = code == 0;
+    n_oob += code == 1;
     u32 home, qfull;
     tg_hash_row(t, g, krow, home, qfull);
     int st = 0, fresh = 0;
     tg_insert_rows(t, g, L, lds_rows, lds_vals, home, qfull, active, st, fresh);
-    if (active && stored) stored[i] = (u8)st;
+    if (inside && stored) stored[i] = (u8)(active ? st : 0);
     n_fresh += fresh;
     n_full += (active && st == 0);
   }
-  dok_block_add2(&t.header[DOK_H_NELEM], n_fresh, &t.header[DOK_H_NFULL], n_full);
+  dok_block_add3(&t.header[DOK_H_NELEM], n_fresh, &t.header[DOK_H_NFULL], n_full, &t.header[DOK_H_NOOB], n_oob);
 }
 
-// ---- table scans: read-out and rehash -----------------------------------------------------------
-#define DOK_CHUNK 256
+// ---- table scans: read-out and rehash (chunks of DOK_CHUNK buckets, as in the packed layout) --------
 
 __device__ __forceinline__ bool tg_scan_load(const DevTable &t, const TgLane &L, i64 b, u64 &w) {
   const bool valid = b < (i64)t.nb;
@@ -641,6 +811,9 @@ __global__ __launch_bounds__(DOK_TPB) void tg_chunk_count_kernel(DevTable t, TgG
   if (L.lane == 0) chunk_counts[wid] = cnt;
 }
 
+// COLS: the key words are coordinates and go out the way a COO tensor holds them, word d of entry
+// `row` at keys_out[d * cap + row].
+template <bool COLS>
 __global__ __launch_bounds__(DOK_TPB) void tg_chunk_write_kernel(DevTable t, TgGeom g, const i64 *chunk_offsets,
                                                                  i64 n_chunks, u8 *keys_out, u8 *values_out, i64 cap) {
   const i64 wid = (i64)blockIdx.x * (DOK_TPB / 64) + (threadIdx.x >> 6);
@@ -657,10 +830,38 @@ __global__ __launch_bounds__(DOK_TPB) void tg_chunk_write_kernel(DevTable t, TgG
     const bool slot_live = L.valid && ((m >> tag_lane) & 1ULL);
     const i64 row = base + __popcll(m & ((1ULL << tag_lane) - 1ULL));
     if (slot_live && row < cap) {
-      if (L.is_key && keys_out) tg_store_word(keys_out + (size_t)row * g.K, L.p - 1, g.K, g.unit_k, w);
+      if (L.is_key && keys_out) {
+        if (COLS) ((u64 *)keys_out)[(i64)(L.p - 1) * cap + row] = w;
+        else tg_store_word(keys_out + (size_t)row * g.K, L.p - 1, g.K, g.unit_k, w);
+      }
       if (L.is_val && values_out) tg_store_word(values_out + (size_t)row * g.V, L.p - 1 - g.KW, g.V, g.unit_v, w);
     }
     base += __popcll(m);
+  }
+}
+
+// dense[row-major offset of the coordinates] = value for every live entry of a coordinate table
+// (strides: row-major element strides of the dense tensor).  The key lanes of a slot hold one
+// coordinate each; the slot's tag lane collects them with lane shuffles.
+struct TgDenseStrides { i64 s[DOK_MAX_DIMS]; };
+__global__ __launch_bounds__(DOK_TPB) void tg_to_dense_kernel(DevTable t, TgGeom g, TgDenseStrides strides, u8 *dense,
+                                                              i64 n_chunks) {
+  const i64 wid = (i64)blockIdx.x * (DOK_TPB / 64) + (threadIdx.x >> 6);
+  if (wid >= n_chunks) return;
+  const TgLane L(g);
+  const int tag_lane = L.gbase + L.tag_lane;
+  for (int s = 0; s < DOK_CHUNK / 4; s++) {
+    u64 w;
+    const bool live_tag = tg_scan_load(t, L, wid * DOK_CHUNK + s * 4 + (L.lane >> 4), w);
+    u64 off = 0;
+    bool ok = true;
+    for (int k = 0; k < g.KW; k++) {
+      const u64 c = dok_shfl64(w, (tag_lane + 1 + k) & 63);
+      ok = ok && c < (u64)t.lin_dims[k];
+      off += c * (u64)strides.s[k];
+    }
+    const u64 val = dok_shfl64(w, (tag_lane + 1 + g.KW) & 63);
+    if (live_tag && ok) tg_store_word(dense + (size_t)off * g.V, 0, g.V, g.V, val);
   }
 }
 
@@ -734,59 +935,88 @@ static size_t tg_lds_insert(const TgGeom &g) { return (size_t)DOK_TPB * (g.KW + 
 #define DOK_TG_REMOVE_GRID 4096u
 #define DOK_TG_SET_GRID 32768u
 
-// fallback: host pointer to the fallback row (NULL = zeros); fb_dev: device pointer to it instead
-static int tg_launch_get(const DevTable &d, const void *keys, i64 n, void *values, const void *fallback,
+// Launch of the lookup kernel for one mode and row source.  fallback: host pointer to the fallback row
+// (NULL = zeros); fb_dev: device pointer to it instead.
+template <class Src>
+static int tg_launch_get(const DevTable &d, const Src &src, i64 n, void *values, const void *fallback,
                          const void *fb_dev, u8 *found, bool stats, hipStream_t s) {
   TgGeom g;
   int rc = tg_geom(d, fallback, g);
   if (rc) return rc;
-  if (!tg_aligned(keys, g.unit_k) || !tg_aligned(values, g.unit_v)) return DOK_EINVAL;
+  if (!tg_aligned(values, g.unit_v)) return DOK_EINVAL;
   if (fb_dev && !tg_aligned(fb_dev, g.unit_v)) return DOK_EINVAL;
   const u8 *fbd = (const u8 *)fb_dev;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
   const unsigned cgrid = grid < 2048u ? grid : 2048u;
   if (stats)
-    tg_lookup_kernel<0, true><<<cgrid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr, fbd);
+    tg_lookup_kernel<0, true, 0, Src><<<cgrid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, src, n, (u8 *)values, found, nullptr, fbd);
   else if (g.unit_v == 8)
-    tg_lookup_kernel<0, false, 8><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr, fbd);
+    tg_lookup_kernel<0, false, 8, Src><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, src, n, (u8 *)values, found, nullptr, fbd);
   else if (g.unit_v == 4)
-    tg_lookup_kernel<0, false, 4><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr, fbd);
+    tg_lookup_kernel<0, false, 4, Src><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, src, n, (u8 *)values, found, nullptr, fbd);
   else
-    tg_lookup_kernel<0, false><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, (u8 *)values, found, nullptr, fbd);
+    tg_lookup_kernel<0, false, 0, Src><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, src, n, (u8 *)values, found, nullptr, fbd);
   return DOK_OK;
 }
 
-static int tg_launch_count(const DevTable &d, const void *keys, i64 n, i64 *count, hipStream_t s) {
+template <class Src>
+static int tg_launch_count(const DevTable &d, const Src &src, i64 n, i64 *count, hipStream_t s) {
   TgGeom g;
   int rc = tg_geom(d, nullptr, g);
   if (rc) return rc;
-  if (!tg_aligned(keys, g.unit_k)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_lookup_kernel<1, false><<<(grid < DOK_TG_COUNT_GRID ? grid : DOK_TG_COUNT_GRID), DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, nullptr, nullptr, count);
+  tg_lookup_kernel<1, false, 0, Src><<<(grid < DOK_TG_COUNT_GRID ? grid : DOK_TG_COUNT_GRID), DOK_TPB, tg_lds_lookup(g), s>>>(d, g, src, n, nullptr, nullptr, count, nullptr);
   return DOK_OK;
 }
 
-static int tg_launch_remove(const DevTable &d, const void *keys, i64 n, u8 *removed, bool unique, hipStream_t s) {
+template <class Src>
+static int tg_launch_remove(const DevTable &d, const Src &src, i64 n, u8 *removed, bool unique, hipStream_t s) {
   TgGeom g;
   int rc = tg_geom(d, nullptr, g);
   if (rc) return rc;
-  if (!tg_aligned(keys, g.unit_k)) return DOK_EINVAL;
   const unsigned tiles = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
   const unsigned grid = tiles < DOK_TG_REMOVE_GRID ? tiles : DOK_TG_REMOVE_GRID;
   if (unique)
-    tg_lookup_kernel<3, false><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, nullptr, removed, nullptr);
+    tg_lookup_kernel<3, false, 0, Src><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, src, n, nullptr, removed, nullptr, nullptr);
   else
-    tg_lookup_kernel<2, false><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, (const u8 *)keys, n, nullptr, removed, nullptr);
+    tg_lookup_kernel<2, false, 0, Src><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, src, n, nullptr, removed, nullptr, nullptr);
   return DOK_OK;
 }
 
-static int tg_launch_set(const DevTable &d, const void *keys, const void *values, i64 n, u8 *stored, hipStream_t s) {
+template <class Src>
+static int tg_launch_set(const DevTable &d, const Src &src, i64 n, u8 *stored, hipStream_t s) {
   TgGeom g;
   int rc = tg_geom(d, nullptr, g);
   if (rc) return rc;
-  if (!tg_aligned(keys, g.unit_k) || !tg_aligned(values, g.unit_v)) return DOK_EINVAL;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
-  tg_set_kernel<<<(grid < DOK_TG_SET_GRID ? grid : DOK_TG_SET_GRID), DOK_TPB, tg_lds_insert(g), s>>>(d, g, (const u8 *)keys, (const u8 *)values, n, stored);
+  tg_set_kernel<Src><<<(grid < DOK_TG_SET_GRID ? grid : DOK_TG_SET_GRID), DOK_TPB, tg_lds_insert(g), s>>>(d, g, src, n, stored);
+  return DOK_OK;
+}
+
+// Key / value row pointers of a batch call, checked against the access granules of the widths.
+static int tg_rows(const DevTable &d, const void *keys, const void *values, TgRows &r) {
+  TgGeom g;
+  int rc = tg_geom(d, nullptr, g);
+  if (rc) return rc;
+  if (!tg_aligned(keys, g.unit_k) || (values && !tg_aligned(values, g.unit_v))) return DOK_EINVAL;
+  r.keys = (const u8 *)keys;
+  r.values = (const u8 *)values;
+  return DOK_OK;
+}
+
+static int tg_launch_getitem_sparse(const DevTable &d, const TgIndexSrc &src, const DevTable &out, hipStream_t s) {
+  TgGeom g;
+  int rc = tg_geom(d, nullptr, g);
+  if (rc) return rc;
+  const i64 n = src.ix.n_elems;
+  const unsigned tiles = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
+  const unsigned grid = tiles < 2048u ? tiles : 2048u;
+  switch (out.value_bytes) {
+    case 1: tg_getitem_sparse_kernel<1><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, src, out); break;
+    case 2: tg_getitem_sparse_kernel<2><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, src, out); break;
+    case 4: tg_getitem_sparse_kernel<4><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, src, out); break;
+    default: tg_getitem_sparse_kernel<8><<<grid, DOK_TPB, tg_lds_lookup(g), s>>>(d, g, src, out); break;
+  }
   return DOK_OK;
 }
 
@@ -798,17 +1028,33 @@ static int tg_launch_rehash(const DevTable &a, const DevTable &b, i64 n_chunks, 
   return DOK_OK;
 }
 
+// cols: coordinate table, keys go out as [ndim][cap] int64 (see tg_chunk_write_kernel)
 static int tg_launch_compact(const DevTable &d, i64 *offs, i64 n_chunks, void *keys_out, void *values_out,
-                             i64 cap, i64 *count_out, hipStream_t s) {
+                             i64 cap, i64 *count_out, bool cols, hipStream_t s) {
   TgGeom g;
   int rc = tg_geom(d, nullptr, g);
   if (rc) return rc;
-  if ((keys_out && !tg_aligned(keys_out, g.unit_k)) || (values_out && !tg_aligned(values_out, g.unit_v)))
+  if ((keys_out && !tg_aligned(keys_out, cols ? 8 : g.unit_k)) || (values_out && !tg_aligned(values_out, g.unit_v)))
     return DOK_EINVAL;
   const unsigned grid = (unsigned)((n_chunks + 3) / 4);
   tg_chunk_count_kernel<<<grid, DOK_TPB, 0, s>>>(d, g, offs, n_chunks);
   dok_scan_kernel<<<1, 1024, 0, s>>>(offs, n_chunks, nullptr, count_out);
-  if (keys_out || values_out)
-    tg_chunk_write_kernel<<<grid, DOK_TPB, 0, s>>>(d, g, offs, n_chunks, (u8 *)keys_out, (u8 *)values_out, cap);
+  if (keys_out || values_out) {
+    if (cols) tg_chunk_write_kernel<true><<<grid, DOK_TPB, 0, s>>>(d, g, offs, n_chunks, (u8 *)keys_out, (u8 *)values_out, cap);
+    else tg_chunk_write_kernel<false><<<grid, DOK_TPB, 0, s>>>(d, g, offs, n_chunks, (u8 *)keys_out, (u8 *)values_out, cap);
+  }
+  return DOK_OK;
+}
+
+static int tg_launch_to_dense(const DevTable &d, void *dense, i64 n_chunks, hipStream_t s) {
+  TgGeom g;
+  int rc = tg_geom(d, nullptr, g);
+  if (rc) return rc;
+  if (!tg_aligned(dense, g.V)) return DOK_EINVAL;
+  TgDenseStrides st;
+  memset(&st, 0, sizeof(st));
+  i64 vol = 1;
+  for (int k = d.lin_ndim - 1; k >= 0; k--) { st.s[k] = vol; vol *= d.lin_dims[k]; }
+  tg_to_dense_kernel<<<(unsigned)((n_chunks + 3) / 4), DOK_TPB, 0, s>>>(d, g, st, (u8 *)dense, n_chunks);
   return DOK_OK;
 }

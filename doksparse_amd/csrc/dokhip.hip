@@ -117,15 +117,20 @@ static void div_magic(u64 d, u64 &magic, int &shift) {
 }
 
 // Validate a table descriptor and build its kernel-argument form.
+// A coordinate table (lin_ndim > 0) states its key format through key_bytes: 8 = the coordinates are
+// linearised into one 8-byte key (packed layout; at most DOK_LIN_DIMS dimensions and fewer than 2^63
+// elements), 8 * lin_ndim = the int64 coordinate rows themselves are the keys (multi-word layout).
 int make_dev_table(const dok_table_t *t, DevTable &d, int &layout) {
   if (!t || !t->buckets || !t->header) return DOK_EINVAL;
   if (t->n_phys_buckets < 1 || t->n_phys_buckets > 0xffffffffLL) return DOK_EINVAL;
   if (((uintptr_t)t->buckets & 127) != 0 || ((uintptr_t)t->header & 7) != 0) return DOK_EINVAL;
   if (t->lin_ndim < 0 || t->lin_ndim > DOK_MAX_DIMS) return DOK_EINVAL;
-  if (t->lin_ndim > 0 && t->key_bytes != 8) return DOK_EINVAL;
+  const bool rows = t->lin_ndim > 0 && (t->lin_ndim > 1 || t->key_bytes != 8) && t->key_bytes == 8 * t->lin_ndim;
+  if (t->lin_ndim > 0 && !rows && t->key_bytes != 8) return DOK_EINVAL;
   layout = layout_of(t->key_bytes, t->value_bytes, nullptr);
   if (layout < 0) return layout;
-  if (t->lin_ndim > 0 && layout != DOK_LAYOUT_PACKED8) return DOK_EUNSUPPORTED;
+  if (rows && layout != DOK_LAYOUT_TAGGED) return DOK_EUNSUPPORTED;
+  if (t->lin_ndim > 0 && !is_pow2_le8(t->value_bytes)) return DOK_EUNSUPPORTED;   // one tensor element per entry
   memset(&d, 0, sizeof(d));
   d.buckets = (u64 *)t->buckets;
   d.header = (i64 *)t->header;
@@ -134,12 +139,15 @@ int make_dev_table(const dok_table_t *t, DevTable &d, int &layout) {
   d.key_bytes = t->key_bytes;
   d.value_bytes = t->value_bytes;
   d.lin_ndim = t->lin_ndim;
-  if (t->lin_ndim > 0) {
+  for (int k = 0; k < t->lin_ndim; k++) {
+    if (t->lin_dims[k] < 0) return DOK_EINVAL;
+    d.lin_dims[k] = t->lin_dims[k];
+  }
+  if (t->lin_ndim > 0 && !rows) {
+    if (t->lin_ndim > DOK_LIN_DIMS) return DOK_EUNSUPPORTED;
     // volume must fit in 63 bits so that a linear key never meets the reserved patterns
     unsigned __int128 vol = 1;
     for (int k = t->lin_ndim - 1; k >= 0; k--) {
-      if (t->lin_dims[k] < 0) return DOK_EINVAL;
-      d.lin_dims[k] = t->lin_dims[k];
       d.lin_strides[k] = (i64)vol;
       if (vol > 1) div_magic((u64)vol, d.lin_magic[k], d.lin_shift[k]);
       vol *= (unsigned __int128)(t->lin_dims[k] > 0 ? t->lin_dims[k] : 1);
@@ -149,11 +157,14 @@ int make_dev_table(const dok_table_t *t, DevTable &d, int &layout) {
   return DOK_OK;
 }
 
-// Validate an index descriptor against the table; build its kernel-argument form.
-int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *src, DevIndex &d) {
+// Validate an index descriptor against the table; build its kernel-argument form: DevIndex for the
+// fused kernels of the packed layout, DevIndexW (more dimensions) for the multi-word layout.
+template <class DI, int MAXD>
+int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *src, DI &d) {
   if (!ix || t.lin_ndim == 0) return DOK_EINVAL;
   if (ix->ndim != t.lin_ndim) return DOK_EINVAL;
   if (ix->sel_ndim < 0 || ix->sel_ndim > DOK_MAX_DIMS) return DOK_EINVAL;
+  if (ix->sel_ndim > MAXD || ix->ndim > MAXD) return DOK_EUNSUPPORTED;
   memset(&d, 0, sizeof(d));
   d.ndim = ix->ndim;
   d.sel_ndim = ix->sel_ndim;
@@ -184,6 +195,15 @@ int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *s
   }
   return DOK_OK;
 }
+int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *src, DevIndex &d) {
+  return make_dev_index<DevIndex, DOK_LIN_DIMS>(t, ix, src, d);
+}
+int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *src, DevIndexW &d) {
+  return make_dev_index<DevIndexW, DOK_MAX_DIMS>(t, ix, src, d);
+}
+// The two kinds of coordinate table.
+inline bool is_lin(const DevTable &d, int layout) { return d.lin_ndim > 0 && layout == DOK_LAYOUT_PACKED8; }
+inline bool is_coord_rows(const DevTable &d, int layout) { return d.lin_ndim > 0 && layout == DOK_LAYOUT_TAGGED; }
 
 // One workgroup per tile of DOK_TPB rows (kernels without counters) ...
 inline unsigned grid_for(i64 n) { return (unsigned)((n + DOK_TPB - 1) / DOK_TPB); }
@@ -274,7 +294,9 @@ static int map_get(const dok_table_t *t, const void *keys, int64_t n, void *valu
       P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_get_kernel<V, false, KF><<<grid_for(n), DOK_TPB, 0, s>>>(d, keys, n, values_out, found, fb, fb_dev)));
     }
   } else {
-    rc = tg_launch_get(d, keys, n, values_out, fallback, fb_dev, found, stats, s);
+    TgRows r;
+    rc = tg_rows(d, keys, nullptr, r);
+    if (!rc) rc = tg_launch_get(d, r, n, values_out, fallback, fb_dev, found, stats, s);
     if (rc) return rc;
   }
   return note_launch();
@@ -310,7 +332,9 @@ int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int6
     const unsigned grid = grid_counting(n);
     P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_set_kernel<V, KF><<<grid, DOK_TPB, 0, s>>>(d, keys, values, n, stored, rows_per_wave(n, grid))));
   } else {
-    rc = tg_launch_set(d, keys, values, n, stored, s);
+    TgRows r;
+    rc = tg_rows(d, keys, values, r);
+    if (!rc) rc = tg_launch_set(d, r, n, stored, s);
     if (rc) return rc;
   }
   return note_launch();
@@ -326,9 +350,16 @@ int dok_coo_set(const dok_table_t *t, const int64_t *indices, const void *values
   if (!indices || !values) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
-  { constexpr int KF = DOK_KF_COLS;
+  if (layout == DOK_LAYOUT_PACKED8) {
+    constexpr int KF = DOK_KF_COLS;
     const unsigned grid = grid_counting(n);
-    P8_DISPATCH(d.value_bytes, (p8_set_kernel<V, KF><<<grid, DOK_TPB, 0, s>>>(d, indices, values, n, nullptr, rows_per_wave(n, grid)))); }
+    P8_DISPATCH(d.value_bytes, (p8_set_kernel<V, KF><<<grid, DOK_TPB, 0, s>>>(d, indices, values, n, nullptr, rows_per_wave(n, grid))));
+  } else {
+    if (((uintptr_t)indices & 7) != 0 || ((uintptr_t)values & (uintptr_t)(d.value_bytes - 1)) != 0) return DOK_EINVAL;
+    const TgCols c{(const i64 *)indices, n, (const u8 *)values};
+    rc = tg_launch_set(d, c, n, nullptr, s);
+    if (rc) return rc;
+  }
   return note_launch();
 }
 
@@ -412,7 +443,9 @@ static int map_remove(const dok_table_t *t, const void *keys, int64_t n, uint8_t
       P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_remove_kernel<V, KF, false><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, removed)));
     }
   } else {
-    rc = tg_launch_remove(d, keys, n, removed, unique, s);
+    TgRows r;
+    rc = tg_rows(d, keys, nullptr, r);
+    if (!rc) rc = tg_launch_remove(d, r, n, removed, unique, s);
     if (rc) return rc;
   }
   return note_launch();
@@ -438,7 +471,9 @@ int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n, in
   if (layout == DOK_LAYOUT_PACKED8) {
     P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_count_kernel<V, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(d, keys, n, (i64 *)count)));
   } else {
-    rc = tg_launch_count(d, keys, n, (i64 *)count, s);
+    TgRows r;
+    rc = tg_rows(d, keys, nullptr, r);
+    if (!rc) rc = tg_launch_count(d, r, n, (i64 *)count, s);
     if (rc) return rc;
   }
   return note_launch();
@@ -468,7 +503,7 @@ int dok_map_compact(const dok_table_t *t, void *keys_out, void *values_out, int6
       P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_chunk_write_kernel<V, KF><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks, keys_out, values_out, capacity_rows)));
     }
   } else {
-    rc = tg_launch_compact(d, offs, n_chunks, keys_out, values_out, capacity_rows, (i64 *)count_out, s);
+    rc = tg_launch_compact(d, offs, n_chunks, keys_out, values_out, capacity_rows, (i64 *)count_out, false, s);
     if (rc) return rc;
   }
   return note_launch();
@@ -502,6 +537,11 @@ int dok_coo_compact(const dok_table_t *t, int64_t *indices_out, void *values_out
   const DeviceScope on_stream_device(s);
   const i64 n_chunks = chunks_of(d);
   i64 *offs = (i64 *)scratch;
+  if (layout != DOK_LAYOUT_PACKED8) {
+    rc = tg_launch_compact(d, offs, n_chunks, indices_out, values_out, capacity, (i64 *)count_out, true, s);
+    if (rc) return rc;
+    return note_launch();
+  }
   P8_DISPATCH(d.value_bytes, (p8_chunk_count_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, offs, n_chunks)));
   dok_scan_kernel<<<1, 1024, 0, s>>>(offs, n_chunks, nullptr, (i64 *)count_out);
   if (indices_out || values_out) {
@@ -578,30 +618,57 @@ int dok_map_rehash_bulk(const dok_table_t *src, const dok_table_t *dst, void *wo
   return note_launch();
 }
 
+// The DOK indexing entry points take both kinds of coordinate table: linearised keys on the packed
+// layout (DevIndex, kernels of dok_packed8.h) and int64 coordinate rows on the multi-word layout
+// (DevIndexW, the kernels of dok_tagged.h fed by an index source).
 int dok_getitem_dense(const dok_table_t *t, const dok_index_t *ix, void *out, void *stream) {
-  DevTable d; int layout; DevIndex di;
+  DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (is_coord_rows(d, layout)) {
+    TgIndexSrc src;
+    rc = make_dev_index(d, ix, nullptr, src.ix);
+    if (rc) return rc;
+    if (src.ix.n_elems == 0) return DOK_OK;
+    if (!out || src.ix.n_elems > kMaxRows) return DOK_EINVAL;
+    const DeviceScope on_stream_device(s);
+    rc = tg_launch_get(d, src, src.ix.n_elems, out, nullptr, nullptr, nullptr, false, s);
+    if (rc) return rc;
+    return note_launch();
+  }
+  DevIndex di;
   rc = make_dev_index(d, ix, nullptr, di);
   if (rc) return rc;
   if (di.n_elems == 0) return DOK_OK;
   if (!out || di.n_elems > kMaxRows) return DOK_EINVAL;
-  hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
   P8_DISPATCH(d.value_bytes, (p8_getitem_kernel<V><<<grid_for(di.n_elems), DOK_TPB, 0, s>>>(d, di, out)));
   return note_launch();
 }
 
 int dok_setitem_dense(const dok_table_t *t, const dok_index_t *ix, const dok_view_t *src, void *stream) {
-  DevTable d; int layout; DevIndex di;
+  DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
   if (!src) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (is_coord_rows(d, layout)) {
+    TgIndexSrc isrc;
+    rc = make_dev_index(d, ix, src, isrc.ix);
+    if (rc) return rc;
+    if (isrc.ix.n_elems == 0) return DOK_OK;
+    if (isrc.ix.n_elems > kMaxRows || ((uintptr_t)src->data & (uintptr_t)(d.value_bytes - 1)) != 0) return DOK_EINVAL;
+    const DeviceScope on_stream_device(s);
+    rc = tg_launch_set(d, isrc, isrc.ix.n_elems, nullptr, s);
+    if (rc) return rc;
+    return note_launch();
+  }
+  DevIndex di;
   rc = make_dev_index(d, ix, src, di);
   if (rc) return rc;
   if (di.n_elems == 0) return DOK_OK;
   if (di.n_elems > kMaxRows) return DOK_EINVAL;
-  hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
   const unsigned grid = grid_counting(di.n_elems);
   P8_DISPATCH(d.value_bytes, (p8_setitem_kernel<V><<<grid, DOK_TPB, 0, s>>>(d, di, rows_per_wave(di.n_elems, grid))));
@@ -609,48 +676,87 @@ int dok_setitem_dense(const dok_table_t *t, const dok_index_t *ix, const dok_vie
 }
 
 int dok_count_items(const dok_table_t *t, const dok_index_t *ix, int64_t *count, void *stream) {
-  DevTable d; int layout; DevIndex di;
+  DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (is_coord_rows(d, layout)) {
+    TgIndexSrc src;
+    rc = make_dev_index(d, ix, nullptr, src.ix);
+    if (rc) return rc;
+    if (src.ix.n_elems == 0) return DOK_OK;
+    if (!count || src.ix.n_elems > kMaxRows) return DOK_EINVAL;
+    const DeviceScope on_stream_device(s);
+    rc = tg_launch_count(d, src, src.ix.n_elems, (i64 *)count, s);
+    if (rc) return rc;
+    return note_launch();
+  }
+  DevIndex di;
   rc = make_dev_index(d, ix, nullptr, di);
   if (rc) return rc;
   if (di.n_elems == 0) return DOK_OK;
   if (!count || di.n_elems > kMaxRows) return DOK_EINVAL;
-  hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
   P8_DISPATCH(d.value_bytes, (p8_countitems_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di, (i64 *)count)));
   return note_launch();
 }
 
 int dok_zero_items(const dok_table_t *t, const dok_index_t *ix, void *stream) {
-  DevTable d; int layout; DevIndex di;
+  DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (is_coord_rows(d, layout)) {
+    TgIndexSrc src;
+    rc = make_dev_index(d, ix, nullptr, src.ix);
+    if (rc) return rc;
+    if (src.ix.n_elems == 0) return DOK_OK;
+    if (src.ix.n_elems > kMaxRows) return DOK_EINVAL;
+    const DeviceScope on_stream_device(s);
+    rc = tg_launch_remove(d, src, src.ix.n_elems, nullptr, false, s);
+    if (rc) return rc;
+    return note_launch();
+  }
+  DevIndex di;
   rc = make_dev_index(d, ix, nullptr, di);
   if (rc) return rc;
   if (di.n_elems == 0) return DOK_OK;
   if (di.n_elems > kMaxRows) return DOK_EINVAL;
-  hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
   P8_DISPATCH(d.value_bytes, (p8_zeroitems_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di)));
   return note_launch();
 }
 
 int dok_getitem_sparse(const dok_table_t *t, const dok_index_t *ix, const dok_table_t *out, void *stream) {
-  DevTable d, o; int layout, lo; DevIndex di;
+  DevTable d, o; int layout, lo;
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
   rc = make_dev_table(out, o, lo);
   if (rc) return rc;
+  // `out` is keyed by the offsets into the index space: a table of linearised coordinates
+  if (!is_lin(o, lo)) return o.lin_ndim > 0 ? DOK_EUNSUPPORTED : DOK_EINVAL;
+  if (o.value_bytes != d.value_bytes || o.buckets == d.buckets) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (is_coord_rows(d, layout)) {
+    TgIndexSrc src;
+    rc = make_dev_index(d, ix, nullptr, src.ix);
+    if (rc) return rc;
+    if (o.lin_ndim != src.ix.sel_ndim) return DOK_EINVAL;
+    for (int j = 0; j < src.ix.sel_ndim; j++) if (o.lin_dims[j] != src.ix.shape[j]) return DOK_EINVAL;
+    if (src.ix.n_elems == 0) return DOK_OK;
+    if (src.ix.n_elems > kMaxRows) return DOK_EINVAL;
+    const DeviceScope on_stream_device(s);
+    rc = tg_launch_getitem_sparse(d, src, o, s);
+    if (rc) return rc;
+    return note_launch();
+  }
+  DevIndex di;
   rc = make_dev_index(d, ix, nullptr, di);
   if (rc) return rc;
-  // `out` must be keyed by the index space itself
-  if (o.lin_ndim != di.sel_ndim || o.lin_ndim == 0 || o.value_bytes != d.value_bytes || o.buckets == d.buckets)
-    return DOK_EINVAL;
+  if (o.lin_ndim != di.sel_ndim) return DOK_EINVAL;
   for (int j = 0; j < di.sel_ndim; j++) if (o.lin_dims[j] != di.shape[j]) return DOK_EINVAL;
   if (di.n_elems == 0) return DOK_OK;
   if (di.n_elems > kMaxRows) return DOK_EINVAL;
-  hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
   P8_DISPATCH(d.value_bytes, (p8_getitem_sparse_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di, o)));
   return note_launch();
@@ -658,15 +764,32 @@ int dok_getitem_sparse(const dok_table_t *t, const dok_index_t *ix, const dok_ta
 
 int dok_setitem_sparse(const dok_table_t *t, const dok_index_t *ix, const int64_t *src_indices,
                        const void *src_values, int64_t n_src, uint64_t nonzero_mask, void *stream) {
-  DevTable d; int layout; DevIndex di;
+  DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (n_src < 0 || n_src > kMaxRows) return DOK_EINVAL;
+  if (is_coord_rows(d, layout)) {
+    TgSparseSrc src;
+    rc = make_dev_index(d, ix, nullptr, src.ix);
+    if (rc) return rc;
+    if (n_src == 0) return DOK_OK;
+    if (!src_values || (!src_indices && src.ix.sel_ndim > 0)) return DOK_EINVAL;
+    if (((uintptr_t)src_indices & 7) != 0 || ((uintptr_t)src_values & (uintptr_t)(d.value_bytes - 1)) != 0) return DOK_EINVAL;
+    src.src_indices = (const i64 *)src_indices;
+    src.src_values = (const u8 *)src_values;
+    src.n_src = n_src;
+    src.nonzero_mask = nonzero_mask;
+    const DeviceScope on_stream_device(s);
+    rc = tg_launch_set(d, src, n_src, nullptr, s);
+    if (rc) return rc;
+    return note_launch();
+  }
+  DevIndex di;
   rc = make_dev_index(d, ix, nullptr, di);
   if (rc) return rc;
-  if (n_src < 0 || n_src > kMaxRows) return DOK_EINVAL;
   if (n_src == 0) return DOK_OK;
   if (!src_values || (!src_indices && di.sel_ndim > 0)) return DOK_EINVAL;
-  hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
   const unsigned grid = grid_counting(n_src);
   P8_DISPATCH(d.value_bytes, (p8_setitem_sparse_kernel<V><<<grid, DOK_TPB, 0, s>>>(
@@ -679,13 +802,22 @@ int dok_to_dense(const dok_table_t *t, void *dense, void *stream) {
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
   if (d.lin_ndim == 0 || !dense) return DOK_EINVAL;
-  i64 volume = 1;
-  for (int k = 0; k < d.lin_ndim; k++) volume *= d.lin_dims[k];
+  unsigned __int128 vol = 1;
+  for (int k = 0; k < d.lin_ndim; k++) {
+    vol *= (unsigned __int128)d.lin_dims[k];
+    if (vol >> 62) return DOK_EINVAL;              // no such dense tensor exists
+  }
+  const i64 volume = (i64)vol;
   if (volume == 0) return DOK_OK;
   hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
   const i64 n_chunks = chunks_of(d);
-  P8_DISPATCH(d.value_bytes, (p8_to_dense_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, dense, n_chunks, volume)));
+  if (layout == DOK_LAYOUT_PACKED8) {
+    P8_DISPATCH(d.value_bytes, (p8_to_dense_kernel<V><<<chunk_grid(n_chunks), DOK_TPB, 0, s>>>(d, dense, n_chunks, volume)));
+  } else {
+    rc = tg_launch_to_dense(d, dense, n_chunks, s);
+    if (rc) return rc;
+  }
   return note_launch();
 }
 

@@ -27,35 +27,26 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from ._lib import DokIndex, DokView, DOK_MAX_DIMS
-from .closed_hashmap import CudaClosedHashmap, _stream_ptr
+from ._lib import DokIndex, DokView, DOK_MAX_DIMS, DOK_LIN_DIMS
+from .closed_hashmap import CudaClosedHashmap, _stream_ptr, coord_rows_needed
 from .util import str2dtype, next_power_of_2, shape_to_stride
 
 _INT_DTYPES = {torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8}
 
-# A tensor whose index space a single 8-byte linear key cannot hold (2^63 elements or more), or
-# with more dimensions than the fused indexing kernels take, keeps its coordinates as they are:
-# the map's key rows are the int64[ndim] coordinate vectors themselves (the reference's own key
-# format, sparse_dok_tensor.py:45-69) on the multi-word table layout, and indexing goes through
-# materialised coordinate rows and the batched get / set / remove kernels.  One tag word, ndim key
-# words and the value word have to fit a 128-byte bucket.
-_WIDE_MAX_DIMS = 14
-
-
-def _is_wide(size):
-    volume = 1
-    for s in size:
-        volume *= max(int(s), 1)
-    return len(size) > DOK_MAX_DIMS or volume >= 2**63
+# The storage of a tensor is a coordinate-keyed map over its size.  Where one 8-byte key can hold a
+# linearised coordinate (at most 8 dimensions, fewer than 2^63 elements) the map stores that; a
+# larger tensor keeps the int64[ndim] coordinate vectors themselves as multi-word keys (the
+# reference's own key format, sparse_dok_tensor.py:45-69).  Every indexing method runs as the same
+# fused kernels on either (the library picks them from the table descriptor).  One tag word, ndim
+# key words and the value word have to fit a 128-byte bucket, hence DOK_MAX_DIMS dimensions at most.
 
 
 def _make_storage(size, n_buckets, device, rehash_factor=2.0, rehash_threshold=0.75):
     """An empty map keyed the way a tensor of this size needs it."""
-    if len(size) > _WIDE_MAX_DIMS:
-        raise NotImplementedError(f"tensors of more than {_WIDE_MAX_DIMS} dimensions: a coordinate row "
+    if len(size) > DOK_MAX_DIMS:
+        raise NotImplementedError(f"tensors of more than {DOK_MAX_DIMS} dimensions: a coordinate row "
                                   "no longer fits a 128-byte bucket")
-    coord_dims = None if _is_wide(size) else tuple(int(s) for s in size)
-    return CudaClosedHashmap(n_buckets=n_buckets, device=device, coord_dims=coord_dims,
+    return CudaClosedHashmap(n_buckets=n_buckets, device=device, coord_dims=tuple(int(s) for s in size),
                              rehash_factor=rehash_factor, rehash_threshold=rehash_threshold)
 
 
@@ -101,7 +92,6 @@ class SparseDOKTensor(object):
         else:
             self._dtype = str2dtype(dtype)
 
-        self._wide = _is_wide(self._size)
         if storage is not None:
             self._hashmap = self._adopt_storage(storage)
         else:
@@ -119,51 +109,24 @@ class SparseDOKTensor(object):
         """Upsert entries given as [ndim, n] coordinates (this view's dimension order must be the
         storage's) and [n, 1] values; coordinates outside the size are skipped."""
         hm = self._hashmap
-        if self._wide:
-            rows = indices.T.contiguous()
-            ok = self._rows_in_range(rows)
-            if not bool(ok.all()):
-                rows, vals = rows[ok], vals[ok]
-            hm.set(rows, vals)
-        elif hm._coord_dims == tuple(self._size):
+        if hm._coord_dims == tuple(self._size):
             hm.set_coo(indices, vals)
         else:
             hm.set(indices.T, vals)
 
     def _adopt_storage(self, storage):
-        """Use `storage` directly if it is keyed the way this tensor needs (linearised coordinates
-        of this size, or plain coordinate rows for a wide tensor); otherwise move its entries
-        into such a map."""
-        if self._wide:
-            if storage._coord_dims is None and (not storage._allocated or (
-                    storage._key_dtype == torch.long and storage._key_shape == (self.ndim,))):
-                return storage
-        elif storage._coord_dims == tuple(self._size):
+        """Use `storage` directly if it is keyed the way this tensor needs (coordinates inside this
+        size); otherwise move its entries into such a map."""
+        if storage._coord_dims == tuple(self._size):
             return storage
         new = _make_storage(self._size, storage.n_buckets, storage.device,
                             storage._rehash_factor, storage._rehash_threshold)
         if storage._allocated:
             keys, values = storage.items()
             if keys.shape[0]:
-                rows = keys.reshape(-1, self.ndim).long()
-                if self._wide:
-                    ok = self._rows_in_range(rows)
-                    rows, values = rows[ok], values[ok]
-                new.set(rows, values)
+                new.set(keys.reshape(-1, self.ndim).long(), values)
+                new._header[_lib.DOK_H_NOOB] = 0      # entries outside this size are dropped
         return new
-
-    # ------------------------------------------------------------------ wide tensors
-    def _storage_sizes(self):
-        """Sizes in the storage's dimension order, as a device tensor."""
-        return torch.tensor(self._to_storage_order(list(self._size)), device=self.device, dtype=torch.long)
-
-    def _rows_in_range(self, rows):
-        return ((rows >= 0) & (rows < self._storage_sizes())).all(dim=1)
-
-    def _wide_rows(self, mats):
-        """[n, ndim] int64 coordinate rows, in the storage's dimension order, of materialised
-        selectors (the reference's stack + transpose, sparse_dok_tensor.py:304-311, in one copy)."""
-        return torch.stack(self._to_storage_order(list(mats)), dim=-1).reshape(-1, self.ndim)
 
     def _ensure_widths(self):
         """Fix the key / value widths of an unallocated map without storing anything."""
@@ -274,11 +237,7 @@ class SparseDOKTensor(object):
 
     def _items_coo_view(self):
         """(indices [ndim, nnz] in this view's dimension order, values [nnz, 1]) from one pass."""
-        if self._wide:
-            keys, values = self._hashmap.items()
-            idx = None if keys is None else keys.T.contiguous()
-        else:
-            idx, values = self._hashmap.items_coo()
+        idx, values = self._hashmap.items_coo()
         if idx is None:
             return (torch.empty(self.ndim, 0, device=self.device, dtype=torch.long),
                     torch.empty(0, 1, device=self.device, dtype=self.dtype))
@@ -317,11 +276,7 @@ class SparseDOKTensor(object):
         hm = self._hashmap
         storage_shape = self._to_storage_order(list(self.shape))
         dense = torch.zeros(tuple(storage_shape), device=self.device, dtype=self.dtype)
-        if self._wide:
-            keys, values = hm.items()
-            if keys is not None and keys.shape[0]:
-                dense[tuple(keys.T)] = values.flatten()
-        elif hm._allocated and dense.numel():
+        if hm._allocated and dense.numel():
             lib = _lib.load()
             _lib.check(lib.dok_to_dense(ctypes.byref(hm._desc), dense.data_ptr(), _stream_ptr(self.device)),
                        "to_dense")
@@ -347,11 +302,9 @@ class SparseDOKTensor(object):
         self._hashmap = new
         self._size = torch.Size(new_size)
         self._perm = tuple(range(len(new_size)))
-        self._wide = _is_wide(self._size)
         if idx is not None:
             self._store_coo(idx.contiguous(), values)
-            if not self._wide:
-                new._header[_lib.DOK_H_NOOB] = 0      # entries outside the new size are dropped
+            new._header[_lib.DOK_H_NOOB] = 0          # entries outside the new size are dropped
 
     # ------------------------------------------------------------------ selectors
     def _normalise_slice(self, sl, dim):
@@ -465,11 +418,15 @@ class SparseDOKTensor(object):
         for j, st in enumerate(strides):
             view.strides[j] = st
 
+    def _max_axes(self):
+        """Most axes an indexing expression's result may have on this tensor's storage."""
+        return DOK_MAX_DIMS if self._hashmap._coord_rows else DOK_LIN_DIMS
+
     def _index_desc(self, selectors):
         """dok_index_t of materialised selectors (the result of _handle_selectors)."""
         out_shape = tuple(selectors[0].shape)
-        if len(out_shape) > DOK_MAX_DIMS or self.ndim > DOK_MAX_DIMS:
-            raise NotImplementedError(f"indexing expressions with more than {DOK_MAX_DIMS} axes")
+        if len(out_shape) > self._max_axes():
+            raise NotImplementedError(f"indexing expressions with more than {self._max_axes()} axes")
         ix = DokIndex()
         ix.ndim = self.ndim
         ix.sel_ndim = len(out_shape)
@@ -489,8 +446,8 @@ class SparseDOKTensor(object):
         shape, scalar positions, tensors to keep alive until the launch)."""
         flat = self._normalise(selectors)
         bshape, first, slice_axis, out_shape, scalar_positions = self._layout(flat)
-        if len(out_shape) > DOK_MAX_DIMS or self.ndim > DOK_MAX_DIMS:
-            raise NotImplementedError(f"indexing expressions with more than {DOK_MAX_DIMS} axes")
+        if len(out_shape) > self._max_axes():
+            raise NotImplementedError(f"indexing expressions with more than {self._max_axes()} axes")
         ix = DokIndex()
         ix.ndim = self.ndim
         ix.sel_ndim = len(out_shape)
@@ -514,8 +471,6 @@ class SparseDOKTensor(object):
 
     # ------------------------------------------------------------------ indexing
     def __getitem__(self, selectors):
-        if self._wide:
-            return self._wide_getitem(selectors)
         ix, out_shape, scalar_positions, keep = self._plan(selectors)
         hm = self._hashmap
         if not hm._allocated:
@@ -532,45 +487,6 @@ class SparseDOKTensor(object):
                 values = values.squeeze(i)
         return values
 
-    def _wide_getitem(self, selectors):
-        mats, scalar_positions = self._handle_selectors(selectors)
-        out_shape = tuple(mats[0].shape)
-        hm = self._hashmap
-        if not hm._allocated or mats[0].numel() == 0:
-            values = torch.zeros(out_shape, device=self.device, dtype=self.dtype)
-        else:
-            values, _ = hm.get(self._wide_rows(mats))          # absent (and out-of-range) coordinates read 0
-            values = values.reshape(out_shape)
-        for i in reversed(scalar_positions):
-            if i < values.ndim:
-                values = values.squeeze(i)
-        return values
-
-    def _wide_set_items_dense(self, src, mats):
-        """`_set_items_dense` for a wide tensor: same growth rule, coordinate rows through the
-        batched upsert."""
-        rows = self._wide_rows(mats)
-        src = src.reshape(-1, 1)
-        n_sel = rows.shape[0]
-        if n_sel == 0:
-            return
-        ok = self._rows_in_range(rows)
-        n_oob = n_sel - int(ok.sum().item())
-        if n_oob:
-            rows, src = rows[ok], src[ok]
-        hm = self._hashmap
-        if rows.shape[0]:
-            if not hm._allocated:
-                hm.set(rows[:1], src[:1].contiguous())            # (sparse_dok_tensor_impl.py:413-416)
-            limit = hm.n_buckets * hm._rehash_threshold
-            if hm._n_upper + n_sel > limit:
-                n_now = hm.n_elements
-                if n_now + n_sel > limit:
-                    hm.rehash(int(np.ceil((n_now + n_sel) * hm._rehash_factor)))
-            hm.set(rows, src.contiguous())
-        if n_oob:
-            raise IndexError(f"{n_oob} coordinates fall outside the tensor of size {tuple(self.shape)}")
-
     def __setitem__(self, selectors, values):
         if isinstance(values, SparseDOKTensor) or (isinstance(values, Tensor) and values.is_sparse):
             mats, _ = self._handle_selectors(selectors)
@@ -578,13 +494,6 @@ class SparseDOKTensor(object):
             assert tuple(values.shape) == out_shape, \
                 f"expecting the value shape to be {out_shape}, got {tuple(values.shape)} instead"
             return self._set_items_sparse(values, mats)
-        if self._wide:
-            mats, _ = self._handle_selectors(selectors)
-            out_shape = tuple(mats[0].shape)
-            if not isinstance(values, Tensor):
-                values = torch.tensor(values, device=self.device, dtype=self.dtype)
-            values = torch.broadcast_to(values.to(device=self.device, dtype=self.dtype), out_shape)
-            return self._wide_set_items_dense(values, mats)
         ix, out_shape, _, keep = self._plan(selectors)
         if not isinstance(values, Tensor):
             values = torch.tensor(values, device=self.device, dtype=self.dtype)
@@ -637,11 +546,13 @@ class SparseDOKTensor(object):
         hm = self._hashmap
         if not hm._allocated:
             return out
-        if self._wide or out._wide:
-            # through coordinate rows: look up, keep the hits, key them by their index vector
+        if coord_rows_needed(out_shape):
+            # an index space of more than 8 axes (its offsets cannot key the result's table): look
+            # the coordinate rows up, keep the hits, key them by their index vector
             n = 0
             if selectors[0].numel():
-                values, found = hm.get(self._wide_rows(selectors))
+                rows = torch.stack(self._to_storage_order(list(selectors)), dim=-1).reshape(-1, self.ndim)
+                values, found = hm.get(rows)
                 at = found.nonzero().flatten()
                 n = int(at.shape[0])
             out._hashmap = _make_storage(out_shape, int(n * 2.0), self.device)
@@ -683,8 +594,6 @@ class SparseDOKTensor(object):
         src_indices = src_indices.to(self.device)
         src_values = src_values.to(device=self.device, dtype=self.dtype).contiguous()
         hm = self._hashmap
-        if self._wide:
-            return self._wide_set_items_sparse(src_indices, src_values, selectors)
         if not hm._allocated:
             # (reference: sparse_dok_tensor_impl.py:237-240)
             first_key = torch.stack([s.reshape(-1)[0] for s in self._to_storage_order(selectors)], dim=0)[None]
@@ -707,41 +616,12 @@ class SparseDOKTensor(object):
                                               src_values.data_ptr(), n_src, mask, stream), "__setitem__")
         hm._n_upper = n_now + n_src
 
-    def _wide_set_items_sparse(self, src_indices, src_values, mats):
-        hm = self._hashmap
-        rows_all = self._wide_rows(mats)
-        if not hm._allocated:
-            first = rows_all[:1]
-            if first.shape[0] and bool(self._rows_in_range(first).all()):
-                hm.set(first, torch.zeros(1, 1, device=self.device, dtype=self.dtype))   # (sparse_dok_tensor_impl.py:237-240)
-            else:
-                self._ensure_widths()
-        if rows_all.shape[0]:
-            hm._remove_rows(rows_all)
-        n_src = int(src_values.shape[0])
-        n_now = hm.n_elements
-        hm.rehash(int(np.ceil((n_now + n_src) * hm._rehash_factor * 2)))
-        if n_src:
-            shape = torch.tensor(tuple(mats[0].shape), device=self.device, dtype=torch.long)[:, None]
-            keep = (src_values != 0) & ((src_indices >= 0) & (src_indices < shape)).all(dim=0)
-            at = tuple(src_indices[:, keep])
-            rows = torch.stack([m[at] for m in self._to_storage_order(list(mats))], dim=-1).reshape(-1, self.ndim)
-            vals = src_values[keep][:, None]
-            ok = self._rows_in_range(rows)
-            if rows.shape[0]:
-                hm.set(rows[ok], vals[ok].contiguous())
-        hm._n_upper = n_now + n_src
-
     def count_items(self, selectors):
         """Number of addressed elements that are stored (reference: count_items,
         sparse_dok_tensor_impl.py:56-108)."""
         selectors, _ = self._handle_selectors(selectors)
         count = torch.zeros(1, device=self.device, dtype=torch.long)
         hm = self._hashmap
-        if self._wide:
-            if hm._allocated and selectors[0].numel():
-                count += hm.count_existing(self._wide_rows(selectors))
-            return count
         if hm._allocated and selectors[0].numel():
             ix, _ = self._index_desc(selectors)
             lib = _lib.load()
@@ -753,10 +633,6 @@ class SparseDOKTensor(object):
         """Remove every addressed element (reference: zero_items, sparse_dok_tensor_impl.py:110-146)."""
         selectors, _ = self._handle_selectors(selectors)
         hm = self._hashmap
-        if self._wide:
-            if hm._allocated and selectors[0].numel():
-                hm._remove_rows(self._wide_rows(selectors))
-            return
         if hm._allocated and selectors[0].numel():
             ix, _ = self._index_desc(selectors)
             lib = _lib.load()

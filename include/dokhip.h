@@ -35,7 +35,7 @@ extern "C" {
 #define DOK_ETOOLARGE    -4   /* the table needs more scratch than dok_map_compact_static owns   */
 
 #define DOK_BUCKET_BYTES  128
-#define DOK_MAX_DIMS      8
+#define DOK_MAX_DIMS      14  /* most dimensions of a coordinate table and of an index space     */
 
 /* Table header: DOK_HEADER_WORDS int64 words in device memory, zeroed by dok_table_clear.     */
 #define DOK_HEADER_WORDS  16
@@ -60,11 +60,20 @@ typedef struct dok_table {
   int64_t *header;             /* device, DOK_HEADER_WORDS int64                                  */
   int64_t  n_phys_buckets;     /* 1 .. 2^32-1                                                     */
   uint64_t seed;               /* hash seed; placement depends on it, results do not              */
-  int32_t  key_bytes;          /* bytes per key row as stored (8 when lin_ndim > 0)               */
+  int32_t  key_bytes;          /* bytes per key row as stored                                     */
   int32_t  value_bytes;        /* bytes per value row                                             */
-  int32_t  lin_ndim;           /* 0: key rows are raw bytes.  n>0: key rows handed to the batch
-                                  entry points are n int64 coordinates that are linearised
-                                  row-major over lin_dims into one 8-byte key                     */
+  int32_t  lin_ndim;           /* 0: key rows are raw bytes.  n>0: a COORDINATE TABLE - key rows
+                                  handed to the entry points are n int64 coordinates inside
+                                  lin_dims (the key format of the reference's SparseDOKTensor,
+                                  sparse_dok_tensor.py:45-69); rows outside lin_dims are skipped
+                                  (lookups: absent; inserts: counted in header[DOK_H_NOOB]).
+                                  key_bytes says how they are stored:
+                                    8      linearised row-major into one 8-byte key (packed
+                                           layout).  Needs n <= 8 and prod(lin_dims) < 2^63, else
+                                           DOK_EUNSUPPORTED.
+                                    8 * n  (n >= 2) the coordinate rows themselves, as multi-word
+                                           keys (n <= DOK_MAX_DIMS, any lin_dims).
+                                  value_bytes must be 1, 2, 4 or 8 (one tensor element).           */
   int32_t  reserved_;
   int64_t  lin_dims[DOK_MAX_DIMS];
 } dok_table_t;
@@ -85,8 +94,10 @@ typedef struct dok_view {
  * tensor dimension: what SparseDOKTensor._handle_selectors (sparse_dok_tensor.py:220-300)
  * produces and get_tensor_accessor_argument_array (util.py:295-310) packs for the kernels. */
 typedef struct dok_index {
-  int32_t    ndim;                     /* tensor dimensions = number of selectors (<= 8)         */
-  int32_t    sel_ndim;                 /* dimensions of the broadcast index space (<= 8)         */
+  int32_t    ndim;                     /* tensor dimensions = number of selectors                */
+  int32_t    sel_ndim;                 /* dimensions of the broadcast index space: at most
+                                          DOK_MAX_DIMS; on a table of linearised keys at most 8
+                                          (else DOK_EUNSUPPORTED)                                */
   int64_t    shape[DOK_MAX_DIMS];      /* broadcast shape                                        */
   dok_view_t sel[DOK_MAX_DIMS];        /* int64 selector views, one per tensor dimension         */
 } dok_index_t;
@@ -242,7 +253,7 @@ int64_t dok_rehash_bulk_workspace_bytes(const dok_table_t *src, const dok_table_
 int dok_map_rehash_bulk(const dok_table_t *src, const dok_table_t *dst, void *workspace,
                         int64_t workspace_bytes, void *stream);
 
-/* ---- COO bridge (tables with lin_ndim > 0) -------------------------------------------------- */
+/* ---- COO bridge (coordinate tables: lin_ndim > 0, either key format) ------------------------ */
 
 /* dok_map_set for coordinates given the way a COO tensor holds them: indices is
  * [lin_ndim][n] int64 (coordinate d of entry i at indices[d*n + i]).  No per-row flag.
@@ -251,7 +262,7 @@ int dok_map_rehash_bulk(const dok_table_t *src, const dok_table_t *dst, void *wo
 int dok_coo_set(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
                 void *stream);
 
-/* dok_coo_set through the bulk path (see dok_map_set_bulk). */
+/* dok_coo_set through the bulk path (see dok_map_set_bulk; tables of linearised keys only). */
 int dok_coo_set_bulk(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
                      void *workspace, int64_t workspace_bytes, void *stream);
 
@@ -265,7 +276,7 @@ int dok_coo_build_bulk(const dok_table_t *t, const int64_t *indices, const void 
 int dok_coo_compact(const dok_table_t *t, int64_t *indices_out, void *values_out, int64_t capacity,
                     int64_t *count_out, void *scratch, void *stream);
 
-/* ---- DOK indexing (tables with lin_ndim > 0) ------------------------------------------------ */
+/* ---- DOK indexing (coordinate tables: lin_ndim > 0, either key format) ---------------------- */
 
 /* out[e] = value stored at the coordinate the selectors give for element e of the broadcast
  * index space, or zero; out is C-contiguous with value_bytes per element.
@@ -288,7 +299,8 @@ int dok_zero_items(const dok_table_t *t, const dok_index_t *ix, void *stream);
 
 /* Sparse-valued gather: every element e of the index space whose coordinate is stored in t is
  * inserted into `out` under the key e.  `out` is a cleared coordinate-keyed table whose
- * lin_dims are the broadcast shape of ix and whose value_bytes equal t's.
+ * lin_dims are the broadcast shape of ix and whose value_bytes equal t's.  `out` must hold
+ * linearised keys (key_bytes 8), else DOK_EUNSUPPORTED; t may be of either key format.
  * Reference: sparse_dok_get_items (sparse_dok_tensor_impl.cu:111-160). */
 int dok_getitem_sparse(const dok_table_t *t, const dok_index_t *ix, const dok_table_t *out,
                        void *stream);
@@ -303,7 +315,7 @@ int dok_setitem_sparse(const dok_table_t *t, const dok_index_t *ix, const int64_
                        const void *src_values, int64_t n_src, uint64_t nonzero_mask, void *stream);
 
 /* dense[linear coordinate] = value for every live entry; `dense` holds prod(lin_dims) elements
- * of value_bytes and must be zero-filled by the caller.
+ * of value_bytes (fewer than 2^62 elements) and must be zero-filled by the caller.
  * Reference: SparseDOKTensor.to_dense (sparse_dok_tensor.py:195-209). */
 int dok_to_dense(const dok_table_t *t, void *dense, void *stream);
 

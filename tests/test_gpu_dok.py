@@ -515,6 +515,22 @@ def test_constructors_clone_resize_and_conversions(cuda):
     assert shrunk._nnz() == int(mask[:10].sum())
 
 
+def _new_dok(shape, idx, vals, dev, rows):
+    """A tensor from COO entries; rows=True: on a storage that keeps the int64 coordinate rows as
+    multi-word keys (what tensors of 2^63 elements and more, or of more than 8 dimensions, get by
+    themselves), so that the kernels of that key format meet every small case as well."""
+    from doksparse_amd import SparseDOKTensor, CudaClosedHashmap
+    from doksparse_amd.util import next_power_of_2
+    from doksparse_amd import _lib
+    storage = None
+    if rows:
+        storage = CudaClosedHashmap(n_buckets=next_power_of_2(vals.shape[0]), device=dev, coord_dims=shape, coord_rows=True)
+    dok = SparseDOKTensor(shape, idx.to(dev), vals.to(dev), device=dev, storage=storage)
+    if rows and len(shape) >= 2:
+        assert dok.storage()._layout == _lib.DOK_LAYOUT_TAGGED and dok.storage()._desc.key_bytes == 8 * len(shape)
+    return dok
+
+
 def _random_selectors(rng, shape):
     """A random indexing expression over the leading dimensions of `shape`: integers, slices,
     index tensors that broadcast to one shape, lists, and at most one 1-D mask (kept apart
@@ -549,7 +565,8 @@ def _random_selectors(rng, shape):
     return tuple(sel)
 
 
-def test_random_selectors_against_the_oracle(cuda):
+@pytest.mark.parametrize("rows", [False, True])
+def test_random_selectors_against_the_oracle(cuda, rows):
     """Differential test: random shapes (1 to 5 dimensions), random contents and random indexing
     expressions; every expression the oracle accepts is read through the HIP path and compared,
     then assigned one value through both and the tensors compared.  (Equal coordinates inside
@@ -564,8 +581,9 @@ def test_random_selectors_against_the_oracle(cuda):
         nnz = max(1, int(rng.integers(0, vol + 1)))
         idx = torch.stack(torch.unravel_index(torch.from_numpy(rng.permutation(vol)[:nnz]), shape))
         vals = torch.from_numpy(rng.integers(1, 100, size=nnz)).float()
-        dok = SparseDOKTensor(shape, idx.to(cuda), vals.to(cuda), device=cuda)
+        dok = _new_dok(shape, idx, vals, cuda, rows)
         ref = RefSparseDOKTensor(shape, idx, vals, rng=np.random.default_rng(case))
+        assert same_entries(dok, ref)
         for _ in range(4):
             sel = _random_selectors(rng, shape)
             dsel = tuple(s.to(cuda) if isinstance(s, torch.Tensor) else s for s in sel)
@@ -587,7 +605,8 @@ def test_random_selectors_against_the_oracle(cuda):
     assert compared > 200
 
 
-def test_random_selectors_through_permuted_views(cuda):
+@pytest.mark.parametrize("rows", [False, True])
+def test_random_selectors_through_permuted_views(cuda, rows):
     """The same differential test through `permute` views: reads and writes through the view must
     equal an oracle tensor built from the permuted coordinates, and the base tensor must see
     the writes (the view shares its table)."""
@@ -601,7 +620,7 @@ def test_random_selectors_through_permuted_views(cuda):
         nnz = max(1, int(rng.integers(0, vol + 1)))
         idx = torch.stack(torch.unravel_index(torch.from_numpy(rng.permutation(vol)[:nnz]), shape))
         vals = torch.from_numpy(rng.integers(1, 100, size=nnz)).float()
-        dok = SparseDOKTensor(shape, idx.to(cuda), vals.to(cuda), device=cuda)
+        dok = _new_dok(shape, idx, vals, cuda, rows)
         perm = [int(x) for x in rng.permutation(nd)]
         view = dok.permute(*perm) if case % 2 else dok.permute(perm)
         pshape = tuple(shape[p] for p in perm)
@@ -630,7 +649,8 @@ def test_random_selectors_through_permuted_views(cuda):
     assert compared > 100
 
 
-def test_random_sparse_valued_indexing_against_the_oracle(cuda):
+@pytest.mark.parametrize("rows", [False, True])
+def test_random_sparse_valued_indexing_against_the_oracle(cuda, rows):
     """Differential test of the sparse-valued paths: `__spgetitem__` of random expressions and
     `__setitem__` with a sparse source of the selection's shape (without repeated coordinates,
     where the winner among equal coordinates is not defined)."""
@@ -651,7 +671,7 @@ def test_random_sparse_valued_indexing_against_the_oracle(cuda):
         nnz = max(1, int(rng.integers(0, vol + 1)))
         idx = torch.stack(torch.unravel_index(torch.from_numpy(rng.permutation(vol)[:nnz]), shape))
         vals = torch.from_numpy(rng.integers(1, 100, size=nnz)).float()
-        dok = SparseDOKTensor(shape, idx.to(cuda), vals.to(cuda), device=cuda)
+        dok = _new_dok(shape, idx, vals, cuda, rows)
         ref = RefSparseDOKTensor(shape, idx, vals, rng=np.random.default_rng(case))
         for _ in range(4):
             sel = _random_selectors(rng, shape)
@@ -702,7 +722,7 @@ def test_wide_index_space_construct_getitem_setitem_roundtrip(cuda, size):
     gather (hits, misses, broadcast and slice selectors), scatter (new and present coordinates,
     with growth), read-out - all against the oracle."""
     dok, ref, idx, vals = _wide_pair(size, 5000, 11, cuda)
-    assert dok._wide and dok._nnz() == ref._nnz() == idx.shape[1]
+    assert dok.storage()._coord_rows and dok._nnz() == ref._nnz() == idx.shape[1]
     assert dok.storage().n_buckets == ref._hashmap.n_buckets
     assert same_entries(dok, ref)
     rng = np.random.default_rng(12)
@@ -764,7 +784,7 @@ def test_wide_many_dimensions_against_the_oracle(cuda):
     from doksparse_amd import SparseDOKTensor
     size = (3, 2, 4, 3, 2, 3, 2, 2, 3, 2)
     dok, ref, idx, vals = _wide_pair(size, 3000, 21, cuda)
-    assert dok._wide and dok.ndim == 10 and same_entries(dok, ref)
+    assert dok.storage()._coord_rows and dok.ndim == 10 and same_entries(dok, ref)
     assert torch.equal(dok.to_dense().cpu(), ref.to_dense())
     rng = np.random.default_rng(22)
     compared = 0
@@ -830,3 +850,119 @@ def test_permuted_dok_tensor_as_sparse_source(cuda):
     a[torch.tensor([7, 1, 0, 9])[:, None].to(cuda), torch.tensor([0, 11, 5, 2, 3, 8])[None, :].to(cuda)] = b.permute(1, 0)
     a_dense[torch.tensor([7, 1, 0, 9])[:, None], torch.tensor([0, 11, 5, 2, 3, 8])[None, :]] = b_dense.t()
     assert torch.equal(a.to_dense().cpu(), a_dense)
+
+
+def test_dok_entry_points_on_coordinate_rows_through_the_c_abi(cuda):
+    """The C entry points themselves on a table of int64 coordinate rows (key_bytes = 8 * ndim):
+    dok_coo_set, dok_getitem_dense, dok_setitem_dense, dok_count_items, dok_zero_items,
+    dok_coo_compact and dok_to_dense called through ctypes with hand-filled descriptors, on a
+    (2^40, 2^40) index space and on a small one that a dense torch tensor can mirror."""
+    import ctypes
+    from doksparse_amd import _lib
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def table(dims, n_buckets, vbytes=4):
+        t = _lib.DokTable()
+        mem = torch.empty(n_buckets * 128, device=cuda, dtype=torch.uint8)
+        header = torch.empty(16, device=cuda, dtype=torch.long)
+        t.buckets, t.header, t.n_phys_buckets, t.seed = mem.data_ptr(), header.data_ptr(), n_buckets, 99
+        t.key_bytes, t.value_bytes, t.lin_ndim = 8 * len(dims), vbytes, len(dims)
+        for i, d in enumerate(dims):
+            t.lin_dims[i] = d
+        assert lib.dok_table_clear(ctypes.byref(t), st) == 0
+        return t, mem, header
+
+    def index(ndim, shape, sels):
+        ix = _lib.DokIndex()
+        ix.ndim, ix.sel_ndim = ndim, len(shape)
+        for j, s in enumerate(shape):
+            ix.shape[j] = s
+        for d, (ptr, base, strides) in enumerate(sels):
+            ix.sel[d].data, ix.sel[d].base = ptr, base
+            for j, sd in enumerate(strides):
+                ix.sel[d].strides[j] = sd
+        return ix
+
+    # ---- (2^40, 2^40): 20,000 entries
+    rng = np.random.default_rng(31)
+    n = 20000
+    coords = np.ascontiguousarray(np.unique(rng.integers(0, 2**40, size=(2, n), dtype=np.int64), axis=1))
+    n = coords.shape[1]
+    vals = rng.standard_normal(n).astype(np.float32)
+    t, mem, header = table((2**40, 2**40), 16384)
+    ci, cv = torch.from_numpy(coords).to(cuda), torch.from_numpy(vals).to(cuda)
+    assert ci.is_contiguous()
+    assert lib.dok_coo_set(ctypes.byref(t), ci.data_ptr(), cv.data_ptr(), n, st) == 0
+    assert int(header[_lib.DOK_H_NELEM]) == n and int(header[_lib.DOK_H_NOOB]) == 0
+    # gather: every stored coordinate in reverse order, plus misses, through two 1-D selectors
+    q = np.concatenate([coords[:, ::-1], rng.integers(0, 2**40, size=(2, 500), dtype=np.int64)], axis=1)
+    qd = torch.from_numpy(np.ascontiguousarray(q)).to(cuda)
+    out = torch.full((q.shape[1],), -1.0, device=cuda)
+    ix = index(2, (q.shape[1],), [(qd[0].data_ptr(), 0, (1,)), (qd[1].data_ptr(), 0, (1,))])
+    assert lib.dok_getitem_dense(ctypes.byref(t), ctypes.byref(ix), out.data_ptr(), st) == 0
+    expect = np.concatenate([vals[::-1], np.zeros(500, dtype=np.float32)])
+    assert np.array_equal(out.cpu().numpy(), expect)
+    cnt = torch.zeros(1, device=cuda, dtype=torch.long)
+    assert lib.dok_count_items(ctypes.byref(t), ctypes.byref(ix), cnt.data_ptr(), st) == 0
+    assert int(cnt) == n
+    # an affine selector without a device tensor: row coords[0, 0], columns coords[1, 0] - 3 .. + 4
+    r0, c0 = int(coords[0, 0]), int(coords[1, 0])
+    lo = max(c0 - 3, 0)
+    ix2 = index(2, (8,), [(None, r0, (0,)), (None, lo, (1,))])
+    out8 = torch.full((8,), -1.0, device=cuda)
+    assert lib.dok_getitem_dense(ctypes.byref(t), ctypes.byref(ix2), out8.data_ptr(), st) == 0
+    model = {(int(a), int(b)): float(v) for a, b, v in zip(coords[0], coords[1], vals)}
+    assert out8.cpu().tolist() == [model.get((r0, lo + k), 0.0) for k in range(8)]
+    # scatter through the same descriptor (8 cells of one row), then remove them again
+    src = torch.arange(1, 9, device=cuda, dtype=torch.float32)
+    view = _lib.DokView()
+    view.data = src.data_ptr()
+    view.strides[0] = 1
+    before = sum((r0, lo + k) in model for k in range(8))
+    assert lib.dok_setitem_dense(ctypes.byref(t), ctypes.byref(ix2), ctypes.byref(view), st) == 0
+    assert int(header[_lib.DOK_H_NELEM]) == n + 8 - before
+    assert lib.dok_getitem_dense(ctypes.byref(t), ctypes.byref(ix2), out8.data_ptr(), st) == 0
+    assert out8.cpu().tolist() == list(range(1, 9))
+    assert lib.dok_zero_items(ctypes.byref(t), ctypes.byref(ix2), st) == 0
+    assert int(header[_lib.DOK_H_NELEM]) == n - before
+    # rows outside the coordinate space: skipped and counted by the insert, absent for the lookups
+    bad = torch.tensor([[2**40, -1, 5], [7, 7, 2**40 + 1]], device=cuda)
+    assert lib.dok_coo_set(ctypes.byref(t), bad.data_ptr(), cv.data_ptr(), 3, st) == 0
+    assert int(header[_lib.DOK_H_NOOB]) == 3 and int(header[_lib.DOK_H_NELEM]) == n - before
+    # read-out in COO layout
+    scratch = torch.empty(int(lib.dok_compact_scratch_bytes(ctypes.byref(t))) // 8, device=cuda, dtype=torch.long)
+    live = n - before
+    oi = torch.zeros(2, live, device=cuda, dtype=torch.long)
+    ov = torch.zeros(live, device=cuda)
+    assert lib.dok_coo_compact(ctypes.byref(t), oi.data_ptr(), ov.data_ptr(), live, cnt.data_ptr(), scratch.data_ptr(), st) == 0
+    assert int(cnt) == live
+    for k in range(8):
+        model.pop((r0, lo + k), None)
+    got = {(int(a), int(b)): float(v) for a, b, v in zip(oi[0].cpu(), oi[1].cpu(), ov.cpu())}
+    assert got == model
+    # a linear key cannot hold this space: the descriptor with key_bytes 8 is refused, not misread
+    t.key_bytes = 8
+    assert lib.dok_getitem_dense(ctypes.byref(t), ctypes.byref(ix), out.data_ptr(), st) == _lib.DOK_EUNSUPPORTED
+
+    # ---- a small 3-D space mirrored by a dense tensor; float16 values
+    dims = (6, 5, 7)
+    dense = torch.zeros(dims, dtype=torch.float16)
+    flat = torch.from_numpy(rng.permutation(6 * 5 * 7)[:90])
+    c3 = torch.stack(torch.unravel_index(flat, dims))
+    v3 = torch.from_numpy(rng.integers(1, 50, size=90)).to(torch.float16)
+    dense[tuple(c3)] = v3
+    t3, mem3, header3 = table(dims, 64, vbytes=2)
+    c3d, v3d = c3.contiguous().to(cuda), v3.to(cuda)
+    assert lib.dok_coo_set(ctypes.byref(t3), c3d.data_ptr(), v3d.data_ptr(), 90, st) == 0
+    dd = torch.zeros(dims, device=cuda, dtype=torch.float16)
+    assert lib.dok_to_dense(ctypes.byref(t3), dd.data_ptr(), st) == 0
+    assert torch.equal(dd.cpu(), dense)
+    # dok[rows[:, None], 1:4, cols[None, :]] -> (3, 2, 3) by the reference's axis rule: block first, slice after
+    rows_ = torch.tensor([4, 0, 5], device=cuda)
+    cols_ = torch.tensor([6, 2], device=cuda)
+    ix3 = index(3, (3, 2, 3), [(rows_.data_ptr(), 0, (1, 0, 0)), (None, 1, (0, 0, 1)), (cols_.data_ptr(), 0, (0, 1, 0))])
+    o3 = torch.zeros(3, 2, 3, device=cuda, dtype=torch.float16)
+    assert lib.dok_getitem_dense(ctypes.byref(t3), ctypes.byref(ix3), o3.data_ptr(), st) == 0
+    want = dense[rows_.cpu()[:, None, None], torch.arange(1, 4)[None, None, :], cols_.cpu()[None, :, None]]
+    assert torch.equal(o3.cpu(), want)

@@ -328,3 +328,80 @@ def test_table_beyond_the_bulk_limit_takes_the_per_row_kernel(cuda, monkeypatch)
     got, found = hm.get(keys)
     assert bool(found.all()) and torch.equal(got, values)
     assert not bool(hm.get(keys + 1)[1].any())
+
+
+def test_coordinate_row_tensor_10m_entries(cuda):
+    """A (2^40, 2^40) tensor - its coordinates cannot be linearised into one 8-byte key and are
+    stored as two-word keys - with 10M entries: construct, gather of 4M elements (half stored, half
+    absent), scatter of 4M (half present, half new, with a growth of the table), sparse-valued
+    gather, read-out.  The independent map is a sorted array: the coordinates are drawn as
+    c = (r << 20) | f(r) with r < 2^20, so that a pair of them has a 40-bit name (r0, r1) of its
+    own that the table never sees."""
+    from doksparse_amd import SparseDOKTensor, _lib
+    gen = torch.Generator(device=cuda).manual_seed(4040)
+    size = (2**40, 2**40)
+
+    def spread(r):
+        return (r << 20) | ((r * 0x9E3779B1) & 0xFFFFF)
+
+    def names(n):
+        lin = torch.unique(torch.randint(0, 2**40, (n,), generator=gen, device=cuda))
+        return lin[torch.randperm(lin.numel(), generator=gen, device=cuda)]
+
+    lin = names(10_000_000)
+    nnz = lin.numel()
+    coords = torch.stack([spread(lin >> 20), spread(lin & 0xFFFFF)])
+    assert int(coords.max()) >= 2**39
+    vals = torch.randn(nnz, generator=gen, device=cuda)
+    dok = SparseDOKTensor(size, coords, vals, device=cuda)
+    hm = dok.storage()
+    assert hm._coord_rows and hm._layout == _lib.DOK_LAYOUT_TAGGED and hm._desc.key_bytes == 16
+    assert dok._nnz() == nnz
+    smap = SortedMap(lin, vals)
+
+    # gather: 2M stored coordinates, 1M absent pairs of the same form, 1M arbitrary coordinates
+    pick = torch.randint(0, nnz, (2_000_000,), generator=gen, device=cuda)
+    other = torch.randint(0, 2**40, (1_000_000,), generator=gen, device=cuda)
+    qlin = torch.cat([lin[pick], other])
+    q = torch.stack([spread(qlin >> 20), spread(qlin & 0xFFFFF)])
+    q = torch.cat([q, torch.randint(0, 2**40, (2, 1_000_000), generator=gen, device=cuda)], dim=1)
+    exp = torch.cat([smap.get(qlin)[0], torch.zeros(1_000_000, device=cuda)])
+    order = torch.randperm(q.shape[1], generator=gen, device=cuda)
+    q, exp = q[:, order].contiguous(), exp[order]
+    got = dok[q[0], q[1]]
+    assert torch.equal(got, exp) and int((exp != 0).sum()) >= 2_000_000
+    # the same as a 2-D expression: 2048 stored rows x 2048 columns (mostly absent cells)
+    rr, cc = coords[0, :2048], coords[1, 5000:7048]
+    got2 = dok[rr[:, None], cc[None, :]]
+    lin2 = ((rr >> 20)[:, None] << 20) + (cc >> 20)[None, :]
+    assert torch.equal(got2.reshape(-1), smap.get(lin2.reshape(-1))[0])
+
+    # scatter: 2M stored + 2M fresh coordinates; the table has to grow
+    flin = names(2_200_000)
+    flin = flin[~smap.get(flin)[1]][:2_000_000]
+    wl = torch.cat([lin[:2_000_000], flin])
+    wl = wl[torch.randperm(wl.numel(), generator=gen, device=cuda)]
+    wc = torch.stack([spread(wl >> 20), spread(wl & 0xFFFFF)])
+    wv = torch.randn(wl.numel(), generator=gen, device=cuda)
+    n_before = hm.n_buckets
+    dok[wc[0], wc[1]] = wv
+    assert dok._nnz() == nnz + flin.numel()
+    assert hm.n_buckets == int(np.ceil((nnz + wl.numel()) * 2.0)) > n_before      # grown as the reference would
+    keep = ~SortedMap(wl, wv).get(lin)[1]
+    smap2 = SortedMap(torch.cat([lin[keep], wl]), torch.cat([vals[keep], wv]))
+    assert torch.equal(dok[q[0], q[1]][order.argsort()][:3_000_000], smap2.get(qlin)[0])
+
+    # read-out: exactly the entries, each once
+    idx, v = dok.indices(), dok.values()
+    assert idx.shape == (2, nnz + flin.numel())
+    assert torch.equal(spread(idx[0] >> 20), idx[0]) and torch.equal(spread(idx[1] >> 20), idx[1])
+    rl = ((idx[0] >> 20) << 20) + (idx[1] >> 20)
+    so = torch.argsort(rl)
+    assert torch.equal(rl[so], smap2.keys) and torch.equal(v[so], smap2.values)
+
+    # count / remove of the first gather's elements
+    n_stored = int(smap2.get(qlin)[1].sum())
+    assert int(dok.count_items((q[0], q[1])).item()) == n_stored
+    dok.zero_items((q[0], q[1]))
+    assert dok._nnz() == nnz + flin.numel() - int(smap2.get(torch.unique(qlin))[1].sum())
+    assert int(dok.count_items((q[0], q[1])).item()) == 0

@@ -47,10 +47,11 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_struct_sizes_match_the_header():
-    # dok_table_t: 2 pointers + 2 x 8 + 4 x 4 + 8 x 8 bytes; dok_view_t: pointer + 8 x 8
-    assert ctypes.sizeof(_lib.DokTable) == 8 + 8 + 8 + 8 + 16 + 64
-    assert ctypes.sizeof(_lib.DokView) == 8 + 8 + 64
-    assert ctypes.sizeof(_lib.DokIndex) == 8 + 64 + 8 * (8 + 8 + 64)
+    # dok_table_t: 2 pointers + 2 x 8 + 4 x 4 + 14 x 8 bytes; dok_view_t: pointer + 8 + 14 x 8
+    assert _lib.DOK_MAX_DIMS == 14
+    assert ctypes.sizeof(_lib.DokTable) == 8 + 8 + 8 + 8 + 16 + 14 * 8
+    assert ctypes.sizeof(_lib.DokView) == 8 + 8 + 14 * 8
+    assert ctypes.sizeof(_lib.DokIndex) == 8 + 14 * 8 + 14 * (8 + 8 + 14 * 8)
 
 
 def test_layout_selection():
