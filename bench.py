@@ -43,6 +43,7 @@ PROFILED = {
     "remove_lf05": 5.688e9,      # p8_remove_kernel, half of the keys, plain-store tombstones
     # bench.py --only-tagged (profiles/tagged_32M_f32x3_i64x5.txt), load factor 0.5
     "tagged_set_lf05": 11.84e9,        # tg_set_kernel, 32M fresh float32[3] -> int64[5] rows
+    "tagged_build_lf05": None,         # dok_fill_kernel + tg_fast_set_kernel + tg_deferred_kernel
     "tagged_overwrite_lf05": None,
     "tagged_get_lf05": 6.07e9,         # tg_lookup_kernel<0, false, 8>, 32M queries
     "tagged_remove_lf05": None,
@@ -354,6 +355,14 @@ def tagged_scale(device, n=32_000_000):
         rem = lambda: _lib.check(lib.dok_map_remove_unique(desc, quarter.data_ptr(), n // 4, out_f.data_ptr(), stream), "remove")
         s_avg, _ = time_kernel(set_, 3, prep=clear)
         assert hm.n_elements == n
+        # the same rows as the first batch of a new map takes them: clear + insert with one
+        # compare-and-swap per row, in one call (dok_map_build_bulk)
+        nws = int(lib.dok_bulk_workspace_bytes(desc, n))
+        ws = torch.empty(nws, device=device, dtype=torch.uint8)
+        build = lambda: _lib.check(lib.dok_map_build_bulk(desc, k.data_ptr(), v.data_ptr(), n, ws.data_ptr(), nws, stream), "build")
+        b_avg, _ = time_kernel(build, 3)
+        assert hm.n_elements == n
+        del ws
         o_avg, _ = time_kernel(set_, 3)
         get()
         assert int(out_f.sum().item()) == n // 2
@@ -361,7 +370,8 @@ def tagged_scale(device, n=32_000_000):
         probe = hm.probe_stats(q)
         r_avg, _ = time_kernel(rem, 1)
         assert hm.n_elements == n - n // 4
-        for nm, ms in (("set", s_avg), ("overwrite", o_avg), ("get", g_avg), ("remove", r_avg)):
+        res[f"tagged_build_mops_{tag}"] = round(n / b_avg / 1e3, 1)
+        for nm, ms in (("set", s_avg), ("build", b_avg), ("overwrite", o_avg), ("get", g_avg), ("remove", r_avg)):
             res[f"tagged_{nm}_ms_{tag}"] = round(ms, 4)
         res[f"tagged_set_mops_{tag}"] = round(n / s_avg / 1e3, 1)
         res[f"tagged_overwrite_mops_{tag}"] = round(n / o_avg / 1e3, 1)
@@ -732,6 +742,7 @@ def main():
         results.update(dk)
         for name, entry, ms, ops in (
                 ("tagged_set_32M_lf05", "tagged_set_lf05", tg["tagged_set_ms_lf05"], nt),
+                ("tagged_build_32M_lf05", "tagged_build_lf05", tg["tagged_build_ms_lf05"], nt),
                 ("tagged_overwrite_32M_lf05", "tagged_overwrite_lf05", tg["tagged_overwrite_ms_lf05"], nt),
                 ("tagged_get_32M_lf05", "tagged_get_lf05", tg["tagged_get_ms_lf05"], nt),
                 ("tagged_remove_8M_lf05", "tagged_remove_lf05", tg["tagged_remove_ms_lf05"], nt // 4),

@@ -91,6 +91,7 @@ SIGNATURES = {
     "dok_map_rehash_bulk": (c_int32, [POINTER(DokTable), POINTER(DokTable), c_void_p, c_int64, c_void_p]),
     "dok_getitem_dense": (c_int32, [POINTER(DokTable), POINTER(DokIndex), c_void_p, c_void_p]),
     "dok_setitem_dense": (c_int32, [POINTER(DokTable), POINTER(DokIndex), POINTER(DokView), c_void_p]),
+    "dok_setitem_dense_bulk": (c_int32, [POINTER(DokTable), POINTER(DokIndex), POINTER(DokView), c_void_p, c_int64, c_void_p]),
     "dok_count_items": (c_int32, [POINTER(DokTable), POINTER(DokIndex), c_void_p, c_void_p]),
     "dok_zero_items": (c_int32, [POINTER(DokTable), POINTER(DokIndex), c_void_p]),
     "dok_getitem_sparse": (c_int32, [POINTER(DokTable), POINTER(DokIndex), POINTER(DokTable), c_void_p]),

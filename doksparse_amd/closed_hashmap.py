@@ -46,6 +46,9 @@ def _stream_ptr(device):
 # million rows into a table at 85 % with tombstones), so there the bulk path pays from fewer
 # rows per bucket on.
 BULK_MIN_ROWS = 1 << 20
+# The multi-word layout's bulk form (one compare-and-swap per new row, a deferred list, two more
+# small launches) pays from a few tens of thousands of rows on.
+TAGGED_FAST_MIN_ROWS = 1 << 15
 BULK_MIN_ROWS_PER_BUCKET = 2.0
 BULK_MIN_ROWS_PER_BUCKET_LOADED = 1.5
 BULK_LOADED_FILL = 0.7
@@ -510,8 +513,10 @@ class CudaClosedHashmap:
         """Workspace tensor for a bulk insert of n rows, or None if the batch should take the
         per-row kernel."""
         if self._layout != _lib.DOK_LAYOUT_PACKED8:
-            return None
-        if not bulk_pays(n, self._n_phys, self._slots_per_bucket, self._n_upper):
+            # served for values of one word, and for the first batch of a new table
+            if n < TAGGED_FAST_MIN_ROWS or not (self._value_bytes <= 8 or self._pending_clear):
+                return None
+        elif not bulk_pays(n, self._n_phys, self._slots_per_bucket, self._n_upper):
             return None
         nbytes = int(_lib.load().dok_bulk_workspace_bytes(ctypes.byref(self._desc), n))
         if nbytes <= 0:

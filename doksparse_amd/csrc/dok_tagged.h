@@ -761,6 +761,239 @@ __device__ __forceinline__ void tg_place_rows(const DevTable &t, const TgGeom &g
   }
 }
 
+// ---- insert with ONE compare-and-swap per new row (batches with a workspace) ------------------------
+// The protocol above costs a new row three write transactions (claim, payload, publish) because a
+// row with the same key on another XCD must never read a half-written slot.  tg_fast_rows drops
+// that guarantee and does not need it: a new row claims an EMPTY slot with one compare-and-swap
+// EMPTY -> FULL and its group writes the payload with plain stores, and a row that cannot tell
+// what it sees is DEFERRED - put on a list in the caller's workspace - and inserted by the protocol
+// above in a second launch, when everything the first one wrote is visible.  Rules per row:
+//   * a slot with the row's tag: compare the key words.  Equal: the key is present (or an equal row
+//     of this batch has just claimed the slot: same bytes either way) - the value, a single 8-byte
+//     word, is overwritten with one store, which cannot tear.  Not equal: a payload in flight or a
+//     fingerprint collision: defer.
+//   * a tag BUSY with the row's fingerprint: a tombstone being re-used (below): look again.
+//   * otherwise the first free slot of the walk, after the displacement checks of tg_insert_rows.
+//     EMPTY: claim -> FULL, payload by plain stores.  A TOMBSTONE keeps the key words of the entry
+//     that was removed, which a concurrent row could mistake for a payload, so it is claimed the
+//     slow way (BUSY, write-through payload, publish).  A claim lost to the row's own tag: defer.
+//   * a row whose key words are all zero is deferred at once: zero is what the key words of a
+//     never-used slot hold, so for every other key "the key words equal mine" proves a payload.
+// Only values of one word can be overwritten without a lock, so this form serves tables with
+// VW == 1 (every coordinate table).  FRESH - the table held nothing when the kernel started, so
+// whatever a row meets was claimed by this kernel - compares nothing, overwrites nothing (a slot with
+// the row's tag: defer) and serves any widths.  (Claiming without looking first - one compare-and-swap
+// per slot tried, the returned tag telling what holds it - was measured and is slower: 32M rows of 52
+// bytes at load factor 0.5 take 3.4 ms against 3.05 ms, at 0.75 5.3 against 3.6 ms: a returning
+// atomic costs more than the loads of a bucket's tags.)
+template <bool FRESH>
+__device__ __forceinline__ void tg_fast_rows(const DevTable &t, const TgGeom &g, const TgLane &L,
+                                             const u64 *lds_rows, const u64 *lds_vals, u32 home, u32 qfull,
+                                             bool pend, int &st, int &fresh, bool &deferred) {
+  const int RS = tg_rs(g);
+  const int wave_row0 = threadIdx.x & ~63;
+  const u64 *krow = lds_rows + threadIdx.x * RS;
+  if (!FRESH && pend) {
+    u64 any = 0;
+    for (int k = 0; k < g.KW; k++) any |= krow[1 + k];
+    if (any == 0) { deferred = true; pend = false; }
+  }
+  if (!pend) home = 0;
+  const u32 qbusy = qfull & ~1u;
+  const u32 fbit = tg_fbit(qfull);
+  const bool has_filter = g.S >= 2;
+  u32 cur = 0, md_home = 0, filt_home = 0;
+  bool chosen = false, slot_tomb = false, far_unb = false;
+  u32 slot_d = 0, slot_w = 0, chk = 0, far_next = 0, far_to = 0;
+
+  u64 pm = dok_ballot(pend);
+  while (pm != 0) {
+    const u32 b = pend ? tg_wrap(home, cur, t.nb) : 0u;
+    u64 *bucket = t.buckets + (u64)b * 16;
+    bool wr = false, wr_slow = false;
+    u32 wr_b = 0, wr_w = 0;
+    u64 tw[DOK_TG_MAXS];
+    #pragma unroll
+    for (int s = 0; s < DOK_TG_MAXS; s++) {
+      tw[s] = 0;
+      if (s < g.S && pend) tw[s] = dok_load_coherent(bucket + s * g.W);
+    }
+    const u32 md = (u32)(tw[0] >> 32);
+    u32 candm = 0, emptym = 0, tombm = 0;
+    bool busy = false;
+    #pragma unroll
+    for (int s = 0; s < DOK_TG_MAXS; s++) {
+      if (s < g.S) {
+        const u32 t32 = (u32)tw[s];
+        candm |= (u32)(t32 == qfull) << s;
+        busy = busy || t32 == qbusy;
+        emptym |= (u32)(t32 == DOK_TG_EMPTY) << s;
+        tombm |= (u32)(t32 == DOK_TG_TOMB) << s;
+      }
+    }
+    if (pend) {
+      if (candm) {
+        // (FRESH: whatever carries this fingerprint was claimed by this kernel, its payload may be in
+        // flight: nothing to compare)
+        bool hit = false;
+        u32 c = FRESH ? 0u : candm;
+        while (c != 0 && !hit) {
+          const int s = __builtin_ctz(c);
+          c &= c - 1;
+          bool eq = true;
+          for (int k = 0; k < g.KW; k++) eq = eq && dok_load_coherent(bucket + s * g.W + 1 + k) == krow[1 + k];
+          if (eq) {
+            bucket[s * g.W + 1 + g.KW] = lds_vals[threadIdx.x * g.VW];       // (VW == 1: one word, one store)
+            hit = true;
+          }
+        }
+        if (hit) st = 1; else deferred = true;
+        pend = false;
+      } else if (busy) {
+        // a tombstone being re-used by a row of this fingerprint: its holder publishes within its turn
+      } else {
+        if (!chosen) {
+          if (cur == 0) { md_home = md; filt_home = (u32)(tw[1] >> 32); }
+          if (tombm | emptym) {
+            chosen = true;
+            slot_tomb = tombm != 0;
+            slot_d = cur;
+            slot_w = (u32)(__builtin_ctz(tombm ? tombm : emptym) * g.W);
+            chk = cur < DOK_TG_NEAR ? (md_home & DOK_TG_NEARMASK & ~((2u << cur) - 1u)) : 0u;
+            far_unb = (md_home & 1u) && (md_home >> 24) == DOK_TG_FARCAP;
+            far_to = (md_home & 1u) ? (far_unb ? 0xffffffffu : (md_home >> 24)) : 0u;
+            far_next = cur + 1 > DOK_TG_NEAR + 1u ? cur + 1 : DOK_TG_NEAR + 1u;
+            if (has_filter && !(filt_home & fbit)) { chk = 0; far_to = 0; }
+            if (FRESH) { chk = 0; far_to = 0; }               // nothing was in the table: nothing to find further on
+          } else if ((u64)cur + 1 >= t.nb) {
+            st = 0; pend = false;                              // no free slot anywhere
+          } else {
+            cur++;
+          }
+        } else if (far_unb && cur > DOK_TG_NEAR && emptym) {
+          far_to = 0;
+        }
+        if (pend && chosen) {
+          bool claim = false;
+          if (chk) { cur = (u32)__builtin_ctz(chk); chk &= chk - 1; }
+          else if (far_next <= far_to && (u64)far_next < t.nb) cur = far_next++;
+          else claim = true;
+          if (claim) {
+            const u32 tb = tg_wrap(home, slot_d, t.nb);
+            u32 *tagp = (u32 *)(t.buckets + (u64)tb * 16 + slot_w);
+            const u32 expect = slot_tomb ? DOK_TG_TOMB : DOK_TG_EMPTY;
+            const u32 old = atomicCAS(tagp, expect, slot_tomb ? qbusy : qfull);
+            if (old == expect) {
+              wr = true; wr_slow = slot_tomb; wr_b = tb; wr_w = slot_w;
+              st = 1; fresh = 1; pend = false;
+              if (slot_d > 0) tg_mark(t.buckets + (u64)home * 16, slot_d, md_home, has_filter ? g.W : 0, fbit, filt_home);
+            } else if ((old | 1u) == qfull) {
+              deferred = true; pend = false;                   // a row with this fingerprint took the slot
+            } else {
+              chosen = false; cur = slot_d;                    // somebody else's key: look at that bucket again
+            }
+          }
+        }
+      }
+    }
+
+    // ---- the slots won in this turn: lane p of the row's group stores word p of the payload
+    const u64 wm = dok_ballot(wr);
+    if (wm != 0) {
+      const u32 wsub = L.grp(wm);
+      u32 wany = (u32)wm | (u32)(wm >> 32);
+      wany = (wany | (wany >> 16)) & 0xffffu;
+      #pragma unroll
+      for (int r = 0; r < 16; r++) {
+        if (!((wany >> r) & 1u)) continue;
+        const int j = L.gbase + r;
+        const u32 qb = dok_shfl32(wr_b, j), qw = dok_shfl32(wr_w, j);
+        const bool slow = dok_shfl32((u32)wr_slow, j) != 0;
+        if (((wsub >> r) & 1u) && L.l >= 1 && L.l < g.W) {
+          const u64 word = L.l <= g.KW ? lds_rows[(wave_row0 + j) * RS + L.l]
+                                       : lds_vals[(wave_row0 + j) * g.VW + L.l - 1 - g.KW];
+          u64 *dst = t.buckets + (u64)qb * 16 + qw + L.l;
+          if (slow) dok_store_coherent(dst, word); else *dst = word;
+        }
+      }
+      if (dok_ballot(wr_slow) != 0) {
+        // re-used tombstones: the payload has completed before the tag is published
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (wr_slow) __hip_atomic_store((u32 *)(t.buckets + (u64)wr_b * 16 + wr_w), qfull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    pm = dok_ballot(pend);
+  }
+}
+
+// Workspace of the fast insert: a counter and the list of the deferred rows' numbers.
+struct TgDeferList {
+  u64 *count;        // [1] (cleared by tg_defer_clear_kernel)
+  i64 *rows;         // [cap]
+  i64 cap;
+};
+__global__ void tg_defer_clear_kernel(TgDeferList dl) { if (threadIdx.x == 0) dl.count[0] = 0; }
+
+template <class Src, bool FRESH>
+__global__ __launch_bounds__(DOK_TPB) void tg_fast_set_kernel(DevTable t, TgGeom g, Src src, i64 n, TgDeferList dl) {
+  extern __shared__ u64 lds[];
+  const int RS = tg_rs(g);
+  u64 *lds_rows = lds;
+  u64 *lds_vals = lds + DOK_TPB * RS;
+  const TgLane L(g);
+  int n_fresh = 0, n_full = 0, n_oob = 0;
+  DOK_TILE_LOOP(n) {
+    const i64 i = DOK_TILE_ROW();
+    const bool inside = i < n;
+    u64 *krow = lds_rows + threadIdx.x * RS;
+    const int code = inside ? src.stage(t, g, i, krow, lds_vals + threadIdx.x * g.VW) : 2;
+    const bool active = code == 0;
+    n_oob += code == 1;
+    u32 home, qfull;
+    tg_hash_row(t, g, krow, home, qfull);
+    int st = 0, fresh = 0;
+    bool deferred = false;
+    tg_fast_rows<FRESH>(t, g, L, lds_rows, lds_vals, home, qfull, active, st, fresh, deferred);
+    // the deferred rows of the wave go on the list with one atomic
+    const u64 dm = dok_ballot(deferred);
+    if (dm != 0) {
+      u64 base = 0;
+      if (L.lane == 0) base = atomicAdd(dl.count, (u64)__popcll(dm));
+      base = dok_shfl64(base, 0);
+      const i64 at = (i64)base + __popcll(dm & ((1ULL << L.lane) - 1ULL));
+      if (deferred && at < dl.cap) dl.rows[at] = i;
+    }
+    n_fresh += fresh;
+    n_full += (active && !deferred && st == 0);
+  }
+  dok_block_add3(&t.header[DOK_H_NELEM], n_fresh, &t.header[DOK_H_NFULL], n_full, &t.header[DOK_H_NOOB], n_oob);
+}
+
+// Second launch of the fast insert: the deferred rows, by the ordinary protocol.
+template <class Src>
+__global__ __launch_bounds__(DOK_TPB) void tg_deferred_kernel(DevTable t, TgGeom g, Src src, TgDeferList dl) {
+  extern __shared__ u64 lds[];
+  const int RS = tg_rs(g);
+  u64 *lds_rows = lds;
+  u64 *lds_vals = lds + DOK_TPB * RS;
+  const TgLane L(g);
+  const i64 n = (i64)dl.count[0] < dl.cap ? (i64)dl.count[0] : dl.cap;
+  int n_fresh = 0, n_full = 0;
+  DOK_TILE_LOOP(n) {
+    const i64 k = DOK_TILE_ROW();
+    const bool inside = k < n;
+    u64 *krow = lds_rows + threadIdx.x * RS;
+    const bool active = inside && src.stage(t, g, dl.rows[k], krow, lds_vals + threadIdx.x * g.VW) == 0;
+    u32 home, qfull;
+    tg_hash_row(t, g, krow, home, qfull);
+    int st = 0, fresh = 0;
+    tg_insert_rows(t, g, L, lds_rows, lds_vals, home, qfull, active, st, fresh);
+    n_fresh += fresh;
+    n_full += (active && st == 0);
+  }
+  dok_block_add2(&t.header[DOK_H_NELEM], n_fresh, &t.header[DOK_H_NFULL], n_full);
+}
+
 // Upsert of the rows a source delivers (see the row sources above).
 template <class Src>
 __global__ __launch_bounds__(DOK_TPB) void tg_set_kernel(DevTable t, TgGeom g, Src src, i64 n, u8 *__restrict__ stored) {
@@ -990,6 +1223,32 @@ static int tg_launch_set(const DevTable &d, const Src &src, i64 n, u8 *stored, h
   if (rc) return rc;
   const unsigned grid = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
   tg_set_kernel<Src><<<(grid < DOK_TG_SET_GRID ? grid : DOK_TG_SET_GRID), DOK_TPB, tg_lds_insert(g), s>>>(d, g, src, n, stored);
+  return DOK_OK;
+}
+
+// Workspace bytes of the fast insert for n rows, and its layout.
+static i64 tg_fast_workspace_bytes(i64 n) { return 256 + 8 * n; }
+// Whether the fast insert serves this table (fresh = it holds nothing: every width; else one-word values).
+static bool tg_fast_serves(const DevTable &d, bool fresh) { return fresh || d.value_bytes <= 8; }
+
+// fresh: the table has just been cleared (or is cleared here: `clear`), nothing else is in it.
+template <class Src>
+static int tg_launch_set_fast(const DevTable &d, const Src &src, i64 n, bool fresh, void *workspace, hipStream_t s) {
+  TgGeom g;
+  int rc = tg_geom(d, nullptr, g);
+  if (rc) return rc;
+  TgDeferList dl;
+  dl.count = (u64 *)workspace;
+  dl.rows = (i64 *)((char *)workspace + 256);
+  dl.cap = n;
+  const unsigned tiles = (unsigned)((n + DOK_TPB - 1) / DOK_TPB);
+  const unsigned grid = tiles < DOK_TG_SET_GRID ? tiles : DOK_TG_SET_GRID;
+  tg_defer_clear_kernel<<<1, 64, 0, s>>>(dl);
+  if (fresh) tg_fast_set_kernel<Src, true><<<grid, DOK_TPB, tg_lds_insert(g), s>>>(d, g, src, n, dl);
+  else tg_fast_set_kernel<Src, false><<<grid, DOK_TPB, tg_lds_insert(g), s>>>(d, g, src, n, dl);
+  // (the deferred rows are few - equal keys inside the batch, re-used fingerprints - and the grid is
+  // sized for a list that nobody knows yet: its workgroups find the count on the device)
+  tg_deferred_kernel<Src><<<(tiles < 1024u ? tiles : 1024u), DOK_TPB, tg_lds_insert(g), s>>>(d, g, src, dl);
   return DOK_OK;
 }
 

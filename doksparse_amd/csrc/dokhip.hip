@@ -367,8 +367,9 @@ int64_t dok_bulk_workspace_bytes(const dok_table_t *t, int64_t n) {
   DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
+  if (layout != DOK_LAYOUT_PACKED8) return n >= 1 && n <= kMaxRows ? tg_fast_workspace_bytes(n) : 0;
   BulkPlan p;
-  if (layout != DOK_LAYOUT_PACKED8 || !bulk_plan(d, n, p)) return 0;
+  if (!bulk_plan(d, n, p)) return 0;
   return (int64_t)p.bytes;
 }
 
@@ -383,8 +384,29 @@ static int set_bulk(const dok_table_t *t, const void *keys, const void *values, 
   if (n < 0) return DOK_EINVAL;
   if (n == 0) return fresh ? DOK_EINVAL : DOK_OK;      // a build writes the table: it needs rows
   if (!keys || !values || !workspace) return DOK_EINVAL;
+  if (layout != DOK_LAYOUT_PACKED8) {
+    // multi-word layout: the insert with one compare-and-swap per new row and a list of deferred rows
+    if (n > kMaxRows || ((uintptr_t)workspace & 255) != 0 || workspace_bytes < tg_fast_workspace_bytes(n)) return DOK_EINVAL;
+    hipStream_t s = (hipStream_t)stream;
+    const DeviceScope on_stream_device(s);
+    if (fresh) {
+      const i64 words = (i64)d.nb * 16;
+      dok_fill_kernel<<<(unsigned)((words / 4 + DOK_TPB - 1) / DOK_TPB), DOK_TPB, 0, s>>>(d.buckets, words, d.header);
+    }
+    if (cols) {
+      if (((uintptr_t)keys & 7) != 0 || ((uintptr_t)values & (uintptr_t)(d.value_bytes - 1)) != 0) return DOK_EINVAL;
+      const TgCols c{(const i64 *)keys, n, (const u8 *)values};
+      rc = tg_fast_serves(d, fresh) ? tg_launch_set_fast(d, c, n, fresh, workspace, s) : tg_launch_set(d, c, n, nullptr, s);
+    } else {
+      TgRows r;
+      rc = tg_rows(d, keys, values, r);
+      if (!rc) rc = tg_fast_serves(d, fresh) ? tg_launch_set_fast(d, r, n, fresh, workspace, s) : tg_launch_set(d, r, n, nullptr, s);
+    }
+    if (rc) return rc;
+    return note_launch();
+  }
   BulkPlan p;
-  if (layout != DOK_LAYOUT_PACKED8 || !bulk_plan(d, n, p)) return DOK_EUNSUPPORTED;
+  if (!bulk_plan(d, n, p)) return DOK_EUNSUPPORTED;
   if (((uintptr_t)workspace & 255) != 0 || workspace_bytes < (int64_t)p.bytes) return DOK_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
@@ -672,6 +694,27 @@ int dok_setitem_dense(const dok_table_t *t, const dok_index_t *ix, const dok_vie
   const DeviceScope on_stream_device(s);
   const unsigned grid = grid_counting(di.n_elems);
   P8_DISPATCH(d.value_bytes, (p8_setitem_kernel<V><<<grid, DOK_TPB, 0, s>>>(d, di, rows_per_wave(di.n_elems, grid))));
+  return note_launch();
+}
+
+int dok_setitem_dense_bulk(const dok_table_t *t, const dok_index_t *ix, const dok_view_t *src, void *workspace,
+                           int64_t workspace_bytes, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (!is_coord_rows(d, layout)) return dok_setitem_dense(t, ix, src, stream);    // (no use for the workspace)
+  if (!src || !workspace) return DOK_EINVAL;
+  TgIndexSrc isrc;
+  rc = make_dev_index(d, ix, src, isrc.ix);
+  if (rc) return rc;
+  const i64 n = isrc.ix.n_elems;
+  if (n == 0) return DOK_OK;
+  if (n > kMaxRows || ((uintptr_t)src->data & (uintptr_t)(d.value_bytes - 1)) != 0) return DOK_EINVAL;
+  if (((uintptr_t)workspace & 255) != 0 || workspace_bytes < tg_fast_workspace_bytes(n)) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
+  rc = tg_launch_set_fast(d, isrc, n, false, workspace, s);
+  if (rc) return rc;
   return note_launch();
 }
 

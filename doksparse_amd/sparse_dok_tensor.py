@@ -526,8 +526,13 @@ class SparseDOKTensor(object):
             if n_now + n_sel > limit:
                 hm.rehash(int(np.ceil((n_now + n_sel) * hm._rehash_factor)))
         lib = _lib.load()
-        _lib.check(lib.dok_setitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), ctypes.byref(view),
-                                         _stream_ptr(self.device)), "__setitem__")
+        ws = hm._bulk_workspace(n_sel) if hm._coord_rows else None
+        if ws is not None:
+            _lib.check(lib.dok_setitem_dense_bulk(ctypes.byref(hm._desc), ctypes.byref(ix), ctypes.byref(view),
+                                                  ws.data_ptr(), ws.numel(), _stream_ptr(self.device)), "__setitem__")
+        else:
+            _lib.check(lib.dok_setitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), ctypes.byref(view),
+                                             _stream_ptr(self.device)), "__setitem__")
         header = hm._read_header()
         hm._n_upper = int(header[_lib.DOK_H_NELEM])
         n_oob = int(header[_lib.DOK_H_NOOB])

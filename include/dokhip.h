@@ -157,12 +157,18 @@ int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int6
  * through `workspace`, each bin of a pass owning a region of fixed capacity there) and every
  * range of buckets is merged in LDS, so the table is streamed through the GPU once.  Rows whose
  * bin's region is full (batches with very many equal keys) take the per-row insert at the end;
- * header[DOK_H_NSPILL] says how many.  Packed layout only.
+ * header[DOK_H_NSPILL] says how many.
+ * On the multi-word layout the bulk entry points run another fast form: a new row claims its slot
+ * with ONE compare-and-swap and plain stores (dok_map_set: claim, payload and publish are three
+ * write transactions); a row that meets its own fingerprint in flight - equal keys inside the batch,
+ * mostly - is put on a list in the workspace and inserted by a second launch.  That form serves
+ * tables with values of at most 8 bytes (every coordinate table) and, for dok_map_build_bulk /
+ * dok_coo_build_bulk, any widths; other tables take the dok_map_set kernel, same result.
  *   dok_bulk_workspace_bytes: device bytes dok_map_set_bulk / dok_coo_set_bulk need for n rows;
- *     0 if the bulk path cannot take this table or n (tagged layout, n >= 2^31, more than
+ *     0 if the bulk path cannot take this table or n (packed layout: n >= 2^31 or more than
  *     2^28 buckets: use dok_map_set), negative on a bad table.
- *     (about 3.4 times the bytes of the batch: two partition buffers with slack and the spill
- *     list, plus 4 bytes per 256 buckets of the table).
+ *     (packed layout: about 3.4 times the bytes of the batch - two partition buffers with slack
+ *     and the spill list - plus 4 bytes per 256 buckets of the table; multi-word layout: 8 n + 256).
  *   workspace: device, 256-byte aligned, at least that many bytes; contents need no
  *     initialisation and are garbage afterwards.  Calls sharing one workspace must be ordered.
  * Reference: the same closed_hashmap_set launch as dok_map_set, at the batch sizes of
@@ -262,7 +268,7 @@ int dok_map_rehash_bulk(const dok_table_t *src, const dok_table_t *dst, void *wo
 int dok_coo_set(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
                 void *stream);
 
-/* dok_coo_set through the bulk path (see dok_map_set_bulk; tables of linearised keys only). */
+/* dok_coo_set through the bulk path (see dok_map_set_bulk). */
 int dok_coo_set_bulk(const dok_table_t *t, const int64_t *indices, const void *values, int64_t n,
                      void *workspace, int64_t workspace_bytes, void *stream);
 
@@ -288,6 +294,14 @@ int dok_getitem_dense(const dok_table_t *t, const dok_index_t *ix, void *out, vo
  * Reference: sparse_dok_set_items_dense (sparse_dok_tensor_impl.cu:271-313). */
 int dok_setitem_dense(const dok_table_t *t, const dok_index_t *ix, const dok_view_t *src,
                       void *stream);
+
+/* dok_setitem_dense for large scatters into a table of coordinate rows (key_bytes = 8 * lin_ndim):
+ * the fast insert of the multi-word layout (see dok_map_set_bulk), which needs a workspace of
+ * dok_bulk_workspace_bytes(t, number of elements of the index space) bytes, 256-byte aligned.  On a
+ * table of linearised keys the call is dok_setitem_dense and the workspace is not used.
+ * Reference: sparse_dok_set_items_dense (sparse_dok_tensor_impl.cu:271-313). */
+int dok_setitem_dense_bulk(const dok_table_t *t, const dok_index_t *ix, const dok_view_t *src,
+                           void *workspace, int64_t workspace_bytes, void *stream);
 
 /* count[0] += number of elements whose coordinate is stored.
  * Reference: sparse_dok_count_items (sparse_dok_tensor_impl.cu:4-56). */

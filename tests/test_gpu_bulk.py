@@ -208,12 +208,15 @@ def test_bulk_entry_point_rejects_bad_arguments(cuda):
     assert lib.dok_map_set_bulk(desc, None, v.data_ptr(), 100, ws.data_ptr(), need, None) == _lib.DOK_EINVAL
     assert lib.dok_map_set_bulk(desc, k.data_ptr(), v.data_ptr(), 0, ws.data_ptr(), need, None) == _lib.DOK_OK
     assert lib.dok_coo_set_bulk(desc, k.data_ptr(), v.data_ptr(), 100, ws.data_ptr(), need, None) == _lib.DOK_EINVAL
-    # the tagged layout has no bulk path
+    # the multi-word layout's bulk form needs the list of deferred rows: 8 bytes per row + 256
     hm2 = CudaClosedHashmap(n_buckets=256, device=cuda)
-    hm2.set(torch.rand(10, 3, device=cuda), torch.zeros(10, 5, device=cuda, dtype=torch.long))
-    assert int(lib.dok_bulk_workspace_bytes(ctypes.byref(hm2._desc), 10)) == 0
-    assert lib.dok_map_set_bulk(ctypes.byref(hm2._desc), k.data_ptr(), v.data_ptr(), 10, ws.data_ptr(), need, None) \
-        == _lib.DOK_EUNSUPPORTED
+    k2, v2 = torch.rand(10, 3, device=cuda), torch.zeros(10, 5, device=cuda, dtype=torch.long)
+    hm2.set(k2, v2)
+    assert int(lib.dok_bulk_workspace_bytes(ctypes.byref(hm2._desc), 10)) == 8 * 10 + 256
+    assert lib.dok_map_set_bulk(ctypes.byref(hm2._desc), k2.data_ptr(), v2.data_ptr(), 10, ws.data_ptr(), 8 * 10 + 248, None) \
+        == _lib.DOK_EINVAL
+    assert lib.dok_coo_set_bulk(ctypes.byref(hm2._desc), k2.data_ptr(), v2.data_ptr(), 10, ws.data_ptr(), need, None) \
+        == _lib.DOK_EINVAL                                   # not a coordinate table
     torch.cuda.synchronize()
     assert hm.n_elements == 100
 
@@ -595,3 +598,126 @@ def test_bulk_and_per_row_agree_on_coordinate_batches(cuda, monkeypatch, size):
         for got in per_layout:
             assert got[2:] == ref[2:]
             assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+
+
+# ---- the multi-word layout's bulk form: one compare-and-swap per new row, deferred rows in a second launch
+
+@pytest.fixture
+def tagged_fast_always(monkeypatch):
+    from doksparse_amd import closed_hashmap as ch
+    monkeypatch.setattr(ch, "TAGGED_FAST_MIN_ROWS", 0)
+    return ch
+
+
+def test_multiword_fast_and_per_row_insert_agree_on_random_configurations(cuda, monkeypatch):
+    """Random configurations of the multi-word layout (key / value widths of one to four slots per
+    bucket, load factors up to 0.95, batches with many repeated keys, the all-zero key, removals in
+    between so that tombstones are re-used): three batches each, once through the per-row protocol
+    and once through the fast form - the first batch of a map as a build into the new table, later
+    ones as upserts where the values are one word wide.  Values are a function of key and batch, so
+    the resulting map is unique and must be the same."""
+    from doksparse_amd import CudaClosedHashmap, closed_hashmap as ch, _lib
+    rng = np.random.default_rng(77)
+    geoms = [(2, torch.int64, 1, torch.float32), (3, torch.float32, 5, torch.int64), (13, torch.int64, 1, torch.float16),
+             (4, torch.int64, 1, torch.int64), (2, torch.int64, 1, torch.int8), (5, torch.int32, 2, torch.int64)]
+
+    def val_of(keys, rnd, vw, dt):
+        x = (keys.to(torch.int64).sum(dim=1) * 2654435761 + rnd * 97) >> 5
+        cols = torch.stack([(x + 13 * c) % 251 - 125 for c in range(vw)], dim=1)
+        return cols.to(dt)
+
+    for case in range(18):
+        kw, kdt, vw, vdt = geoms[case % len(geoms)]
+        n = int(10 ** rng.uniform(2.5, 5.3))
+        lf = float(rng.uniform(0.2, 0.95))
+        universe = int(n * rng.uniform(0.3, 1.5)) + 10
+        cap = int(universe / lf) + 16
+        g = torch.Generator(device=cuda); g.manual_seed(case)
+        if kdt.is_floating_point:
+            keyspace = torch.randint(-2**20, 2**20, (universe, kw), generator=g, device=cuda).to(kdt)
+        else:
+            keyspace = torch.randint(-2**30, 2**30, (universe, kw), generator=g, device=cuda).to(kdt)
+        keyspace[0] = 0                                  # the all-zero key (always deferred by the fast form)
+        keyspace = torch.unique(keyspace, dim=0)
+        universe = keyspace.shape[0]
+        maps = []
+        for fast in (False, True):
+            monkeypatch.setattr(ch, "TAGGED_FAST_MIN_ROWS", 0 if fast else 1 << 62)
+            hm = CudaClosedHashmap(n_buckets=cap, device=cuda, rehash_threshold=1e9, seed=501 + case)
+            gg = torch.Generator(device=cuda); gg.manual_seed(2000 + case)
+            for rnd in range(3):
+                pick = torch.randint(0, universe, (n,), generator=gg, device=cuda)
+                pick[:3] = 0                             # the zero key, three times in every batch
+                k = keyspace[pick]
+                hm.set(k, val_of(k, rnd, vw, vdt))
+                assert hm._layout == _lib.DOK_LAYOUT_TAGGED
+                if rnd < 2:
+                    gone = keyspace[torch.randint(0, universe, (n // 4,), generator=gg, device=cuda)]
+                    hm._remove_rows(gone.contiguous())
+            h = hm._header.cpu()
+            keys, vals = hm.items()
+            kb = keys.contiguous().view(torch.uint8).reshape(keys.shape[0], -1).cpu().numpy()
+            order = np.lexsort(kb.T[::-1])
+            maps.append((kb[order], vals.cpu().numpy()[order], int(h[0]), int(h[1])))
+        a, b = maps
+        assert a[2] == b[2] == a[0].shape[0] and a[3] == b[3] == 0, (case, a[2:], b[2:])
+        assert np.array_equal(a[0], b[0]), f"case {case}: key sets differ"
+        assert np.array_equal(a[1].view(np.uint8), b[1].view(np.uint8)), f"case {case}: values differ"
+        assert len({r.tobytes() for r in a[0]}) == a[0].shape[0], f"case {case}: a key is stored twice"
+
+
+def test_multiword_fast_insert_with_nothing_but_equal_keys(cuda, tagged_fast_always):
+    """A batch of 200,000 rows that holds 5 distinct keys (every row but five is deferred), as the
+    first batch of a map and as an upsert: one slot per key, an untorn value of one of its rows."""
+    from doksparse_amd import CudaClosedHashmap
+    g = torch.Generator(device=cuda).manual_seed(9)
+    base = torch.randint(-2**40, 2**40, (5, 2), generator=g, device=cuda)
+    pick = torch.randint(0, 5, (200_000,), generator=g, device=cuda)
+    rowv = torch.arange(200_000, device=cuda, dtype=torch.float32)[:, None]
+    for first in (True, False):
+        hm = CudaClosedHashmap(n_buckets=4096, device=cuda)
+        if not first:
+            hm.set(torch.randint(2**41, 2**42, (1000, 2), generator=g, device=cuda), torch.zeros(1000, 1, device=cuda))
+        hm.set(base[pick], rowv)
+        assert hm.n_elements == 5 + (0 if first else 1000)
+        v, f = hm.get(base)
+        assert bool(f.all())
+        for j in range(5):
+            r = int(v[j, 0].item())
+            assert int(pick[r].item()) == j             # the stored value is the row number of a row of that key
+
+
+def test_multiword_bulk_entry_points_through_the_c_abi(cuda):
+    """dok_bulk_workspace_bytes / dok_map_set_bulk / dok_map_build_bulk on a multi-word table, called
+    through ctypes: the build takes the table as uninitialised memory, bad workspaces are refused."""
+    from doksparse_amd import CudaClosedHashmap, _lib
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    lib = _lib.load()
+    rng = np.random.default_rng(3)
+    n = 50_000
+    keys = np.unique(rng.random((n, 3), dtype=np.float32), axis=0)
+    n = keys.shape[0]
+    vals = rng.integers(0, 2**62, size=(n, 5), dtype=np.int64)
+    hm = CudaClosedHashmap(n_buckets=2 * n, device=cuda, rehash_threshold=1e9)
+    k, v = _to(cuda, keys, vals)
+    hm.set(k[:4], v[:4])
+    desc, st = ctypes.byref(hm._desc), _stream_ptr(cuda)
+    need = int(lib.dok_bulk_workspace_bytes(desc, n))
+    assert need == 8 * n + 256
+    ws = torch.empty(need, device=cuda, dtype=torch.uint8)
+    hm._table.fill_(0xA5)                                # garbage: the build must not read it
+    hm._header.fill_(-77)
+    assert lib.dok_map_build_bulk(desc, k.data_ptr(), v.data_ptr(), n, ws.data_ptr(), need, st) == 0
+    ref = RefClosedHashmap(n_buckets=2 * n, rng=np.random.default_rng(8))
+    ref.set(keys, vals)
+    assert hm.n_elements == ref.n_elements == n
+    _assert_same_map(hm, ref)
+    # upsert with 40-byte values: no fast form for them, the per-row protocol runs instead - same result
+    vals2 = vals + 1
+    assert lib.dok_map_set_bulk(desc, k.data_ptr(), torch.from_numpy(vals2).to(cuda).data_ptr(), n, ws.data_ptr(), need, st) == 0
+    ref.set(keys, vals2)
+    _assert_same_map(hm, ref)
+    assert lib.dok_map_set_bulk(desc, k.data_ptr(), v.data_ptr(), n, ws.data_ptr(), need - 8, st) == _lib.DOK_EINVAL
+    assert lib.dok_map_set_bulk(desc, k.data_ptr(), v.data_ptr(), n, ws.data_ptr() + 8, need, st) == _lib.DOK_EINVAL
+    assert lib.dok_map_set_bulk(desc, k.data_ptr(), v.data_ptr(), n, None, need, st) == _lib.DOK_EINVAL
+    _assert_same_map(hm, ref)

@@ -565,14 +565,18 @@ def _random_selectors(rng, shape):
     return tuple(sel)
 
 
-@pytest.mark.parametrize("rows", [False, True])
-def test_random_selectors_against_the_oracle(cuda, rows):
+@pytest.mark.parametrize("rows", [False, True, "fast"])
+def test_random_selectors_against_the_oracle(cuda, rows, monkeypatch):
     """Differential test: random shapes (1 to 5 dimensions), random contents and random indexing
     expressions; every expression the oracle accepts is read through the HIP path and compared,
     then assigned one value through both and the tensors compared.  (Equal coordinates inside
     one assignment: the reference over-counts its element counter, so the entry count is compared
     with the oracle's distinct coordinates.)"""
-    from doksparse_amd import SparseDOKTensor
+    from doksparse_amd import SparseDOKTensor, closed_hashmap as ch
+    if rows == "fast":
+        # every insert through the form with one compare-and-swap per new row and a deferred list
+        # (by itself only batches of tens of thousands of rows take it)
+        monkeypatch.setattr(ch, "TAGGED_FAST_MIN_ROWS", 0)
     rng = np.random.default_rng(20)
     compared = 0
     for case in range(80):
