@@ -442,6 +442,31 @@ def dok_scale(device):
     return res
 
 
+def gather_scale(device, n):
+    """Uniformly random, naturally aligned granules of 128, 64 and 32 bytes of the default workload's
+    load-factor-0.5 table (n keys, 13.4M buckets = 1.72 GB at n = 2^26), n granules per launch: what
+    a lookup could cost at most if a probe needed only half or a quarter of a bucket line."""
+    from doksparse_amd import _lib
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    lib = _lib.load()
+    gen = torch.Generator(device=device)
+    gen.manual_seed(1003)
+    keys = make_unique_keys(n, gen, device)
+    values = torch.randn(n, generator=gen, device=device, dtype=torch.float32)
+    hm = build_map(keys, values, 2 * n, device)
+    out = torch.empty(n, device=device, dtype=torch.int32)
+    res = {"gather_table_bytes": hm._n_phys * 128, "gather_granules_per_launch": n}
+    for gb in (128, 64, 32):
+        fn = lambda: _lib.check(lib.dok_line_gather_granule(ctypes.byref(hm._desc), n, 12345, gb, out.data_ptr(),
+                                                            _stream_ptr(device)), "gather")
+        fn()
+        avg, _ = time_kernel(fn, 10)
+        res[f"gather_{gb}B_ms"] = round(avg, 4)
+        res[f"gather_{gb}B_ggranules_s"] = round(n / avg / 1e6, 2)
+        res[f"gather_{gb}B_payload_gbs"] = round(n * gb / avg / 1e6, 1)
+    return res
+
+
 def dok_wide_scale(device, nnz=10_000_000, n_q=1 << 22):
     """A tensor whose coordinates do not fit one 8-byte key, (2^40, 2^40), beside one of the same
     content whose do, (2^20, 2^20): the same 10M entries (the small tensor's coordinates, spread
@@ -497,6 +522,9 @@ def main():
     ap.add_argument("--tagged", action="store_true", help="(kept for old command lines: this leg now always runs)")
     ap.add_argument("--only-tagged", action="store_true",
                     help="run nothing but the --tagged leg and print its figures (for profiling that leg)")
+    ap.add_argument("--only-gather", action="store_true",
+                    help="run nothing but the random-granule gather (128, 64 and 32 bytes) over the "
+                         "load-factor-0.5 table of the default workload, and print its rates")
     ap.add_argument("--only-wide", action="store_true",
                     help="run nothing but the wide-tensor legs of --only-dok")
     ap.add_argument("--only-dok", action="store_true",
@@ -518,6 +546,9 @@ def main():
     torch.cuda.set_device(device)
     if args.only_tagged:
         print(json.dumps({"extra": tagged_scale(device)}), flush=True)
+        return
+    if args.only_gather:
+        print(json.dumps({"extra": gather_scale(device, args.keys)}), flush=True)
         return
     if args.only_wide:
         print(json.dumps({"extra": dok_wide_scale(device)}), flush=True)

@@ -99,6 +99,7 @@ SIGNATURES = {
                                      c_uint64, c_void_p]),
     "dok_to_dense": (c_int32, [POINTER(DokTable), c_void_p, c_void_p]),
     "dok_line_gather": (c_int32, [POINTER(DokTable), c_int64, c_uint64, c_void_p, c_void_p]),
+    "dok_line_gather_granule": (c_int32, [POINTER(DokTable), c_int64, c_uint64, c_int32, c_void_p, c_void_p]),
 }
 
 _lib = None

@@ -160,27 +160,30 @@ __global__ __launch_bounds__(DOK_TPB) void dok_fill_kernel(u64 *p, i64 words, i6
   if (blockIdx.x == 0 && threadIdx.x < DOK_HEADER_WORDS) header[threadIdx.x] = 0;
 }
 
-// Measurement aid: every 16-lane group loads `per_group` pseudo-random 128-byte lines of the
-// bucket array (8 bytes per lane, eight independent loads in flight) and folds what it read into
-// one word per line.  This is the access pattern of a lookup with the probing taken out, so its
-// rate is the practical ceiling of the lookup kernels on a given table.
-__global__ __launch_bounds__(DOK_TPB) void dok_line_gather_kernel(const u64 *__restrict__ lines, u64 n_lines,
+// Measurement aid: every group of LANES adjacent lanes loads pseudo-random, naturally aligned
+// granules of LANES * 8 bytes of the bucket array (8 bytes per lane, eight independent loads in
+// flight) and folds what it read into one word per granule.  With 16 lanes this is the access
+// pattern of a lookup with the probing taken out - one 128-byte bucket line per row - so its rate is
+// the practical ceiling of the lookup kernels on a given table; 8 and 4 lanes answer what a probe
+// of half or a quarter of a line would cost instead.
+template <int LANES>
+__global__ __launch_bounds__(DOK_TPB) void dok_line_gather_kernel(const u64 *__restrict__ lines, u64 n_granules,
                                                                   i64 n, u64 seed, u32 *__restrict__ out) {
-  const int l = threadIdx.x & 15;
-  const i64 group = ((i64)blockIdx.x * DOK_TPB + threadIdx.x) >> 4;
-  const i64 n_groups = ((i64)gridDim.x * DOK_TPB) >> 4;
+  const int l = threadIdx.x & (LANES - 1);
+  const i64 group = ((i64)blockIdx.x * DOK_TPB + threadIdx.x) / LANES;
+  const i64 n_groups = ((i64)gridDim.x * DOK_TPB) / LANES;
   for (i64 base = group * 8; base < n; base += n_groups * 8) {
     u64 v[8];
 #pragma unroll
     for (int u = 0; u < 8; u++) {
-      const u64 line = dok_reduce(dok_fmix64((u64)(base + u) ^ seed), n_lines);
-      v[u] = lines[line * 16 + l];
+      const u64 gi = dok_reduce(dok_fmix64((u64)(base + u) ^ seed), n_granules);
+      v[u] = lines[gi * LANES + l];
     }
 #pragma unroll
     for (int u = 0; u < 8; u++) {
       u32 x = (u32)v[u] ^ (u32)(v[u] >> 32);
-      x ^= __shfl_xor(x, 8, 16); x ^= __shfl_xor(x, 4, 16);
-      x ^= __shfl_xor(x, 2, 16); x ^= __shfl_xor(x, 1, 16);
+#pragma unroll
+      for (int o = LANES / 2; o > 0; o >>= 1) x ^= __shfl_xor(x, o, LANES);
       if (l == 0 && base + u < n) out[base + u] = x;
     }
   }

@@ -864,19 +864,31 @@ int dok_to_dense(const dok_table_t *t, void *dense, void *stream) {
   return note_launch();
 }
 
-int dok_line_gather(const dok_table_t *t, int64_t n, uint64_t seed, uint32_t *out, void *stream) {
+int dok_line_gather_granule(const dok_table_t *t, int64_t n, uint64_t seed, int32_t granule_bytes, uint32_t *out,
+                            void *stream) {
   DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);
   if (rc) return rc;
   if (n < 0 || (n > 0 && !out)) return DOK_EINVAL;
+  if (granule_bytes != 128 && granule_bytes != 64 && granule_bytes != 32) return DOK_EINVAL;
   if (n == 0) return DOK_OK;
+  const int lanes = granule_bytes / 8;
+  const u64 n_granules = d.nb * (u64)(128 / granule_bytes);
+  if (n_granules > 0xffffffffULL) return DOK_EUNSUPPORTED;
   const i64 groups = (n + 7) / 8;
-  i64 blocks = (groups * 16 + DOK_TPB - 1) / DOK_TPB;
+  i64 blocks = (groups * lanes + DOK_TPB - 1) / DOK_TPB;
   if (blocks > 16384) blocks = 16384;
-  const DeviceScope on_stream_device((hipStream_t)stream);
-  dok_line_gather_kernel<<<(unsigned)blocks, DOK_TPB, 0, (hipStream_t)stream>>>(
-      (const u64 *)d.buckets, d.nb, n, seed, out);
+  hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
+  const u64 *lines = (const u64 *)d.buckets;
+  if (lanes == 16) dok_line_gather_kernel<16><<<(unsigned)blocks, DOK_TPB, 0, s>>>(lines, n_granules, n, seed, out);
+  else if (lanes == 8) dok_line_gather_kernel<8><<<(unsigned)blocks, DOK_TPB, 0, s>>>(lines, n_granules, n, seed, out);
+  else dok_line_gather_kernel<4><<<(unsigned)blocks, DOK_TPB, 0, s>>>(lines, n_granules, n, seed, out);
   return note_launch();
+}
+
+int dok_line_gather(const dok_table_t *t, int64_t n, uint64_t seed, uint32_t *out, void *stream) {
+  return dok_line_gather_granule(t, n, seed, 128, out, stream);
 }
 
 }  // extern "C"

@@ -339,6 +339,12 @@ int dok_to_dense(const dok_table_t *t, void *dense, void *stream);
  * for lookups on this table; the benchmark reports it beside the published HBM peak. */
 int dok_line_gather(const dok_table_t *t, int64_t n, uint64_t seed, uint32_t *out, void *stream);
 
+/* The same with granules of 128, 64 or 32 bytes (naturally aligned pieces of the bucket array, read
+ * by 16, 8 or 4 lanes): what a probe of half or a quarter of a bucket line would cost.  No
+ * counterpart in the reference. */
+int dok_line_gather_granule(const dok_table_t *t, int64_t n, uint64_t seed, int32_t granule_bytes,
+                            uint32_t *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -452,9 +452,11 @@ def test_completely_full_tables_exercise_far_displacements(cuda, vdtype):
         _assert_same_map(hm, ref)
 
 
-def test_line_gather_measurement_kernel_reads_the_lines_it_claims(cuda):
-    """dok_line_gather: out[i] = XOR of the sixteen 8-byte words (folded to 32 bits) of bucket
-    (fmix64(i ^ seed) >> 32) * n_buckets >> 32, recomputed here from a copy of the table."""
+@pytest.mark.parametrize("granule", [128, 64, 32])
+def test_line_gather_measurement_kernel_reads_the_lines_it_claims(cuda, granule):
+    """dok_line_gather / dok_line_gather_granule: out[i] = XOR of the 8-byte words (folded to 32 bits)
+    of granule (fmix64(i ^ seed) >> 32) * n_granules >> 32 of the bucket array, recomputed here from
+    a copy of the table."""
     import ctypes
     from doksparse_amd import CudaClosedHashmap, _lib
     from doksparse_amd.closed_hashmap import _stream_ptr
@@ -464,9 +466,15 @@ def test_line_gather_measurement_kernel_reads_the_lines_it_claims(cuda):
     hm.set(torch.from_numpy(k[:, None]).to(cuda), torch.from_numpy(k[:, None].astype(np.float32)).to(cuda))
     n, seed = 4099, 987654321
     out = torch.zeros(n, device=cuda, dtype=torch.int32)
-    _lib.check(_lib.load().dok_line_gather(ctypes.byref(hm._desc), n, seed, out.data_ptr(), _stream_ptr(cuda)),
-               "line_gather")
-    table = hm._table.view(torch.int64).reshape(hm._n_phys, 16).cpu().numpy().view(np.uint64)
+    lib = _lib.load()
+    if granule == 128:
+        _lib.check(lib.dok_line_gather(ctypes.byref(hm._desc), n, seed, out.data_ptr(), _stream_ptr(cuda)), "line_gather")
+    else:
+        _lib.check(lib.dok_line_gather_granule(ctypes.byref(hm._desc), n, seed, granule, out.data_ptr(),
+                                               _stream_ptr(cuda)), "line_gather")
+    words = granule // 8
+    n_gran = hm._n_phys * (128 // granule)
+    table = hm._table.view(torch.int64).reshape(n_gran, words).cpu().numpy().view(np.uint64)
     M = (1 << 64) - 1
     expect = np.empty(n, dtype=np.uint32)
     for i in range(n):
@@ -474,10 +482,11 @@ def test_line_gather_measurement_kernel_reads_the_lines_it_claims(cuda):
         x ^= x >> 33; x = (x * 0xff51afd7ed558ccd) & M
         x ^= x >> 33; x = (x * 0xc4ceb9fe1a85ec53) & M
         x ^= x >> 33
-        line = ((x >> 32) * hm._n_phys) >> 32
+        line = ((x >> 32) * n_gran) >> 32
         w = int(np.bitwise_xor.reduce(table[line]))
         expect[i] = (w ^ (w >> 32)) & 0xffffffff
     assert np.array_equal(out.cpu().numpy().view(np.uint32), expect)
+    assert lib.dok_line_gather_granule(ctypes.byref(hm._desc), n, seed, 48, out.data_ptr(), None) == _lib.DOK_EINVAL
 
 
 def test_calls_replay_inside_a_hip_graph(cuda):
