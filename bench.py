@@ -408,7 +408,8 @@ def dok_scale(device):
     n_g = 1 << 26
     pick = torch.randint(0, lin.numel(), (n_g,), generator=gen, device=device)
     r, c = coords[0][pick].contiguous(), coords[1][pick].contiguous()
-    ix, out_shape, _, keep = dok._plan((r, c))
+    plan, keep = dok._plan((r, c))
+    ix = plan.ix
     out = torch.empty(n_g, device=device, dtype=torch.float32)
     gather = lambda: _lib.check(lib.dok_getitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), out.data_ptr(), stream), "getitem")
     gather()
@@ -416,12 +417,13 @@ def dok_scale(device):
     g_avg, _ = time_kernel(gather, 5)
     res["dok_getitem_2p26_ms"] = round(g_avg, 4)
     res["dok_getitem_2p26_mops"] = round(n_g / g_avg / 1e3, 1)
-    del pick, r, c, out, ix, keep
+    del pick, r, c, out, ix, keep, plan
     # scatter: 5M present + 5M new coordinates
     sc = torch.cat([coords[:, :5_000_000], torch.randint(0, 10**6, (2, 5_000_000), generator=gen, device=device)], dim=1)
     sc = sc[:, torch.randperm(sc.shape[1], generator=gen, device=device)].contiguous()
     sv = torch.randn(sc.shape[1], generator=gen, device=device)
-    ix, _, _, keep = dok._plan((sc[0], sc[1]))
+    plan, keep = dok._plan((sc[0], sc[1]))
+    ix = plan.ix
     view = _lib.DokView()
     view.data = sv.data_ptr()
     view.strides[0] = 1
@@ -436,7 +438,7 @@ def dok_scale(device):
     ro, _ = timed(lambda: hm.items_coo())
     res["dok_readout_ms"] = round(ro, 4)
     res["dok_entries"] = hm.n_elements
-    del dok, hm, coords, vals, lin, sc, sv, ix, keep
+    del dok, hm, coords, vals, lin, sc, sv, ix, keep, plan
     torch.cuda.empty_cache()
     res.update(dok_wide_scale(device))
     return res

@@ -144,7 +144,7 @@ class _TableState:
 
 _SHARED = ("_table", "_header", "_desc", "_n_phys", "_slots_per_bucket", "_layout", "_n_buckets",
            "_key_shape", "_key_dtype", "_value_shape", "_value_dtype", "_key_bytes", "_value_bytes",
-           "_n_upper", "_seed", "_pending_clear")
+           "_n_upper", "_n_exact", "_seed", "_pending_clear")
 
 
 def _forward(name):
@@ -218,8 +218,10 @@ class CudaClosedHashmap:
         self._value_dtype = None
         self._key_bytes = 0
         self._value_bytes = 0
-        # host-side upper bound of n_elements; lets set() skip the device read-back
+        # host-side upper bound of n_elements; lets set() skip the device read-back.  _n_exact: the
+        # bound IS the count (read from the table header, nothing enqueued since that could change it)
         self._n_upper = 0
+        self._n_exact = True
         # True only inside set()/set_coo(), between the allocation of the table and its first
         # insert: the bucket memory is still uninitialised (a bulk build writes all of it)
         self._pending_clear = False
@@ -316,7 +318,16 @@ class CudaClosedHashmap:
     def n_elements(self):
         n = int(self._read_header()[_lib.DOK_H_NELEM])
         self._n_upper = n
+        self._n_exact = True
         return n
+
+    def _touch(self):
+        """Called by whatever enqueues a kernel that may change the number of entries."""
+        self._n_exact = False
+
+    def _count_now(self):
+        """n_elements, without the device read-back when the host already knows it."""
+        return self._n_upper if self._n_exact else self.n_elements
 
     @property
     def n_buckets(self):
@@ -531,6 +542,7 @@ class CudaClosedHashmap:
         lib = _lib.load()
         n = keys.shape[1] if coo else keys.shape[0]
         desc, stream = ctypes.byref(self._desc), _stream_ptr(self.device)
+        self._touch()
         ws = self._bulk_workspace(n)
         if ws is not None and self._pending_clear:
             # first insert into a new table: the build writes every bucket, no clear needed
@@ -596,7 +608,7 @@ class CudaClosedHashmap:
             self._launch_checked(lambda: self._launch_set(keys, values), n)
             return
         self._ensure_cleared()
-        n_old = self.n_elements
+        n_old = self._count_now()
         if n_old + n <= limit:
             self._launch_checked(lambda: self._launch_set(keys, values), n)
             return
@@ -614,6 +626,8 @@ class CudaClosedHashmap:
         n_miss = n - int(self.count_existing(keys).item())
         if n_old + n_miss <= limit:
             self._launch_checked(lambda: self._launch_set(keys, values), n_miss)
+            if n_miss == 0:
+                self._n_exact = True          # every key was present: the batch only overwrites values
             return
         # otherwise count the distinct new keys exactly, as the reference does
         _, is_found = self.get(keys)
@@ -656,7 +670,7 @@ class CudaClosedHashmap:
             self._launch_checked(launch, n)
             return
         self._ensure_cleared()
-        n_old = self.n_elements
+        n_old = self._count_now()
         if n_old + n <= limit:
             self._launch_checked(launch, n)
         elif n_old + n <= int(0.9 * self._physical_slots()):
@@ -772,6 +786,7 @@ class CudaClosedHashmap:
         n = keys.shape[0]
         is_removed = torch.empty(n, device=self.device, dtype=torch.bool)
         lib = _lib.load()
+        self._touch()
         fn = lib.dok_map_remove_unique if unique else lib.dok_map_remove
         _lib.check(fn(ctypes.byref(self._desc), keys.data_ptr(), n,
                       is_removed.data_ptr(), _stream_ptr(self.device)), "remove")

@@ -70,9 +70,34 @@ def _mask_indices(mask, device):
     return idx
 
 
+class _Plan(object):
+    """A filled dok_index_t and what goes with it.  Plans are kept per tensor, keyed by the
+    STRUCTURE of the indexing expression (kinds of the selectors, slice bounds, shapes and strides of
+    the index tensors, identity and version of masks): a later expression of the same structure
+    only refreshes the integer bases and the data pointers (`patches`) instead of normalising the
+    selectors, laying out the result and filling the descriptor again - which is most of the host
+    time of a small indexing call."""
+    __slots__ = ("ix", "ref", "views", "out_shape", "final_shape", "scalar_positions", "patches", "masks")
+
+
+_PLAN_CACHE_SIZE = 32
+
+try:
+    _raw_stream = torch._C._cuda_getCurrentRawStream
+except AttributeError:                                     # (older torch: the documented way)
+    _raw_stream = None
+
+
+def _stream_of(device):
+    if _raw_stream is not None:
+        return _raw_stream(device.index or 0)
+    return torch.cuda.current_stream(device).cuda_stream
+
+
 class SparseDOKTensor(object):
     def __init__(self, size, indices=None, values=None, device=None, dtype=None, storage=None):
         assert isinstance(size, (list, tuple))
+        self._plans = {}
         self._size = torch.Size(size)
         # view dimension i addresses dimension _perm[i] of the storage (identity unless the tensor
         # was made by permute/transpose, which share the storage)
@@ -229,6 +254,7 @@ class SparseDOKTensor(object):
         new = SparseDOKTensor(size=tuple(self._size), device=self.device, dtype=self.dtype)
         new._hashmap = self._hashmap.clone(deepclone=deepclone)
         new._perm = self._perm
+        new._plans = {}
         return new
 
     # ------------------------------------------------------------------ read-out
@@ -302,6 +328,7 @@ class SparseDOKTensor(object):
         self._hashmap = new
         self._size = torch.Size(new_size)
         self._perm = tuple(range(len(new_size)))
+        self._plans = {}
         if idx is not None:
             self._store_coo(idx.contiguous(), values)
             new._header[_lib.DOK_H_NOOB] = 0          # entries outside the new size are dropped
@@ -439,11 +466,57 @@ class SparseDOKTensor(object):
             keep.append(sel)
         return ix, out_shape
 
+    def _plan_key(self, selectors):
+        """Hashable structure of an indexing expression, or None when it holds selectors that are
+        converted on the way (lists, numpy arrays, tensors of another dtype or on another device)."""
+        key = []
+        for sel in selectors:
+            t = type(sel)
+            if t is int:
+                key.append(0)
+            elif t is slice:
+                key.append((sel.start, sel.stop, sel.step))
+            elif t is Tensor:
+                if sel.device != self.device:
+                    return None
+                if sel.dtype is torch.bool:
+                    key.append((id(sel), sel._version, None))
+                elif sel.dtype is torch.long:
+                    key.append((sel.shape, sel.stride()))
+                else:
+                    return None
+            else:
+                return None
+        return tuple(key)
+
     def _plan(self, selectors):
         """dok_index_t straight from the expression: integers and slices become affine
         selectors that need no device tensor (no arange kernel, no host-to-device copy of a
-        scalar); only real index tensors are passed by pointer.  Returns (descriptor, result
-        shape, scalar positions, tensors to keep alive until the launch)."""
+        scalar); only real index tensors are passed by pointer.  Returns (plan, tensors to keep alive
+        until the launch)."""
+        if not isinstance(selectors, tuple):
+            selectors = (selectors,)
+        key = self._plan_key(selectors)
+        plan = self._plans.get(key) if key is not None else None
+        if plan is not None:
+            keep = []
+            views = plan.views
+            for code, pos, sd in plan.patches:
+                sel = selectors[pos]
+                if code == 0:
+                    views[sd].base = sel
+                elif code == 1:
+                    views[sd].data = sel.data_ptr()
+                else:
+                    if plan.masks[pos]() is not sel:          # another tensor at a recycled address
+                        plan = None
+                        break
+                    idx = _mask_indices(sel, self.device)
+                    for m, d in enumerate(sd):
+                        views[d].data = idx[m].data_ptr()
+                    keep.append(idx)
+            if plan is not None:
+                return plan, keep
         flat = self._normalise(selectors)
         bshape, first, slice_axis, out_shape, scalar_positions = self._layout(flat)
         if len(out_shape) > self._max_axes():
@@ -467,24 +540,49 @@ class SparseDOKTensor(object):
                 strides[first:first + len(bshape)] = view.stride()
                 self._fill_index(ix, self._perm[d], view.data_ptr(), 0, strides)
                 keep.append(view)
-        return ix, out_shape, scalar_positions, keep
+        plan = _Plan()
+        plan.ix, plan.ref = ix, ctypes.byref(ix)
+        plan.views = [ix.sel[d] for d in range(self.ndim)]
+        plan.out_shape, plan.scalar_positions = out_shape, scalar_positions
+        # the reference squeezes the output axis numbered like each scalar selector's position
+        final = list(out_shape)
+        for i in reversed(scalar_positions):
+            if i < len(final) and final[i] == 1:
+                del final[i]
+        plan.final_shape = tuple(final)
+        if key is not None:
+            # which tensor dimension(s) every selector of the expression feeds (a mask of k
+            # dimensions stands for k of them)
+            plan.patches, plan.masks, d = [], {}, 0
+            for pos, sel in enumerate(selectors):
+                if type(sel) is int:
+                    plan.patches.append((0, pos, self._perm[d]))
+                    d += 1
+                elif type(sel) is slice:
+                    d += 1
+                elif sel.dtype is torch.bool:
+                    plan.patches.append((2, pos, tuple(self._perm[d + m] for m in range(sel.ndim))))
+                    plan.masks[pos] = weakref.ref(sel)
+                    d += sel.ndim
+                else:
+                    plan.patches.append((1, pos, self._perm[d]))
+                    d += 1
+            if len(self._plans) >= _PLAN_CACHE_SIZE:
+                self._plans.pop(next(iter(self._plans)))
+            self._plans[key] = plan
+        return plan, keep
 
     # ------------------------------------------------------------------ indexing
     def __getitem__(self, selectors):
-        ix, out_shape, scalar_positions, keep = self._plan(selectors)
+        plan, keep = self._plan(selectors)
         hm = self._hashmap
         if not hm._allocated:
-            values = torch.zeros(out_shape, device=self.device, dtype=self.dtype)
-        else:
-            values = torch.empty(out_shape, device=self.device, dtype=self.dtype)
-            if values.numel():
-                lib = _lib.load()
-                _lib.check(lib.dok_getitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), values.data_ptr(),
-                                                 _stream_ptr(self.device)), "__getitem__")
-        # the reference squeezes the output axis numbered like each scalar selector's position
-        for i in reversed(scalar_positions):
-            if i < values.ndim:
-                values = values.squeeze(i)
+            return torch.zeros(plan.final_shape, device=self.device, dtype=self._dtype)
+        values = torch.empty(plan.final_shape, device=self.device, dtype=self._dtype)
+        if values.numel():
+            rc = _lib.load().dok_getitem_dense(ctypes.byref(hm._desc), plan.ref, values.data_ptr(), _stream_of(self.device))
+            if rc:
+                _lib.check(rc, "__getitem__")
         return values
 
     def __setitem__(self, selectors, values):
@@ -494,11 +592,11 @@ class SparseDOKTensor(object):
             assert tuple(values.shape) == out_shape, \
                 f"expecting the value shape to be {out_shape}, got {tuple(values.shape)} instead"
             return self._set_items_sparse(values, mats)
-        ix, out_shape, _, keep = self._plan(selectors)
+        plan, keep = self._plan(selectors)
         if not isinstance(values, Tensor):
             values = torch.tensor(values, device=self.device, dtype=self.dtype)
-        values = torch.broadcast_to(values.to(device=self.device, dtype=self.dtype), out_shape)
-        self._set_items_dense(values, ix, selectors)
+        values = torch.broadcast_to(values.to(device=self.device, dtype=self.dtype), plan.out_shape)
+        self._set_items_dense(values, plan.ix, selectors)
 
     def _set_items_dense(self, src, ix, expr):
         """Reference: SparseDOKTensorImplCuda.set_items_dense (sparse_dok_tensor_impl.py:412-474).
@@ -526,6 +624,7 @@ class SparseDOKTensor(object):
             if n_now + n_sel > limit:
                 hm.rehash(int(np.ceil((n_now + n_sel) * hm._rehash_factor)))
         lib = _lib.load()
+        hm._touch()
         ws = hm._bulk_workspace(n_sel) if hm._coord_rows else None
         if ws is not None:
             _lib.check(lib.dok_setitem_dense_bulk(ctypes.byref(hm._desc), ctypes.byref(ix), ctypes.byref(view),
@@ -534,7 +633,7 @@ class SparseDOKTensor(object):
             _lib.check(lib.dok_setitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), ctypes.byref(view),
                                              _stream_ptr(self.device)), "__setitem__")
         header = hm._read_header()
-        hm._n_upper = int(header[_lib.DOK_H_NELEM])
+        hm._n_upper, hm._n_exact = int(header[_lib.DOK_H_NELEM]), True
         n_oob = int(header[_lib.DOK_H_NOOB])
         if n_oob:
             hm._header[_lib.DOK_H_NOOB] = 0
@@ -580,7 +679,7 @@ class SparseDOKTensor(object):
         if n:
             _lib.check(lib.dok_getitem_sparse(ctypes.byref(hm._desc), ctypes.byref(ix), ctypes.byref(om._desc),
                                               stream), "__spgetitem__")
-        om._n_upper = n
+        om._n_upper, om._n_exact = n, False
         out._hashmap = om
         return out
 
@@ -607,6 +706,7 @@ class SparseDOKTensor(object):
         ix, _ = self._index_desc(selectors)
         lib = _lib.load()
         stream = _stream_ptr(self.device)
+        hm._touch()
         if selectors[0].numel():
             _lib.check(lib.dok_zero_items(ctypes.byref(hm._desc), ctypes.byref(ix), stream), "zero_items")
         n_src = int(src_values.shape[0])
@@ -619,7 +719,7 @@ class SparseDOKTensor(object):
                 mask >>= 1                                   # minus zero counts as zero
             _lib.check(lib.dok_setitem_sparse(ctypes.byref(hm._desc), ctypes.byref(ix), src_indices.data_ptr(),
                                               src_values.data_ptr(), n_src, mask, stream), "__setitem__")
-        hm._n_upper = n_now + n_src
+        hm._n_upper, hm._n_exact = n_now + n_src, False
 
     def count_items(self, selectors):
         """Number of addressed elements that are stored (reference: count_items,
@@ -641,6 +741,7 @@ class SparseDOKTensor(object):
         if hm._allocated and selectors[0].numel():
             ix, _ = self._index_desc(selectors)
             lib = _lib.load()
+            hm._touch()
             _lib.check(lib.dok_zero_items(ctypes.byref(hm._desc), ctypes.byref(ix), _stream_ptr(self.device)),
                        "zero_items")
 
@@ -705,6 +806,7 @@ class SparseDOKTensor(object):
         assert sorted(ordering) == list(range(self.ndim))
         self._perm = tuple(self._perm[o] for o in ordering)
         self._size = torch.Size(self._size[o] for o in ordering)
+        self._plans = {}
         return self
 
     def permute(self, *ordering):

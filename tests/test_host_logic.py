@@ -228,7 +228,8 @@ def test_affine_plan_equals_materialised_selectors(case):
     sel = SELECTOR_CASES[case](r, c, m)
     dok = SparseDOKTensor(size=(13, 17), device="cpu")
     mats, sc1 = dok._handle_selectors(sel)
-    ix, out_shape, sc2, keep = dok._plan(sel)
+    plan, keep = dok._plan(sel)
+    ix, out_shape, sc2 = plan.ix, plan.out_shape, plan.scalar_positions
     assert sc1 == sc2 and tuple(mats[0].shape) == out_shape
     if int(np.prod(out_shape)) == 0:
         return
@@ -243,7 +244,8 @@ def test_affine_plan_4d_and_views():
     for sel in [(slice(None), i, slice(None), k), (i, slice(None), k), (4, slice(0, 3), i[:2], k[:2]),
                 (2, slice(1, 5), i[:, None], mask), (3,), (3, 2, 1, 0), (slice(2, 2),)]:
         mats, sc1 = dok._handle_selectors(sel)
-        ix, out_shape, sc2, keep = dok._plan(sel)
+        plan, keep = dok._plan(sel)
+        ix, out_shape, sc2 = plan.ix, plan.out_shape, plan.scalar_positions
         assert sc1 == sc2 and tuple(mats[0].shape) == out_shape
         if int(np.prod(out_shape)) == 0:
             continue
@@ -251,10 +253,49 @@ def test_affine_plan_4d_and_views():
             assert np.array_equal(got, exp.reshape(-1).numpy())
     # a permuted view fills the descriptor in the storage's dimension order
     v = dok.permute(2, 0, 3, 1)
-    ix, out_shape, _, keep = v._plan((1, slice(None), 2, slice(0, 3)))
+    plan, keep = v._plan((1, slice(None), 2, slice(0, 3)))
+    ix, out_shape = plan.ix, plan.out_shape
     assert out_shape == (6, 3)
     assert ix.sel[2].base == 1 and ix.sel[3].base == 2          # view dims 0, 2 -> storage dims 2, 3
     assert list(ix.sel[0].strides)[:2] == [1, 0] and list(ix.sel[1].strides)[:2] == [0, 1]
+
+
+def test_plans_are_reused_by_structure_and_refreshed_by_value():
+    """An expression of a structure seen before takes the cached descriptor with only its integer
+    bases and data pointers refreshed: the coordinates it yields must be those of a fresh plan, for
+    other integers, other index tensors of the same shape, and a mask that was changed in place."""
+    dok = SparseDOKTensor(size=(6, 7, 5, 4), device="cpu")
+    idx_a, idx_b = torch.tensor([[0], [3], [4]]), torch.tensor([[2], [2], [1]])
+    mask = torch.tensor([True, False, True, True])
+    first, _ = dok._plan((2, slice(1, 5), idx_a, mask))
+    for i, idx in ((2, idx_a), (5, idx_b), (0, idx_a.clone())):
+        sel = (i, slice(1, 5), idx, mask)
+        plan, keep = dok._plan(sel)
+        assert plan is first                                   # same structure: the cached plan
+        mats, sc = dok._handle_selectors(sel)
+        assert sc == plan.scalar_positions and tuple(mats[0].shape) == plan.out_shape
+        for got, exp in zip(_coords_from_plan(plan.ix, plan.out_shape, 4), mats):
+            assert np.array_equal(got, exp.reshape(-1).numpy())
+    assert dok[2, 1:5, idx_a, mask].shape == first.final_shape
+    # other slice bounds, another index shape: other plans
+    assert dok._plan((2, slice(0, 5), idx_a, mask))[0] is not first
+    assert dok._plan((2, slice(1, 5), idx_a[:2], mask))[0] is not first
+    # a mask changed in place selects other columns: its version is part of the structure
+    mask[1] = True
+    plan2, keep = dok._plan((2, slice(1, 5), idx_a, mask))
+    assert plan2 is not first and plan2.out_shape[-1] == 4 or plan2.out_shape != first.out_shape
+    mats, _ = dok._handle_selectors((2, slice(1, 5), idx_a, mask))
+    for got, exp in zip(_coords_from_plan(plan2.ix, plan2.out_shape, 4), mats):
+        assert np.array_equal(got, exp.reshape(-1).numpy())
+    # selectors that are converted on the way (lists, int32 tensors) are planned afresh every time
+    p1, _ = dok._plan(([1, 2], 0))
+    p2, _ = dok._plan(([1, 2], 0))
+    assert p1 is not p2
+    # a permuted view keeps plans of its own
+    v = dok.permute(3, 2, 1, 0)
+    assert v._plans == {} and len(dok._plans) >= 3
+    dok.permute_(1, 0, 2, 3)
+    assert dok._plans == {}
 
 
 def test_bulk_path_decision():
