@@ -41,6 +41,7 @@ PROFILED = {
     "build_lf09": 5.124e9,
     "set_cas_lf05": 1.615e10,    # p8_set_kernel (one compare-and-swap per row)
     "remove_lf05": 5.688e9,      # p8_remove_kernel, half of the keys, plain-store tombstones
+    "remove_bulk_lf05": None,    # the partitioned removal's kernels together, half of the keys
     # bench.py --only-tagged (profiles/tagged_32M_f32x3_i64x5.txt), load factor 0.5
     "tagged_set_lf05": 11.84e9,        # tg_set_kernel, 32M fresh float32[3] -> int64[5] rows
     "tagged_build_lf05": None,         # dok_fill_kernel + tg_fast_set_kernel + tg_deferred_kernel
@@ -318,7 +319,8 @@ def other_configs(device):
     torch.cuda.synchronize()
     n_gone = lin.numel() // 5
     gone = coords[:, :n_gone].T.contiguous()
-    res["cfg5_remove_20M_ms"] = round(timed(lambda: dok.storage()._remove_rows(gone, unique=True))[0], 3)
+    # (`del storage[keys]`: no per-row flags asked for, so the partitioned removal runs)
+    res["cfg5_remove_20M_ms"] = round(timed(lambda: dok.storage().__delitem__(gone))[0], 3)
     fresh = torch.stack([torch.randint(0, s, (n_gone,), generator=gen, device=device) for s in size], dim=1)
     fv = torch.randn(n_gone, 1, generator=gen, device=device).half()
     res["cfg5_reinsert_20M_ms"] = round(timed(lambda: dok.storage().set(fresh, fv))[0], 3)
@@ -698,6 +700,19 @@ def main():
                                                 _stream_ptr(device)), "remove")
         rc_avg, _ = time_kernel(raw_remove_cas, 3, prep=lambda: raw_set(half, values[: n // 2]))
         results["remove_cas_mops_lf05"] = round((n // 2) / rc_avg / 1e3, 1)
+        # the same removal without per-row flags, partitioned by table range (what `del map[keys]` runs)
+        nws = int(_dl.load().dok_bulk_workspace_bytes(ctypes.byref(hm._desc), n // 2))
+        if nws > 0:
+            rws = torch.empty(nws, device=device, dtype=torch.uint8)
+            def raw_remove_bulk():
+                _dl.check(_dl.load().dok_map_remove_bulk(ctypes.byref(hm._desc), half.data_ptr(), n // 2, rws.data_ptr(),
+                                                         nws, _stream_ptr(device)), "remove_bulk")
+            raw_set(half, values[: n // 2]); raw_remove_bulk()
+            assert hm.n_elements == n - n // 2
+            rb_avg, _ = time_kernel(raw_remove_bulk, 5, prep=lambda: raw_set(half, values[: n // 2]))
+            results["remove_bulk_ms_lf05"] = round(rb_avg, 4)
+            results["remove_bulk_mops_lf05"] = round((n // 2) / rb_avg / 1e3, 1)
+            del rws
         del half, rem_f
         del hm
         torch.cuda.empty_cache()
@@ -807,7 +822,8 @@ def main():
                                          ("set_lf09", "set_bulk_lf09", "set_bulk_ms_lf09", n),
                                          ("build_lf09", "build_lf09", "build_ms_lf09", n),
                                          ("set_per_row_lf05", "set_cas_lf05", "set_cas_kernel_ms_lf05", n),
-                                         ("remove_lf05", "remove_lf05", "remove_ms_lf05", n // 2)):
+                                         ("remove_lf05", "remove_lf05", "remove_ms_lf05", n // 2),
+                                         ("remove_bulk_lf05", "remove_bulk_lf05", "remove_bulk_ms_lf05", n // 2)):
             ms = results.get(ms_key)
             m = measured(entry, ms)
             if ms is not None:

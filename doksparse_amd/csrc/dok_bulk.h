@@ -225,7 +225,9 @@ __global__ __launch_bounds__(DOK_BULK_CTPB) void bulk_linearise_kernel(DevTable 
 
 // ---- scatter: LEVEL 1 moves the caller's rows into first-level bins (keysA/valsA), LEVEL 2 moves
 // the rows of each first-level bin into their ranges (keysB/valsB) ---------------------------------
-template <int V, int KF, int LEVEL, int SL = DOK_BULK_SUBLOG, int ND = 0, bool SMALLT = false>
+// REMOVE: the rows are keys to be removed - no values travel with them, a key that lives in a side
+// slot of the header is removed on the spot, rows outside the coordinate space are dropped silently.
+template <int V, int KF, int LEVEL, int SL = DOK_BULK_SUBLOG, int ND = 0, bool SMALLT = false, bool REMOVE = false>
 __global__ __launch_bounds__(bulk_tpb(LEVEL, KF, ND)) void bulk_scatter_kernel(DevTable t, const void *__restrict__ keys_in,
                                                                     const void *__restrict__ vals_in, i64 n, BulkWs ws) {
   typedef typename ValT<V>::type VT;
@@ -293,7 +295,8 @@ __global__ __launch_bounds__(bulk_tpb(LEVEL, KF, ND)) void bulk_scatter_kernel(D
           bulk_fetch<KF, ND>(t, kin, i, n, r);
           k[j] = r.w[0];
         }
-        if (KF == DOK_KF_TABLE) {                     // value i & 15 of bucket i >> 4 of the source
+        if (REMOVE) {
+        } else if (KF == DOK_KF_TABLE) {              // value i & 15 of bucket i >> 4 of the source
           if ((int)(i & 15) < P8<V>::S)
             v[j] = *(const VT *)((const char *)kin + (i >> 4) * 128 + 8 * P8<V>::S + V * (i & 15));
         } else {
@@ -333,10 +336,11 @@ __global__ __launch_bounds__(bulk_tpb(LEVEL, KF, ND)) void bulk_scatter_kernel(D
     #pragma unroll
     for (int j = 0; j < RPT; j++) {
       bn[j] = -1; rk[j] = 0;
-      if (st[j] == 2) n_oob++;
+      if (st[j] == 2 && !REMOVE) n_oob++;
       if (st[j] == 1) {
         if (LEVEL == 1 && (k[j] ^ DOK_P8_XOR) < 2) {
-          n_fresh += p8_side_set(t, k[j] ^ DOK_P8_XOR, (u64)v[j]);
+          if (REMOVE) n_fresh -= atomicExch((u64 *)&t.header[DOK_H_SIDE_STATE + (k[j] ^ DOK_P8_XOR)], 0ULL) != 0;
+          else n_fresh += p8_side_set(t, k[j] ^ DOK_P8_XOR, (u64)v[j]);
         } else {
           const u32 r = bulk_range_of(k[j], t);
           bn[j] = LEVEL == 1 ? (int)(r >> ws.sublog) : (int)(r & (NB - 1));
@@ -397,11 +401,14 @@ __global__ __launch_bounds__(bulk_tpb(LEVEL, KF, ND)) void bulk_scatter_kernel(D
         const u32 r = pos - off[b];
         if (r < room[b]) {
           out_keys[gbase[b] + r] = skeys[pos];
-          out_vals[gbase[b] + r] = svals[pos];
+          if (!REMOVE) out_vals[gbase[b] + r] = svals[pos];
         } else {
           // the bin's region is full: the row goes to the ordinary insert
           const u32 at = atomicAdd(ws.spill_cnt, 1u);
-          if (at < ws.spill_cap) { ws.spill_keys[at] = skeys[pos]; ((VT *)ws.spill_vals)[at] = svals[pos]; }
+          if (at < ws.spill_cap) {
+            ws.spill_keys[at] = skeys[pos];
+            if (!REMOVE) ((VT *)ws.spill_vals)[at] = svals[pos];
+          }
         }
       }
     }
@@ -1075,6 +1082,169 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void bulk_deferred_kerne
   });
 }
 
+// ---- bulk removal ---------------------------------------------------------------------------------
+// The keys of a large removal, partitioned by the range of their home bucket like the rows of a bulk
+// insert, meet their buckets in table order: a workgroup works through the ranges of its block, its
+// lookups read every bucket line of a range once (and mostly from the caches, the rows of a range
+// arriving together), and the tombstones of a line leave the GPU as one write-back - where the
+// per-row kernel pays a random line read and a partial write per key.
+// Equal keys of a batch have one home, so they meet in one workgroup, which lets exactly one of them
+// count: a bit per slot of the range in LDS.  (A key found outside the range of its home - placed
+// far from it, near the range's end - is settled by a compare-and-swap on the slot instead.)
+#define DOK_BULK_RM_CHUNK 2048                      // keys of a range sorted and looked up at a time
+template <int V>
+__global__ __launch_bounds__(DOK_TPB) void bulk_remove_kernel(DevTable t, BulkWs ws) {
+  constexpr int CH = DOK_BULK_RM_CHUNK, RPT = CH / DOK_TPB;
+  static_assert(DOK_BULK_R == DOK_TPB, "one counter of the bucket sort per thread");
+  __shared__ u32 taken[DOK_BULK_R * 16 / 32];       // one bit per (bucket of the range, word of the bucket)
+  __shared__ u64 skeys[CH];                         // the chunk's keys in bucket order
+  __shared__ u32 cnt[DOK_BULK_R], off[DOK_BULK_R], wsum[16];
+  const int tid = threadIdx.x;
+  const u32 per = (ws.n_part + gridDim.x - 1) / gridDim.x;
+  const u32 p_lo = blockIdx.x * per < ws.n_part ? blockIdx.x * per : ws.n_part;
+  const u32 p_hi = p_lo + per < ws.n_part ? p_lo + per : ws.n_part;
+  int n_removed = 0;
+  // The work items are (range, chunk of its keys); the keys of the next item are loaded into
+  // registers while the current one is looked up.
+  u32 p = p_lo, c0 = 0;
+  while (p < p_hi && bulk_part_n(ws, p) == 0) p++;
+  u64 k[RPT];
+  auto load_keys = [&](u32 pp, u32 cc) {
+    const u32 n_pp = bulk_part_n(ws, pp);
+    const u64 *rows = ws.keysB + (u64)pp * ws.part_cap + cc;
+    const u32 mm = n_pp - cc < (u32)CH ? n_pp - cc : (u32)CH;
+    #pragma unroll
+    for (int j = 0; j < RPT; j++) {
+      const u32 i = (u32)j * DOK_TPB + tid;
+      k[j] = i < mm ? rows[i] : 0;
+    }
+  };
+  if (p < p_hi) load_keys(p, 0);
+  while (p < p_hi) {
+    const u32 n_p = bulk_part_n(ws, p);
+    const u64 b0 = (u64)p << DOK_BULK_RLOG;
+    if (c0 == 0)
+      for (int q = tid; q < DOK_BULK_R * 16 / 32; q += DOK_TPB) taken[q] = 0;
+    u32 pn = p, cn = c0 + CH;                          // the item after this one
+    if (cn >= n_p) {
+      cn = 0; pn = p + 1;
+      while (pn < p_hi && bulk_part_n(ws, pn) == 0) pn++;
+    }
+    {
+      const u32 m = n_p - c0 < (u32)CH ? n_p - c0 : (u32)CH;
+      // The keys of a range arrive in no order.  Sorted by home bucket (a counting sort in LDS),
+      // the keys of one bucket sit in neighbouring lanes, so every bucket line is fetched once, by
+      // one wave instruction, instead of once per key and whenever a key's turn comes.
+      cnt[tid] = 0;
+      u32 lb[RPT], rk[RPT];
+      __syncthreads();
+      #pragma unroll
+      for (int j = 0; j < RPT; j++) {
+        const u32 i = (u32)j * DOK_TPB + tid;
+        lb[j] = 0; rk[j] = 0;
+        if (i < m) {
+          lb[j] = (p8_home(k[j] ^ DOK_P8_XOR, t) - (u32)b0) & (DOK_BULK_R - 1);
+          rk[j] = atomicAdd(&cnt[lb[j]], 1u);
+        }
+      }
+      __syncthreads();
+      u32 total;
+      const u32 ex = bulk_block_scan(cnt[tid], wsum, total);
+      off[tid] = ex;
+      __syncthreads();
+      #pragma unroll
+      for (int j = 0; j < RPT; j++)
+        if ((u32)j * DOK_TPB + tid < m) skeys[off[lb[j]] + rk[j]] = k[j];
+      __syncthreads();
+      if (pn < p_hi) load_keys(pn, cn);                 // (in flight during the lookups below)
+      for (u32 i0 = 0; i0 < m; i0 += DOK_TPB) {
+        const u32 i = i0 + tid;
+        const bool active = i < m;
+        const u64 sk = (active ? skeys[i] : 0) ^ DOK_P8_XOR;
+        bool found = false, removed = false;
+        u64 val = 0;
+        u32 sb = 0; int ss = 0, nprobe = 0;
+        const u64 h = p8_hash(sk, t);
+        const u32 home = active ? dok_reduce(h, t.nb) : 0u;
+        // Every lane reads the key words of its own key's home bucket (neighbouring lanes read the
+        // same line: the keys are in bucket order): a dozen instructions per key, where the
+        // cooperative probe of p8_lookup - made for keys in no order, one line per 16 lanes and
+        // round - takes some forty and would bound this kernel by instruction issue.  Only a key that
+        // is not in its home bucket although the bucket's metadata says it may sit further on takes
+        // the general lookup.
+        bool more = false;
+        {
+          const ulonglong2 *hb = (const ulonglong2 *)(t.buckets + (u64)home * 16);
+          ulonglong2 w[8];
+          #pragma unroll
+          for (int q = 0; q < 8; q++) w[q] = hb[q];
+          u32 gm = 0;
+          #pragma unroll
+          for (int q = 0; q < 8; q++) {
+            if (2 * q < P8<V>::S) gm |= (u32)(w[q].x == sk) << (2 * q);
+            if (2 * q + 1 < P8<V>::S) gm |= (u32)(w[q].y == sk) << (2 * q + 1);
+          }
+          const u64 meta = w[7].y;
+          if (active && gm) { found = true; sb = home; ss = __builtin_ctz(gm); }
+          more = active && !gm && (u32)meta != 0 && ((u32)(meta >> 32) & p8_fbit(h)) != 0;
+        }
+        if (dok_ballot(more) != 0) {
+          bool f2 = false;
+          u32 sb2 = 0; int ss2 = 0;
+          p8_lookup<V, false>(t.buckets, t.nb, sk, more ? home : 0u, p8_fbit(h), more, f2, val, sb2, ss2, nprobe);
+          if (more && f2) { found = true; sb = sb2; ss = ss2; }
+        }
+        if (found) {
+          const u64 lbk = (u64)sb - b0;
+          if (lbk < (u64)DOK_BULK_R) {
+            const u32 bit = (u32)lbk * 16 + (u32)ss;
+            removed = !(atomicOr(&taken[bit >> 5], 1u << (bit & 31)) & (1u << (bit & 31)));
+            if (removed) t.buckets[(u64)sb * 16 + ss] = DOK_P8_TOMB;
+          } else {
+            removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
+          }
+        }
+        n_removed += removed;
+      }
+      __syncthreads();                                // skeys, cnt and (next range) the bits are reused
+    }
+    p = pn; c0 = cn;
+  }
+  dok_block_add1(&t.header[DOK_H_NELEM], -n_removed);
+}
+
+// The keys that found their bin's region full during the partition (batches with very many equal
+// keys), after everything else: one compare-and-swap per row found.
+template <int V>
+__global__ __launch_bounds__(DOK_TPB) void bulk_remove_spill_kernel(DevTable t, BulkWs ws) {
+  const i64 n = ws.spill_cnt[0] < ws.spill_cap ? ws.spill_cnt[0] : ws.spill_cap;
+  int n_removed = 0;
+  DOK_TILE_LOOP(n) {
+    const i64 i = DOK_TILE_ROW();
+    const bool active = i < n;
+    const u64 sk = (active ? ws.spill_keys[i] : 0) ^ DOK_P8_XOR;
+    bool found = false, removed = false;
+    u64 val = 0;
+    u32 sb = 0; int ss = 0, nprobe = 0;
+    const u64 h = p8_hash(sk, t);
+    p8_lookup<V>(t.buckets, t.nb, sk, active ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), active, found, val, sb, ss, nprobe);
+    if (found) removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
+    n_removed += removed;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) t.header[DOK_H_NSPILL] = n;
+  dok_block_add1(&t.header[DOK_H_NELEM], -n_removed);
+}
+
+// Batch keys of any format as one 8-byte word per row in keysB (all ones: a row outside the
+// coordinate space), for the first scatter of a removal.
+template <int KF>
+__global__ __launch_bounds__(DOK_TPB) void bulk_keys_to_words_kernel(DevTable t, const void *__restrict__ keys, i64 n, BulkWs ws) {
+  for (i64 i = (i64)blockIdx.x * DOK_TPB + threadIdx.x; i < n; i += (i64)gridDim.x * DOK_TPB) {
+    u64 key = 0;
+    ws.keysB[i] = dok_load_key8<KF>(t, keys, i, n, key) ? key : ~0ULL;
+  }
+}
+
 // ---- host side -----------------------------------------------------------------------------------
 struct BulkPlan {
   u32 n_part, n_big, sublog, ch, g1, gm;
@@ -1264,4 +1434,28 @@ static void bulk_launch(const DevTable &d, const void *keys, const void *values,
   } else {
     bulk_launch_nd<V, KF, 0, FRESH>(d, keys, values, n, p, workspace, s);
   }
+}
+
+// Bulk removal of n keys (key rows in the table's batch format; no per-row flags).
+template <int V>
+static void bulk_launch_remove(const DevTable &d, const void *keys, i64 n, const BulkPlan &p, void *workspace, hipStream_t s) {
+  BulkWs ws;
+  bulk_bind(p, workspace, ws);
+  bulk_init_kernel<<<64, DOK_TPB, 0, s>>>(ws, nullptr);
+  // (the scatters move no values: their instantiation for one-byte values serves every table)
+  if (d.lin_ndim == 0 && d.key_bytes == 8) {
+    bulk_scatter_kernel<1, DOK_KF_U64, 1, DOK_BULK_SUBLOG, 0, false, true><<<p.g1, bulk_tpb(1, DOK_KF_U64, 0), 0, s>>>(d, keys, nullptr, n, ws);
+  } else {
+    const unsigned g = (unsigned)((n + DOK_TPB - 1) / DOK_TPB < 8192 ? (n + DOK_TPB - 1) / DOK_TPB : 8192);
+    if (d.lin_ndim > 0) bulk_keys_to_words_kernel<DOK_KF_ROWS><<<g, DOK_TPB, 0, s>>>(d, keys, n, ws);
+    else bulk_keys_to_words_kernel<DOK_KF_RAW><<<g, DOK_TPB, 0, s>>>(d, keys, n, ws);
+    bulk_scatter_kernel<1, DOK_KF_LIN, 1, DOK_BULK_SUBLOG, 0, false, true><<<p.g1, bulk_tpb(1, DOK_KF_LIN, 0), 0, s>>>(d, ws.keysB, nullptr, n, ws);
+  }
+  if (p.sublog == DOK_BULK_SUBLOG)
+    bulk_scatter_kernel<1, DOK_KF_U64, 2, DOK_BULK_SUBLOG, 0, false, true><<<p.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
+  else
+    bulk_scatter_kernel<1, DOK_KF_U64, 2, DOK_BULK_SUBLOG_WIDE, 0, false, true><<<p.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
+  const u32 grid = p.n_part < 2048u ? p.n_part : 2048u;
+  bulk_remove_kernel<V><<<grid, DOK_TPB, 0, s>>>(d, ws);
+  bulk_remove_spill_kernel<V><<<256, DOK_TPB, 0, s>>>(d, ws);
 }

@@ -150,7 +150,9 @@ __device__ __forceinline__ int p8_pick(u32 free_mask, int start) {   // free_mas
 #define DOK_P8_U 8
 #define DOK_P8_WL 2  // rows per group per phase-2 turn of the lookup
 #define DOK_P8_WI 4  // rows per group per phase-2 turn of the insert
-template <int V>
+// WANT_VALUE = false: the caller only needs to know whether and where the key is (removal, counts);
+// the value is then not read, which takes one dependent load off every hit.
+template <int V, bool WANT_VALUE = true>
 __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 nb, u64 sk, u32 b, u32 fbit,
                                           bool pend, bool &found, u64 &val, u32 &slot_b,
                                           int &slot_s, int &nprobe) {
@@ -195,7 +197,7 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
     const int s1 = __builtin_ctz(my_gm | 0x10000u);
     // the bucket line was fetched a moment ago: the owner reads the value of the matching slot
     // from it (cheaper than shuffling a value out of the group in every round)
-    if (hit1) {
+    if (WANT_VALUE && hit1) {
       typedef typename ValT<V>::type T;
       my_v = *(const T *)((const char *)(buckets + (u64)home * 16) + 8 * P8<V>::S + V * s1);
     }
@@ -284,7 +286,7 @@ __device__ __forceinline__ void p8_lookup(const u64 *__restrict__ buckets, u64 n
   if (hit2) {
     typedef typename ValT<V>::type T;
     found = true;
-    val = *(const T *)((const char *)(buckets + (u64)slot_b * 16) + 8 * P8<V>::S + V * slot_s);
+    if (WANT_VALUE) val = *(const T *)((const char *)(buckets + (u64)slot_b * 16) + 8 * P8<V>::S + V * slot_s);
   }
 }
 
@@ -718,7 +720,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_remove_kernel(DevTable t, const vo
     }
     u32 sb = 0; int ss = 0, nprobe = 0;
     const u64 h = p8_hash(sk, t);
-    p8_lookup<V>(t.buckets, t.nb, sk, pend ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), pend, found, val, sb, ss, nprobe);
+    p8_lookup<V, false>(t.buckets, t.nb, sk, pend ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), pend, found, val, sb, ss, nprobe);
     if (found) {
       if (UNIQUE) { t.buckets[(u64)sb * 16 + ss] = DOK_P8_TOMB; removed = true; }
       else removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
@@ -745,7 +747,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_count_kernel(DevTable t, const voi
     if (ok && sk < 2) { found = p8_side_get(t, sk, val); pend = false; }
     u32 sb = 0; int ss = 0, nprobe = 0;
     const u64 h = p8_hash(sk, t);
-    p8_lookup<V>(t.buckets, t.nb, sk, pend ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), pend, found, val, sb, ss, nprobe);
+    p8_lookup<V, false>(t.buckets, t.nb, sk, pend ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), pend, found, val, sb, ss, nprobe);
     n_found += found;
   }
   dok_block_add1(count, n_found);
@@ -955,7 +957,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_countitems_kernel(DevTable t, DevI
     u64 val = 0;
     u32 sb = 0; int ss = 0, nprobe = 0;
     const u64 h = p8_hash(sk, t);
-    p8_lookup<V>(t.buckets, t.nb, sk, ok ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), ok, found, val, sb, ss, nprobe);
+    p8_lookup<V, false>(t.buckets, t.nb, sk, ok ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), ok, found, val, sb, ss, nprobe);
     n_found += found;
   }
   dok_block_add1(count, n_found);
@@ -974,7 +976,7 @@ __global__ __launch_bounds__(DOK_TPB) void p8_zeroitems_kernel(DevTable t, DevIn
     u64 val = 0;
     u32 sb = 0; int ss = 0, nprobe = 0;
     const u64 h = p8_hash(sk, t);
-    p8_lookup<V>(t.buckets, t.nb, sk, ok ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), ok, found, val, sb, ss, nprobe);
+    p8_lookup<V, false>(t.buckets, t.nb, sk, ok ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), ok, found, val, sb, ss, nprobe);
     if (found) removed = atomicCAS(t.buckets + (u64)sb * 16 + ss, sk, DOK_P8_TOMB) == sk;
     n_removed += removed;
   }

@@ -481,6 +481,24 @@ int dok_map_remove_unique(const dok_table_t *t, const void *keys, int64_t n, uin
   return map_remove(t, keys, n, removed, true, stream);
 }
 
+int dok_map_remove_bulk(const dok_table_t *t, const void *keys, int64_t n, void *workspace, int64_t workspace_bytes,
+                        void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (n < 0) return DOK_EINVAL;
+  if (n == 0) return DOK_OK;
+  if (!keys || !workspace) return DOK_EINVAL;
+  BulkPlan p;
+  if (layout != DOK_LAYOUT_PACKED8 || !bulk_plan(d, n, p)) return DOK_EUNSUPPORTED;
+  if (((uintptr_t)workspace & 255) != 0 || workspace_bytes < (int64_t)p.bytes) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
+  { constexpr int KF = DOK_KF_U64;
+    P8_DISPATCH(d.value_bytes, (bulk_plan_for<V, KF>(d, n, p), bulk_launch_remove<V>(d, keys, n, p, workspace, s))); }
+  return note_launch();
+}
+
 int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n, int64_t *count, void *stream) {
   DevTable d; int layout;
   int rc = make_dev_table(t, d, layout);

@@ -205,6 +205,17 @@ int dok_map_remove(const dok_table_t *t, const void *keys, int64_t n,
 int dok_map_remove_unique(const dok_table_t *t, const void *keys, int64_t n,
                           uint8_t *removed, void *stream);
 
+/* dok_map_remove without per-row flags for a batch that is large against the table (rule of
+ * thumb: a million keys and more, more than one per physical bucket): the keys are partitioned by
+ * table range through `workspace` (dok_bulk_workspace_bytes(t, n) bytes, 256-byte aligned, as for
+ * dok_map_set_bulk) and every range's keys are looked up together, so the table is read in order
+ * and each bucket line written back once.  Equal keys inside the batch count once.  Packed layout
+ * only (else DOK_EUNSUPPORTED: use dok_map_remove).
+ * Reference: closed_hashmap_remove (closed_hashmap_impl.cu:159-220) at the batch sizes of
+ * `del hashmap[keys]` (cuda_closed_hashmap.py:476-477), which discards the flags. */
+int dok_map_remove_bulk(const dok_table_t *t, const void *keys, int64_t n, void *workspace,
+                        int64_t workspace_bytes, void *stream);
+
 /* count[0] += number of rows whose key is present.  count is a device int64.
  * Reference: ClosedHashmap::exists (closed_hashmap_impl_class.cu:253-278). */
 int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n,

@@ -20,6 +20,7 @@ def bulk_always(monkeypatch):
     from doksparse_amd import closed_hashmap as ch
     monkeypatch.setattr(ch, "BULK_MIN_ROWS", 0)
     monkeypatch.setattr(ch, "BULK_MIN_ROWS_PER_BUCKET", 0.0)
+    monkeypatch.setattr(ch, "BULK_REMOVE_MIN_ROWS_PER_BUCKET", 0.0)
     return ch
 
 
@@ -721,3 +722,81 @@ def test_multiword_bulk_entry_points_through_the_c_abi(cuda):
     assert lib.dok_map_set_bulk(desc, k.data_ptr(), v.data_ptr(), n, ws.data_ptr() + 8, need, st) == _lib.DOK_EINVAL
     assert lib.dok_map_set_bulk(desc, k.data_ptr(), v.data_ptr(), n, None, need, st) == _lib.DOK_EINVAL
     _assert_same_map(hm, ref)
+
+
+# ---- bulk removal: keys partitioned by table range, lookups in table order, no per-row flags
+
+@pytest.mark.parametrize("key_dtype,value_dtype", [(np.int64, np.float32), (np.int64, np.int64), (np.int32, np.float16),
+                                                   (np.int16, np.int8)])
+def test_bulk_removal_matches_oracle(cuda, bulk_always, key_dtype, value_dtype):
+    """`del map[keys]` through dok_map_remove_bulk (thresholds lowered): batches with absent keys,
+    keys given several times, the two key patterns that live in the table header, on tables of a few
+    ranges and of many; entry count and remaining map against the oracle after every batch."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(5)
+    lim = min(2**62, int(np.iinfo(key_dtype).max))
+    for n, cap in ((40000, 65536), (3000, 3300), (200000, 1 << 20), (40, 64)):
+        n = min(n, lim // 2)
+        pool = np.unique(rng.integers(-lim, lim, size=3 * n, dtype=np.int64).astype(key_dtype))
+        rng.shuffle(pool)
+        keys = pool[:n].copy()
+        special = np.array([0x9E3779B97F4A7C15, 0x9E3779B97F4A7C14], dtype=np.uint64).view(np.int64)
+        if key_dtype == np.int64:
+            keys[:2] = special                               # stored words 0 and 1: the header's side slots
+            keys = np.unique(keys)
+            n = keys.shape[0]
+        vals = rng.integers(-100, 100, size=(n, 1)).astype(value_dtype)
+        hm = CudaClosedHashmap(n_buckets=cap, device=cuda, rehash_threshold=1e9)
+        ref = RefClosedHashmap(n_buckets=cap, rehash_threshold=1e9, rng=np.random.default_rng(9))
+        hm.set(*_to(cuda, keys[:, None], vals))
+        ref.set(keys[:, None], vals)
+        for frac in (0.3, 0.5):
+            m = int(n * frac)
+            gone = np.concatenate([keys[rng.permutation(n)[:m]], pool[n:n + m // 3], keys[:m // 4]])   # present, absent, repeats
+            if key_dtype == np.int64:
+                gone = np.concatenate([gone, special[:1], special[:1]])
+            rng.shuffle(gone)
+            del hm[torch.from_numpy(gone[:, None]).to(cuda)]
+            ref.remove(gone[:, None])
+            assert hm.n_elements == ref.n_elements
+            _assert_same_map(hm, ref)
+            _check_get(hm, ref, np.concatenate([keys, pool[n:2 * n]])[:, None], cuda, fallback=-1)
+        # what was removed can be stored again (tombstones re-used), and removed again
+        hm.set(*_to(cuda, keys[:, None], vals))
+        ref.set(keys[:, None], vals)
+        assert hm.n_elements == ref.n_elements == n
+        del hm[torch.from_numpy(keys[:, None]).to(cuda)]
+        assert hm.n_elements == 0 and hm.items()[0].shape[0] == 0
+
+
+def test_bulk_removal_of_coordinate_rows_and_rejections(cuda, bulk_always):
+    """The same on a coordinate-keyed tensor (key rows are linearised on the way; rows outside the
+    size are ignored), and the entry point's argument checks."""
+    from doksparse_amd import SparseDOKTensor, _lib
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(3)
+    size = (300, 40, 25)
+    flat = torch.randperm(300 * 40 * 25, generator=g)[:60000]
+    idx = torch.stack(torch.unravel_index(flat, size))
+    vals = torch.randn(60000, generator=g)
+    dok = SparseDOKTensor(size, idx.to(cuda), vals.to(cuda), device=cuda)
+    hm = dok.storage()
+    gone = torch.cat([idx[:, :25000].T, torch.tensor([[300, 0, 0], [-1, 5, 5], [5, 40, 1]]), idx[:, :100].T]).contiguous().to(cuda)
+    del hm[gone]
+    assert dok._nnz() == 35000
+    dense = torch.zeros(size)
+    dense[tuple(idx[:, 25000:])] = vals[25000:]
+    assert torch.equal(dok.to_dense().cpu(), dense)
+    desc = ctypes.byref(hm._desc)
+    need = int(lib.dok_bulk_workspace_bytes(desc, gone.shape[0]))
+    ws = torch.empty(need, device=cuda, dtype=torch.uint8)
+    assert lib.dok_map_remove_bulk(desc, gone.data_ptr(), gone.shape[0], ws.data_ptr(), need - 1, None) == _lib.DOK_EINVAL
+    assert lib.dok_map_remove_bulk(desc, None, gone.shape[0], ws.data_ptr(), need, None) == _lib.DOK_EINVAL
+    assert lib.dok_map_remove_bulk(desc, gone.data_ptr(), 0, ws.data_ptr(), need, None) == _lib.DOK_OK
+    from doksparse_amd import CudaClosedHashmap
+    hm2 = CudaClosedHashmap(n_buckets=256, device=cuda)
+    hm2.set(torch.rand(10, 3, device=cuda), torch.zeros(10, 5, device=cuda, dtype=torch.long))
+    assert lib.dok_map_remove_bulk(ctypes.byref(hm2._desc), gone.data_ptr(), 10, ws.data_ptr(), need, None) == _lib.DOK_EUNSUPPORTED
+    torch.cuda.synchronize()
+    assert dok._nnz() == 35000
