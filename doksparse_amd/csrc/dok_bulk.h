@@ -25,6 +25,12 @@
 //   5. the handful of rows left (overflow of the per-range lists, keys that may sit at far
 //      displacements) are handed, packed, to the ordinary insert, which runs last.
 //
+// The two levels address 1024 x 1024 ranges = 2^28 buckets.  A larger table is worked through in
+// windows of that many buckets, steps 2 to 5 once per window: the first scatter reads the whole
+// batch each time and keeps the rows whose range lies in the window.  The rows that run out of a
+// window's last range are placed by step 5's ordinary insert, in the next window's buckets before
+// that window's merge - so the merge of a table of several windows always reads its ranges.
+//
 // Every step is exact for any input: a bin that receives more rows than its region holds spills
 // the surplus, and a batch whose rows all fall into one range merely degrades to step 5's
 // ordinary insert.
@@ -36,6 +42,7 @@
 #define DOK_BULK_SUBLOG 8                   // log2 of the ranges per first-level bin ...
 #define DOK_BULK_SUBLOG_WIDE 10             // ... and for tables of more than 1024 << 8 ranges
 #define DOK_BULK_MAXBIG 1024                // first-level bins at most
+#define DOK_BULK_WINDOW ((u64)DOK_BULK_MAXBIG << DOK_BULK_SUBLOG_WIDE)   // ranges one run of the passes takes: 2^28 buckets
 // Threads per scatter workgroup.  One workgroup per CU with the large tiles either way (a tile
 // fills the LDS); 16 waves instead of 8 make the second pass, whose workgroups take one or two
 // tiles each, 12 % faster and the first pass over plain keys 3 %; the first pass over coordinate
@@ -73,7 +80,12 @@ struct BulkWs {
   u32 *def_cnt;             // [GRID] rows each merge workgroup handed to the ordinary insert
   u32 *meta_cnt;            // [GRID] displacement marks each merge workgroup left to be applied
   u32 *edge_cnt;            // [GRID] rows each merge workgroup could not place in the last range of its block
-  u32 n_big, n_part;
+  u32 n_big, n_part;        // first-level bins and ranges OF THE CURRENT WINDOW (see range_base)
+  u32 range_base;           // A table of more than 2^28 buckets is worked through in windows of
+                            // DOK_BULK_WINDOW ranges, one run of the passes per window: range_base is the
+                            // window's first range; range numbers inside the passes are relative to it,
+  u32 first_window;         // and the rows outside the window are skipped by the first scatter.  first_window:
+                            // this run also looks after what belongs to no range (side-slot keys, row counts)
   u32 sublog;               // log2 of the ranges per first-level bin
   u32 g1;                   // workgroups of the first pass (a multiple of 64, at most DOK_BULK_GRID)
   u32 ch;                   // stretches (workgroups) per first-level bin in the second pass
@@ -336,14 +348,16 @@ __global__ __launch_bounds__(bulk_tpb(LEVEL, KF, ND)) void bulk_scatter_kernel(D
     #pragma unroll
     for (int j = 0; j < RPT; j++) {
       bn[j] = -1; rk[j] = 0;
-      if (st[j] == 2 && !REMOVE) n_oob++;
+      if (st[j] == 2 && !REMOVE && ws.first_window) n_oob++;
       if (st[j] == 1) {
         if (LEVEL == 1 && (k[j] ^ DOK_P8_XOR) < 2) {
-          if (REMOVE) n_fresh -= atomicExch((u64 *)&t.header[DOK_H_SIDE_STATE + (k[j] ^ DOK_P8_XOR)], 0ULL) != 0;
+          if (!ws.first_window) {
+          } else if (REMOVE) n_fresh -= atomicExch((u64 *)&t.header[DOK_H_SIDE_STATE + (k[j] ^ DOK_P8_XOR)], 0ULL) != 0;
           else n_fresh += p8_side_set(t, k[j] ^ DOK_P8_XOR, (u64)v[j]);
         } else {
-          const u32 r = bulk_range_of(k[j], t);
-          bn[j] = LEVEL == 1 ? (int)(r >> ws.sublog) : (int)(r & (NB - 1));
+          const u32 r = bulk_range_of(k[j], t) - ws.range_base;        // (a row before the window wraps to a huge number)
+          if (LEVEL == 2) bn[j] = (int)(r & (NB - 1));
+          else if (r < ws.n_part) bn[j] = (int)(r >> ws.sublog);
         }
       }
     }
@@ -501,7 +515,7 @@ __global__ __launch_bounds__(DOK_BULK_R, 3) void bulk_merge_kernel(DevTable t, B
     const u32 carried = n_carry;                     // rows handed on by the range before (they sit
                                                      // at the head of the list already)
     if (!FRESH && lo == hi && carried == 0) continue;   // nothing to do in this range
-    const u64 b0 = (u64)p << DOK_BULK_RLOG;
+    const u64 b0 = ((u64)p + ws.range_base) << DOK_BULK_RLOG;
     const u64 left = t.nb - b0;
     const u32 nbk = left < (u64)R ? (u32)left : (u32)R;
     ulonglong2 *g = (ulonglong2 *)(t.buckets + b0 * 16);
@@ -953,7 +967,7 @@ __global__ __launch_bounds__(DOK_BULK_R) void bulk_edge_kernel(DevTable t, BulkW
   const u32 guests = per < 2 ? per : 2;
   for (u32 gi = 0; gi < guests && p_hi + gi < ws.n_part; gi++) {
     const u32 p = p_hi + gi;
-    const u64 b0 = (u64)p << DOK_BULK_RLOG;
+    const u64 b0 = ((u64)p + ws.range_base) << DOK_BULK_RLOG;
     const u64 left = t.nb - b0;
     const u32 nbk = left < (u64)R ? (u32)left : (u32)R;
     ulonglong2 *g = (ulonglong2 *)(t.buckets + b0 * 16);
@@ -1122,7 +1136,7 @@ __global__ __launch_bounds__(DOK_TPB) void bulk_remove_kernel(DevTable t, BulkWs
   if (p < p_hi) load_keys(p, 0);
   while (p < p_hi) {
     const u32 n_p = bulk_part_n(ws, p);
-    const u64 b0 = (u64)p << DOK_BULK_RLOG;
+    const u64 b0 = ((u64)p + ws.range_base) << DOK_BULK_RLOG;
     if (c0 == 0)
       for (int q = tid; q < DOK_BULK_R * 16 / 32; q += DOK_TPB) taken[q] = 0;
     u32 pn = p, cn = c0 + CH;                          // the item after this one
@@ -1247,7 +1261,10 @@ __global__ __launch_bounds__(DOK_TPB) void bulk_keys_to_words_kernel(DevTable t,
 
 // ---- host side -----------------------------------------------------------------------------------
 struct BulkPlan {
-  u32 n_part, n_big, sublog, ch, g1, gm;
+  u64 n_part_all;            // ranges of the whole table
+  u32 n_windows;             // runs of the passes: windows of DOK_BULK_WINDOW ranges
+  u32 n_part, n_big;         // ranges / first-level bins of a (full) window
+  u32 sublog, ch, g1, gm;
   u32 big_cap, part_cap, spill_cap;
   i64 share;
   size_t o_keysA, o_keysB, o_valsA, o_valsB, o_big_cnt, o_part_cnt, o_spill_keys, o_spill_vals, o_spill_cnt,
@@ -1274,10 +1291,12 @@ static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p, u32 g1 = DOK_BULK_G
   if (n_cap < 0) n_cap = n;
   if (n < 1 || n > 0x7fff0000LL) return false;
   p.g1 = g1;
-  const u64 n_part = (d.nb + DOK_BULK_R - 1) >> DOK_BULK_RLOG;
+  const u64 n_part_all = (d.nb + DOK_BULK_R - 1) >> DOK_BULK_RLOG;
+  p.n_part_all = n_part_all;
+  p.n_windows = (u32)((n_part_all + DOK_BULK_WINDOW - 1) / DOK_BULK_WINDOW);     // (at most 16: a table has < 2^32 buckets)
+  const u64 n_part = n_part_all < DOK_BULK_WINDOW ? n_part_all : DOK_BULK_WINDOW;
   p.sublog = n_part <= ((u64)DOK_BULK_MAXBIG << DOK_BULK_SUBLOG) ? DOK_BULK_SUBLOG : DOK_BULK_SUBLOG_WIDE;
   const u64 n_big = (n_part + (1u << p.sublog) - 1) >> p.sublog;
-  if (n_big > DOK_BULK_MAXBIG) return false;
   p.n_part = (u32)n_part;
   p.n_big = (u32)n_big;
   // second pass: about 4096 workgroups in all, 16 to 256 per first-level bin
@@ -1321,7 +1340,8 @@ static bool bulk_plan(const DevTable &d, i64 n, BulkPlan &p, u32 g1 = DOK_BULK_G
   return true;
 }
 
-static void bulk_bind(const BulkPlan &p, void *workspace, BulkWs &ws) {
+// Device view of the workspace for window `win` of the table.
+static void bulk_bind(const BulkPlan &p, void *workspace, BulkWs &ws, u32 win = 0) {
   char *w = (char *)workspace;
   ws.keysA = (u64 *)(w + p.o_keysA);
   ws.keysB = (u64 *)(w + p.o_keysB);
@@ -1338,8 +1358,12 @@ static void bulk_bind(const BulkPlan &p, void *workspace, BulkWs &ws) {
   ws.def_cnt = (u32 *)(w + p.o_def_cnt);
   ws.meta_cnt = (u32 *)(w + p.o_meta_cnt);
   ws.edge_cnt = (u32 *)(w + p.o_edge_cnt);
-  ws.n_big = p.n_big;
-  ws.n_part = p.n_part;
+  const u64 base = (u64)win * DOK_BULK_WINDOW;
+  const u64 parts = p.n_part_all - base < DOK_BULK_WINDOW ? p.n_part_all - base : DOK_BULK_WINDOW;
+  ws.range_base = (u32)base;
+  ws.first_window = win == 0;
+  ws.n_part = (u32)parts;
+  ws.n_big = (u32)((parts + (1u << p.sublog) - 1) >> p.sublog);
   ws.sublog = p.sublog;
   ws.g1 = p.g1;
   ws.ch = p.ch;
@@ -1393,9 +1417,10 @@ __global__ void bulk_side_slots_kernel(DevTable src, DevTable dst) {
 template <int V, int KF, int ND, bool FRESH>
 static void bulk_launch_nd(const DevTable &d, const void *keys, const void *values, i64 n, const BulkPlan &p,
                            void *workspace, hipStream_t s) {
+  for (u32 win = 0; win < p.n_windows; win++) {
   BulkWs ws;
-  bulk_bind(p, workspace, ws);
-  bulk_init_kernel<<<64, DOK_TPB, 0, s>>>(ws, FRESH ? d.header : nullptr);
+  bulk_bind(p, workspace, ws, win);
+  bulk_init_kernel<<<64, DOK_TPB, 0, s>>>(ws, FRESH && win == 0 ? d.header : nullptr);
   // coordinate rows of three and more dimensions are linearised first (see bulk_linearise_kernel)
   constexpr bool LIN = ND >= 3;
   if constexpr (LIN) {
@@ -1405,16 +1430,18 @@ static void bulk_launch_nd(const DevTable &d, const void *keys, const void *valu
     bulk_scatter_kernel<V, KF, 1, DOK_BULK_SUBLOG, ND><<<p.g1, bulk_tpb(1, KF, ND), 0, s>>>(d, keys, values, n, ws);
   }
   // narrow values: small second-pass tiles when the workgroups' stretches are short
-  const bool smallt = V <= 2 && n / ((i64)p.n_big * p.ch) < DOK_BULK_T2S_BELOW;
+  const bool smallt = V <= 2 && n / ((i64)p.n_big * p.ch * p.n_windows) < DOK_BULK_T2S_BELOW;
   if (p.sublog == DOK_BULK_SUBLOG) {
-    if (smallt) bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG, 0, V <= 2><<<p.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
-    else bulk_scatter_kernel<V, DOK_KF_U64, 2><<<p.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
+    if (smallt) bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG, 0, V <= 2><<<ws.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
+    else bulk_scatter_kernel<V, DOK_KF_U64, 2><<<ws.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
   } else {
-    bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG_WIDE><<<p.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
+    bulk_scatter_kernel<V, DOK_KF_U64, 2, DOK_BULK_SUBLOG_WIDE><<<ws.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
   }
-  bulk_merge_kernel<V, FRESH><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
-  if (p.gm > 1) bulk_edge_kernel<V><<<p.gm, DOK_BULK_R, 0, s>>>(d, ws);
-  bulk_deferred_kernel<V><<<p.gm, DOK_TPB, 0, s>>>(d, ws);
+  const u32 gm = ws.n_part < p.gm ? ws.n_part : p.gm;
+  bulk_merge_kernel<V, FRESH><<<gm, DOK_BULK_R, 0, s>>>(d, ws);
+  if (gm > 1) bulk_edge_kernel<V><<<gm, DOK_BULK_R, 0, s>>>(d, ws);
+  bulk_deferred_kernel<V><<<gm, DOK_TPB, 0, s>>>(d, ws);
+  }
 }
 
 template <int V, int KF, bool FRESH = false>
@@ -1439,8 +1466,9 @@ static void bulk_launch(const DevTable &d, const void *keys, const void *values,
 // Bulk removal of n keys (key rows in the table's batch format; no per-row flags).
 template <int V>
 static void bulk_launch_remove(const DevTable &d, const void *keys, i64 n, const BulkPlan &p, void *workspace, hipStream_t s) {
+  for (u32 win = 0; win < p.n_windows; win++) {
   BulkWs ws;
-  bulk_bind(p, workspace, ws);
+  bulk_bind(p, workspace, ws, win);
   bulk_init_kernel<<<64, DOK_TPB, 0, s>>>(ws, nullptr);
   // (the scatters move no values: their instantiation for one-byte values serves every table)
   if (d.lin_ndim == 0 && d.key_bytes == 8) {
@@ -1452,10 +1480,11 @@ static void bulk_launch_remove(const DevTable &d, const void *keys, i64 n, const
     bulk_scatter_kernel<1, DOK_KF_LIN, 1, DOK_BULK_SUBLOG, 0, false, true><<<p.g1, bulk_tpb(1, DOK_KF_LIN, 0), 0, s>>>(d, ws.keysB, nullptr, n, ws);
   }
   if (p.sublog == DOK_BULK_SUBLOG)
-    bulk_scatter_kernel<1, DOK_KF_U64, 2, DOK_BULK_SUBLOG, 0, false, true><<<p.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
+    bulk_scatter_kernel<1, DOK_KF_U64, 2, DOK_BULK_SUBLOG, 0, false, true><<<ws.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
   else
-    bulk_scatter_kernel<1, DOK_KF_U64, 2, DOK_BULK_SUBLOG_WIDE, 0, false, true><<<p.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
-  const u32 grid = p.n_part < 2048u ? p.n_part : 2048u;
+    bulk_scatter_kernel<1, DOK_KF_U64, 2, DOK_BULK_SUBLOG_WIDE, 0, false, true><<<ws.n_big * p.ch, bulk_tpb(2, DOK_KF_U64, 0), 0, s>>>(d, nullptr, nullptr, n, ws);
+  const u32 grid = ws.n_part < 2048u ? ws.n_part : 2048u;
   bulk_remove_kernel<V><<<grid, DOK_TPB, 0, s>>>(d, ws);
   bulk_remove_spill_kernel<V><<<256, DOK_TPB, 0, s>>>(d, ws);
+  }
 }

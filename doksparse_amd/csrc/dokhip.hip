@@ -411,8 +411,16 @@ static int set_bulk(const dok_table_t *t, const void *keys, const void *values, 
   hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
   // the launch plan shares the workspace layout of the sizing plan above and only narrows the grids
+  // A table of several windows (more than 2^28 buckets) is built as "clear, then upsert": the rows
+  // that leave a window are placed in the next one before that one's merge, which therefore has to
+  // read its ranges instead of taking them as empty.
+  const bool build = fresh && p.n_windows == 1;
+  if (fresh && !build) {
+    const i64 words = (i64)d.nb * 16;
+    dok_fill_kernel<<<(unsigned)((words / 4 + DOK_TPB - 1) / DOK_TPB), DOK_TPB, 0, s>>>(d.buckets, words, d.header);
+  }
 #define BULK_GO (bulk_plan_for<V, KF>(d, n, p),                                                    \
-                 fresh ? bulk_launch<V, KF, true>(d, keys, values, n, p, workspace, s)             \
+                 build ? bulk_launch<V, KF, true>(d, keys, values, n, p, workspace, s)             \
                        : bulk_launch<V, KF, false>(d, keys, values, n, p, workspace, s))
   if (cols) {
     constexpr int KF = DOK_KF_COLS;
@@ -652,8 +660,14 @@ int dok_map_rehash_bulk(const dok_table_t *src, const dok_table_t *dst, void *wo
   hipStream_t s = (hipStream_t)stream;
   const DeviceScope on_stream_device(s);
   constexpr int KF = DOK_KF_TABLE;
+  const bool build = p.n_windows == 1;           // (several windows: clear, then upsert - see set_bulk)
+  if (!build) {
+    const i64 words = (i64)b.nb * 16;
+    dok_fill_kernel<<<(unsigned)((words / 4 + DOK_TPB - 1) / DOK_TPB), DOK_TPB, 0, s>>>(b.buckets, words, b.header);
+  }
   P8_DISPATCH(b.value_bytes, (bulk_plan_for<V, KF>(b, n_in, p, n_cap),
-                              bulk_launch<V, KF, true>(b, a.buckets, nullptr, n_in, p, workspace, s)));
+                              build ? bulk_launch<V, KF, true>(b, a.buckets, nullptr, n_in, p, workspace, s)
+                                    : bulk_launch<V, KF, false>(b, a.buckets, nullptr, n_in, p, workspace, s)));
   bulk_side_slots_kernel<<<1, 64, 0, s>>>(a, b);
   return note_launch();
 }

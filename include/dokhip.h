@@ -165,8 +165,11 @@ int dok_map_set(const dok_table_t *t, const void *keys, const void *values, int6
  * tables with values of at most 8 bytes (every coordinate table) and, for dok_map_build_bulk /
  * dok_coo_build_bulk, any widths; other tables take the dok_map_set kernel, same result.
  *   dok_bulk_workspace_bytes: device bytes dok_map_set_bulk / dok_coo_set_bulk need for n rows;
- *     0 if the bulk path cannot take this table or n (packed layout: n >= 2^31 or more than
- *     2^28 buckets: use dok_map_set), negative on a bad table.
+ *     0 if the bulk path cannot take this table or n (packed layout: n >= 2^31: use
+ *     dok_map_set), negative on a bad table.  A table of more than 2^28 buckets (32 GiB) is
+ *     worked through in windows of 2^28 buckets, one run of the passes per window, each reading
+ *     the whole batch and keeping the rows of its window; dok_map_build_bulk then clears the table
+ *     first and merges into it like dok_map_set_bulk.
  *     (packed layout: about 3.4 times the bytes of the batch - two partition buffers with slack
  *     and the spill list - plus 4 bytes per 256 buckets of the table; multi-word layout: 8 n + 256).
  *   workspace: device, 256-byte aligned, at least that many bytes; contents need no

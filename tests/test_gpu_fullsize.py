@@ -310,24 +310,72 @@ def test_bulk_path_with_the_wide_second_level(cuda, monkeypatch):
     assert int(ks.sum()) % (1 << 64) == (total * (total - 1) // 2 * odd) % (1 << 64)
 
 
-def test_table_beyond_the_bulk_limit_takes_the_per_row_kernel(cuda, monkeypatch):
-    """More than 2^28 buckets (a table of 36 GB): the bulk path declines (its two partition levels
-    address at most 1024 x 1024 ranges), and a batch that would otherwise qualify is inserted row
-    by row."""
-    from doksparse_amd import CudaClosedHashmap
+def test_table_of_several_bulk_windows(cuda, monkeypatch):
+    """More than 2^28 buckets (a table of 36 GB): the two partition levels address 1024 x 1024
+    ranges, so the bulk path works through such a table in windows of 2^28 buckets, one run of its
+    passes per window.  Bulk build of 700M rows, bulk upsert of 50M stored + 50M new keys, bulk
+    removal of 100M (half of them absent), then get / count / read-out checksum; bulk rehash of a
+    smaller table into one of two windows."""
+    from doksparse_amd import CudaClosedHashmap, _lib
     from doksparse_amd import closed_hashmap as ch
     monkeypatch.setattr(ch, "BULK_MIN_ROWS", 0)
     monkeypatch.setattr(ch, "BULK_MIN_ROWS_PER_BUCKET", 0.0)
+    monkeypatch.setattr(ch, "BULK_REMOVE_MIN_ROWS_PER_BUCKET", 0.0)
+    odd = -7046029254386353131
+    def rows(lo, hi, bump):
+        i = torch.arange(lo, hi, device=cuda, dtype=torch.long)
+        return (i * odd)[:, None], ((i % (1 << 24)).float() + bump)[:, None]
+
     hm = CudaClosedHashmap(n_buckets=2_800_000_000, device=cuda, rehash_threshold=1.0)
-    n = 20_000_000
-    i = torch.arange(n, device=cuda, dtype=torch.long)
-    keys, values = (i * -7046029254386353131)[:, None], (i % (1 << 24)).float()[:, None]
-    hm.set(keys, values)
-    assert hm._n_phys > 2**28 and hm._bulk_workspace(n) is None
-    assert hm.n_elements == n
-    got, found = hm.get(keys)
-    assert bool(found.all()) and torch.equal(got, values)
-    assert not bool(hm.get(keys + 1)[1].any())
+    n1 = 700_000_000
+    k1, v1 = rows(0, n1, 0.0)
+    hm.set(k1, v1)                                          # build
+    assert hm._n_phys > 2**28 and hm._bulk_workspace(n1) is not None
+    assert hm.n_elements == n1
+    got, found = hm.get(k1)
+    assert bool(found.all()) and torch.equal(got, v1)
+    del got, found
+    k2, v2 = rows(n1 - 50_000_000, n1 + 50_000_000, 1.0)
+    hm.set(k2, v2)                                          # upsert into the populated table
+    total = n1 + 50_000_000
+    assert hm.n_elements == total
+    got, found = hm.get(k2)
+    assert bool(found.all()) and torch.equal(got, v2)
+    got, found = hm.get(k1[: n1 - 50_000_000])
+    assert bool(found.all()) and torch.equal(got, v1[: n1 - 50_000_000])
+    del got, found, k2, v2
+    assert not bool(hm.get(rows(total, total + 10_000_000, 0.0)[0])[1].any())
+    k3 = rows(total - 50_000_000, total + 50_000_000, 0.0)[0]
+    del hm[k3]                                              # bulk removal: 50M stored, 50M absent
+    total -= 50_000_000
+    assert hm.n_elements == total
+    assert not bool(hm.get(k3)[1].any())
+    del k3
+    got, found = hm.get(k1[: n1 - 50_000_000])
+    assert bool(found.all()) and torch.equal(got, v1[: n1 - 50_000_000])
+    del got, found
+    ks = hm.keys()
+    assert ks.shape[0] == total
+    assert int(ks.sum()) % (1 << 64) == (total * (total - 1) // 2 * odd) % (1 << 64)
+    del ks, hm
+
+    # bulk rehash from a table of one window (the source's words are the rows: 2^27 buckets at
+    # most) into one of two
+    hm = CudaClosedHashmap(n_buckets=1_300_000_000, device=cuda, rehash_threshold=1.0)
+    hm.set(k1, v1)
+    assert hm._n_phys <= 2**27
+    lib = _lib.load()
+    calls = []
+    real = lib.dok_map_rehash_bulk
+    monkeypatch.setattr(lib, "dok_map_rehash_bulk", lambda *a: (calls.append(1), real(*a))[1])
+    hm.rehash(2_700_000_000)                                # (2.5 entries per bucket and more: the bulk rehash)
+    assert calls and hm._n_phys > 2**28 and hm.n_elements == n1
+    got, found = hm.get(k1)
+    assert bool(found.all()) and torch.equal(got, v1)
+    del got, found
+    ks = hm.keys()
+    assert ks.shape[0] == n1
+    assert int(ks.sum()) % (1 << 64) == (n1 * (n1 - 1) // 2 * odd) % (1 << 64)
 
 
 def test_coordinate_row_tensor_10m_entries(cuda):
