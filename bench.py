@@ -26,33 +26,17 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the default workload's kernels (2^26 keys / queries), from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs of this file, scaled against a table scan and a table clear of known
-# size: profiles/hashmap_get_64M_int64_f32_lf05.txt and profiles/hashmap_set_bulk_64M_int64_f32.txt
-# hold the runs.  The figures belong to one state of the kernel sources, named by `csrc_sha16`
-# (see csrc_sha16()): when the sources have changed since, nothing measured is reported.
+# HBM bytes per measured leg (everything the leg launches, per repetition), from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs of `bench.py --markers --no-cpu --calibrate --steps 10`, the counter
+# units scaled against a table scan and a table clear of known size (the files under profiles/ hold
+# the runs).  The figures belong to one state of the kernel sources, named by `csrc_sha16` (see
+# csrc_sha16()): when the sources have changed since, nothing measured is reported.
+# PROFILED-BEGIN
 PROFILED = {
     "csrc_sha16": "d3e6f388efff7039",
-    "get_lf05": 6.661e9,         # p8_get_kernel, load factor 0.5
-    "get_lf09": 7.075e9,         # p8_get_kernel, load factor 0.9 (mean over four builds)
-    "set_bulk_lf05": 7.611e9,    # the bulk upsert's kernels together, into a cleared table
-    "build_lf05": 5.891e9,       # the bulk build's kernels together, into uninitialised memory
-    "set_bulk_lf09": 6.081e9,
-    "build_lf09": 5.124e9,
-    "set_cas_lf05": 1.615e10,    # p8_set_kernel (one compare-and-swap per row)
-    "remove_lf05": 5.688e9,      # p8_remove_kernel, half of the keys, plain-store tombstones
-    "remove_bulk_lf05": None,    # the partitioned removal's kernels together, half of the keys
-    # bench.py --only-tagged (profiles/tagged_32M_f32x3_i64x5.txt), load factor 0.5
-    "tagged_set_lf05": 11.84e9,        # tg_set_kernel, 32M fresh float32[3] -> int64[5] rows
-    "tagged_build_lf05": None,         # dok_fill_kernel + tg_fast_set_kernel + tg_deferred_kernel
-    "tagged_overwrite_lf05": None,
-    "tagged_get_lf05": 6.07e9,         # tg_lookup_kernel<0, false, 8>, 32M queries
-    "tagged_remove_lf05": None,
-    # bench.py --only-dok (profiles/dok_indexing_50M_2d_f32.txt)
-    "dok_getitem_2p26": 10.69e9,       # p8_getitem_kernel<4>, 2^26 stored coordinates of a 2-D tensor
-    "dok_setitem_10M": 2.24e9,         # p8_setitem_kernel<4>, 10M coordinates, half of them new
-    "dok_readout": None,
+    "bytes": {},
 }
+# PROFILED-END
 # algorithmic bytes per op for 8-byte keys and 4-byte values: one 128-byte bucket line per op,
 # plus the batch row and the outputs
 B_GET = 8 + 128 + 4 + 1           # key in, bucket line, value out, flag out
@@ -69,14 +53,22 @@ def csrc_sha16():
     return h.hexdigest()[:16]
 
 
-def measured(entry, kernel_ms):
-    """Roofline figures from profiled HBM bytes per launch and the live kernel duration; None
-    where no profile of the current sources exists."""
-    nbytes = PROFILED.get(entry) if PROFILED["csrc_sha16"] == csrc_sha16() else None
+def measured(leg, kernel_ms):
+    """Roofline figures of a leg from its profiled HBM bytes and the live duration; None where no
+    profile of the current sources exists."""
+    nbytes = PROFILED["bytes"].get(leg) if PROFILED["csrc_sha16"] == csrc_sha16() else None
     if nbytes is None or kernel_ms is None:
         return None
     gbs = nbytes / (kernel_ms * 1e-3) / 1e9
     return {"traffic": nbytes, "gbs": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4)}
+
+
+def leg_entry(leg, ms, ops, level):
+    """One entry of roofline.other_legs."""
+    m = measured(leg, ms)
+    return {"ms": ms, "mops": round(ops / ms / 1e3, 1), "level": level,
+            "traffic": m and m["traffic"], "bytes_per_op": m and round(m["traffic"] / ops, 1),
+            "measured_gbs": m and m["gbs"], "frac_measured": m and m["frac"]}
 
 
 def make_unique_keys(n, gen, device):
@@ -107,18 +99,58 @@ def make_queries(keys, n_q, gen, device, zipf_s=1.1):
     return q, n_hit
 
 
-def time_kernel(fn, reps, prep=None):
+class LegMarks:
+    """--markers (profiling runs): every measured leg is bracketed by two tiny launches of the
+    library's clear kernel on a scratch table, whose grid sizes say which leg begins (leg number
+    x 256 threads, numbers from 3) and that it ends (256 threads), so that a kernel trace or a counter
+    run can be cut into legs without knowing the launch sequence.  The numbers are printed at the end
+    (`{"leg_ids": ...}`).  The markers sit outside the timed regions."""
+    ids = {}
+    state = None
+
+    @classmethod
+    def enable(cls, device):
+        from doksparse_amd import CudaClosedHashmap
+        hm = CudaClosedHashmap(n_buckets=1 << 17, device=device)
+        hm.set(torch.arange(8, device=device)[:, None], torch.zeros(8, 1, device=device))
+        cls.state = (hm, device)
+
+    @classmethod
+    def _launch(cls, number):
+        from doksparse_amd import _lib
+        from doksparse_amd.closed_hashmap import _stream_ptr
+        hm, device = cls.state
+        desc = _lib.DokTable.from_buffer_copy(hm._desc)
+        desc.n_phys_buckets = 64 * number                  # (the clear kernel: one workgroup per 64 buckets)
+        assert desc.n_phys_buckets <= hm._n_phys
+        _lib.check(_lib.load().dok_table_clear(ctypes.byref(desc), _stream_ptr(device)), "marker")
+
+    @classmethod
+    def begin(cls, leg):
+        if cls.state is not None and leg is not None:
+            cls._launch(cls.ids.setdefault(leg, 3 + len(cls.ids)))
+
+    @classmethod
+    def end(cls, leg):
+        if cls.state is not None and leg is not None:
+            cls._launch(1)
+
+
+def time_kernel(fn, reps, prep=None, leg=None):
     """Average / min milliseconds of fn() over reps, measured with events on the current stream
-    (the stream the library launches on).  prep() runs untimed before each rep."""
+    (the stream the library launches on).  prep() runs untimed before each rep.  leg: the name
+    the measurement goes by in a profile (see LegMarks)."""
     times = []
     for _ in range(reps):
         if prep is not None:
             prep()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
+        LegMarks.begin(leg)
         e0.record()
         fn()
         e1.record()
+        LegMarks.end(leg)
         e1.synchronize()
         times.append(e0.elapsed_time(e1))
     return float(np.mean(times)), float(np.min(times))
@@ -210,13 +242,15 @@ def cpu_baseline(keys, vals, q, n_hit, seed, what):
     }
 
 
-def timed(fn):
+def timed(fn, leg=None):
     """Milliseconds of fn() (everything it enqueues on the current stream), by events."""
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    LegMarks.begin(leg)
     e0.record()
     out = fn()
     e1.record()
+    LegMarks.end(leg)
     e1.synchronize()
     return e0.elapsed_time(e1), out
 
@@ -235,9 +269,16 @@ def other_configs(device):
     gen.manual_seed(1001)
     k = make_unique_keys(131072, gen, device)
     v = torch.randint(-2**62, 2**62, (65536, 1), generator=gen, device=device)
-    hm = CudaClosedHashmap(n_buckets=131072, device=device)
-    hm.set(k[:8, None], v[:8]); hm.get(k[:8, None]); hm.remove(k[:8, None])   # warm-up (allocation, first launches)
-    res["cfg1_set_ms"] = round(timed(lambda: hm.set(k[:65536, None], v))[0], 4)
+    # (the configuration's set is the first large one of a map; one call is a few tens of
+    # microseconds, so it is taken as the best of five maps)
+    k1 = k[:65536, None]
+    best = None
+    for _ in range(5):
+        hm = CudaClosedHashmap(n_buckets=131072, device=device)
+        hm.set(k[:8, None], v[:8]); hm.get(k[:8, None]); hm.remove(k[:8, None])   # warm-up (allocation, first launches)
+        ms = timed(lambda: hm.set(k1, v), leg="cfg1_set_65536")[0]
+        best = ms if best is None else min(best, ms)
+    res["cfg1_set_ms"] = round(best, 4)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(50):
@@ -245,8 +286,8 @@ def other_configs(device):
     res["cfg1_set_host_us_per_call"] = round((time.perf_counter() - t0) / 50 * 1e6, 1)
     torch.cuda.synchronize()
     hm.get(k[:, None])                  # (the first call of a size pays for the allocation of its outputs)
-    res["cfg1_get_ms"] = round(timed(lambda: hm.get(k[:, None]))[0], 4)
-    res["cfg1_remove_ms"] = round(timed(lambda: hm._remove_rows(k[:32768, None].contiguous(), unique=True))[0], 4)
+    res["cfg1_get_ms"] = round(timed(lambda: hm.get(k[:, None]), leg="cfg1_get_131072")[0], 4)
+    res["cfg1_remove_ms"] = round(timed(lambda: hm._remove_rows(k[:32768, None].contiguous(), unique=True), leg="cfg1_remove_32768")[0], 4)
 
     # cfg2: 1M float32[3] keys -> int64[5], capacity 2^21 (tagged layout)
     gen.manual_seed(1002)
@@ -260,12 +301,12 @@ def other_configs(device):
     warm.set(k2, v2); warm.get(k2[:8]); warm._remove_rows(k2[:8].contiguous()); warm.set(k2[:8], v2[:8])
     del warm
     hm2 = CudaClosedHashmap(n_buckets=2**21, device=device)
-    res["cfg2_set_ms"] = round(timed(lambda: hm2.set(k2, v2))[0], 4)
+    res["cfg2_set_ms"] = round(timed(lambda: hm2.set(k2, v2), leg="cfg2_set_1M_f32x3_i64x5")[0], 4)
     assert hm2.n_elements == 1_000_000
-    res["cfg2_upsert_ms"] = round(timed(lambda: hm2.set(k2, v2))[0], 4)
+    res["cfg2_upsert_ms"] = round(timed(lambda: hm2.set(k2, v2), leg="cfg2_upsert_1M")[0], 4)
     hm2.get(q2)
-    res["cfg2_get_ms"] = round(timed(lambda: hm2.get(q2))[0], 4)
-    res["cfg2_remove_ms"] = round(timed(lambda: hm2._remove_rows(k2[:250_000].contiguous(), unique=True))[0], 4)
+    res["cfg2_get_ms"] = round(timed(lambda: hm2.get(q2), leg="cfg2_get_2M")[0], 4)
+    res["cfg2_remove_ms"] = round(timed(lambda: hm2._remove_rows(k2[:250_000].contiguous(), unique=True), leg="cfg2_remove_250K")[0], 4)
     del hm, hm2, k2, v2, q2
 
     # cfg4: 2-D 1e6 x 1e6 float32, 50M entries
@@ -277,20 +318,20 @@ def other_configs(device):
     # from torch's caching allocator instead of hipMalloc: allocation is not part of the path)
     del_me = SparseDOKTensor((10**6, 10**6), coords, vals, device=device)
     del del_me
-    ms, dok = timed(lambda: SparseDOKTensor((10**6, 10**6), coords, vals, device=device))
+    ms, dok = timed(lambda: SparseDOKTensor((10**6, 10**6), coords, vals, device=device), leg="cfg4_construct_50M")
     res["cfg4_construct_50M_ms"] = round(ms, 3)
     res["cfg4_entries"] = int(lin.numel())
     rows = torch.randint(0, 10**6, (4096, 1), generator=gen, device=device)
     cols = torch.randint(0, 10**6, (1, 256), generator=gen, device=device)
     dok[rows, cols]
-    res["cfg4_getitem_4096x256_ms"] = round(min(timed(lambda: dok[rows, cols])[0] for _ in range(5)), 4)
+    res["cfg4_getitem_4096x256_ms"] = round(min(timed(lambda: dok[rows, cols], leg="cfg4_getitem_4096x256")[0] for _ in range(5)), 4)
     sc = torch.cat([coords[:, :5_000_000], torch.randint(0, 10**6, (2, 5_000_000), generator=gen, device=device)], dim=1)
     sv = torch.randn(sc.shape[1], generator=gen, device=device)
     def scatter():
         dok[sc[0], sc[1]] = sv
-    res["cfg4_setitem_10M_ms"] = round(timed(scatter)[0], 3)           # includes the growth to 120M slots
-    res["cfg4_setitem_10M_again_ms"] = round(timed(scatter)[0], 3)     # all overwrites, no growth
-    res["cfg4_readout_ms"] = round(timed(lambda: dok.storage().items())[0], 3)
+    res["cfg4_setitem_10M_ms"] = round(timed(scatter, leg="cfg4_setitem_10M_with_growth")[0], 3)           # includes the growth to 120M slots
+    res["cfg4_setitem_10M_again_ms"] = round(timed(scatter, leg="cfg4_setitem_10M_overwrite")[0], 3)     # all overwrites, no growth
+    res["cfg4_readout_ms"] = round(timed(lambda: dok.storage().items(), leg="cfg4_readout")[0], 3)
     del dok, coords, vals, lin, sc, sv
 
     # cfg5: 4-D (4096, 4096, 64, 8) float16, 100M entries at load factor 0.85
@@ -305,7 +346,7 @@ def other_configs(device):
     del_me = SparseDOKTensor(size, coords, vals, device=device, storage=new_store())    # (as for cfg4)
     del del_me
     store = new_store()
-    ms, dok = timed(lambda: SparseDOKTensor(size, coords, vals, device=device, storage=store))
+    ms, dok = timed(lambda: SparseDOKTensor(size, coords, vals, device=device, storage=store), leg="cfg5_construct_100M")
     res["cfg5_construct_100M_ms"] = round(ms, 3)
     res["cfg5_entries"] = int(lin.numel())
     i_list = torch.randint(0, 4096, (64,), generator=gen, device=device).tolist()
@@ -316,7 +357,7 @@ def other_configs(device):
             dok[i, :512, idx, mask]
     gets()
     res["cfg5_lookups_per_64_getitems"] = 64 * 512 * 128 * int(mask.sum().item())
-    res["cfg5_64_getitems_ms"] = round(timed(gets)[0], 3)
+    res["cfg5_64_getitems_ms"] = round(timed(gets, leg="cfg5_64_getitems")[0], 3)
     # the host's share: time to enqueue the 64 calls (selector normalisation, descriptor, launch),
     # without waiting for the GPU
     torch.cuda.synchronize()
@@ -327,10 +368,10 @@ def other_configs(device):
     n_gone = lin.numel() // 5
     gone = coords[:, :n_gone].T.contiguous()
     # (`del storage[keys]`: no per-row flags asked for, so the partitioned removal runs)
-    res["cfg5_remove_20M_ms"] = round(timed(lambda: dok.storage().__delitem__(gone))[0], 3)
+    res["cfg5_remove_20M_ms"] = round(timed(lambda: dok.storage().__delitem__(gone), leg="cfg5_remove_20M")[0], 3)
     fresh = torch.stack([torch.randint(0, s, (n_gone,), generator=gen, device=device) for s in size], dim=1)
     fv = torch.randn(n_gone, 1, generator=gen, device=device).half()
-    res["cfg5_reinsert_20M_ms"] = round(timed(lambda: dok.storage().set(fresh, fv))[0], 3)
+    res["cfg5_reinsert_20M_ms"] = round(timed(lambda: dok.storage().set(fresh, fv), leg="cfg5_reinsert_20M")[0], 3)
     res["cfg5_64_getitems_after_churn_ms"] = round(timed(gets)[0], 3)
     return res
 
@@ -362,22 +403,22 @@ def tagged_scale(device, n=32_000_000):
         get = lambda: _lib.check(lib.dok_map_get(desc, q.data_ptr(), n, out_v.data_ptr(), None,
                                                  out_f.data_ptr(), stream), "get")
         rem = lambda: _lib.check(lib.dok_map_remove_unique(desc, quarter.data_ptr(), n // 4, out_f.data_ptr(), stream), "remove")
-        s_avg, _ = time_kernel(set_, 3, prep=clear)
+        s_avg, _ = time_kernel(set_, 3, prep=clear, leg=f"tagged_set_{tag}")
         assert hm.n_elements == n
         # the same rows as the first batch of a new map takes them: clear + insert with one
         # compare-and-swap per row, in one call (dok_map_build_bulk)
         nws = int(lib.dok_bulk_workspace_bytes(desc, n))
         ws = torch.empty(nws, device=device, dtype=torch.uint8)
         build = lambda: _lib.check(lib.dok_map_build_bulk(desc, k.data_ptr(), v.data_ptr(), n, ws.data_ptr(), nws, stream), "build")
-        b_avg, _ = time_kernel(build, 3)
+        b_avg, _ = time_kernel(build, 3, leg=f"tagged_build_{tag}")
         assert hm.n_elements == n
         del ws
-        o_avg, _ = time_kernel(set_, 3)
+        o_avg, _ = time_kernel(set_, 3, leg=f"tagged_overwrite_{tag}")
         get()
         assert int(out_f.sum().item()) == n // 2
-        g_avg, _ = time_kernel(get, 5)
+        g_avg, _ = time_kernel(get, 5, leg=f"tagged_get_{tag}")
         probe = hm.probe_stats(q)
-        r_avg, _ = time_kernel(rem, 1)
+        r_avg, _ = time_kernel(rem, 1, leg=f"tagged_remove_{tag}")
         assert hm.n_elements == n - n // 4
         res[f"tagged_build_mops_{tag}"] = round(n / b_avg / 1e3, 1)
         for nm, ms in (("set", s_avg), ("build", b_avg), ("overwrite", o_avg), ("get", g_avg), ("remove", r_avg)):
@@ -423,7 +464,7 @@ def dok_scale(device):
     gather = lambda: _lib.check(lib.dok_getitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), out.data_ptr(), stream), "getitem")
     gather()
     assert torch.equal(out, vals[pick])
-    g_avg, _ = time_kernel(gather, 5)
+    g_avg, _ = time_kernel(gather, 5, leg="dok_getitem_2p26")
     res["dok_getitem_2p26_ms"] = round(g_avg, 4)
     res["dok_getitem_2p26_mops"] = round(n_g / g_avg / 1e3, 1)
     del pick, r, c, out, ix, keep, plan
@@ -437,14 +478,14 @@ def dok_scale(device):
     view.data = sv.data_ptr()
     view.strides[0] = 1
     scatter = lambda: _lib.check(lib.dok_setitem_dense(ctypes.byref(hm._desc), ctypes.byref(ix), ctypes.byref(view), stream), "setitem")
-    s_first, _ = timed(scatter)                   # half of the rows are new
-    s_avg, _ = time_kernel(scatter, 3)            # every row present
+    s_first, _ = timed(scatter, leg="dok_setitem_10M")    # half of the rows are new
+    s_avg, _ = time_kernel(scatter, 3, leg="dok_setitem_10M_overwrite")            # every row present
     res["dok_setitem_10M_ms"] = round(s_first, 4)
     res["dok_setitem_10M_overwrite_ms"] = round(s_avg, 4)
     assert hm.n_elements > nnz
     # read-out of every entry as [ndim, nnz] coordinates + values
     ro, _ = timed(lambda: hm.items_coo())
-    ro, _ = timed(lambda: hm.items_coo())
+    ro, _ = timed(lambda: hm.items_coo(), leg="dok_readout")
     res["dok_readout_ms"] = round(ro, 4)
     res["dok_entries"] = hm.n_elements
     del dok, hm, coords, vals, lin, sc, sv, ix, keep, plan
@@ -471,7 +512,7 @@ def gather_scale(device, n):
         fn = lambda: _lib.check(lib.dok_line_gather_granule(ctypes.byref(hm._desc), n, 12345, gb, out.data_ptr(),
                                                             _stream_ptr(device)), "gather")
         fn()
-        avg, _ = time_kernel(fn, 10)
+        avg, _ = time_kernel(fn, 10, leg=f"gather_{gb}B")
         res[f"gather_{gb}B_ms"] = round(avg, 4)
         res[f"gather_{gb}B_ggranules_s"] = round(n / avg / 1e6, 2)
         res[f"gather_{gb}B_payload_gbs"] = round(n * gb / avg / 1e6, 1)
@@ -498,14 +539,14 @@ def dok_wide_scale(device, nnz=10_000_000, n_q=1 << 22):
         coords, q = (small << shift).contiguous(), (qs << shift).contiguous()
         best = {"construct": 1e9, "getitem": 1e9, "setitem": 1e9}
         for _ in range(3):
-            ms, dok = timed(lambda: SparseDOKTensor(size, coords, vals, device=device))
+            ms, dok = timed(lambda: SparseDOKTensor(size, coords, vals, device=device), leg=f"{tag}_construct_10M")
             best["construct"] = min(best["construct"], ms)
             dok.storage().rehash(4 * lin.numel())          # room for the scatter: no growth inside the timed call
             got = dok[q[0], q[1]]
-            best["getitem"] = min(best["getitem"], timed(lambda: dok[q[0], q[1]])[0])
+            best["getitem"] = min(best["getitem"], timed(lambda: dok[q[0], q[1]], leg=f"{tag}_getitem_4M")[0])
             def scatter():
                 dok[q[0], q[1]] = sv
-            best["setitem"] = min(best["setitem"], timed(scatter)[0])
+            best["setitem"] = min(best["setitem"], timed(scatter, leg=f"{tag}_setitem_4M")[0])
             # (a coordinate the random half happens to hold twice keeps either of its two values)
             assert int((dok[q[0], q[1]] != sv).sum().item()) <= 16
             del dok
@@ -540,6 +581,9 @@ def main():
                     help="run nothing but the wide-tensor legs of --only-dok")
     ap.add_argument("--only-dok", action="store_true",
                     help="run nothing but the DOK indexing kernels at scale and print their figures (for profiling)")
+    ap.add_argument("--markers", action="store_true",
+                    help="profiling runs: bracket every measured leg with marker launches (see LegMarks) and "
+                         "print the leg numbers at the end")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one read-only pass over the whole table (the live-entry count of "
                          "the read-out path); with the table clear that every run does, this gives "
@@ -555,6 +599,10 @@ def main():
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.markers:
+        import atexit
+        LegMarks.enable(device)
+        atexit.register(lambda: print(json.dumps({"leg_ids": LegMarks.ids}), file=sys.stderr, flush=True))
     if args.only_tagged:
         print(json.dumps({"extra": tagged_scale(device)}), flush=True)
         return
@@ -618,7 +666,7 @@ def main():
     get_mops = n / (ms_per_step * 1e-3) / 1e6
 
     # kernel-only duration for the roofline
-    k_avg, k_min = time_kernel(lambda: raw_get(queries, out_v, out_f), max(args.steps, 5))
+    k_avg, k_min = time_kernel(lambda: raw_get(queries, out_v, out_f), max(args.steps, 5), leg="get_lf05")
     results["get_kernel_ms_lf05"] = round(k_avg, 4)
     results["get_mops_lf05"] = round(n / k_avg / 1e3, 1)
     results["probe_len_lf05"] = round(hm.probe_stats(queries[:, None]), 4)
@@ -629,7 +677,7 @@ def main():
         _dl.check(_dl.load().dok_line_gather(ctypes.byref(hm._desc), n, 12345, chk32.data_ptr(),
                                              _stream_ptr(device)), "line_gather")
     line_gather()
-    lg_avg, _ = time_kernel(line_gather, 5)
+    lg_avg, _ = time_kernel(line_gather, 5, leg="line_gather_lf05")
     results["line_gather_glines_s_lf05"] = round(n / lg_avg / 1e6, 2)
     results["line_gather_gbs_lf05"] = round(n * 128 / lg_avg / 1e6, 1)
     del chk32
@@ -656,7 +704,7 @@ def main():
         # set of all n keys into the cleared table: the per-row compare-and-swap kernel, and the
         # bulk path (partition by table range + merge in LDS) that CudaClosedHashmap.set picks
         # for a batch of this size
-        s_avg, s_min = time_kernel(lambda: raw_set(keys, values), 5, prep=raw_clear)
+        s_avg, s_min = time_kernel(lambda: raw_set(keys, values), 5, prep=raw_clear, leg="set_cas_lf05")
         results["set_cas_kernel_ms_lf05"] = round(s_avg, 4)
         results["set_cas_mops_lf05"] = round(n / s_avg / 1e3, 1)
         assert hm.n_elements == n
@@ -670,7 +718,7 @@ def main():
                                                    vv.data_ptr(), None, ff.data_ptr(), _stream_ptr(device)), "get_stats")
             assert bool(ff.all()) and torch.equal(vv, chk_expect), "bulk insert stored a wrong value"
             del vv, ff
-            b_avg, _ = time_kernel(lambda: bulk(keys, values), 5, prep=raw_clear)
+            b_avg, _ = time_kernel(lambda: bulk(keys, values), 5, prep=raw_clear, leg="set_bulk_lf05")
             results["set_bulk_ms_lf05"] = round(b_avg, 4)
             s_avg = min(s_avg, b_avg)
             # the same rows into a table taken as uninitialised memory (what the first set of a
@@ -679,7 +727,7 @@ def main():
             bulk = raw_bulk_set(hm, n, build=True)
             bulk(keys, values)
             assert hm.n_elements == n
-            bb_avg, _ = time_kernel(lambda: bulk(keys, values), 5)
+            bb_avg, _ = time_kernel(lambda: bulk(keys, values), 5, leg="build_lf05")
             results["build_ms_lf05"] = round(bb_avg, 4)
             results["build_mops_lf05"] = round(n / bb_avg / 1e3, 1)
         results["set_ms_lf05"] = round(s_avg, 4)
@@ -687,7 +735,7 @@ def main():
         assert hm.n_elements == n
         del bulk
         # overwrite pass (every key present)
-        o_avg, _ = time_kernel(lambda: raw_set(keys, values), 5)
+        o_avg, _ = time_kernel(lambda: raw_set(keys, values), 5, leg="overwrite_cas_lf05")
         results["overwrite_mops_lf05"] = round(n / o_avg / 1e3, 1)
         # remove of a random half of the keys (the keys are in random order); the removed rows
         # are stored again outside the timed region
@@ -699,13 +747,13 @@ def main():
                                                        rem_f.data_ptr(), _stream_ptr(device)), "remove")
         raw_remove()
         assert bool(rem_f.all()) and hm.n_elements == n - n // 2
-        r_avg, _ = time_kernel(raw_remove, 5, prep=lambda: raw_set(half, values[: n // 2]))
+        r_avg, _ = time_kernel(raw_remove, 5, prep=lambda: raw_set(half, values[: n // 2]), leg="remove_lf05")
         results["remove_ms_lf05"] = round(r_avg, 4)
         results["remove_mops_lf05"] = round((n // 2) / r_avg / 1e3, 1)
         def raw_remove_cas():                  # any batch, equal keys allowed: one compare-and-swap per row
             _dl.check(_dl.load().dok_map_remove(ctypes.byref(hm._desc), half.data_ptr(), n // 2, rem_f.data_ptr(),
                                                 _stream_ptr(device)), "remove")
-        rc_avg, _ = time_kernel(raw_remove_cas, 3, prep=lambda: raw_set(half, values[: n // 2]))
+        rc_avg, _ = time_kernel(raw_remove_cas, 3, prep=lambda: raw_set(half, values[: n // 2]), leg="remove_cas_lf05")
         results["remove_cas_mops_lf05"] = round((n // 2) / rc_avg / 1e3, 1)
         # the same removal without per-row flags, partitioned by table range (what `del map[keys]` runs)
         nws = int(_dl.load().dok_bulk_workspace_bytes(ctypes.byref(hm._desc), n // 2))
@@ -716,7 +764,7 @@ def main():
                                                          nws, _stream_ptr(device)), "remove_bulk")
             raw_set(half, values[: n // 2]); raw_remove_bulk()
             assert hm.n_elements == n - n // 2
-            rb_avg, _ = time_kernel(raw_remove_bulk, 5, prep=lambda: raw_set(half, values[: n // 2]))
+            rb_avg, _ = time_kernel(raw_remove_bulk, 5, prep=lambda: raw_set(half, values[: n // 2]), leg="remove_bulk_lf05")
             results["remove_bulk_ms_lf05"] = round(rb_avg, 4)
             results["remove_bulk_mops_lf05"] = round((n // 2) / rb_avg / 1e3, 1)
             del rws
@@ -738,24 +786,24 @@ def main():
                 v, f = hm9.get(queries[:, None])
                 assert int(f.sum().item()) == n_hit
                 del v, f
-            g9s.append(time_kernel(lambda: raw_get9(queries, out_v, out_f), 5)[0])
+            g9s.append(time_kernel(lambda: raw_get9(queries, out_v, out_f), 5, leg="get_lf09")[0])
             p9s.append(hm9.probe_stats(queries[:, None]))
             if rep < 3:
                 del hm9, raw_get9, raw_set9, raw_clear9
         g9 = float(np.mean(g9s))
         results["get_kernel_ms_lf09_builds"] = [round(x, 4) for x in g9s]
         results["probe_len_lf09_builds"] = [round(x, 4) for x in p9s]
-        s9, _ = time_kernel(lambda: raw_set9(keys, values), 3, prep=raw_clear9)
+        s9, _ = time_kernel(lambda: raw_set9(keys, values), 3, prep=raw_clear9, leg="set_cas_lf09")
         results["set_cas_mops_lf09"] = round(n / s9 / 1e3, 1)
         bulk9 = raw_bulk_set(hm9, n)
         if bulk9 is not None:
-            b9, _ = time_kernel(lambda: bulk9(keys, values), 3, prep=raw_clear9)
+            b9, _ = time_kernel(lambda: bulk9(keys, values), 3, prep=raw_clear9, leg="set_bulk_lf09")
             assert hm9.n_elements == n
             results["set_bulk_ms_lf09"] = round(b9, 4)
             s9 = min(s9, b9)
             del bulk9
             bulk9 = raw_bulk_set(hm9, n, build=True)
-            bb9, _ = time_kernel(lambda: bulk9(keys, values), 3)
+            bb9, _ = time_kernel(lambda: bulk9(keys, values), 3, leg="build_lf09")
             assert hm9.n_elements == n
             results["build_ms_lf09"] = round(bb9, 4)
         del bulk9
@@ -783,11 +831,14 @@ def main():
                                   ("cfg4_getitem_4096x256", "cfg4_getitem_4096x256_ms", 4096 * 256),
                                   ("cfg4_setitem_10M_with_growth", "cfg4_setitem_10M_ms", 10_000_000),
                                   ("cfg4_setitem_10M_overwrite", "cfg4_setitem_10M_again_ms", 10_000_000),
+                                  ("cfg4_readout", "cfg4_readout_ms", cfg["cfg4_entries"]),
                                   ("cfg5_construct_100M", "cfg5_construct_100M_ms", cfg["cfg5_entries"]),
                                   ("cfg5_64_getitems", "cfg5_64_getitems_ms", cfg["cfg5_lookups_per_64_getitems"]),
                                   ("cfg5_remove_20M", "cfg5_remove_20M_ms", cfg["cfg5_entries"] // 5),
                                   ("cfg5_reinsert_20M", "cfg5_reinsert_20M_ms", cfg["cfg5_entries"] // 5)):
-            legs[name] = {"ms": cfg[ms_key], "mops": round(ops / cfg[ms_key] / 1e3, 1), "level": "api"}
+            # (API level: the time holds the host's share of the call; the bytes are those of every
+            # kernel the call launches)
+            legs[name] = leg_entry(name, cfg[ms_key], ops, "api")
         torch.cuda.empty_cache()
         # the multi-word layout and the DOK indexing kernels at scale: kernel level, with profiled bytes
         tg = tagged_scale(device)
@@ -796,29 +847,29 @@ def main():
         torch.cuda.empty_cache()
         dk = dok_scale(device)
         results.update(dk)
-        for name, entry, ms, ops in (
+        for name, leg, ms, ops in (
                 ("tagged_set_32M_lf05", "tagged_set_lf05", tg["tagged_set_ms_lf05"], nt),
                 ("tagged_build_32M_lf05", "tagged_build_lf05", tg["tagged_build_ms_lf05"], nt),
                 ("tagged_overwrite_32M_lf05", "tagged_overwrite_lf05", tg["tagged_overwrite_ms_lf05"], nt),
                 ("tagged_get_32M_lf05", "tagged_get_lf05", tg["tagged_get_ms_lf05"], nt),
                 ("tagged_remove_8M_lf05", "tagged_remove_lf05", tg["tagged_remove_ms_lf05"], nt // 4),
-                ("tagged_set_32M_lf075", None, tg["tagged_set_ms_lf075"], nt),
-                ("tagged_get_32M_lf075", None, tg["tagged_get_ms_lf075"], nt),
+                ("tagged_set_32M_lf075", "tagged_set_lf075", tg["tagged_set_ms_lf075"], nt),
+                ("tagged_build_32M_lf075", "tagged_build_lf075", tg["tagged_build_ms_lf075"], nt),
+                ("tagged_get_32M_lf075", "tagged_get_lf075", tg["tagged_get_ms_lf075"], nt),
                 ("dok_getitem_2p26", "dok_getitem_2p26", dk["dok_getitem_2p26_ms"], 1 << 26),
                 ("dok_setitem_10M", "dok_setitem_10M", dk["dok_setitem_10M_ms"], 10_000_000),
+                ("dok_setitem_10M_overwrite", "dok_setitem_10M_overwrite", dk["dok_setitem_10M_overwrite_ms"], 10_000_000),
                 ("dok_readout_55M", "dok_readout", dk["dok_readout_ms"], dk["dok_entries"]),
-                ("dok_lin_2p20x2p20_getitem_4M", None, dk.get("dok_lin_getitem_4M_ms"), 1 << 22),
-                ("dok_lin_2p20x2p20_setitem_4M", None, dk.get("dok_lin_setitem_4M_ms"), 1 << 22),
-                ("dok_lin_2p20x2p20_construct_10M", None, dk.get("dok_lin_construct_10M_ms"), 10_000_000),
-                ("dok_wide_2p40x2p40_getitem_4M", None, dk.get("dok_wide_getitem_4M_ms"), 1 << 22),
-                ("dok_wide_2p40x2p40_setitem_4M", None, dk.get("dok_wide_setitem_4M_ms"), 1 << 22),
-                ("dok_wide_2p40x2p40_construct_10M", None, dk.get("dok_wide_construct_10M_ms"), 10_000_000)):
+                ("dok_lin_2p20x2p20_getitem_4M", "dok_lin_getitem_4M", dk.get("dok_lin_getitem_4M_ms"), 1 << 22),
+                ("dok_lin_2p20x2p20_setitem_4M", "dok_lin_setitem_4M", dk.get("dok_lin_setitem_4M_ms"), 1 << 22),
+                ("dok_lin_2p20x2p20_construct_10M", "dok_lin_construct_10M", dk.get("dok_lin_construct_10M_ms"), 10_000_000),
+                ("dok_wide_2p40x2p40_getitem_4M", "dok_wide_getitem_4M", dk.get("dok_wide_getitem_4M_ms"), 1 << 22),
+                ("dok_wide_2p40x2p40_setitem_4M", "dok_wide_setitem_4M", dk.get("dok_wide_setitem_4M_ms"), 1 << 22),
+                ("dok_wide_2p40x2p40_construct_10M", "dok_wide_construct_10M", dk.get("dok_wide_construct_10M_ms"), 10_000_000)):
             if ms is None:
                 continue
-            m = measured(entry, ms) if entry else None
-            legs[name] = {"ms": ms, "mops": round(ops / ms / 1e3, 1), "level": "kernel",
-                          "traffic": m and m["traffic"], "bytes_per_op": m and round(m["traffic"] / ops, 1),
-                          "measured_gbs": m and m["gbs"], "frac_measured": m and m["frac"]}
+            # (the two construct / getitem / setitem triples of the wide-tensor comparison are API level)
+            legs[name] = leg_entry(leg, ms, ops, "api" if leg.startswith(("dok_lin_", "dok_wide_")) else "kernel")
 
     line_model_gbs = n * B_GET / (k_avg * 1e-3) / 1e9
     m_get = measured("get_lf05", k_avg) if default_workload else None
@@ -833,11 +884,8 @@ def main():
                                          ("remove_lf05", "remove_lf05", "remove_ms_lf05", n // 2),
                                          ("remove_bulk_lf05", "remove_bulk_lf05", "remove_bulk_ms_lf05", n // 2)):
             ms = results.get(ms_key)
-            m = measured(entry, ms)
             if ms is not None:
-                legs[name] = {"ms": ms, "mops": round(ops / ms / 1e3, 1),
-                              "traffic": m and m["traffic"], "bytes_per_op": m and round(m["traffic"] / ops, 1),
-                              "measured_gbs": m and m["gbs"], "frac_measured": m and m["frac"]}
+                legs[name] = leg_entry(entry, ms, ops, "kernel")
     line = {
         "metric": "hashmap get/set Mops/s at 64M keys LF 0.5/0.9; achieved HBM GB/s % of peak",
         "value": round(get_mops, 1),

@@ -82,18 +82,6 @@ class _Plan(object):
 
 _PLAN_CACHE_SIZE = 32
 
-try:
-    _raw_stream = torch._C._cuda_getCurrentRawStream
-except AttributeError:                                     # (older torch: the documented way)
-    _raw_stream = None
-
-
-def _stream_of(device):
-    if _raw_stream is not None:
-        return _raw_stream(device.index or 0)
-    return torch.cuda.current_stream(device).cuda_stream
-
-
 class SparseDOKTensor(object):
     def __init__(self, size, indices=None, values=None, device=None, dtype=None, storage=None):
         assert isinstance(size, (list, tuple))
@@ -580,7 +568,7 @@ class SparseDOKTensor(object):
             return torch.zeros(plan.final_shape, device=self.device, dtype=self._dtype)
         values = torch.empty(plan.final_shape, device=self.device, dtype=self._dtype)
         if values.numel():
-            rc = _lib.load().dok_getitem_dense(ctypes.byref(hm._desc), plan.ref, values.data_ptr(), _stream_of(self.device))
+            rc = _lib.load().dok_getitem_dense(ctypes.byref(hm._desc), plan.ref, values.data_ptr(), _stream_ptr(self.device))
             if rc:
                 _lib.check(rc, "__getitem__")
         return values
