@@ -151,6 +151,25 @@ def unique_rows(keys):
     return uniq
 
 
+def unique_rows_inverse(keys):
+    """`unique_rows` together with, for every row of `keys`, the position of its key among the
+    distinct rows."""
+    n = keys.shape[0]
+    ordered = _ordered_bits(keys).reshape(n, -1)
+    uniq, inverse = ordered.unique(dim=0, return_inverse=True)
+    uniq = uniq.reshape(-1, *keys.shape[1:])
+    if keys.dtype.is_floating_point:
+        uniq = _ordered_bits(uniq.view(keys.dtype)).view(keys.dtype)
+    return uniq, inverse
+
+
+def _row_fits(keys, values):
+    """Whether a table can hold key and value rows of these shapes inside its 128-byte buckets."""
+    kb = int(np.prod(keys.shape[1:], dtype=np.int64)) * keys.element_size()
+    vb = int(np.prod(values.shape[1:], dtype=np.int64)) * values.element_size()
+    return _lib.load().dok_layout_of(kb, vb, ctypes.byref(ctypes.c_int32(0))) >= 0
+
+
 class _TableState:
     """Physical state of one table.  Shallow clones of a map share one instance, so a rehash or
     an insert through any of them is seen by all."""
@@ -159,7 +178,8 @@ class _TableState:
 
 _SHARED = ("_table", "_header", "_desc", "_n_phys", "_slots_per_bucket", "_layout", "_n_buckets",
            "_key_shape", "_key_dtype", "_value_shape", "_value_dtype", "_key_bytes", "_value_bytes",
-           "_n_upper", "_n_exact", "_seed", "_pending_clear")
+           "_n_upper", "_n_exact", "_seed", "_pending_clear",
+           "_rows", "_rows_used", "_row_shape", "_row_dtype")
 
 
 def _forward(name):
@@ -240,6 +260,11 @@ class CudaClosedHashmap:
         # True only inside set()/set_coo(), between the allocation of the table and its first
         # insert: the bucket memory is still uninitialised (a bulk build writes all of it)
         self._pending_clear = False
+        # value rows kept outside the table (see _OutOfLineValuesMap); unused by this class
+        self._rows = None
+        self._rows_used = 0
+        self._row_shape = None
+        self._row_dtype = None
 
     # ------------------------------------------------------------------ physical table
     for _name in _SHARED:
@@ -600,6 +625,10 @@ class CudaClosedHashmap:
         if not self._allocated:
             assert new_keys.device == new_values.device == self.device, \
                 f"keys on {new_keys.device}, values on {new_values.device}, the map is on {self.device}"
+            if type(self) is CudaClosedHashmap and self._coord_dims is None and not _row_fits(new_keys, new_values):
+                # key + value rows wider than a bucket: the values move to a side array
+                self.__class__ = _OutOfLineValuesMap
+                return self.set(new_keys, new_values)
             self._init_storage(new_keys, new_values)
         else:
             self._check_keys(new_keys)
@@ -933,11 +962,14 @@ class CudaClosedHashmap:
             rehash_factor=self._rehash_factor, rehash_threshold=self._rehash_threshold,
             coord_dims=self._coord_dims, seed=self._seed, coord_rows=self._coord_rows or None,
         )
+        new.__class__ = self.__class__
         if not deepclone:
             new._st = self._st
             return new
         for name in _SHARED:
             setattr(new, name, getattr(self, name))
+        if self._rows is not None:
+            new._rows = self._rows.clone()
         if self._allocated:
             new._table = self._table.clone()
             new._header = self._header.clone()
@@ -977,3 +1009,132 @@ class CudaClosedHashmap:
             return
         self._check_keys(keys)
         self._remove_rows_no_mask(self._prep_rows(keys, "keys"))
+
+
+class _OutOfLineValuesMap(CudaClosedHashmap):
+    """The map for rows that do not fit a 128-byte bucket (8 * (1 + ceil(K/8) + ceil(V/8)) > 128):
+    the table maps each key to the int64 number of a row of a side array `_rows`
+    [capacity, *value_shape], and the value rows live there.  A CudaClosedHashmap turns into this
+    class in its first `set`, when the widths are known; everything that deals with keys only
+    (remove, keys, rehash, the growth rule, the counts) is the base class working on the
+    key -> row-number table.  The reference compiles its kernels for any KeySize / ValueSize
+    (closed_hashmap_impl_class.cu:7); this keeps every value width usable.  Keys wider than 112
+    bytes still do not fit (a slot needs the tag word, the key words and the row number).
+    Rows of removed keys stay allocated until the side array is compacted, which `set` does when it
+    is full and more than half of it is garbage.  This path is composed from the batched kernels
+    and torch indexing; it is not tuned."""
+
+    @property
+    def value_shape(self):
+        assert self._allocated
+        return torch.Size(self._row_shape)
+
+    @property
+    def value_type(self):
+        return self._row_dtype
+
+    def _reserve_rows(self, n_new):
+        """Room for n_new more value rows.  True if the rows of the present keys were renumbered."""
+        need = self._rows_used + n_new
+        if need <= self._rows.shape[0]:
+            return False
+        if self._rows_used > 2 * self.n_elements:
+            # more than half of the rows belong to removed keys: renumber the live ones 0 .. n-1
+            keys, numbers = CudaClosedHashmap.items(self)
+            n = keys.shape[0]
+            live = self._rows[numbers.reshape(-1)]
+            self._rows = torch.empty(max(2 * (n + n_new), 16), *self._row_shape, device=self.device, dtype=self._row_dtype)
+            self._rows[:n] = live
+            self._rows_used = n
+            if n:
+                CudaClosedHashmap.set(self, keys.reshape(n, *self._key_shape),
+                                      torch.arange(n, device=self.device)[:, None])
+            return True
+        grown = torch.empty(max(need, 2 * self._rows.shape[0]), *self._row_shape, device=self.device, dtype=self._row_dtype)
+        grown[: self._rows_used] = self._rows[: self._rows_used]
+        self._rows = grown
+        return False
+
+    def set(self, new_keys, new_values):
+        assert new_keys.shape[0] == new_values.shape[0], \
+            f"{new_keys.shape[0]} key rows but {new_values.shape[0]} value rows"
+        if self._rows is None:
+            assert new_keys.device == new_values.device == self.device, \
+                f"keys on {new_keys.device}, values on {new_values.device}, the map is on {self.device}"
+            self._row_shape = tuple(new_values.shape[1:])
+            self._row_dtype = new_values.dtype
+            row_bytes = max(int(np.prod(self._row_shape, dtype=np.int64)) * new_values.element_size(), 1)
+            self._rows = torch.empty(max(16, min(1024, (1 << 24) // row_bytes)), *self._row_shape,
+                                     device=self.device, dtype=self._row_dtype)
+            self._rows_used = 0
+            if new_keys.shape[0] == 0:
+                # (the table is allocated by the first set even if the batch is empty, as in the reference)
+                CudaClosedHashmap.set(self, new_keys, torch.empty(0, 1, device=self.device, dtype=torch.long))
+        else:
+            assert new_values.dtype == self._row_dtype, f"values are {new_values.dtype}, the map holds {self._row_dtype}"
+            assert new_values.device == self.device, f"values are on {new_values.device}, the map is on {self.device}"
+            assert tuple(new_values.shape[1:]) == self._row_shape, \
+                f"value rows have shape {tuple(new_values.shape[1:])}, the map holds {self._row_shape}"
+        n = new_keys.shape[0]
+        if n == 0:
+            return
+        if self._allocated:
+            self._check_keys(new_keys)
+        # one row per distinct key of the batch (equal keys: one of their rows wins, whole)
+        keys, inverse = unique_rows_inverse(new_keys)
+        m = keys.shape[0]
+        winner = torch.empty(m, device=self.device, dtype=torch.long)
+        winner.scatter_(0, inverse, torch.arange(n, device=self.device))
+        if self._allocated:
+            numbers, found = CudaClosedHashmap.get(self, keys)
+            numbers = numbers.reshape(-1)
+            missing = ~found
+            n_new = m - int(found.sum().item())
+        else:
+            numbers = torch.empty(m, device=self.device, dtype=torch.long)
+            missing = torch.ones(m, device=self.device, dtype=torch.bool)
+            n_new = m
+        if n_new:
+            if self._reserve_rows(n_new) and n_new < m:
+                numbers = CudaClosedHashmap.get(self, keys)[0].reshape(-1)
+            fresh = torch.arange(self._rows_used, self._rows_used + n_new, device=self.device)
+            numbers = numbers.masked_scatter(missing, fresh)
+            self._rows_used += n_new
+            CudaClosedHashmap.set(self, keys[missing], fresh[:, None])
+        self._rows.index_copy_(0, numbers, new_values[winner])
+
+    def get(self, keys, fallback_value=None):
+        if not self._allocated:
+            raise RuntimeError("store something first")
+        if keys.shape[0] == 0:
+            return (torch.empty(0, *self._row_shape, device=self.device, dtype=self._row_dtype),
+                    torch.empty(0, device=self.device, dtype=torch.bool))
+        numbers, found = CudaClosedHashmap.get(self, keys)            # (row 0 for absent keys)
+        values = self._rows[numbers.reshape(-1)]
+        if fallback_value is None:
+            fallback = torch.zeros((), device=self.device, dtype=self._row_dtype)
+        elif isinstance(fallback_value, Tensor):
+            assert fallback_value.dtype == self._row_dtype
+            fallback = fallback_value.to(self.device)
+        else:
+            fallback = torch.tensor(fallback_value, dtype=self._row_dtype, device=self.device)
+        fallback = torch.broadcast_to(fallback, self._row_shape)
+        values = torch.where(found.reshape(-1, *([1] * len(self._row_shape))), values, fallback)
+        return values, found
+
+    def values(self):
+        if not self._allocated:
+            return None
+        _, numbers = self._compact(False, True)
+        return self._rows[numbers.reshape(-1)]
+
+    def items(self):
+        if not self._allocated:
+            return None, None
+        keys, numbers = CudaClosedHashmap.items(self)
+        return keys, self._rows[numbers.reshape(-1)]
+
+    def set_values(self, selectors, new_values):
+        keys, values = self.items()
+        values[selectors] = new_values
+        self.set(keys.reshape(-1, *self._key_shape), values)

@@ -911,3 +911,105 @@ def test_device_resident_fallback_row(cuda, vshape, vdt):
     # a NULL device row is refused
     assert lib.dok_map_get_dev_fallback(desc, q.data_ptr(), q.shape[0], out_v.data_ptr(), None, out_f.data_ptr(),
                                         None) == _lib.DOK_EINVAL
+
+
+def test_rows_wider_than_a_bucket_against_a_dict(cuda):
+    """Key + value rows that do not fit a 128-byte bucket (the reference compiles its kernels for
+    any KeySize / ValueSize, closed_hashmap_impl_class.cu:7): the values then live in a side array
+    and the table holds row numbers.  Differential test against a Python dict over several rounds of
+    set (with equal keys in a batch), get (hits, misses, fallback row), remove (mask over the sorted
+    distinct keys) and growth from 64 slots; then read-out, set_values, clones and the compaction of
+    the side array after heavy churn."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(77)
+    geoms = [((1,), np.int64, (40,), np.float32), ((3,), np.float32, (20,), np.int64), ((8,), np.int64, (64,), np.int16),
+             ((2,), np.int64, (4, 8), np.float32), ((), np.int64, (33,), np.float64)]
+    for case, (ks, kdt, vs, vdt) in enumerate(geoms):
+        universe = int(10 ** rng.uniform(2.5, 3.8))
+        grow = case % 2 == 0
+        cap = 64 if grow else 2 * universe
+        pool = rng.integers(-2**30, 2**30, size=(universe, *ks)).astype(kdt)
+        pool = np.unique(pool.reshape(universe, -1), axis=0).reshape(-1, *ks)
+        universe = pool.shape[0]
+        hm = CudaClosedHashmap(n_buckets=cap, device=cuda, rehash_threshold=0.75 if grow else 1e9)
+        model = {}
+        for rnd in range(4):
+            n = int(universe * rng.uniform(0.2, 0.9)) + 1
+            idx = rng.integers(0, universe, size=n)
+            v = rng.integers(-100, 100, size=(n, *vs)).astype(vdt)
+            hm.set(*_to(cuda, pool[idx], v))
+            assert tuple(hm.value_shape) == vs and hm.value_type == torch.from_numpy(v).dtype
+            rows_of = {}
+            for i, key in enumerate(idx.tolist()):
+                rows_of.setdefault(key, []).append(i)
+            uk = np.array(sorted(rows_of))
+            got, f = hm.get(torch.from_numpy(pool[uk]).to(cuda))
+            got = got.cpu().numpy()
+            assert bool(f.all()) and got.shape == (len(uk), *vs)
+            for j, key in enumerate(uk.tolist()):       # each key holds the value of ONE of its rows, untorn
+                assert any(np.array_equal(v[r], got[j]) for r in rows_of[key]), (case, rnd, key)
+                model[key] = got[j].copy()
+            assert hm.n_elements == len(model) == len(hm)
+            # remove: mask over the sorted distinct keys of the batch
+            gidx = rng.integers(0, universe, size=int(universe * rng.uniform(0.05, 0.6)) + 1)
+            gk = torch.from_numpy(pool[gidx]).to(cuda)
+            mask = hm.remove(gk).cpu().numpy()
+            distinct = np.unique(pool[gidx].reshape(len(gidx), -1), axis=0)
+            index_of = {bytes(np.ascontiguousarray(pool[i]).reshape(-1)): i for i in set(gidx.tolist())}
+            expect = np.array([index_of[bytes(np.ascontiguousarray(r.astype(kdt)))] in model for r in distinct])
+            assert mask.shape == expect.shape and np.array_equal(mask, expect), (case, rnd)
+            for key in set(gidx.tolist()):
+                model.pop(key, None)
+            assert hm.n_elements == len(model)
+            # every key of the pool, with a fallback row for the absent ones
+            fb = np.full(vs, 7, dtype=vdt)
+            allv, allf = hm.get(torch.from_numpy(pool).to(cuda), fallback_value=torch.from_numpy(fb).to(cuda))
+            allv, allf = allv.cpu().numpy(), allf.cpu().numpy()
+            present = np.zeros(universe, dtype=bool)
+            present[list(model)] = True
+            assert np.array_equal(allf, present), (case, rnd)
+            for key in range(universe):
+                assert np.array_equal(allv[key], model[key] if key in model else fb), (case, rnd, key)
+        # read-out: keys() / values() / items() in one order, equal to the model as a set of rows
+        k, vals = hm.items()
+        assert k.shape[0] == len(model) and vals.shape == (len(model), *vs)
+        assert torch.equal(hm.values(), vals) and torch.equal(hm.keys(), k)
+        back = {bytes(np.ascontiguousarray(pool[i]).reshape(-1)): val for i, val in model.items()}
+        kn, vn = k.cpu().numpy(), vals.cpu().numpy()
+        for j in range(kn.shape[0]):
+            assert np.array_equal(vn[j], back[bytes(np.ascontiguousarray(kn[j]))])
+        # clones: the shallow one shares the entries, the deep one keeps its own
+        shallow, deep = hm.clone(), hm.clone(deepclone=True)
+        some = pool[: min(50, universe)]
+        nv = rng.integers(-5, 5, size=(some.shape[0], *vs)).astype(vdt)
+        hm.set(*_to(cuda, some, nv))
+        assert torch.equal(shallow.get(torch.from_numpy(some).to(cuda))[0].cpu(), torch.from_numpy(nv))
+        dv, df = deep.get(torch.from_numpy(some).to(cuda))
+        for j in range(some.shape[0]):
+            if j in model:
+                assert bool(df[j]) and np.array_equal(dv[j].cpu().numpy(), model[j])
+            else:
+                assert not bool(df[j])
+        # set_values: overwrite the first entry of the read-out order
+        k, vals = hm.items()
+        first = rng.integers(-9, 9, size=vs).astype(vdt)
+        hm.set_values(slice(0, 1), torch.from_numpy(first).to(cuda))
+        assert torch.equal(hm.get(k[:1].reshape(1, *ks))[0][0].cpu(), torch.from_numpy(first))
+        # churn: remove everything and insert again, several times - the side array is compacted instead of growing
+        for _ in range(6):
+            del hm[torch.from_numpy(pool).to(cuda)]
+            assert hm.n_elements == 0
+            v = rng.integers(-100, 100, size=(universe, *vs)).astype(vdt)
+            hm.set(*_to(cuda, pool, v))
+            assert hm.n_elements == universe
+        assert hm._rows.shape[0] <= 6 * universe + 2048
+        got, f = hm.get(torch.from_numpy(pool).to(cuda))
+        assert bool(f.all()) and np.array_equal(got.cpu().numpy(), v)
+
+
+def test_keys_wider_than_a_bucket_are_refused(cuda):
+    """A key row of more than 112 bytes cannot be stored whatever the value width."""
+    from doksparse_amd import CudaClosedHashmap
+    hm = CudaClosedHashmap(n_buckets=64, device=cuda)
+    with pytest.raises((RuntimeError, NotImplementedError, ValueError, AssertionError)):
+        hm.set(torch.zeros(4, 15, device=cuda, dtype=torch.long), torch.zeros(4, 1, device=cuda))

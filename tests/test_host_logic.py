@@ -317,3 +317,24 @@ def test_bulk_path_decision():
     assert bulk_pays(16 * M, nb, S, int(0.6 * nb * S))        # ends 76 % full
     # ... but not below 1.5 rows per bucket
     assert not bulk_pays(12 * M, nb, S, int(0.8 * nb * S))
+
+
+def test_row_width_rule_and_unique_rows_inverse():
+    """Which rows fit a 128-byte bucket (tag word + key words + value words), and the bit-pattern
+    unique with its inverse that the out-of-line value path groups a batch by."""
+    import torch
+    from doksparse_amd import closed_hashmap as ch
+    k1, k3, k15 = torch.zeros(2, 1, dtype=torch.long), torch.zeros(2, 3), torch.zeros(2, 15, dtype=torch.long)
+    assert ch._row_fits(k1, torch.zeros(2, 1))                                  # packed layout
+    assert ch._row_fits(k3, torch.zeros(2, 5, dtype=torch.long))                # 8 * (1 + 2 + 5) = 64
+    assert ch._row_fits(k1, torch.zeros(2, 14, dtype=torch.long))               # 8 * (1 + 1 + 14) = 128
+    assert not ch._row_fits(k1, torch.zeros(2, 15, dtype=torch.long))
+    assert not ch._row_fits(k3, torch.zeros(2, 40))
+    assert not ch._row_fits(k15, torch.zeros(2, 1))                             # the key alone is too wide
+    nan = float("nan")
+    keys = torch.tensor([[0.0, 1.0], [-0.0, 1.0], [nan, 2.0], [0.0, 1.0], [nan, 2.0], [-3.0, 0.5]])
+    uniq, inv = ch.unique_rows_inverse(keys)
+    assert uniq.shape == (4, 2) and inv.shape == (6,)
+    assert torch.equal(uniq.view(torch.int32), ch.unique_rows(keys).view(torch.int32))
+    assert torch.equal(uniq[inv].view(torch.int32), keys.view(torch.int32))     # -0.0 and +0.0 apart, equal NaNs together
+    assert inv[0] == inv[3] and inv[2] == inv[4] and inv[0] != inv[1]
