@@ -773,8 +773,11 @@ __device__ __forceinline__ void tg_place_rows(const DevTable &t, const TgGeom &g
 //     EMPTY: claim -> FULL, payload by plain stores.  A TOMBSTONE keeps the key words of the entry
 //     that was removed, which a concurrent row could mistake for a payload, so it is claimed the
 //     slow way (BUSY, write-through payload, publish).  A claim lost to the row's own tag: defer.
-//   * a row whose key words are all zero is deferred at once: zero is what the key words of a
-//     never-used slot hold, so for every other key "the key words equal mine" proves a payload.
+//   * a row with a key word that is zero is deferred at once.  Zero is what the key words of a
+//     never-used slot hold, and the words of a payload in flight become visible in any order: a slot
+//     claimed by another key of the same fingerprint shows, word by word, either that key's word or
+//     zero.  A row without a zero word can only find "the key words equal mine" when every word has
+//     arrived and the keys are equal, so the comparison is exact.
 // Only values of one word can be overwritten without a lock, so this form serves tables with
 // VW == 1 (every coordinate table).  FRESH - the table held nothing when the kernel started, so
 // whatever a row meets was claimed by this kernel - compares nothing, overwrites nothing (a slot with
@@ -793,9 +796,9 @@ __device__ __forceinline__ void tg_fast_rows(const DevTable &t, const TgGeom &g,
   const int wave_row0 = threadIdx.x & ~63;
   const u64 *krow = lds_rows + threadIdx.x * RS;
   if (!FRESH && pend) {
-    u64 any = 0;
-    for (int k = 0; k < g.KW; k++) any |= krow[1 + k];
-    if (any == 0) { deferred = true; pend = false; }
+    bool zero_word = false;
+    for (int k = 0; k < g.KW; k++) zero_word = zero_word || krow[1 + k] == 0;
+    if (zero_word) { deferred = true; pend = false; }
   }
   if (!pend) home = 0;
   const u32 qbusy = qfull & ~1u;

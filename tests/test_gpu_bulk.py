@@ -612,7 +612,7 @@ def tagged_fast_always(monkeypatch):
 
 def test_multiword_fast_and_per_row_insert_agree_on_random_configurations(cuda, monkeypatch):
     """Random configurations of the multi-word layout (key / value widths of one to four slots per
-    bucket, load factors up to 0.95, batches with many repeated keys, the all-zero key, removals in
+    bucket, load factors up to 0.95, batches with many repeated keys, keys with zero words, removals in
     between so that tombstones are re-used): three batches each, once through the per-row protocol
     and once through the fast form - the first batch of a map as a build into the new table, later
     ones as upserts where the values are one word wide.  Values are a function of key and batch, so
@@ -638,7 +638,8 @@ def test_multiword_fast_and_per_row_insert_agree_on_random_configurations(cuda, 
             keyspace = torch.randint(-2**20, 2**20, (universe, kw), generator=g, device=cuda).to(kdt)
         else:
             keyspace = torch.randint(-2**30, 2**30, (universe, kw), generator=g, device=cuda).to(kdt)
-        keyspace[0] = 0                                  # the all-zero key (always deferred by the fast form)
+        keyspace[0] = 0                                  # the all-zero key ...
+        keyspace[1: min(200, universe // 4), case % kw] = 0   # ... and keys with one zero word (the fast form defers both kinds)
         keyspace = torch.unique(keyspace, dim=0)
         universe = keyspace.shape[0]
         maps = []
