@@ -350,9 +350,13 @@ def other_configs(device):
     warm = CudaClosedHashmap(n_buckets=2**21, device=device)
     warm.set(k2, v2); warm.get(k2[:8]); warm._remove_rows(k2[:8].contiguous()); warm.set(k2[:8], v2[:8])
     del warm
-    hm2 = CudaClosedHashmap(n_buckets=2**21, device=device)
-    res["cfg2_set_ms"] = round(timed(lambda: hm2.set(k2, v2), leg="cfg2_set_1M_f32x3_i64x5")[0], 4)
-    assert hm2.n_elements == 1_000_000
+    best = None
+    for _ in range(3):                  # (best of three new maps, like configuration 1's first set)
+        hm2 = CudaClosedHashmap(n_buckets=2**21, device=device)
+        ms = timed(lambda: hm2.set(k2, v2), leg="cfg2_set_1M_f32x3_i64x5")[0]
+        best = ms if best is None else min(best, ms)
+        assert hm2.n_elements == 1_000_000
+    res["cfg2_set_ms"] = round(best, 4)
     res["cfg2_upsert_ms"] = round(timed(lambda: hm2.set(k2, v2), leg="cfg2_upsert_1M")[0], 4)
     hm2.get(q2)
     res["cfg2_get_ms"] = round(timed(lambda: hm2.get(q2), leg="cfg2_get_2M")[0], 4)
