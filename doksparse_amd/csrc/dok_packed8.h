@@ -512,7 +512,9 @@ __global__ __launch_bounds__(DOK_TPB) void p8_get_kernel(DevTable t, const void 
 // The header counters are updated once per workgroup at the end (dok_block_add3: every thread of
 // the workgroup has to reach the end of this function, exactly once per kernel).
 // The core works through the rows [next, end) that the caller assigns to this wave.
-template <int V, class Src>
+// RETRY: see the claim below; switched on where it costs no registers (it takes three more in the
+// indexing kernel, which already spills).
+template <int V, bool RETRY = false, class Src>
 __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 next, i64 end,
                                                       u8 *__restrict__ stored, Src src) {
   const P8Lane L;
@@ -650,7 +652,22 @@ __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 nex
         const u64 expect = slot_tomb ? DOK_P8_TOMB : DOK_P8_EMPTY;
         const u64 tbb = (u64)home + td;
         u64 *tp = buckets + (tbb >= nb ? tbb - nb : tbb) * 16;
-        const u64 old = atomicCAS(tp + slot_s, expect, sk);
+        u64 old = atomicCAS(tp + slot_s, expect, sk);
+        if (RETRY && dcur == td) {
+          // The claim follows the choice in the same pass (nothing marked to look at first), so the
+          // pass's view of the slot's bucket is still at hand: a slot lost to another key is
+          // followed at once by the other free slots of the same kind that the view showed, in the
+          // order every row of this key tries them, instead of by another pass that loads the
+          // bucket again.  (Rows that arrive at one bucket together - a batch that is large
+          // against a small table - otherwise pay a load and a claim, one after the other, per
+          // lost slot.)
+          u32 cand = (slot_tomb ? gt : ge) & ~(1u << slot_s);
+          while (old != expect && old != sk && cand != 0) {
+            slot_s = p8_pick(cand, p8_slot_start<V>(sk));
+            cand &= ~(1u << slot_s);
+            old = atomicCAS(tp + slot_s, expect, sk);
+          }
+        }
         if (old == expect) {
           P8<V>::store(tp, slot_s, val);
           if (td > 0) p8_mark(buckets + (u64)home * 16 + DOK_P8_META, td, fbit, ((u64)far_home << 32) | md_home);
@@ -676,7 +693,7 @@ __device__ __forceinline__ void p8_stream_insert_rows(const DevTable &t, i64 nex
 }
 
 // Rows [0, n) split into one contiguous share per wave of the grid.
-template <int V, class Src>
+template <int V, bool RETRY = false, class Src>
 __device__ __forceinline__ void p8_stream_insert(const DevTable &t, i64 n, i64 rows_per_wave,
                                                  u8 *__restrict__ stored, Src src) {
   const i64 wave = ((i64)blockIdx.x * DOK_TPB + threadIdx.x) >> 6;
@@ -684,14 +701,14 @@ __device__ __forceinline__ void p8_stream_insert(const DevTable &t, i64 n, i64 r
   i64 end = next + rows_per_wave;
   if (end > n) end = n;
   if (next > end) next = end;
-  p8_stream_insert_rows<V>(t, next, end, stored, src);
+  p8_stream_insert_rows<V, RETRY>(t, next, end, stored, src);
 }
 
 template <int V, int KF>
 __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void p8_set_kernel(DevTable t, const void *__restrict__ keys,
                                                          const void *__restrict__ values, i64 n,
                                                          u8 *__restrict__ stored, i64 rows_per_wave) {
-  p8_stream_insert<V>(t, n, rows_per_wave, stored, [&](i64 i, u64 &key, u64 &val) -> int {
+  p8_stream_insert<V, KF == DOK_KF_RAW>(t, n, rows_per_wave, stored, [&](i64 i, u64 &key, u64 &val) -> int {
     if (!dok_load_key8<KF>(t, keys, i, n, key)) return 1;
     val = dok_load_val<V>(values, i);
     return 0;
