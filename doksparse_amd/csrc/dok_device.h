@@ -61,19 +61,27 @@ __device__ __forceinline__ u64 dok_div_stride(u64 n, u64 magic, int shift) {
   return (((n - q) >> 1) + q) >> shift;
 }
 
-// Kernel-argument form of dok_index_t (+ optional source-value view).
-struct DevIndex {
+// Kernel-argument form of dok_index_t (+ optional source-value view), for tensors and index spaces
+// of up to MAXD dimensions.  The descriptor travels by value and the kernels read it with scalar
+// loads, each of which a use waits for: with arrays for 8 dimensions (8 x 8 selector strides) a
+// gather of a few thousand elements spends 4 of its 12 microseconds there, so tensors of up to 4
+// dimensions indexed over up to 4 axes - nearly all - take the small form.
+template <int MAXD>
+struct DevIndexT {
+  static constexpr int DIMS = MAXD;
   int ndim;
   int sel_ndim;
   i64 n_elems;
-  i64 shape[DOK_LIN_DIMS];
-  i64 estride[DOK_LIN_DIMS];       // C-contiguous strides of `shape`
-  const i64 *sel[DOK_LIN_DIMS];              // NULL: the coordinate is sbase + offset itself
-  i64 sbase[DOK_LIN_DIMS];
-  i64 sstride[DOK_LIN_DIMS][DOK_LIN_DIMS];
+  i64 shape[MAXD];
+  i64 estride[MAXD];               // C-contiguous strides of `shape`
+  const i64 *sel[MAXD];            // NULL: the coordinate is sbase + offset itself
+  i64 sbase[MAXD];
+  i64 sstride[MAXD][MAXD];
   const void *src;
-  i64 vstride[DOK_LIN_DIMS];
+  i64 vstride[MAXD];
 };
+typedef DevIndexT<DOK_LIN_DIMS> DevIndex;
+typedef DevIndexT<4> DevIndex4;
 
 __device__ __forceinline__ u64 dok_fmix64(u64 x) {
   x ^= x >> 33; x *= 0xff51afd7ed558ccdULL;
@@ -300,19 +308,24 @@ template <int V> __device__ __forceinline__ void dok_store_val(void *values, i64
 // `voff` receives the element offset into the source view.  Loops run to the compile-time
 // maximum with uniform guards so that idx[] stays in registers; the host zeroes the strides of
 // unused axes.
-__device__ __forceinline__ bool dok_gather_at(const DevTable &t, const DevIndex &ix,
-                                              const i64 (&idx)[DOK_LIN_DIMS], u64 &key, i64 &voff) {
+template <class IX>
+__device__ __forceinline__ bool dok_gather_at(const DevTable &t, const IX &ix,
+                                              const i64 (&idx)[IX::DIMS], u64 &key, i64 &voff) {
+  constexpr int DIMS = IX::DIMS;
+  // The small form runs its stride loops without guards: the unused strides are zero, and nothing
+  // then stands between the descriptor's scalar loads and the head of the kernel.
+  constexpr bool GUARD = DIMS > 4;
   // first every dimension's selector is read, then the values are used: a use next to its load
   // would make the loads of the dimensions wait for one another
-  i64 g[DOK_LIN_DIMS];
+  i64 g[DIMS];
   #pragma unroll
-  for (int d = 0; d < DOK_LIN_DIMS; d++) {
+  for (int d = 0; d < DIMS; d++) {
     g[d] = 0;
-    if (d < ix.ndim) {
+    if (!GUARD || d < ix.ndim) {
       i64 off = 0;
       #pragma unroll
-      for (int j = 0; j < DOK_LIN_DIMS; j++)
-        if (j < ix.sel_ndim) off += idx[j] * ix.sstride[d][j];
+      for (int j = 0; j < DIMS; j++)
+        if (!GUARD || j < ix.sel_ndim) off += idx[j] * ix.sstride[d][j];
       const i64 *sp = ix.sel[d];
       g[d] = off;
       if (sp) g[d] = sp[off];
@@ -321,7 +334,7 @@ __device__ __forceinline__ bool dok_gather_at(const DevTable &t, const DevIndex 
   bool ok = true;
   u64 k = 0;
   #pragma unroll
-  for (int d = 0; d < DOK_LIN_DIMS; d++) {
+  for (int d = 0; d < DIMS; d++) {
     if (d < ix.ndim) {
       const i64 c = ix.sbase[d] + g[d];
       ok = ok && ((u64)c < (u64)t.lin_dims[d]);
@@ -330,23 +343,26 @@ __device__ __forceinline__ bool dok_gather_at(const DevTable &t, const DevIndex 
   }
   i64 vo = 0;
   #pragma unroll
-  for (int j = 0; j < DOK_LIN_DIMS; j++)
-    if (j < ix.sel_ndim) vo += idx[j] * ix.vstride[j];
+  for (int j = 0; j < DIMS; j++)
+    if (!GUARD || j < ix.sel_ndim) vo += idx[j] * ix.vstride[j];
   voff = vo;
   key = k;
   return ok;
 }
 
 // The same for element e (row-major offset) of the index space: unravel e over `shape` first.
-__device__ __forceinline__ bool dok_gather_key(const DevTable &t, const DevIndex &ix, i64 e,
+template <class IX>
+__device__ __forceinline__ bool dok_gather_key(const DevTable &t, const IX &ix, i64 e,
                                                u64 &key, i64 &voff) {
-  i64 idx[DOK_LIN_DIMS];
+  constexpr int DIMS = IX::DIMS;
+  constexpr bool GUARD = DIMS > 4;           // (the divisors of unused axes are 1)
+  i64 idx[DIMS];
   if (ix.n_elems <= 0x7fffffffLL) {
     u32 rem = (u32)e;
     #pragma unroll
-    for (int j = 0; j < DOK_LIN_DIMS; j++) {
+    for (int j = 0; j < DIMS; j++) {
       idx[j] = 0;
-      if (j < ix.sel_ndim) {
+      if (!GUARD || j < ix.sel_ndim) {
         u32 s = (u32)ix.estride[j];
         u32 q = rem / s;
         rem -= q * s;
@@ -356,7 +372,7 @@ __device__ __forceinline__ bool dok_gather_key(const DevTable &t, const DevIndex
   } else {
     u64 rem = (u64)e;
     #pragma unroll
-    for (int j = 0; j < DOK_LIN_DIMS; j++) {
+    for (int j = 0; j < DIMS; j++) {
       idx[j] = 0;
       if (j < ix.sel_ndim) {
         u64 s = (u64)ix.estride[j];

@@ -934,8 +934,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_to_dense_kernel(DevTable t, void *
 
 // ---- DOK indexing kernels: gather coordinate -> linear key -> table op ----------------------
 
-template <int V>
-__global__ __launch_bounds__(DOK_TPB) void p8_getitem_kernel(DevTable t, DevIndex ix, void *__restrict__ out) {
+template <int V, class IX>
+__global__ __launch_bounds__(DOK_TPB) void p8_getitem_kernel(DevTable t, IX ix, void *__restrict__ out) {
   DOK_TILE_LOOP(ix.n_elems) {
     const i64 e = DOK_TILE_ROW();
     const bool active = e < ix.n_elems;
@@ -951,8 +951,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_getitem_kernel(DevTable t, DevInde
   }
 }
 
-template <int V>
-__global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void p8_setitem_kernel(DevTable t, DevIndex ix, i64 rows_per_wave) {
+template <int V, class IX>
+__global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void p8_setitem_kernel(DevTable t, IX ix, i64 rows_per_wave) {
   p8_stream_insert<V>(t, ix.n_elems, rows_per_wave, nullptr, [&](i64 e, u64 &key, u64 &val) -> int {
     i64 voff = 0;
     if (!dok_gather_key(t, ix, e, key, voff)) return 1;
@@ -961,8 +961,8 @@ __global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void p8_setitem_kernel(D
   });
 }
 
-template <int V>
-__global__ __launch_bounds__(DOK_TPB) void p8_countitems_kernel(DevTable t, DevIndex ix, i64 *count) {
+template <int V, class IX>
+__global__ __launch_bounds__(DOK_TPB) void p8_countitems_kernel(DevTable t, IX ix, i64 *count) {
   int n_found = 0;
   DOK_TILE_LOOP(ix.n_elems) {
     const i64 e = DOK_TILE_ROW();
@@ -980,8 +980,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_countitems_kernel(DevTable t, DevI
   dok_block_add1(count, n_found);
 }
 
-template <int V>
-__global__ __launch_bounds__(DOK_TPB) void p8_zeroitems_kernel(DevTable t, DevIndex ix) {
+template <int V, class IX>
+__global__ __launch_bounds__(DOK_TPB) void p8_zeroitems_kernel(DevTable t, IX ix) {
   int n_removed = 0;
   DOK_TILE_LOOP(ix.n_elems) {
     const i64 e = DOK_TILE_ROW();
@@ -1002,8 +1002,8 @@ __global__ __launch_bounds__(DOK_TPB) void p8_zeroitems_kernel(DevTable t, DevIn
 
 // Sparse-valued getitem: every element of the index space whose coordinate is stored in `t` is
 // inserted into `out`, a coordinate-keyed table over the index space itself (key = e).
-template <int V>
-__global__ __launch_bounds__(DOK_TPB) void p8_getitem_sparse_kernel(DevTable t, DevIndex ix, DevTable out) {
+template <int V, class IX>
+__global__ __launch_bounds__(DOK_TPB) void p8_getitem_sparse_kernel(DevTable t, IX ix, DevTable out) {
   int n_fresh = 0, n_full = 0;
   DOK_TILE_LOOP(ix.n_elems) {
     const i64 e = DOK_TILE_ROW();
@@ -1029,17 +1029,17 @@ __global__ __launch_bounds__(DOK_TPB) void p8_getitem_sparse_kernel(DevTable t, 
 // Sparse-valued setitem: source entry k has index vector src_indices[j*n_src + k] (j over the
 // axes of the index space) and value src_values[k]; entries whose value is zero under
 // `nonzero_mask` (all ones for integers, sign bit cleared for floating values) are skipped.
-template <int V>
-__global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void p8_setitem_sparse_kernel(DevTable t, DevIndex ix,
+template <int V, class IX>
+__global__ __launch_bounds__(DOK_TPB, DOK_STREAM_WAVES) void p8_setitem_sparse_kernel(DevTable t, IX ix,
                                                                     const i64 *__restrict__ src_indices,
                                                                     const void *__restrict__ src_values,
                                                                     i64 n_src, u64 nonzero_mask,
                                                                     i64 rows_per_wave) {
   p8_stream_insert<V>(t, n_src, rows_per_wave, nullptr, [&](i64 k, u64 &key, u64 &val) -> int {
-    i64 idx[DOK_LIN_DIMS];
+    i64 idx[IX::DIMS];
     bool inside = true;
     #pragma unroll
-    for (int j = 0; j < DOK_LIN_DIMS; j++) {
+    for (int j = 0; j < IX::DIMS; j++) {
       idx[j] = 0;
       if (j < ix.sel_ndim) {
         idx[j] = src_indices[(i64)j * n_src + k];

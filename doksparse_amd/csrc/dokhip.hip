@@ -177,6 +177,7 @@ int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *s
     if (n >> 62) return DOK_EINVAL;
   }
   d.n_elems = (i64)n;
+  for (int j = ix->sel_ndim; j < MAXD; j++) d.estride[j] = 1;      // (divisors of the unused axes)
   for (int k = 0; k < ix->ndim; k++) {
     d.sel[k] = (const i64 *)ix->sel[k].data;
     d.sbase[k] = ix->sel[k].base;
@@ -198,6 +199,11 @@ int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *s
 int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *src, DevIndex &d) {
   return make_dev_index<DevIndex, DOK_LIN_DIMS>(t, ix, src, d);
 }
+int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *src, DevIndex4 &d) {
+  return make_dev_index<DevIndex4, 4>(t, ix, src, d);
+}
+// Whether the small descriptor form serves this index.
+inline bool small_index(const dok_index_t *ix) { return ix && ix->ndim <= 4 && ix->sel_ndim >= 0 && ix->sel_ndim <= 4; }
 int make_dev_index(const DevTable &t, const dok_index_t *ix, const dok_view_t *src, DevIndexW &d) {
   return make_dev_index<DevIndexW, DOK_MAX_DIMS>(t, ix, src, d);
 }
@@ -242,6 +248,80 @@ const i64 kMaxRows = (i64)0x7fffffff * DOK_TPB;
 #define P8_DISPATCH_LIN(vb, lin, CALL)                                          \
   if (lin) { constexpr int KF = DOK_KF_ROWS; P8_DISPATCH(vb, CALL) }            \
   else { constexpr int KF = DOK_KF_RAW; P8_DISPATCH(vb, CALL) }
+
+// The fused kernels of the packed layout, for either size of the index descriptor.
+template <class IX>
+int getitem_dense_lin(const DevTable &d, const dok_index_t *ix, void *out, hipStream_t s) {
+  IX di;
+  int rc = make_dev_index(d, ix, nullptr, di);
+  if (rc) return rc;
+  if (di.n_elems == 0) return DOK_OK;
+  if (!out || di.n_elems > kMaxRows) return DOK_EINVAL;
+  const DeviceScope on_stream_device(s);
+  P8_DISPATCH(d.value_bytes, (p8_getitem_kernel<V, IX><<<grid_for(di.n_elems), DOK_TPB, 0, s>>>(d, di, out)));
+  return note_launch();
+}
+template <class IX>
+int setitem_dense_lin(const DevTable &d, const dok_index_t *ix, const dok_view_t *src, hipStream_t s) {
+  IX di;
+  int rc = make_dev_index(d, ix, src, di);
+  if (rc) return rc;
+  if (di.n_elems == 0) return DOK_OK;
+  if (di.n_elems > kMaxRows) return DOK_EINVAL;
+  const DeviceScope on_stream_device(s);
+  const unsigned grid = grid_counting(di.n_elems);
+  P8_DISPATCH(d.value_bytes, (p8_setitem_kernel<V, IX><<<grid, DOK_TPB, 0, s>>>(d, di, rows_per_wave(di.n_elems, grid))));
+  return note_launch();
+}
+template <class IX>
+int count_items_lin(const DevTable &d, const dok_index_t *ix, int64_t *count, hipStream_t s) {
+  IX di;
+  int rc = make_dev_index(d, ix, nullptr, di);
+  if (rc) return rc;
+  if (di.n_elems == 0) return DOK_OK;
+  if (!count || di.n_elems > kMaxRows) return DOK_EINVAL;
+  const DeviceScope on_stream_device(s);
+  P8_DISPATCH(d.value_bytes, (p8_countitems_kernel<V, IX><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di, (i64 *)count)));
+  return note_launch();
+}
+template <class IX>
+int zero_items_lin(const DevTable &d, const dok_index_t *ix, hipStream_t s) {
+  IX di;
+  int rc = make_dev_index(d, ix, nullptr, di);
+  if (rc) return rc;
+  if (di.n_elems == 0) return DOK_OK;
+  if (di.n_elems > kMaxRows) return DOK_EINVAL;
+  const DeviceScope on_stream_device(s);
+  P8_DISPATCH(d.value_bytes, (p8_zeroitems_kernel<V, IX><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di)));
+  return note_launch();
+}
+template <class IX>
+int getitem_sparse_lin(const DevTable &d, const dok_index_t *ix, const DevTable &o, hipStream_t s) {
+  IX di;
+  int rc = make_dev_index(d, ix, nullptr, di);
+  if (rc) return rc;
+  if (o.lin_ndim != di.sel_ndim) return DOK_EINVAL;
+  for (int j = 0; j < di.sel_ndim; j++) if (o.lin_dims[j] != di.shape[j]) return DOK_EINVAL;
+  if (di.n_elems == 0) return DOK_OK;
+  if (di.n_elems > kMaxRows) return DOK_EINVAL;
+  const DeviceScope on_stream_device(s);
+  P8_DISPATCH(d.value_bytes, (p8_getitem_sparse_kernel<V, IX><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di, o)));
+  return note_launch();
+}
+template <class IX>
+int setitem_sparse_lin(const DevTable &d, const dok_index_t *ix, const int64_t *src_indices,
+                              const void *src_values, int64_t n_src, uint64_t nonzero_mask, hipStream_t s) {
+  IX di;
+  int rc = make_dev_index(d, ix, nullptr, di);
+  if (rc) return rc;
+  if (n_src == 0) return DOK_OK;
+  if (!src_values || (!src_indices && di.sel_ndim > 0)) return DOK_EINVAL;
+  const DeviceScope on_stream_device(s);
+  const unsigned grid = grid_counting(n_src);
+  P8_DISPATCH(d.value_bytes, (p8_setitem_sparse_kernel<V, IX><<<grid, DOK_TPB, 0, s>>>(
+      d, di, (const i64 *)src_indices, src_values, n_src, nonzero_mask, rows_per_wave(n_src, grid))));
+  return note_launch();
+}
 
 }  // namespace
 
@@ -691,14 +771,7 @@ int dok_getitem_dense(const dok_table_t *t, const dok_index_t *ix, void *out, vo
     if (rc) return rc;
     return note_launch();
   }
-  DevIndex di;
-  rc = make_dev_index(d, ix, nullptr, di);
-  if (rc) return rc;
-  if (di.n_elems == 0) return DOK_OK;
-  if (!out || di.n_elems > kMaxRows) return DOK_EINVAL;
-  const DeviceScope on_stream_device(s);
-  P8_DISPATCH(d.value_bytes, (p8_getitem_kernel<V><<<grid_for(di.n_elems), DOK_TPB, 0, s>>>(d, di, out)));
-  return note_launch();
+  return small_index(ix) ? getitem_dense_lin<DevIndex4>(d, ix, out, s) : getitem_dense_lin<DevIndex>(d, ix, out, s);
 }
 
 int dok_setitem_dense(const dok_table_t *t, const dok_index_t *ix, const dok_view_t *src, void *stream) {
@@ -718,15 +791,7 @@ int dok_setitem_dense(const dok_table_t *t, const dok_index_t *ix, const dok_vie
     if (rc) return rc;
     return note_launch();
   }
-  DevIndex di;
-  rc = make_dev_index(d, ix, src, di);
-  if (rc) return rc;
-  if (di.n_elems == 0) return DOK_OK;
-  if (di.n_elems > kMaxRows) return DOK_EINVAL;
-  const DeviceScope on_stream_device(s);
-  const unsigned grid = grid_counting(di.n_elems);
-  P8_DISPATCH(d.value_bytes, (p8_setitem_kernel<V><<<grid, DOK_TPB, 0, s>>>(d, di, rows_per_wave(di.n_elems, grid))));
-  return note_launch();
+  return small_index(ix) ? setitem_dense_lin<DevIndex4>(d, ix, src, s) : setitem_dense_lin<DevIndex>(d, ix, src, s);
 }
 
 int dok_setitem_dense_bulk(const dok_table_t *t, const dok_index_t *ix, const dok_view_t *src, void *workspace,
@@ -766,14 +831,7 @@ int dok_count_items(const dok_table_t *t, const dok_index_t *ix, int64_t *count,
     if (rc) return rc;
     return note_launch();
   }
-  DevIndex di;
-  rc = make_dev_index(d, ix, nullptr, di);
-  if (rc) return rc;
-  if (di.n_elems == 0) return DOK_OK;
-  if (!count || di.n_elems > kMaxRows) return DOK_EINVAL;
-  const DeviceScope on_stream_device(s);
-  P8_DISPATCH(d.value_bytes, (p8_countitems_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di, (i64 *)count)));
-  return note_launch();
+  return small_index(ix) ? count_items_lin<DevIndex4>(d, ix, count, s) : count_items_lin<DevIndex>(d, ix, count, s);
 }
 
 int dok_zero_items(const dok_table_t *t, const dok_index_t *ix, void *stream) {
@@ -792,14 +850,7 @@ int dok_zero_items(const dok_table_t *t, const dok_index_t *ix, void *stream) {
     if (rc) return rc;
     return note_launch();
   }
-  DevIndex di;
-  rc = make_dev_index(d, ix, nullptr, di);
-  if (rc) return rc;
-  if (di.n_elems == 0) return DOK_OK;
-  if (di.n_elems > kMaxRows) return DOK_EINVAL;
-  const DeviceScope on_stream_device(s);
-  P8_DISPATCH(d.value_bytes, (p8_zeroitems_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di)));
-  return note_launch();
+  return small_index(ix) ? zero_items_lin<DevIndex4>(d, ix, s) : zero_items_lin<DevIndex>(d, ix, s);
 }
 
 int dok_getitem_sparse(const dok_table_t *t, const dok_index_t *ix, const dok_table_t *out, void *stream) {
@@ -825,16 +876,7 @@ int dok_getitem_sparse(const dok_table_t *t, const dok_index_t *ix, const dok_ta
     if (rc) return rc;
     return note_launch();
   }
-  DevIndex di;
-  rc = make_dev_index(d, ix, nullptr, di);
-  if (rc) return rc;
-  if (o.lin_ndim != di.sel_ndim) return DOK_EINVAL;
-  for (int j = 0; j < di.sel_ndim; j++) if (o.lin_dims[j] != di.shape[j]) return DOK_EINVAL;
-  if (di.n_elems == 0) return DOK_OK;
-  if (di.n_elems > kMaxRows) return DOK_EINVAL;
-  const DeviceScope on_stream_device(s);
-  P8_DISPATCH(d.value_bytes, (p8_getitem_sparse_kernel<V><<<grid_counting(di.n_elems), DOK_TPB, 0, s>>>(d, di, o)));
-  return note_launch();
+  return small_index(ix) ? getitem_sparse_lin<DevIndex4>(d, ix, o, s) : getitem_sparse_lin<DevIndex>(d, ix, o, s);
 }
 
 int dok_setitem_sparse(const dok_table_t *t, const dok_index_t *ix, const int64_t *src_indices,
@@ -860,16 +902,8 @@ int dok_setitem_sparse(const dok_table_t *t, const dok_index_t *ix, const int64_
     if (rc) return rc;
     return note_launch();
   }
-  DevIndex di;
-  rc = make_dev_index(d, ix, nullptr, di);
-  if (rc) return rc;
-  if (n_src == 0) return DOK_OK;
-  if (!src_values || (!src_indices && di.sel_ndim > 0)) return DOK_EINVAL;
-  const DeviceScope on_stream_device(s);
-  const unsigned grid = grid_counting(n_src);
-  P8_DISPATCH(d.value_bytes, (p8_setitem_sparse_kernel<V><<<grid, DOK_TPB, 0, s>>>(
-      d, di, (const i64 *)src_indices, src_values, n_src, nonzero_mask, rows_per_wave(n_src, grid))));
-  return note_launch();
+  return small_index(ix) ? setitem_sparse_lin<DevIndex4>(d, ix, src_indices, src_values, n_src, nonzero_mask, s)
+                         : setitem_sparse_lin<DevIndex>(d, ix, src_indices, src_values, n_src, nonzero_mask, s);
 }
 
 int dok_to_dense(const dok_table_t *t, void *dense, void *stream) {

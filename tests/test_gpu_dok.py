@@ -580,7 +580,9 @@ def test_random_selectors_against_the_oracle(cuda, rows, monkeypatch):
     rng = np.random.default_rng(20)
     compared = 0
     for case in range(80):
-        shape = tuple(int(x) for x in rng.integers(1, 9, size=int(rng.integers(1, 6))))
+        # (one to eight dimensions: up to four take the small index descriptor, more the large one)
+        nd = int(rng.integers(1, 9))
+        shape = tuple(int(x) for x in rng.integers(1, 9 if nd <= 5 else 4, size=nd))
         vol = int(np.prod(shape))
         nnz = max(1, int(rng.integers(0, vol + 1)))
         idx = torch.stack(torch.unravel_index(torch.from_numpy(rng.permutation(vol)[:nnz]), shape))
@@ -595,7 +597,11 @@ def test_random_selectors_against_the_oracle(cuda, rows, monkeypatch):
                 exp = ref[sel]
             except Exception:
                 continue                          # rejected by the oracle, as by the reference
-            got = dok[dsel]
+            try:
+                got = dok[dsel]
+            except NotImplementedError as err:    # (an index space of more axes than a descriptor holds)
+                assert "axes" in str(err) and len(shape) >= 6
+                continue
             assert got.shape == exp.shape and torch.equal(got.cpu(), exp), (shape, sel)
             val = float(rng.integers(-50, 50))
             try:
