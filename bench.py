@@ -33,37 +33,37 @@ HBM_PEAK_GBS = 8000.0
 # csrc_sha16()): when the sources have changed since, nothing measured is reported.
 # PROFILED-BEGIN
 PROFILED = {
-    "csrc_sha16": "678f2bfc273c2769",
+    "csrc_sha16": "b1aa32e3f1b8762c",
     "bytes": {
-        "get_lf05": 6.653e+09,
-        "line_gather_lf05": 8.878e+09,
+        "get_lf05": 6.656e+09,
+        "line_gather_lf05": 8.877e+09,
         "set_cas_lf05": 1.599e+10,
-        "set_bulk_lf05": 7.691e+09,
-        "build_lf05": 5.973e+09,
+        "set_bulk_lf05": 7.692e+09,
+        "build_lf05": 5.972e+09,
         "overwrite_cas_lf05": 1.177e+10,
         "remove_lf05": 5.688e+09,
         "remove_cas_lf05": 6.769e+09,
-        "remove_bulk_lf05": 3.561e+09,
-        "get_lf09": 7.133e+09,
+        "remove_bulk_lf05": 3.563e+09,
+        "get_lf09": 7.065e+09,
         "set_cas_lf09": 1.923e+10,
-        "set_bulk_lf09": 6.143e+09,
-        "build_lf09": 5.191e+09,
-        "cfg1_set_65536": 1.639e+07,
-        "cfg1_get_131072": 1.354e+07,
-        "cfg1_remove_32768": 5.188e+06,
-        "cfg2_set_1M_f32x3_i64x5": 4.808e+08,
-        "cfg2_upsert_1M": 5.447e+08,
-        "cfg2_get_2M": 3.72e+08,
+        "set_bulk_lf09": 6.149e+09,
+        "build_lf09": 5.187e+09,
+        "cfg1_set_65536": 1.638e+07,
+        "cfg1_get_131072": 1.355e+07,
+        "cfg1_remove_32768": 5.206e+06,
+        "cfg2_set_1M_f32x3_i64x5": 4.804e+08,
+        "cfg2_upsert_1M": 5.523e+08,
+        "cfg2_get_2M": 3.721e+08,
         "cfg2_remove_250K": 4.348e+07,
-        "cfg4_construct_50M": 4.416e+09,
-        "cfg4_getitem_4096x256": 1.408e+08,
-        "cfg4_setitem_10M_with_growth": 7.353e+09,
-        "cfg4_setitem_10M_overwrite": 1.979e+09,
+        "cfg4_construct_50M": 4.415e+09,
+        "cfg4_getitem_4096x256": 1.406e+08,
+        "cfg4_setitem_10M_with_growth": 7.215e+09,
+        "cfg4_setitem_10M_overwrite": 1.865e+09,
         "cfg4_readout": 4.207e+09,
-        "cfg5_construct_100M": 1.071e+10,
-        "cfg5_64_getitems": 1.075e+09,
-        "cfg5_remove_20M": 4.722e+09,
-        "cfg5_reinsert_20M": 4.394e+09,
+        "cfg5_construct_100M": 1.07e+10,
+        "cfg5_64_getitems": 1.06e+09,
+        "cfg5_remove_20M": 4.723e+09,
+        "cfg5_reinsert_20M": 4.398e+09,
         "tagged_set_lf05": 1.184e+10,
         "tagged_build_lf05": 1.492e+10,
         "tagged_overwrite_lf05": 1.165e+10,
@@ -74,13 +74,13 @@ PROFILED = {
         "tagged_overwrite_lf075": 1.362e+10,
         "tagged_get_lf075": 6.433e+09,
         "tagged_remove_lf075": 1.682e+09,
-        "dok_getitem_2p26": 1.084e+10,
-        "dok_setitem_10M": 2.346e+09,
-        "dok_setitem_10M_overwrite": 1.979e+09,
+        "dok_getitem_2p26": 1.161e+10,
+        "dok_setitem_10M": 2.192e+09,
+        "dok_setitem_10M_overwrite": 1.865e+09,
         "dok_readout": 4.25e+09,
-        "dok_lin_construct_10M": 9.887e+08,
-        "dok_lin_getitem_4M": 6.294e+08,
-        "dok_lin_setitem_4M": 9.837e+08,
+        "dok_lin_construct_10M": 9.79e+08,
+        "dok_lin_getitem_4M": 6.519e+08,
+        "dok_lin_setitem_4M": 8.995e+08,
         "dok_wide_construct_10M": 3.174e+09,
         "dok_wide_getitem_4M": 6.207e+08,
         "dok_wide_setitem_4M": 9.101e+08,
