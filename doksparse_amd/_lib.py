@@ -81,6 +81,7 @@ SIGNATURES = {
     "dok_map_remove_unique": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p]),
     "dok_map_remove_bulk": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "dok_map_count_existing": (c_int32, [POINTER(DokTable), c_void_p, c_int64, c_void_p, c_void_p]),
+    "dok_map_update_existing": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "dok_compact_scratch_bytes": (c_int64, [POINTER(DokTable)]),
     "dok_map_compact": (c_int32, [POINTER(DokTable), c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "dok_static_scratch_bytes": (c_int64, []),

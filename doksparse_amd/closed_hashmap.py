@@ -179,7 +179,7 @@ class _TableState:
 _SHARED = ("_table", "_header", "_desc", "_n_phys", "_slots_per_bucket", "_layout", "_n_buckets",
            "_key_shape", "_key_dtype", "_value_shape", "_value_dtype", "_key_bytes", "_value_bytes",
            "_n_upper", "_n_exact", "_seed", "_pending_clear",
-           "_rows", "_rows_used", "_row_shape", "_row_dtype")
+           "_rows", "_rows_used", "_row_shape", "_row_dtype", "_miss_counter", "_miss_seen")
 
 
 def _forward(name):
@@ -260,6 +260,10 @@ class CudaClosedHashmap:
         # True only inside set()/set_coo(), between the allocation of the table and its first
         # insert: the bucket memory is still uninitialised (a bulk build writes all of it)
         self._pending_clear = False
+        # device counter that _update_existing adds to (never reset: the host keeps the last value
+        # it read, which saves a fill launch per call)
+        self._miss_counter = None
+        self._miss_seen = 0
         # value rows kept outside the table (see _OutOfLineValuesMap); unused by this class
         self._rows = None
         self._rows_used = 0
@@ -666,8 +670,14 @@ class CudaClosedHashmap:
             return
         # the batch may not fit.  Rows that miss bound the distinct new keys from above; if even
         # that bound stays under the threshold nothing can grow and no sort is needed
-        # (counted by a kernel that writes one number: no value rows, no flags)
-        n_miss = n - int(self.count_existing(keys).item())
+        # (counted by a kernel that writes one number: no value rows, no flags).  On the packed
+        # layout the counting kernel also overwrites the values of the keys it finds, so a batch
+        # that only updates present keys - the usual case in a table this full - is done with it
+        n_miss = self._update_existing(keys, values)
+        if n_miss == 0:
+            return                            # every key was present and holds its new value
+        if n_miss < 0:
+            n_miss = n - int(self.count_existing(keys).item())
         if n_old + n_miss <= limit:
             self._launch_checked(lambda: self._launch_set(keys, values), n_miss)
             if n_miss == 0:
@@ -852,6 +862,22 @@ class CudaClosedHashmap:
                       is_removed.data_ptr(), _stream_ptr(self.device)), "remove")
         return is_removed
 
+    def _update_existing(self, keys, values):
+        """Overwrite the values of the rows of an upsert batch whose keys are present; returns the
+        number of rows whose key is absent (nothing is inserted), or -1 where the layout has no
+        such kernel.  The entry count cannot change."""
+        if self._layout != _lib.DOK_LAYOUT_PACKED8:
+            return -1
+        if self._miss_counter is None:
+            self._miss_counter = torch.zeros((), device=self.device, dtype=torch.long)
+            self._miss_seen = 0
+        _lib.check(_lib.load().dok_map_update_existing(ctypes.byref(self._desc), keys.data_ptr(), values.data_ptr(),
+                                                       keys.shape[0], self._miss_counter.data_ptr(),
+                                                       _stream_ptr(self.device)), "set")
+        total = int(self._miss_counter.item())
+        n_miss, self._miss_seen = total - self._miss_seen, total
+        return n_miss
+
     def count_existing(self, keys):
         """How many rows of ``keys`` are present (device int64 scalar)."""
         if not self._allocated:
@@ -970,6 +996,7 @@ class CudaClosedHashmap:
             setattr(new, name, getattr(self, name))
         if self._rows is not None:
             new._rows = self._rows.clone()
+        new._miss_counter, new._miss_seen = None, 0
         if self._allocated:
             new._table = self._table.clone()
             new._header = self._header.clone()

@@ -770,6 +770,38 @@ __global__ __launch_bounds__(DOK_TPB) void p8_count_kernel(DevTable t, const voi
   dok_block_add1(count, n_found);
 }
 
+// The keys of the batch that are present get their values overwritten; the others are only counted
+// (missing[0] += their number) and nothing is inserted.  A batch of nothing but present keys - the
+// usual update of a map - is then done in one pass at the rate of a lookup, with no compare-and-swap.
+// (Equal keys in the batch store into one slot, each store a whole value.)
+template <int V, int KF>
+__global__ __launch_bounds__(DOK_TPB) void p8_update_kernel(DevTable t, const void *__restrict__ keys,
+                                                            const void *__restrict__ values, i64 n, i64 *missing) {
+  int n_missing = 0;
+  DOK_TILE_LOOP(n) {
+    const i64 i = DOK_TILE_ROW();
+    const bool active = i < n;
+    u64 key = 0;
+    const bool ok = active && dok_load_key8<KF>(t, keys, i, n, key);
+    const u64 sk = key ^ DOK_P8_XOR;
+    const u64 mine = ok ? dok_load_val<V>(values, i) : 0;
+    bool found = false;
+    u64 val = 0;
+    bool pend = ok;
+    if (ok && sk < 2) {
+      found = t.header[DOK_H_SIDE_STATE + sk] != 0;
+      if (found) t.header[DOK_H_SIDE_VALUE + sk] = (i64)mine;
+      pend = false;
+    }
+    u32 sb = 0; int ss = 0, nprobe = 0;
+    const u64 h = p8_hash(sk, t);
+    p8_lookup<V, false>(t.buckets, t.nb, sk, pend ? dok_reduce(h, t.nb) : 0u, p8_fbit(h), pend, found, val, sb, ss, nprobe);
+    if (pend && found) P8<V>::store(t.buckets + (u64)sb * 16, ss, mine);
+    n_missing += active && !found;             // (a row outside the coordinate space is not present either)
+  }
+  dok_block_add1(missing, n_missing);
+}
+
 // ---- table scans: read-out, rehash, densify ------------------------------------------------
 // Each wave walks DOK_CHUNK consecutive buckets, four per step (one per 16-lane group), so the
 // live entries of a chunk are met in slot order and a per-chunk prefix sum gives every entry a

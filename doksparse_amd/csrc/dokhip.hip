@@ -607,6 +607,23 @@ int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n, in
   return note_launch();
 }
 
+int dok_map_update_existing(const dok_table_t *t, const void *keys, const void *values, int64_t n,
+                            int64_t *missing, void *stream) {
+  DevTable d; int layout;
+  int rc = make_dev_table(t, d, layout);
+  if (rc) return rc;
+  if (layout != DOK_LAYOUT_PACKED8) return DOK_EUNSUPPORTED;
+  if (n < 0 || n > kMaxRows) return DOK_EINVAL;
+  if (n == 0) return DOK_OK;
+  if (!keys || !values || !missing) return DOK_EINVAL;
+  if (((uintptr_t)values & (uintptr_t)(d.value_bytes - 1)) != 0) return DOK_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  const DeviceScope on_stream_device(s);
+  P8_DISPATCH_LIN(d.value_bytes, d.lin_ndim > 0, (p8_update_kernel<V, KF><<<grid_counting(n), DOK_TPB, 0, s>>>(
+      d, keys, values, n, (i64 *)missing)));
+  return note_launch();
+}
+
 int64_t dok_compact_scratch_bytes(const dok_table_t *t) {
   if (!t || t->n_phys_buckets < 1) return DOK_EINVAL;
   const i64 n_chunks = (t->n_phys_buckets + DOK_CHUNK - 1) / DOK_CHUNK;

@@ -224,6 +224,18 @@ int dok_map_remove_bulk(const dok_table_t *t, const void *keys, int64_t n, void 
 int dok_map_count_existing(const dok_table_t *t, const void *keys, int64_t n,
                            int64_t *count, void *stream);
 
+/* Overwrite the values of the rows whose key is present and count the others:
+ * missing[0] += number of rows whose key is absent (a device int64); nothing is inserted.
+ * What a caller runs before an upsert whose growth decision needs the number of new keys anyway
+ * (the reference's get + unique pre-pass, cuda_closed_hashmap.py:350-366): when the answer is 0 -
+ * a batch that only updates existing keys - the upsert is already done, at the rate of a lookup.
+ * Otherwise follow with dok_map_set of the whole batch (the rows already written are written
+ * again; equal keys keep one whole value either way).  Packed layout only (DOK_EUNSUPPORTED
+ * otherwise: use dok_map_count_existing).
+ * Reference: the overwrite branch of ClosedHashmap::set (closed_hashmap_impl_class.cu:383-388). */
+int dok_map_update_existing(const dok_table_t *t, const void *keys, const void *values, int64_t n,
+                            int64_t *missing, void *stream);
+
 /* ---- read-out ----------------------------------------------------------------------------- */
 
 /* Bytes of device scratch dok_map_compact needs for this table. */

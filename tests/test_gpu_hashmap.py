@@ -1013,3 +1013,49 @@ def test_keys_wider_than_a_bucket_are_refused(cuda):
     hm = CudaClosedHashmap(n_buckets=64, device=cuda)
     with pytest.raises((RuntimeError, NotImplementedError, ValueError, AssertionError)):
         hm.set(torch.zeros(4, 15, device=cuda, dtype=torch.long), torch.zeros(4, 1, device=cuda))
+
+
+@pytest.mark.parametrize("vdt", [np.float32, np.int64, np.float16])
+def test_update_existing_overwrites_present_keys_and_counts_the_rest(cuda, vdt):
+    """dok_map_update_existing through the C ABI: present keys take their new values, absent keys
+    are counted and not inserted (the two side-slot keys included); and `set` in a table too full
+    to skip the growth check: a batch of present keys only changes values and keeps the count, a
+    batch with new keys still grows the table by the reference's rule."""
+    import ctypes
+    from doksparse_amd import CudaClosedHashmap, _lib
+    from doksparse_amd.closed_hashmap import _stream_ptr
+    from oracle.ref_hashmap import RefClosedHashmap
+    rng = np.random.default_rng(5)
+    n = 20_000
+    keys = _unique_i64(rng, n)
+    keys[:2] = np.array([0x9E3779B97F4A7C15, 0x9E3779B97F4A7C14], dtype=np.uint64).view(np.int64)   # the side-slot keys
+    vals = rng.integers(-1000, 1000, size=(n, 1)).astype(vdt)
+    hm = CudaClosedHashmap(n_buckets=16_000, device=cuda)          # (threshold 12,000 entries)
+    ref = RefClosedHashmap(n_buckets=16_000)
+    half = n // 2
+    hm.set(*_to(cuda, keys[:half, None], vals[:half]))
+    ref.set(keys[:half, None], vals[:half])
+    # C ABI: rows 0 .. n-1, of which the first half is present
+    newv = rng.integers(-1000, 1000, size=(n, 1)).astype(vdt)
+    k, v = _to(cuda, keys[:, None], newv)
+    missing = torch.zeros((), device=cuda, dtype=torch.long)
+    lib = _lib.load()
+    _lib.check(lib.dok_map_update_existing(ctypes.byref(hm._desc), k.data_ptr(), v.data_ptr(), n, missing.data_ptr(),
+                                           _stream_ptr(cuda)), "update")
+    assert int(missing.item()) == n - half and hm.n_elements == half
+    ref.set(keys[:half, None], newv[:half])
+    _assert_same_map(hm, ref)
+    _check_get(hm, ref, keys[:, None], cuda)
+    # a batch of present keys in a table whose growth check cannot be skipped
+    assert hm._n_upper + half > hm._growth_limit()
+    again = rng.integers(-1000, 1000, size=(half, 1)).astype(vdt)
+    buckets_before = hm.n_buckets
+    hm.set(*_to(cuda, keys[:half, None], again))
+    ref.set(keys[:half, None], again)
+    assert hm.n_buckets == buckets_before == ref.n_buckets and hm._n_exact and hm.n_elements == half
+    _assert_same_map(hm, ref)
+    # and one with new keys among them: grows like the reference
+    hm.set(*_to(cuda, keys[:, None], newv))
+    ref.set(keys[:, None], newv)
+    assert hm.n_buckets == ref.n_buckets and hm.n_elements == ref.n_elements == n
+    _assert_same_map(hm, ref)
