@@ -33,37 +33,38 @@ HBM_PEAK_GBS = 8000.0
 # csrc_sha16()): when the sources have changed since, nothing measured is reported.
 # PROFILED-BEGIN
 PROFILED = {
-    "csrc_sha16": "b1aa32e3f1b8762c",
+    "csrc_sha16": "aa601f8a2352ca93",
     "bytes": {
-        "get_lf05": 6.656e+09,
+        "get_lf05": 6.657e+09,
         "line_gather_lf05": 8.877e+09,
         "set_cas_lf05": 1.599e+10,
-        "set_bulk_lf05": 7.692e+09,
-        "build_lf05": 5.972e+09,
+        "set_bulk_lf05": 7.69e+09,
+        "build_lf05": 5.971e+09,
         "overwrite_cas_lf05": 1.177e+10,
+        "update_existing_lf05": 1.157e+10,
         "remove_lf05": 5.688e+09,
         "remove_cas_lf05": 6.769e+09,
-        "remove_bulk_lf05": 3.563e+09,
+        "remove_bulk_lf05": 3.561e+09,
         "get_lf09": 7.065e+09,
         "set_cas_lf09": 1.923e+10,
-        "set_bulk_lf09": 6.149e+09,
-        "build_lf09": 5.187e+09,
-        "cfg1_set_65536": 1.638e+07,
-        "cfg1_get_131072": 1.355e+07,
-        "cfg1_remove_32768": 5.206e+06,
-        "cfg2_set_1M_f32x3_i64x5": 4.804e+08,
-        "cfg2_upsert_1M": 5.523e+08,
-        "cfg2_get_2M": 3.721e+08,
+        "set_bulk_lf09": 6.144e+09,
+        "build_lf09": 5.188e+09,
+        "cfg1_set_65536": 1.639e+07,
+        "cfg1_get_131072": 1.352e+07,
+        "cfg1_remove_32768": 5.211e+06,
+        "cfg2_set_1M_f32x3_i64x5": 4.802e+08,
+        "cfg2_upsert_1M": 5.45e+08,
+        "cfg2_get_2M": 3.722e+08,
         "cfg2_remove_250K": 4.348e+07,
-        "cfg4_construct_50M": 4.415e+09,
+        "cfg4_construct_50M": 4.421e+09,
         "cfg4_getitem_4096x256": 1.406e+08,
-        "cfg4_setitem_10M_with_growth": 7.215e+09,
+        "cfg4_setitem_10M_with_growth": 7.219e+09,
         "cfg4_setitem_10M_overwrite": 1.865e+09,
         "cfg4_readout": 4.207e+09,
         "cfg5_construct_100M": 1.07e+10,
         "cfg5_64_getitems": 1.06e+09,
-        "cfg5_remove_20M": 4.723e+09,
-        "cfg5_reinsert_20M": 4.398e+09,
+        "cfg5_remove_20M": 4.717e+09,
+        "cfg5_reinsert_20M": 4.396e+09,
         "tagged_set_lf05": 1.184e+10,
         "tagged_build_lf05": 1.492e+10,
         "tagged_overwrite_lf05": 1.165e+10,
@@ -78,12 +79,12 @@ PROFILED = {
         "dok_setitem_10M": 2.192e+09,
         "dok_setitem_10M_overwrite": 1.865e+09,
         "dok_readout": 4.25e+09,
-        "dok_lin_construct_10M": 9.79e+08,
-        "dok_lin_getitem_4M": 6.519e+08,
-        "dok_lin_setitem_4M": 8.995e+08,
+        "dok_lin_construct_10M": 9.805e+08,
+        "dok_lin_getitem_4M": 6.526e+08,
+        "dok_lin_setitem_4M": 8.994e+08,
         "dok_wide_construct_10M": 3.174e+09,
         "dok_wide_getitem_4M": 6.207e+08,
-        "dok_wide_setitem_4M": 9.101e+08,
+        "dok_wide_setitem_4M": 9.103e+08,
     },
 }
 # PROFILED-END
@@ -791,6 +792,17 @@ def main():
         # overwrite pass (every key present)
         o_avg, _ = time_kernel(lambda: raw_set(keys, values), 5, leg="overwrite_cas_lf05")
         results["overwrite_mops_lf05"] = round(n / o_avg / 1e3, 1)
+        # the same overwrite as `set` runs it when the table is too full to skip the growth check:
+        # one pass that overwrites present keys and counts absent ones (none here)
+        miss = torch.zeros((), device=device, dtype=torch.long)
+        def raw_update():
+            _dl.check(_dl.load().dok_map_update_existing(ctypes.byref(hm._desc), keys.data_ptr(), values.data_ptr(), n,
+                                                         miss.data_ptr(), _stream_ptr(device)), "update")
+        raw_update()
+        assert int(miss.item()) == 0
+        u_avg, _ = time_kernel(raw_update, 5, leg="update_existing_lf05")
+        results["update_existing_ms_lf05"] = round(u_avg, 4)
+        results["update_existing_mops_lf05"] = round(n / u_avg / 1e3, 1)
         # remove of a random half of the keys (the keys are in random order); the removed rows
         # are stored again outside the timed region
         half = keys[: n // 2]
@@ -935,6 +947,7 @@ def main():
                                          ("set_lf09", "set_bulk_lf09", "set_bulk_ms_lf09", n),
                                          ("build_lf09", "build_lf09", "build_ms_lf09", n),
                                          ("set_per_row_lf05", "set_cas_lf05", "set_cas_kernel_ms_lf05", n),
+                                         ("update_existing_lf05", "update_existing_lf05", "update_existing_ms_lf05", n),
                                          ("remove_lf05", "remove_lf05", "remove_ms_lf05", n // 2),
                                          ("remove_bulk_lf05", "remove_bulk_lf05", "remove_bulk_ms_lf05", n // 2)):
             ms = results.get(ms_key)
