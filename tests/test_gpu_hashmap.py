@@ -1059,3 +1059,28 @@ def test_update_existing_overwrites_present_keys_and_counts_the_rest(cuda, vdt):
     ref.set(keys[:, None], newv)
     assert hm.n_buckets == ref.n_buckets and hm.n_elements == ref.n_elements == n
     _assert_same_map(hm, ref)
+
+
+def test_update_pass_on_a_coordinate_keyed_map(cuda):
+    """The same pre-pass of `set` on a map whose keys are coordinate rows linearised by the table:
+    a batch of present coordinates in a table too full to skip the growth check only changes
+    values; one with new coordinates grows the table."""
+    from doksparse_amd import CudaClosedHashmap
+    rng = np.random.default_rng(6)
+    dims = (300, 200, 7)
+    lin = rng.permutation(int(np.prod(dims)))[:20_000]
+    rows = np.stack(np.unravel_index(lin, dims), axis=1).astype(np.int64)
+    vals = rng.standard_normal((20_000, 1)).astype(np.float32)
+    hm = CudaClosedHashmap(n_buckets=16_000, device=cuda, coord_dims=dims)
+    k, v = _to(cuda, rows, vals)
+    hm.set(k[:10_000], v[:10_000])
+    assert hm.n_elements == 10_000 and hm._n_upper + 10_000 > hm._growth_limit()
+    v2 = torch.from_numpy(rng.standard_normal((10_000, 1)).astype(np.float32)).to(cuda)
+    hm.set(k[:10_000], v2)                                   # only present coordinates
+    assert hm.n_buckets == 16_000 and hm.n_elements == 10_000 and hm._n_exact
+    got, found = hm.get(k)
+    assert bool(found[:10_000].all()) and not bool(found[10_000:].any()) and torch.equal(got[:10_000], v2)
+    hm.set(k, v)                                             # half of them new: the table grows
+    assert hm.n_elements == 20_000 and hm.n_buckets == int((10_000 + 10_000) * 2.0)
+    got, found = hm.get(k)
+    assert bool(found.all()) and torch.equal(got, v)
